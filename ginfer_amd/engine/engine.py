@@ -1,0 +1,115 @@
+"""The engine: requests in, token ids out.  Field names of the configuration are the reference's
+(ginfer/engine/config.h:8-21); `generate` and `step` follow ginfer/engine/engine.cc:93-151, without the
+tokenizer: prompts are lists of token ids and so are the results."""
+import time
+from dataclasses import dataclass
+from typing import List, Optional
+
+from ..sampling import SamplingParams, Sampler
+from .runner import ModelRunner, StepEntry
+from .scheduler import Scheduler
+from .sequence import Sequence
+
+
+@dataclass
+class EngineConfig:
+    model_path: str
+    dtype: str = "bfloat16"               # "bfloat16" or "float32" (everything in true 32-bit)
+    max_num_batched_tokens: int = 2048    # token budget of one step
+    max_num_seqs: int = 64                # requests running at a time
+    max_seq_len: int = 4096               # longest sequence (prompt + output) a request may reach
+    gpu_memory_utilization: float = 0.9   # share of the free device memory that becomes cache pages
+    kvcache_block_size: int = 16          # tokens per cache page
+    num_kvcache_blocks: Optional[int] = None   # pages per cache group; None: from free memory
+
+
+@dataclass
+class RequestOutput:
+    request_id: int
+    prompt_token_ids: List[int]
+    token_ids: List[int]
+    finish_reason: str
+    ttft: Optional[float]
+    tpot: Optional[float]
+    evictions: int
+
+
+class Engine:
+    def __init__(self, config: EngineConfig):
+        self.config = config
+        self.runner = ModelRunner(config.model_path, dtype=config.dtype, page_size=config.kvcache_block_size,
+                                  num_pages=config.num_kvcache_blocks, max_requests=config.max_num_seqs,
+                                  max_model_len=config.max_seq_len,
+                                  gpu_memory_utilization=config.gpu_memory_utilization)
+        self.scheduler = Scheduler(self.runner.cache, config.max_num_seqs, config.max_num_batched_tokens,
+                                   self.runner.spec.eos_token_ids, self.runner.max_model_len)
+        self.sampler = Sampler(self.runner.device)
+        self._next_id = 0
+        self.stats = dict(prefill_tokens=0, prefill_time=0.0, decode_tokens=0, decode_time=0.0, steps=0)
+
+    def add_request(self, prompt_token_ids, params: Optional[SamplingParams] = None):
+        params = params or SamplingParams()
+        params.validate()
+        ids = [int(t) for t in prompt_token_ids]
+        V = self.runner.vocab_size
+        if any(not 0 <= t < V for t in ids):
+            raise ValueError("prompt holds a token id outside [0, %d)" % V)
+        rid = self._next_id
+        self._next_id += 1
+        self.scheduler.add(Sequence(rid, ids, len(ids), params))
+        return rid
+
+    def has_unfinished(self):
+        return not self.scheduler.is_finished()
+
+    def step(self) -> List[RequestOutput]:
+        """One scheduled batch through the model; returns the requests that finished in it."""
+        t0 = time.perf_counter()
+        scheduled = self.scheduler.schedule()
+        entries = []
+        for sc in scheduled:
+            s = sc.seq
+            toks = s.token_ids[s.num_computed:s.num_computed + sc.num_tokens]
+            entries.append(StepEntry(s.request_id, toks, [sc.num_tokens - 1] if sc.samples else []))
+        logits = self.runner.step(entries)
+        sampling = [sc.seq for sc in scheduled if sc.samples]
+        tokens = self.sampler.sample(logits, [s.params for s in sampling],
+                                     [s.num_output_tokens for s in sampling])
+        now = time.perf_counter()
+        finished = self.scheduler.postprocess(scheduled, tokens, now)
+        dt = now - t0
+        n_prefill = sum(sc.num_tokens for sc in scheduled if sc.num_tokens > 1 or sc.seq.num_computed == sc.num_tokens)
+        n_decode = sum(sc.num_tokens for sc in scheduled) - n_prefill
+        st = self.stats
+        st["steps"] += 1
+        # a mixed step's time is shared out by tokens
+        total = max(n_prefill + n_decode, 1)
+        st["prefill_tokens"] += n_prefill
+        st["decode_tokens"] += n_decode
+        st["prefill_time"] += dt * n_prefill / total
+        st["decode_time"] += dt * n_decode / total
+        return [self._output(s) for s in finished]
+
+    @staticmethod
+    def _output(s):
+        ttft = None if s.first_token_ts is None else s.first_token_ts - s.request_ts
+        tpot = None
+        if s.finish_ts is not None and s.first_token_ts is not None and s.num_output_tokens > 1:
+            tpot = (s.finish_ts - s.first_token_ts) / (s.num_output_tokens - 1)
+        return RequestOutput(s.request_id, s.token_ids[:s.num_prompt_tokens], s.output_ids, s.finish_reason,
+                             ttft, tpot, s.evictions)
+
+    def generate(self, prompts, params=None) -> List[RequestOutput]:
+        """prompts: lists of token ids; params: one SamplingParams for all, or one per prompt.  Returns the
+        outputs in the order of the prompts."""
+        if params is None or isinstance(params, SamplingParams):
+            params = [params] * len(prompts)
+        if len(params) != len(prompts):
+            raise ValueError("%d prompts but %d sampling parameter sets" % (len(prompts), len(params)))
+        import copy
+        ids = [self.add_request(p, copy.copy(sp)) for p, sp in zip(prompts, params)]
+        done = {}
+        while self.has_unfinished():
+            for out in self.step():
+                done[out.request_id] = out
+        return [done[i] for i in ids]

@@ -1,0 +1,180 @@
+"""The scheduler: admits requests, cuts prompts into portions under a token budget, decodes,
+finishes and frees.
+
+Every step is one mixed batch.  First every running request that is decoding gets its one token;
+then what is left of the budget goes to prompt portions, first of running requests whose prompt is
+not through yet, then of waiting requests in arrival order, while fewer than max_num_seqs requests
+run and a state slot is free.  A portion is cut to what the budget and the free pages allow.  The
+reference runs prompts whole and never beside decoding (ginfer/engine/scheduler.cc:20-71); its queues,
+its finishing rule (:83-99) and its answer to a full cache are kept:
+
+When pages run out for a decoding request, the newest running request is evicted: its pages are given
+back, it keeps its tokens, returns to the FRONT of the waiting queue and is later fed again from its
+first token, prompt and output alike (recompute; ginfer/engine/scheduler.cc:47-56 and :73-77, where the
+evicted sequence goes to the back of the queue instead).  If the request that cannot grow is the only
+one running, it is evicted itself.  A request that could never fit the pool alone is refused when it
+is added, so eviction always ends.
+"""
+from collections import deque
+from dataclasses import dataclass
+from typing import List
+
+from ..cache import OutOfPages
+from .sequence import Sequence, State
+
+
+@dataclass
+class Scheduled:
+    seq: Sequence
+    num_tokens: int          # tokens of seq.token_ids[num_computed:] that run in this step
+    samples: bool            # the portion reaches the end of the known tokens: a token is sampled
+
+
+class Scheduler:
+    def __init__(self, cache, max_num_seqs, max_num_batched_tokens, eos_token_ids, max_model_len):
+        if max_num_batched_tokens < 1 or max_num_seqs < 1:
+            raise ValueError("max_num_seqs and max_num_batched_tokens must be positive")
+        self.cache = cache
+        self.max_num_seqs, self.max_num_batched_tokens = int(max_num_seqs), int(max_num_batched_tokens)
+        self.eos_token_ids = set(eos_token_ids)
+        self.max_model_len = int(max_model_len)
+        self.waiting = deque()
+        self.running: List[Sequence] = []
+        self.num_evictions = 0
+
+    # ---- requests
+    def add(self, seq):
+        total = seq.num_prompt_tokens + seq.params.max_tokens
+        if seq.num_prompt_tokens < 1:
+            raise ValueError("request %r has an empty prompt" % (seq.request_id,))
+        if seq.num_prompt_tokens + 1 > self.max_model_len:
+            raise ValueError("request %r: prompt of %d tokens leaves no room under max_model_len %d"
+                             % (seq.request_id, seq.num_prompt_tokens, self.max_model_len))
+        need = -(-min(total, self.max_model_len) // self.cache.page_size)
+        for gi, g in enumerate(self.cache.groups):
+            if g.window is None and need > g.pool.num_pages:
+                raise ValueError("request %r can grow to %d tokens (%d pages) but the cache has %d pages; "
+                                 "it could never finish" % (seq.request_id, min(total, self.max_model_len), need,
+                                                            g.pool.num_pages))
+        seq.state = State.WAITING
+        self.waiting.append(seq)
+
+    def is_finished(self):
+        return not self.waiting and not self.running
+
+    # ---- one step
+    def schedule(self) -> List[Scheduled]:
+        cache = self.cache
+        budget = self.max_num_batched_tokens
+        out: List[Scheduled] = []
+
+        # 1. decoding requests, oldest first; evict the newest when pages run out
+        decoding = [s for s in self.running if s.remaining == 1 and s.num_computed > 0]
+        i = 0
+        while i < len(decoding) and budget > 0:
+            seq = decoding[i]
+            if seq.state is not State.RUNNING:      # evicted earlier in this loop
+                i += 1
+                continue
+            try:
+                cache.append(seq.request_id, 1)
+            except OutOfPages:
+                victim = self.running[-1]
+                if any(sc.seq is victim for sc in out):
+                    # the newest already holds its reservation for this step: undo it
+                    out = [sc for sc in out if sc.seq is not victim]
+                    budget += 1
+                self._evict(victim)
+                if victim is seq:
+                    i += 1
+                continue
+            out.append(Scheduled(seq, 1, True))
+            budget -= 1
+            i += 1
+
+        # 2. prompt portions of running requests (prompts not yet through)
+        for seq in self.running:
+            if budget <= 0:
+                break
+            if seq.remaining > 1 or seq.num_computed == 0:
+                if any(sc.seq is seq for sc in out):
+                    continue
+                n = self._portion(seq, budget)
+                if n > 0:
+                    out.append(Scheduled(seq, n, n == seq.remaining))
+                    budget -= n
+
+        # 3. admissions in arrival order; no skipping ahead of the head of the queue
+        while self.waiting and budget > 0 and len(self.running) < self.max_num_seqs and cache.can_admit():
+            seq = self.waiting[0]
+            cache.admit(seq.request_id)
+            n = self._portion(seq, budget)
+            if n == 0:
+                cache.release(seq.request_id)
+                break
+            self.waiting.popleft()
+            seq.state = State.RUNNING
+            self.running.append(seq)
+            out.append(Scheduled(seq, n, n == seq.remaining))
+            budget -= n
+
+        if not out and not self.is_finished():
+            # nothing fits: only possible when running prompts hold every page among them
+            victim = self.running[-1] if self.running else None
+            if victim is None or len(self.running) == 1:
+                raise OutOfPages("no request can take a step: the cache is too small for the work in flight")
+            self._evict(victim)
+            return self.schedule()
+        return out
+
+    def _portion(self, seq, budget):
+        """Reserves the largest portion of the request's remaining tokens that budget and pages allow."""
+        n = min(seq.remaining, budget, self.cache.free_tokens(seq.request_id))
+        while n > 0:
+            try:
+                self.cache.append(seq.request_id, n)
+                return n
+            except OutOfPages:
+                n -= 1
+        return 0
+
+    def _evict(self, seq):
+        self.cache.release(seq.request_id)
+        self.running.remove(seq)
+        seq.state = State.WAITING
+        seq.num_computed = 0
+        seq.evictions += 1
+        self.num_evictions += 1
+        self.waiting.appendleft(seq)
+
+    # ---- after the step
+    def postprocess(self, scheduled: List[Scheduled], tokens: List[int], now=None) -> List[Sequence]:
+        """tokens: one sampled token for every scheduled item that samples, in order.  Appends them,
+        finishes what is done (end-of-sequence id unless ignore_eos, max_tokens, max_model_len), frees
+        their pages.  Returns the sequences that finished."""
+        finished = []
+        it = iter(tokens)
+        for sc in scheduled:
+            seq = sc.seq
+            self.cache.commit(seq.request_id) if self.cache.pending(seq.request_id) else None
+            seq.num_computed += sc.num_tokens
+            if not sc.samples:
+                continue
+            tok = int(next(it))
+            seq.token_ids.append(tok)
+            if seq.first_token_ts is None:
+                seq.first_token_ts = now
+            stops = self.eos_token_ids if seq.params.stop_token_ids is None else set(seq.params.stop_token_ids)
+            reason = None
+            if not seq.params.ignore_eos and tok in stops:
+                reason = "eos"
+            elif seq.num_output_tokens >= seq.params.max_tokens:
+                reason = "max_tokens"
+            elif seq.num_tokens >= self.max_model_len:
+                reason = "max_model_len"
+            if reason:
+                seq.state, seq.finish_reason, seq.finish_ts = State.FINISHED, reason, now
+                self.cache.release(seq.request_id)
+                self.running.remove(seq)
+                finished.append(seq)
+        return finished

@@ -1,0 +1,173 @@
+"""Compiling and loading the HIP kernels.
+
+Each source under `ginfer_amd/csrc/` becomes one shared library, built with hipcc for gfx950 and
+loaded with ctypes (the entry points are `extern "C"`; tensors cross as raw device pointers and the
+launches go to the stream the caller names).  A library is built when it is first asked for and its
+source (or common header, or flags) has changed since the last build; the build goes into
+`csrc/_build/` inside the package, or, when that folder cannot be written, into a per-user folder
+under the system's temporary directory.  There is no fallback: if a library can neither be found nor
+built, loading raises.
+"""
+import ctypes
+import hashlib
+import os
+import shutil
+import subprocess
+import sys
+import tempfile
+import threading
+import time
+
+CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "csrc")
+ARCH = "gfx950"
+# packed 32-bit float instructions are switched off for all device code
+FLAGS = ["--offload-arch=" + ARCH, "-O3", "-std=c++17", "-shared", "-fPIC",
+         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
+MODULES = ("embedding", "norm", "rope_kv", "attention_generic", "attention_decode",
+           "attention_prefill", "gemm", "gemm_skinny", "activation", "sampling")
+
+_loaded = {}
+_lock = threading.Lock()
+
+
+class KernelBuildError(RuntimeError):
+    pass
+
+
+def available_modules():
+    return [m for m in MODULES if os.path.isfile(os.path.join(CSRC, m + ".hip"))]
+
+
+def _hipcc():
+    for cand in (os.environ.get("HIPCC"), shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
+        if cand and os.path.isfile(cand):
+            return cand
+    return None
+
+
+def _digest(module):
+    h = hashlib.sha256()
+    for name in (module + ".hip", "common.cuh"):
+        with open(os.path.join(CSRC, name), "rb") as f:
+            h.update(f.read())
+    h.update(" ".join(FLAGS).encode())
+    return h.hexdigest()[:16]
+
+
+def _build_dirs():
+    dirs = [os.path.join(CSRC, "_build")]
+    tmp = os.path.join(tempfile.gettempdir(), "ginfer_amd_build_%d" % os.getuid())
+    dirs.append(tmp)
+    return dirs
+
+
+def _writable_dir():
+    for d in _build_dirs():
+        try:
+            os.makedirs(d, exist_ok=True)
+            probe = os.path.join(d, ".probe_%d" % os.getpid())
+            with open(probe, "w"):
+                pass
+            os.remove(probe)
+            return d
+        except OSError:
+            continue
+    raise KernelBuildError("no writable folder for built kernels (tried %s)" % ", ".join(_build_dirs()))
+
+
+def _find_built(module, digest):
+    for d in _build_dirs():
+        so = os.path.join(d, "lib%s.so" % module)
+        stamp = os.path.join(d, "%s.stamp" % module)
+        try:
+            with open(stamp) as f:
+                if f.read().strip() == digest and os.path.isfile(so):
+                    return so
+        except OSError:
+            pass
+    return None
+
+
+def _say(msg):
+    sys.stderr.write("[ginfer_amd] %s\n" % msg)
+    sys.stderr.flush()
+
+
+def compile_module(module, out_dir=None, quiet=False):
+    """Runs hipcc for one module; returns the library's path."""
+    hipcc = _hipcc()
+    if hipcc is None:
+        raise KernelBuildError("hipcc not found: cannot build kernel library %r" % module)
+    out_dir = out_dir or _writable_dir()
+    so = os.path.join(out_dir, "lib%s.so" % module)
+    tmp = so + ".%d.tmp" % os.getpid()
+    cmd = [hipcc] + FLAGS + ["-I", CSRC, "-o", tmp, os.path.join(CSRC, module + ".hip")]
+    env = dict(os.environ)
+    env.setdefault("HOME", tempfile.gettempdir())   # hipcc wants a home for its caches
+    t0 = time.time()
+    proc = subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, env=env, text=True)
+    # a line now and then while a long compile runs
+    out = []
+    reader = threading.Thread(target=lambda: out.append(proc.stdout.read()), daemon=True)
+    reader.start()
+    while proc.poll() is None:
+        try:
+            proc.wait(timeout=20)
+        except subprocess.TimeoutExpired:
+            if not quiet:
+                _say("still compiling %s (%.0f s)" % (module, time.time() - t0))
+    reader.join()
+    log = "".join(out)
+    if proc.returncode != 0:
+        if os.path.exists(tmp):
+            os.remove(tmp)
+        raise KernelBuildError("hipcc failed for %s:\n%s" % (module, log))
+    os.replace(tmp, so)
+    with open(os.path.join(out_dir, "%s.stamp" % module), "w") as f:
+        f.write(_digest(module))
+    return so
+
+
+def build_all(force=False, modules=None, quiet=False):
+    """Builds every module (in parallel); with force, also those already built."""
+    from concurrent.futures import ThreadPoolExecutor
+    modules = list(modules or available_modules())
+    todo = [m for m in modules if force or _find_built(m, _digest(m)) is None]
+    if not todo:
+        return
+    out_dir = _writable_dir()
+    if not quiet:
+        _say("compiling %d kernel librar%s for %s: %s" % (len(todo), "y" if len(todo) == 1 else "ies",
+                                                        ARCH, ", ".join(todo)))
+    done = []
+
+    def one(m):
+        compile_module(m, out_dir, quiet=quiet)
+        done.append(m)
+        if not quiet:
+            _say("compiled %s (%d/%d)" % (m, len(done), len(todo)))
+    workers = max(1, min(len(todo), (os.cpu_count() or 4), 8))
+    with ThreadPoolExecutor(workers) as ex:
+        list(ex.map(one, todo))
+
+
+def load(module):
+    """The ctypes library of a module, building it first if it is missing or stale."""
+    with _lock:
+        if module in _loaded:
+            return _loaded[module]
+        if not os.path.isfile(os.path.join(CSRC, module + ".hip")):
+            raise KernelBuildError("no kernel source for module %r in %s" % (module, CSRC))
+        digest = _digest(module)
+        so = _find_built(module, digest)
+        if so is None:
+            _say("kernel library %r is not built yet; compiling it for %s" % (module, ARCH))
+            so = compile_module(module)
+            _say("compiled %s" % module)
+        import torch  # noqa: F401  the HIP runtime that torch loaded is the one the library binds to
+        try:
+            lib = ctypes.CDLL(so)
+        except OSError as e:
+            raise KernelBuildError("cannot load kernel library %s: %s" % (so, e))
+        _loaded[module] = lib
+        return lib

@@ -1,0 +1,66 @@
+"""Attention over the paged cache: grouped queries, rotary positions, all keys or a window."""
+import math
+
+import torch
+
+from ..kernels import ops
+from ..weights.loader import WeightSpec
+from .base import Part, KVCacheSpec
+from .linear import linear
+from .registry import register_mixer
+
+
+@register_mixer("attention")
+class Attention(Part):
+    """q/k/v projections (one fused product over the stacked weights; results equal the three separate
+    ones of ginfer/core/layer/transformer/attention.cc:61-63), rotation of q and k and the cache write
+    (:69-72, :32-33), attention over the request's pages (:34), output projection (:80-81).
+    score scale 1/sqrt(head_dim) unless `scale` is given; `window` None attends to all earlier keys."""
+
+    def __init__(self, hidden_size, num_heads, num_kv_heads, head_dim, qkv_bias, out_bias, window, position,
+                 scale, dtype, device):
+        if num_heads % num_kv_heads:
+            raise ValueError("num_heads %d is not a multiple of num_kv_heads %d" % (num_heads, num_kv_heads))
+        if head_dim % 16 or not 0 < head_dim <= 256:
+            raise ValueError("head_dim %d is not supported: the attention kernels take multiples of 16 up to 256"
+                             % head_dim)
+        self.hidden_size, self.nh, self.nkv, self.hd = hidden_size, num_heads, num_kv_heads, head_dim
+        self.qkv_bias, self.out_bias = bool(qkv_bias), bool(out_bias)
+        self.window = int(window) if window else None
+        self.position = position
+        self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(head_dim)
+        self.dtype, self.device = dtype, device
+        self.w_qkv = self.b_qkv = self.w_o = self.b_o = None
+
+    def cache_spec(self):
+        return KVCacheSpec(self.nkv, self.hd, self.window)
+
+    def weight_specs(self):
+        H, q, kv = self.hidden_size, self.nh * self.hd, self.nkv * self.hd
+        specs = {"q_proj.weight": WeightSpec((q, H)), "k_proj.weight": WeightSpec((kv, H)),
+                 "v_proj.weight": WeightSpec((kv, H)), "o_proj.weight": WeightSpec((H, q))}
+        if self.qkv_bias:
+            specs.update({"q_proj.bias": WeightSpec((q,)), "k_proj.bias": WeightSpec((kv,)),
+                          "v_proj.bias": WeightSpec((kv,))})
+        if self.out_bias:
+            specs["o_proj.bias"] = WeightSpec((H,))
+        return specs
+
+    def bind_weights(self, t):
+        self.w_qkv = torch.cat([t["q_proj.weight"], t["k_proj.weight"], t["v_proj.weight"]], dim=0).contiguous()
+        self.b_qkv = (torch.cat([t["q_proj.bias"], t["k_proj.bias"], t["v_proj.bias"]], dim=0).contiguous()
+                      if self.qkv_bias else None)
+        self.w_o = t["o_proj.weight"]
+        self.b_o = t.get("o_proj.bias") if self.out_bias else None
+
+    def kernel_modules(self):
+        return ["rope_kv", "attention_generic", "attention_decode", "attention_prefill", "gemm", "gemm_skinny"]
+
+    def forward(self, x, step, cache):
+        qkv = linear(x, self.w_qkv, self.b_qkv)
+        cos, sin = self.position.tables()
+        ops.rope_kv_write(qkv, step.positions, cos, sin, cache.slot_mapping, cache.k_pages, cache.v_pages,
+                          self.nh, self.nkv, self.hd, write_kv=cache.owner)
+        a = ops.paged_attention(qkv, cache.k_pages, cache.v_pages, cache.block_table, step, self.nh, self.nkv,
+                                self.hd, self.scale, self.window)
+        return linear(a, self.w_o, self.b_o)

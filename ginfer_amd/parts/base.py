@@ -1,0 +1,55 @@
+"""Interfaces of the parts a model is put together from.
+
+Every part
+  * is constructed as `cls(dtype=..., device=..., **spec.params)` (a position encoding, where a mixer
+    has one, arrives already built under the parameter `position`);
+  * says which tensors it needs: `weight_specs() -> {local name: WeightSpec}`; local names are joined
+    to the part's prefix by the model, e.g. "model.layers.3.self_attn" + "." + "q_proj.weight";
+  * receives them, already on the device and in the right dtype: `bind_weights({local name: tensor})`;
+  * names the kernel libraries it launches: `kernel_modules() -> [module, ...]`.
+
+Mixer         forward(x [T, H], step, cache) -> [T, H]
+              cache_spec() -> KVCacheSpec | StateSpec | None: what one run of this mixer keeps per
+              request; `cache` in forward is the matching view (`KVView`, `StateView` or None) of the
+              schedule entry that is running.  `step` is the `StepContext` of the batch.
+FeedForward   forward(x [T, H]) -> [T, H]
+Norm          forward(residual float32 [T, H], delta [T, H] | None, rows=None) -> [R or T, H]
+              adds delta into the 32-bit residual stream and returns the normalised rows; with `rows`
+              (int32 indices) only those rows are returned and the residual is left as it is.
+Position      what the mixer's kernel needs to encode positions (for rotary kinds: `tables()`).
+Embedding     forward(token_ids int32 [T]) -> float32 [T, H] (the start of the residual stream)
+Head          forward(x [R, H]) -> float32 logits [R, V]
+Arrangement   how a layer's parts are ordered around the residual stream (see block.py).
+"""
+from dataclasses import dataclass
+from typing import Optional, Tuple
+
+import torch
+
+
+@dataclass(frozen=True)
+class KVCacheSpec:
+    """Keys and values in pages: per token, num_kv_heads * head_dim of each.  window: None keeps all
+    keys; an integer w keeps only what queries can still see (positions > p - w)."""
+    num_kv_heads: int
+    head_dim: int
+    window: Optional[int] = None
+
+
+@dataclass(frozen=True)
+class StateSpec:
+    """State of fixed size per request: one tensor of `shape` and `dtype` in a slot."""
+    shape: Tuple[int, ...]
+    dtype: torch.dtype = torch.float32
+
+
+class Part:
+    def weight_specs(self):
+        return {}
+
+    def bind_weights(self, tensors):
+        if tensors:
+            raise ValueError("%s takes no weights, got %s" % (type(self).__name__, sorted(tensors)))
+
+    def kernel_modules(self):
+        return []

@@ -1,0 +1,25 @@
+"""How a layer's parts are arranged around the residual stream."""
+from .registry import register_arrangement
+
+
+@register_arrangement("prenorm")
+class PreNormBlock:
+    """n = norm1(x); h = x + mixer(n); n = norm2(h); x = h + feed_forward(n)
+    (ginfer/core/layer/transformer/encoder.cc:33-39).  The residual stream is kept in 32-bit and every add
+    is fused into the norm that follows it, so a block takes the previous block's output as a pending
+    `delta` and returns its own feed-forward output as the next one."""
+
+    def __init__(self, mixer, feed_forward, mixer_norm, feed_forward_norm):
+        self.mixer, self.feed_forward = mixer, feed_forward
+        self.mixer_norm, self.feed_forward_norm = mixer_norm, feed_forward_norm
+
+    def parts(self):
+        """(role, part): the roles are the keys of `LayerSpec.names`, which gives each its tensor prefix."""
+        return [("mixer", self.mixer), ("feed_forward", self.feed_forward), ("mixer_norm", self.mixer_norm),
+                ("feed_forward_norm", self.feed_forward_norm)]
+
+    def forward(self, residual, delta, step, cache):
+        n = self.mixer_norm.forward(residual, delta)
+        a = self.mixer.forward(n, step, cache)
+        n = self.feed_forward_norm.forward(residual, a)
+        return self.feed_forward.forward(n)

@@ -1,0 +1,26 @@
+"""Next tokens from logits, on the device."""
+import numpy as np
+import torch
+
+from ..kernels import ops
+from .rng import uniform
+
+
+class Sampler:
+    def __init__(self, device):
+        self.device = device
+
+    def sample(self, logits, params, output_positions):
+        """logits float32 [R, V]; params: R SamplingParams; output_positions: which output token of its
+        request each row decides (indexes the request's random stream).  Returns a list of R ints."""
+        R = logits.shape[0]
+        if R == 0:
+            return []
+        if all(p.temperature <= 0 for p in params):
+            out = ops.sample_rows(logits)
+        else:
+            temp = torch.tensor([float(p.temperature) for p in params], dtype=torch.float32, device=self.device)
+            uni = torch.tensor(np.asarray([uniform(p.seed, n) for p, n in zip(params, output_positions)],
+                                          dtype=np.float32), device=self.device)
+            out = ops.sample_rows(logits, temp, uni)
+        return out.cpu().tolist()

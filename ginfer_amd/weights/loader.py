@@ -1,0 +1,84 @@
+"""Binding weights to a model by tensor name.
+
+The model says which tensors it expects (`model.weight_specs()`: full name -> `WeightSpec`); the
+file says which it holds.  Every disagreement (missing, unexpected, wrong shape, wrong kind of
+dtype) is collected and raised as ONE error.  Floating tensors are kept in the compute dtype
+(bfloat16 or float32); integer tables become int32; a tensor whose spec says `keep_32bit` stays in
+32-bit when the file stores it so.  The reference binds the same names without checking shapes
+(ginfer/model/qwen2.cc:34-46, ginfer/model/loader/safetensor_loader.cc:44-81).
+"""
+from dataclasses import dataclass
+from typing import Tuple
+
+import torch
+
+from .safetensors_file import open_model_files
+
+
+@dataclass
+class WeightSpec:
+    shape: Tuple[int, ...]
+    kind: str = "float"          # "float" or "int"
+    init: str = "normal"         # "normal" N(0, std), "one_plus_normal" 1 + N(0, std), "zeros", "ones"
+    std: float = 0.02
+    keep_32bit: bool = False     # a tensor stored in 32-bit stays in 32-bit
+
+
+class WeightError(ValueError):
+    pass
+
+
+def check_against(specs, available, where):
+    """specs: name -> WeightSpec; available: name -> (dtype, shape).  Raises one WeightError that
+    lists everything that is wrong, or returns."""
+    missing = [n for n in specs if n not in available]
+    unexpected = [n for n in available if n not in specs]
+    wrong = []
+    for n, s in specs.items():
+        if n not in available:
+            continue
+        dtype, shape = available[n]
+        if tuple(shape) != tuple(s.shape):
+            wrong.append("%s: expected shape %s, found %s" % (n, list(s.shape), list(shape)))
+        elif s.kind == "float" and not dtype.is_floating_point:
+            wrong.append("%s: expected a floating tensor, found %s" % (n, dtype))
+        elif s.kind == "int" and (dtype.is_floating_point or dtype == torch.bool):
+            wrong.append("%s: expected an integer tensor, found %s" % (n, dtype))
+    if not (missing or unexpected or wrong):
+        return
+    lines = ["weights in %s do not match the model:" % where]
+    if missing:
+        lines.append("  missing tensors (%d): %s" % (len(missing), ", ".join(sorted(missing))))
+    if unexpected:
+        lines.append("  unexpected tensors (%d): %s" % (len(unexpected), ", ".join(sorted(unexpected))))
+    if wrong:
+        lines.append("  wrong tensors (%d):" % len(wrong))
+        lines.extend("    " + w for w in wrong)
+    err = WeightError("\n".join(lines))
+    err.missing, err.unexpected, err.wrong = sorted(missing), sorted(unexpected), wrong
+    raise err
+
+
+def target_dtype(spec, stored_dtype, compute_dtype):
+    if spec.kind == "int":
+        return torch.int32
+    if spec.keep_32bit and stored_dtype == torch.float32:
+        return torch.float32
+    return compute_dtype
+
+
+def load_weights(model, folder, device):
+    """Reads every tensor the model expects from `folder`, converts, uploads, and hands the
+    dictionary to `model.bind_weights`."""
+    specs = model.weight_specs()
+    files = open_model_files(folder)
+    available = {n: f.info(n) for n, f in files.items()}
+    check_against(specs, available, folder)
+    tensors = {}
+    for name, spec in specs.items():
+        cpu = files[name].tensor(name)
+        dt = target_dtype(spec, cpu.dtype, model.dtype)
+        # upload in the stored dtype, convert on the device: no host copy of a large checkpoint
+        tensors[name] = cpu.to(device=device).to(dt).contiguous()
+    model.bind_weights(tensors)
+    return model

@@ -1,0 +1,58 @@
+"""Random-weights mode: a model folder (config.json, model.safetensors) from a configuration and
+a seed.  The reference has no such mode (it loads checkpoints only, ginfer/model/qwen2.cc:28-49).
+
+Matrices, embeddings and biases are drawn from N(0, std); norm gains from 1 + N(0, std), as each
+part's `WeightSpec.init` says.  Every tensor has a generator of its own, seeded by the seed and the
+tensor's name, so a tensor's values do not depend on which other tensors the model has.
+"""
+import hashlib
+import json
+import os
+
+import torch
+
+from .safetensors_file import write_safetensors
+
+_STORAGE = {"bfloat16": torch.bfloat16, "float32": torch.float32, "float16": torch.float16}
+
+
+def _tensor_seed(seed, name):
+    h = hashlib.sha256(("%d:%s" % (seed, name)).encode()).digest()
+    return int.from_bytes(h[:8], "little") & ((1 << 63) - 1)
+
+
+def draw(spec, seed, name, dtype):
+    g = torch.Generator(device="cpu")
+    g.manual_seed(_tensor_seed(seed, name))
+    if spec.kind == "int":
+        return torch.zeros(spec.shape, dtype=torch.int32)
+    if spec.init == "zeros":
+        t = torch.zeros(spec.shape, dtype=torch.float32)
+    elif spec.init == "ones":
+        t = torch.ones(spec.shape, dtype=torch.float32)
+    else:
+        t = torch.empty(spec.shape, dtype=torch.float32).normal_(0.0, spec.std, generator=g)
+        if spec.init == "one_plus_normal":
+            t += 1.0
+        elif spec.init != "normal":
+            raise ValueError("unknown init %r for %s" % (spec.init, name))
+    return t.to(dtype)
+
+
+def write_random_model(folder, config, seed, dtype="bfloat16"):
+    """Writes `folder/config.json` and `folder/model.safetensors`; returns the folder."""
+    from ..parts.model import build_model
+    if dtype not in _STORAGE:
+        raise ValueError("dtype must be one of %s" % sorted(_STORAGE))
+    os.makedirs(folder, exist_ok=True)
+    d = config.to_dict()
+    d["torch_dtype"] = dtype
+    with open(os.path.join(folder, "config.json"), "w") as f:
+        json.dump(d, f, indent=1, sort_keys=True)
+    model = build_model(config.model_spec(), _STORAGE[dtype], device=None)
+    tensors = {}
+    for name, spec in model.weight_specs().items():
+        tensors[name] = draw(spec, seed, name, _STORAGE[dtype])
+    write_safetensors(os.path.join(folder, "model.safetensors"), tensors,
+                      metadata={"format": "pt", "seed": seed})
+    return folder
