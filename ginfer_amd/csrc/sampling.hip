@@ -36,8 +36,11 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(
     if (tid < s) {
       const float a = part_f[tid], b = part_f[tid + s];
       const int ai = part_i[tid], bi = part_i[tid + s];
-      // lower half holds lower indices: take the upper only if strictly greater (or lower is empty)
-      if (bi != 0x7fffffff && (ai == 0x7fffffff || b > a)) { part_f[tid] = b; part_i[tid] = bi; }
+      // among equal values the lower index wins (the two halves interleave index ranges)
+      if (bi != 0x7fffffff && (ai == 0x7fffffff || b > a || (b == a && bi < ai))) {
+        part_f[tid] = b;
+        part_i[tid] = bi;
+      }
     }
     __syncthreads();
   }

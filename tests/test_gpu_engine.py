@@ -1,0 +1,155 @@
+"""The engine against the plain implementation, on the GPU: every way of cutting and batching, in
+32-bit and in bfloat16, at three tiny configurations."""
+import numpy as np
+import pytest
+import torch
+
+import helpers as H
+import plain_model as pm
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    out = {}
+    for name, (cfg, seed, _) in H.TINY.items():
+        out[name] = H.make_model_folder(tmp_path_factory.mktemp("tiny" + name), cfg, seed, "float32")
+    return out
+
+
+def _requests(name, lengths, seed=10):
+    vocab = H.TINY[name][0]["vocab_size"]
+    return {"r%d" % i: H.random_tokens(n, vocab, seed + i) for i, n in enumerate(lengths)}
+
+
+def _runner(folder, name, dtype, pages, max_requests=8):
+    from ginfer_amd import ModelRunner
+    return ModelRunner(folder, dtype=dtype, page_size=H.TINY[name][2], num_pages=pages, max_requests=max_requests)
+
+
+LENGTHS = {"A": [5, 17, 33, 70, 131], "B": [1, 9, 40, 64, 100, 150], "C": [3, 50, 97, 160]}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_whole_last_decoded_and_portions(folders, name, dtype):
+    reqs = _requests(name, LENGTHS[name])
+    ps = H.TINY[name][2]
+    runner = _runner(folders[name], name, dtype, pages=-(-256 // ps))
+    results = {}
+    for what, steps in (("whole", H.steps_whole(reqs)), ("last 32 decoded", H.steps_last_decoded(reqs)),
+                        ("portions", H.steps_portions(reqs))):
+        got = H.run_steps(runner, steps)
+        runner.cache.check()
+        assert not runner.cache.requests
+        H.compare_with_plain(got, reqs, folders[name], H.TOL[dtype], "%s %s %s" % (name, dtype, what))
+        results[what] = got
+    if dtype == "float32":
+        # in 32-bit every reduction has a fixed order: the cuttings agree to the last bit
+        for what in ("last 32 decoded", "portions"):
+            for key, row in results["whole"].items():
+                assert np.array_equal(row, results[what][key]), "%s: %r differs in bits from whole" % (what, key)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_mixed_with_pages_used_again(folders, name, dtype):
+    lengths = {"A": [40, 75, 110, 33, 90, 61, 130], "B": [9, 100, 64, 31, 150, 77, 18], "C": [60, 97, 140, 45, 120, 80]}
+    reqs = _requests(name, lengths[name], seed=40)
+    steps = H.steps_mixed(reqs, max_live=4, seed=3)
+    assert any(len(s["entries"]) > 1 and any(len(e["tokens"]) == 1 for e in s["entries"])
+               and any(len(e["tokens"]) > 1 for e in s["entries"]) for s in steps)
+    ps = H.TINY[name][2]
+    pages = -(-H.max_live_tokens(steps) // ps)
+    assert pages * ps < sum(len(v) for v in reqs.values()), "the pool is not small enough to reuse pages"
+    runner = _runner(folders[name], name, dtype, pages=pages)
+    got = H.run_steps(runner, steps)
+    runner.cache.check()
+    H.compare_with_plain(got, reqs, folders[name], H.TOL[dtype], "%s %s mixed" % (name, dtype))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_program(folders, tmp_path, dtype):
+    """bin/trace_run as a user runs it: whole, then mixed with few pages, in one process."""
+    name = "B"
+    reqs = _requests(name, [70, 33, 120, 64, 90], seed=70)
+    whole = H.steps_whole(reqs)
+    mixed = H.steps_mixed({k + "m": v for k, v in reqs.items()}, max_live=4, seed=5)
+    steps = whole + mixed
+    got = H.run_trace(folders[name], dtype, steps, tmp_path / "out", H.max_live_tokens(steps), page_size=H.TINY[name][2])
+    both = dict(reqs)
+    both.update({k + "m": v for k, v in reqs.items()})
+    H.compare_with_plain(got, both, folders[name], H.TOL[dtype], "trace_run %s" % dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding(folders, dtype):
+    """Three hundred tokens one by one after a short prompt, across many page edges."""
+    name = "B"
+    reqs = _requests(name, [330], seed=90)
+    steps = H.steps_last_decoded(reqs, last=320)
+    runner = _runner(folders[name], name, dtype, pages=48)
+    got = H.run_steps(runner, steps)
+    H.compare_with_plain(got, reqs, folders[name], H.TOL[dtype], "long decoding %s" % dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "C"])
+def test_first_tokens(folders, name, dtype):
+    """The first tokens of a sequence, one at a time from position 0."""
+    reqs = _requests(name, [6], seed=95)
+    runner = _runner(folders[name], name, dtype, pages=8)
+    got = H.run_steps(runner, H.steps_last_decoded(reqs, last=6))
+    H.compare_with_plain(got, reqs, folders[name], H.TOL[dtype], "first tokens")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_greedy_generation_through_the_entry_point(folders, dtype):
+    from ginfer_amd import Engine, EngineConfig, SamplingParams
+    name = "B"
+    folder = folders[name]
+    vocab = H.TINY[name][0]["vocab_size"]
+    prompts = [H.random_tokens(n, vocab, 200 + n) for n in (1, 9, 40, 64, 100)]
+    eng = Engine(EngineConfig(model_path=folder, dtype=dtype, max_num_batched_tokens=24, max_num_seqs=4,
+                              max_seq_len=256, kvcache_block_size=8, num_kvcache_blocks=40))
+    outs = eng.generate(prompts, SamplingParams(max_tokens=12, ignore_eos=True))
+    eng.runner.cache.check()
+    assert not eng.runner.cache.requests
+    cfg, w = pm.read_config(folder), pm.read_weights(folder)
+    for p, o in zip(prompts, outs):
+        assert o.prompt_token_ids == p and len(o.token_ids) == 12 and o.finish_reason == "max_tokens"
+        # every generated token is the plain implementation's greedy choice given the engine's own
+        # prefix, unless the plain top two are within rounding of each other
+        ids = p + o.token_ids
+        logits = pm.forward(cfg, w, ids[:-1])
+        for k, tok in enumerate(o.token_ids):
+            row = logits[len(p) - 1 + k]
+            best = int(torch.argmax(row))
+            if tok != best:
+                gap = float(row[best] - row[tok]) / float(row.abs().max())
+                assert gap <= H.TOL[dtype], "token %d of prompt %d: engine %d, plain %d, gap %.3g" % (k, len(p), tok, best, gap)
+
+
+def test_temperature_sampling_matches_plain_with_same_uniforms(folders):
+    from ginfer_amd import Engine, EngineConfig, SamplingParams
+    from ginfer_amd.sampling import uniform
+    name = "B"
+    folder = folders[name]
+    vocab = H.TINY[name][0]["vocab_size"]
+    prompts = [H.random_tokens(n, vocab, 300 + n) for n in (1, 9, 40, 64, 100)]
+    eng = Engine(EngineConfig(model_path=folder, dtype="float32", max_num_batched_tokens=24, max_num_seqs=5,
+                              max_seq_len=256, kvcache_block_size=8, num_kvcache_blocks=60))
+    params = [SamplingParams(max_tokens=12, temperature=0.8, seed=7 + i, ignore_eos=True) for i in range(5)]
+    outs = eng.generate(prompts, params)
+    cfg, w = pm.read_config(folder), pm.read_weights(folder)
+    agree = total = 0
+    for p, sp, o in zip(prompts, params, outs):
+        ids = p + o.token_ids
+        logits = pm.forward(cfg, w, ids[:-1])
+        for k, tok in enumerate(o.token_ids):
+            total += 1
+            agree += int(pm.sample_token(logits[len(p) - 1 + k], 0.8, uniform(sp.seed, k)) == tok)
+    # the inverse CDF is a step function of the uniform number; only a draw within rounding of a step may differ
+    assert agree >= total - 1, "%d of %d sampled tokens agree with the plain sampler" % (agree, total)
+    assert len({tuple(o.token_ids) for o in outs}) > 1

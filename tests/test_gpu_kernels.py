@@ -1,0 +1,309 @@
+"""Each kernel alone against a plain PyTorch 32-bit statement of the same operation, at sizes other
+than the engine tests' (shapes taken from the reference's own kernel tests where it has them,
+python/test/test_op.py and python/test/test_page_attn.py)."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import plain_model as pm
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [(torch.float32, 1e-5), (torch.bfloat16, 1e-2)]   # the reference's tolerances for these dtypes
+
+
+def dev():
+    return torch.device("cuda:0")
+
+
+def rnd(shape, dtype, seed, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * scale).to(dtype).to(dev())
+
+
+def close(got, ref, tol):
+    got, ref = got.float().cpu(), ref.float().cpu()
+    assert torch.isfinite(got).all()
+    err = (got - ref).abs().max().item() / max(ref.abs().max().item(), 1e-30)
+    assert err <= tol, "error %.3g > %.3g" % (err, tol)
+
+
+@pytest.mark.parametrize("dtype,tol", DTYPES)
+@pytest.mark.parametrize("T,V,H", [(32, 1000, 128), (64, 5000, 256), (127, 10000, 510), (3, 77, 88)])
+def test_embedding(dtype, tol, T, V, H):
+    from ginfer_amd.kernels import ops
+    table = rnd((V, H), dtype, 1)
+    ids = torch.randint(0, V, (T,), dtype=torch.int32, device=dev())
+    ids[0], ids[-1] = V - 1, 0
+    out = ops.embedding_gather(table, ids)
+    assert out.dtype == torch.float32
+    assert torch.equal(out, table[ids.long()].float())
+
+
+@pytest.mark.parametrize("dtype,tol", DTYPES)
+@pytest.mark.parametrize("T,H,eps", [(3 * 127, 128, 1e-5), (5, 1536, 1e-6), (17, 88, 3e-6), (2, 8192, 1e-6)])
+def test_add_rmsnorm(dtype, tol, T, H, eps):
+    from ginfer_amd.kernels import ops
+    res = rnd((T, H), torch.float32, 2)
+    delta = rnd((T, H), dtype, 3)
+    gain = (1 + 0.1 * rnd((H,), torch.float32, 4)).to(dtype)
+    h = res.double() + delta.double()
+    ref = pm.rms_norm(h, gain.double(), eps)
+    res_in = res.clone()
+    out = ops.add_rmsnorm(res_in, delta, gain, eps, dtype)
+    close(out, ref, tol)
+    close(res_in, h, 1e-6)                                  # the residual stream took the add, in 32-bit
+    # without delta: plain norm, residual untouched
+    res2 = res.clone()
+    out = ops.add_rmsnorm(res2, None, gain, eps, dtype)
+    close(out, pm.rms_norm(res.double(), gain.double(), eps), tol)
+    assert torch.equal(res2, res)
+    # with rows: gathers, may name a row twice, leaves the residual alone
+    rows = torch.tensor([T - 1, 0, T - 1], dtype=torch.int32, device=dev())
+    res3 = res.clone()
+    out = ops.add_rmsnorm(res3, delta, gain, eps, dtype, rows=rows)
+    close(out, ref[rows.long()], tol)
+    assert torch.equal(res3, res)
+    # a 32-bit gain beside bfloat16 activations
+    if dtype == torch.bfloat16:
+        out = ops.add_rmsnorm(res.clone(), delta, gain.float(), eps, dtype)
+        close(out, ref, tol)
+
+
+@pytest.mark.parametrize("dtype,tol", DTYPES)
+@pytest.mark.parametrize("T,I", [(4 * 128, 256), (2 * 511, 1024), (1023, 2048), (3, 136), (1, 8960)])
+def test_silu_mul(dtype, tol, T, I):
+    from ginfer_amd.kernels import ops
+    gu = rnd((T, 2 * I), dtype, 5, scale=3.0)
+    ref = torch.nn.functional.silu(gu[:, :I].double()) * gu[:, I:].double()
+    close(ops.silu_mul(gu), ref, tol)
+    edge = torch.tensor([[0.0, 50.0, -50.0, 1.0, 2.0, 3.0]], dtype=dtype, device=dev())
+    out = ops.silu_mul(edge).float().cpu()
+    assert out[0, 0] == 0 and abs(out[0, 1] - 100.0) < 1 and abs(out[0, 2]) < 1e-6
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 5e-5), (torch.bfloat16, 1e-2)])
+@pytest.mark.parametrize("M,N,K,bias", [(2, 8, 9, True), (1031, 2000, 408, False), (512, 1024, 256, True),
+                                        (130, 1001, 1000, True), (1, 1000, 128, True), (1, 197, 4216, False),
+                                        (64, 64, 16, False), (65, 63, 17, True)])
+def test_gemm_nt(dtype, tol, M, N, K, bias):
+    from ginfer_amd.kernels import ops
+    a, w = rnd((M, K), dtype, 6), rnd((N, K), dtype, 7)
+    b = rnd((N,), dtype, 8) if bias else None
+    ref = a.double() @ w.double().t() + (b.double() if bias else 0)
+    close(ops.gemm_nt(a, w, b), ref, tol)
+    if dtype == torch.bfloat16:
+        out = ops.gemm_nt(a, w, b, out_dtype=torch.float32)
+        assert out.dtype == torch.float32
+        close(out, ref, 1e-5)
+
+
+def test_gemm_nt_rows_do_not_depend_on_the_batch():
+    """A row of the 32-bit product has the same bits alone and inside a larger product."""
+    from ginfer_amd.kernels import ops
+    a, w, b = rnd((200, 333), torch.float32, 9), rnd((129, 333), torch.float32, 10), rnd((129,), torch.float32, 11)
+    full = ops.gemm_nt(a, w, b)
+    for r in (0, 63, 64, 199):
+        assert torch.equal(ops.gemm_nt(a[r:r + 1].contiguous(), w, b)[0], full[r])
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-4), (torch.bfloat16, 1e-2)])
+@pytest.mark.parametrize("T,nh,nkv,hd,rd,theta", [(128, 32, 8, 128, 128, 1e4), (64, 12, 12, 64, 64, 1e4),
+                                                  (9, 6, 3, 48, 48, 5e5), (5, 4, 2, 32, 16, 1e6)])
+def test_rope_and_cache_write(dtype, tol, T, nh, nkv, hd, rd, theta):
+    from ginfer_amd.kernels import ops
+    ps, pages = 8, 64
+    qkv = rnd((T, (nh + 2 * nkv) * hd), dtype, 12)
+    positions = torch.randint(0, 300, (T,), dtype=torch.int32, device=dev())
+    positions[0] = 0
+    sin, cos = pm.rope_tables(theta, rd, 300)
+    slots = torch.randperm(pages * ps)[:T].to(torch.int64)
+    slots[1] = -1 if T > 1 else slots[1]
+    kp = rnd((pages, nkv, ps, hd), dtype, 13)
+    vp = rnd((pages, nkv, ps, hd), dtype, 14)
+    kp0, vp0 = kp.clone(), vp.clone()
+    x = qkv.clone()
+    ops.rope_kv_write(x, positions, cos.to(dev()), sin.to(dev()), slots.to(dev()), kp, vp, nh, nkv, hd)
+    q = qkv[:, :nh * hd].double().cpu().view(T, nh, hd)
+    k = qkv[:, nh * hd:(nh + nkv) * hd].double().cpu().view(T, nkv, hd)
+    v = qkv[:, (nh + nkv) * hd:].cpu().view(T, nkv, hd)
+    qr = pm.apply_rope(q, positions.cpu().tolist(), sin.double(), cos.double())
+    kr = pm.apply_rope(k, positions.cpu().tolist(), sin.double(), cos.double())
+    close(x[:, :nh * hd], qr.reshape(T, -1), tol)
+    close(x[:, nh * hd:(nh + nkv) * hd], kr.reshape(T, -1), tol)
+    assert torch.equal(x[:, (nh + nkv) * hd:], qkv[:, (nh + nkv) * hd:])          # v is not rotated
+    assert torch.equal(x[0, :nh * hd], qkv[0, :nh * hd])                           # position 0 is the identity
+    # the cache took the rotated keys and the values at the named slots, and nothing else changed
+    kexp, vexp = kp0.clone().cpu(), vp0.clone().cpu()
+    xk = x[:, nh * hd:(nh + nkv) * hd].cpu().view(T, nkv, hd)
+    for t in range(T):
+        s = int(slots[t])
+        if s < 0:
+            continue
+        kexp[s // ps, :, s % ps, :] = xk[t]
+        vexp[s // ps, :, s % ps, :] = v[t]
+    assert torch.equal(kp.cpu(), kexp) and torch.equal(vp.cpu(), vexp)
+    # a run that reads another layer's cache writes nothing
+    kp1, vp1 = kp0.clone(), vp0.clone()
+    ops.rope_kv_write(qkv.clone(), positions, cos.to(dev()), sin.to(dev()), slots.to(dev()), kp1, vp1, nh, nkv, hd,
+                      write_kv=False)
+    assert torch.equal(kp1, kp0) and torch.equal(vp1, vp0)
+
+
+# ----------------------------------------------------------------------------- attention
+
+def _paged_case(seqs, nh, nkv, hd, ps, dtype, seed, window=None, spike=None):
+    """seqs: list of (q_len, kv_len).  Builds a scrambled paged cache (pages in random order, unused
+    slots filled with NaN) and the step's arrays; returns the operands and the plain result."""
+    g = torch.Generator().manual_seed(seed)
+    E = len(seqs)
+    blocks = [-(-kv // ps) for _, kv in seqs]
+    num_pages = sum(blocks) + 3
+    perm = torch.randperm(num_pages, generator=g).tolist()
+    width = max(blocks) + 1
+    bt = torch.full((E, width), -1, dtype=torch.int32)
+    kp = torch.full((num_pages, nkv, ps, hd), float("nan"))
+    vp = torch.full((num_pages, nkv, ps, hd), float("nan"))
+    T = sum(q for q, _ in seqs)
+    q = torch.randn((T, nh, hd), generator=g)
+    ent, pos = [], []
+    refs = []
+    o = 0
+    for e, (ql, kv) in enumerate(seqs):
+        k = torch.randn((kv, nkv, hd), generator=g)
+        v = torch.randn((kv, nkv, hd), generator=g)
+        qpos = list(range(kv - ql, kv))
+        if spike is not None:
+            # one far key that the last query of the request must find: its score stands out
+            c = spike(e, ql, kv)
+            if c is not None:
+                k[c, :, :] = 0
+                k[c, :, 0] = 40.0
+                q[o + ql - 1, :, :] = 0
+                q[o + ql - 1, :, 0] = math.sqrt(hd)       # score 40 at key c, about N(0, 1) elsewhere
+                v[c, :, :] = 7.0
+        k, v, = k.to(dtype).float(), v.to(dtype).float()
+        pages = [perm.pop() for _ in range(blocks[e])]
+        bt[e, :len(pages)] = torch.tensor(pages, dtype=torch.int32)
+        for c in range(kv):
+            kp[pages[c // ps], :, c % ps, :] = k[c]
+            vp[pages[c // ps], :, c % ps, :] = v[c]
+        qe = q[o:o + ql].to(dtype).float()
+        refs.append(pm.attention(qe.double(), k.double(), v.double(), qpos, window))
+        ent += [e] * ql
+        pos += qpos
+        o += ql
+    d = dev()
+    ops_in = dict(q=q.to(dtype).reshape(T, nh * hd).to(d), k_pages=kp.to(dtype).to(d), v_pages=vp.to(dtype).to(d),
+                  block_table=bt.to(d), token_entry=torch.tensor(ent, dtype=torch.int32, device=d),
+                  positions=torch.tensor(pos, dtype=torch.int32, device=d))
+    return ops_in, torch.cat(refs).reshape(T, nh * hd), seqs
+
+
+ATTN_HEADS = [(32, 8, 128), (12, 12, 64), (12, 2, 128), (6, 1, 32), (4, 2, 16), (6, 3, 48), (5, 5, 80)]
+ATTN_SEQS = [[(1, 128), (1, 256)], [(64, 64), (128, 128)], [(1, 500), (9, 9)], [(125, 260), (63, 63)],
+             [(1, 1), (2, 2), (1, 17), (33, 40)], [(1, 1280), (1, 2561)]]
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-5), (torch.bfloat16, 2e-2)])
+@pytest.mark.parametrize("nh,nkv,hd", ATTN_HEADS)
+@pytest.mark.parametrize("seqs", ATTN_SEQS)
+def test_paged_attention_generic(dtype, tol, nh, nkv, hd, seqs):
+    from ginfer_amd.kernels import ops
+    if sum(kv for _, kv in seqs) * nkv * hd > 3e6:
+        if (nh, nkv, hd) not in ((12, 2, 128), (6, 1, 32)):
+            pytest.skip("large case kept for two head shapes")
+    for ps in (16, 8) if hd <= 48 else (16,):
+        a, ref, _ = _paged_case(seqs, nh, nkv, hd, ps, dtype, seed=hd + ps)
+        out = ops.paged_attention_generic(a["q"], a["k_pages"], a["v_pages"], a["block_table"], a["token_entry"],
+                                          a["positions"], nh, nkv, hd, 1.0 / math.sqrt(hd))
+        close(out, ref, tol)
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-5), (torch.bfloat16, 2e-2)])
+@pytest.mark.parametrize("window", [1, 5, 16, 40, 64, 100])
+def test_paged_attention_window(dtype, tol, window):
+    from ginfer_amd.kernels import ops
+    nh, nkv, hd, ps = 6, 3, 48, 16
+    seqs = [(1, 200), (30, 90), (7, 7), (1, window), (1, window + 1), (50, 130)]
+    a, ref, _ = _paged_case(seqs, nh, nkv, hd, ps, dtype, seed=window, window=window)
+    out = ops.paged_attention_generic(a["q"], a["k_pages"], a["v_pages"], a["block_table"], a["token_entry"],
+                                      a["positions"], nh, nkv, hd, 1.0 / math.sqrt(hd), window=window)
+    close(out, ref, tol)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("where", ["first", "page_edge", "before_page_edge", "tile_edge", "last", "window_edge",
+                                   "behind_window"])
+def test_paged_attention_finds_one_far_key(dtype, where):
+    """Random keys hide a skipped key among hundreds; here one key carries nearly all the weight, so
+    the output is that key's value (7) if and only if the kernel reads it."""
+    from ginfer_amd.kernels import ops
+    nh, nkv, hd, ps = 4, 2, 32, 16
+    kv = 300
+    window = 100 if "window" in where else None
+    place = {"first": 0, "page_edge": 16 * 9, "before_page_edge": 16 * 9 - 1, "tile_edge": 64 * 3, "last": kv - 1,
+             "window_edge": kv - 100, "behind_window": kv - 101}[where]
+    seqs = [(1, kv), (20, kv)]
+    a, ref, _ = _paged_case(seqs, nh, nkv, hd, ps, dtype, seed=5, window=window, spike=lambda e, ql, n: place)
+    out = ops.paged_attention_generic(a["q"], a["k_pages"], a["v_pages"], a["block_table"], a["token_entry"],
+                                      a["positions"], nh, nkv, hd, 1.0 / math.sqrt(hd), window=window)
+    close(out, ref, 1e-5 if dtype == torch.float32 else 2e-2)
+    last_rows = out.float().cpu()[[0, 20]]
+    if where == "behind_window":
+        assert (last_rows.abs() < 3).all()
+    else:
+        assert (last_rows - 7.0).abs().max() < 0.1
+
+
+@pytest.mark.parametrize("R,V", [(1, 128), (1, 1024), (1, 4096), (2, 128), (17, 1024), (33, 4096), (3, 777), (2, 151936)])
+def test_argmax_lowest_index(R, V):
+    from ginfer_amd.kernels import ops
+    x = rnd((R, V), torch.float32, 20)
+    out = ops.sample_rows(x).cpu().numpy()
+    assert (out == np.argmax(x.cpu().numpy(), axis=1)).all()
+    # ties: the lowest index wins, wherever the equal values lie
+    y = torch.zeros((3, V), device=dev())
+    y[1, V - 1] = y[1, V // 2] = 5.0
+    y[2, V // 3] = y[2, V // 3 + 1] = 2.0
+    assert ops.sample_rows(y).cpu().tolist() == [0, V // 2, V // 3]
+
+
+@pytest.mark.parametrize("V", [777, 4096, 151936])
+def test_temperature_sampling(V):
+    from ginfer_amd.kernels import ops
+    R = 64
+    x = rnd((R, V), torch.float32, 21, scale=2.0)
+    temps = torch.full((R,), 0.8, device=dev())
+    temps[::7] = 0.0
+    g = torch.Generator().manual_seed(3)
+    uni = torch.rand((R,), generator=g).to(dev())
+    out = ops.sample_rows(x, temps, uni).cpu().tolist()
+    agree = 0
+    for r in range(R):
+        agree += int(out[r] == pm.sample_token(x[r].cpu(), float(temps[r]), float(uni[r])))
+    assert agree >= R - 1, "%d of %d draws agree with the plain sampler" % (agree, R)
+    # temperature -> 0 tends to the argmax
+    cold = ops.sample_rows(x, torch.full((R,), 1e-4, device=dev()), uni).cpu().tolist()
+    assert cold == x.argmax(dim=1).cpu().tolist()
+    # uniform number 0 picks the first token with mass; just below 1 the last
+    one = torch.zeros((1, V), device=dev())
+    assert ops.sample_rows(one, torch.ones(1, device=dev()), torch.zeros(1, device=dev())).item() == 0
+    assert ops.sample_rows(one, torch.ones(1, device=dev()), torch.full((1,), 0.9999999, device=dev())).item() == V - 1
+
+
+def test_kernels_refuse_what_they_cannot_take():
+    from ginfer_amd.kernels import ops, KernelError
+    with pytest.raises(KernelError):
+        ops.gemm_nt(rnd((4, 8), torch.float32, 1), rnd((4, 9), torch.float32, 2))
+    with pytest.raises(KernelError):
+        ops.add_rmsnorm(rnd((4, 8), torch.float32, 1), rnd((4, 9), torch.float32, 2), rnd((8,), torch.float32, 3), 1e-6,
+                        torch.float32)
+    with pytest.raises(KernelError):
+        ops.embedding_gather(rnd((10, 8), torch.float32, 1), torch.zeros(3, dtype=torch.int64, device=dev()))
+    with pytest.raises(KernelError):
+        ops.silu_mul(rnd((4, 7), torch.float32, 1))
+    with pytest.raises(KernelError):
+        ops.add_rmsnorm(torch.zeros(4, 8), None, torch.ones(8), 1e-6, torch.float32)      # CPU tensors

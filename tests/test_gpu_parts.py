@@ -1,0 +1,265 @@
+"""Each part alone against its plain function, and the generality of the assembly: a toy mixer with
+state of its own, a layer named twice, a layer that reads another layer's cache."""
+import math
+from dataclasses import dataclass
+
+import numpy as np
+import pytest
+import torch
+
+import helpers as H
+import plain_model as pm
+
+pytestmark = pytest.mark.gpu
+
+
+def dev():
+    return torch.device("cuda:0")
+
+
+def rnd(shape, seed, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randn(shape, generator=g) * scale
+
+
+def close(got, ref, tol):
+    got, ref = got.float().cpu(), ref.float().cpu()
+    assert torch.isfinite(got).all()
+    err = (got - ref).abs().max().item() / max(ref.abs().max().item(), 1e-30)
+    assert err <= tol, "error %.3g > %.3g" % (err, tol)
+
+
+PART_DTYPES = [(torch.float32, 1e-5), (torch.bfloat16, 2e-2)]
+
+
+@pytest.mark.parametrize("dtype,tol", PART_DTYPES)
+@pytest.mark.parametrize("T", [1, 7, 200])
+def test_swiglu_part(dtype, tol, T):
+    from ginfer_amd.parts import lookup
+    Hd, I = 88, 136
+    part = lookup("feed_forward", "swiglu")(hidden_size=Hd, intermediate_size=I, dtype=dtype, device=dev())
+    w = {n: rnd(s.shape, i, 0.1).to(dtype) for i, (n, s) in enumerate(part.weight_specs().items())}
+    part.bind_weights({n: t.to(dev()) for n, t in w.items()})
+    x = rnd((T, Hd), 9).to(dtype)
+    wd = {"p." + n: t.double() for n, t in w.items()}
+    ref = pm.feed_forward(x.double(), wd, "p")
+    close(part.forward(x.to(dev())), ref, tol)
+
+
+@pytest.mark.parametrize("dtype,tol", PART_DTYPES)
+def test_norm_part(dtype, tol):
+    from ginfer_amd.parts import lookup
+    part = lookup("norm", "rmsnorm")(size=96, eps=1e-5, dtype=dtype, device=dev())
+    g = (1 + rnd((96,), 1, 0.1)).to(dtype)
+    part.bind_weights({"weight": g.to(dev())})
+    res, delta = rnd((11, 96), 2), rnd((11, 96), 3).to(dtype)
+    ref = pm.rms_norm(res.double() + delta.double(), g.double(), 1e-5)
+    r = res.to(dev())
+    close(part.forward(r, delta.to(dev())), ref, tol)
+    close(r, res.double() + delta.double(), 1e-6)
+
+
+@pytest.mark.parametrize("dtype,tol", PART_DTYPES)
+@pytest.mark.parametrize("tied", [True, False])
+def test_embedding_and_head_parts(dtype, tol, tied):
+    from ginfer_amd.parts import lookup
+    V, Hd = 301, 72
+    emb = lookup("embedding", "embedding")(vocab_size=V, hidden_size=Hd, dtype=dtype, device=dev())
+    head = lookup("head", "lm_head")(vocab_size=V, hidden_size=Hd, tied=tied, dtype=dtype, device=dev())
+    E = rnd((V, Hd), 1).to(dtype)
+    emb.bind_weights({"weight": E.to(dev())})
+    assert (head.weight_specs() == {}) == tied
+    Wh = E if tied else rnd((V, Hd), 2).to(dtype)
+    if tied:
+        head.tie(emb.weight)
+        assert head.weight.data_ptr() == emb.weight.data_ptr()       # one device copy
+    else:
+        head.bind_weights({"weight": Wh.to(dev())})
+    ids = torch.tensor([0, 300, 5, 5], dtype=torch.int32)
+    assert torch.equal(emb.forward(ids.to(dev())).cpu(), E[ids.long()].float())
+    x = rnd((3, Hd), 4).to(dtype)
+    logits = head.forward(x.to(dev()))
+    assert logits.dtype == torch.float32
+    close(logits, x.double() @ Wh.double().t(), 1e-5 if dtype == torch.float32 else 1e-4)
+
+
+@pytest.mark.parametrize("dtype,tol", PART_DTYPES)
+@pytest.mark.parametrize("window", [None, 12])
+def test_attention_part_in_portions(dtype, tol, window):
+    """The mixer alone, fed one request in three portions through a hand-made cache view, equals the
+    plain attention block on the whole sequence."""
+    from ginfer_amd.config import PartSpec
+    from ginfer_amd.parts import lookup, KVView, StepContext
+    Hd, nh, nkv, hd, ps, T = 80, 4, 2, 32, 8, 45
+    pos = lookup("position", "rope_neox")(theta=1e4, rotary_dim=hd, max_positions=64, device=dev())
+    part = lookup("mixer", "attention")(hidden_size=Hd, num_heads=nh, num_kv_heads=nkv, head_dim=hd, qkv_bias=True,
+                                        out_bias=False, window=window, position=pos, scale=None, dtype=dtype,
+                                        device=dev())
+    w = {n: rnd(s.shape, i, 0.15).to(dtype) for i, (n, s) in enumerate(part.weight_specs().items())}
+    part.bind_weights({n: t.to(dev()) for n, t in w.items()})
+    x = rnd((T, Hd), 20).to(dtype)
+    cfg = dict(num_attention_heads=nh, num_key_value_heads=nkv, head_dim=hd)
+    sin, cos = pm.rope_tables(1e4, hd, 64)
+    ref, _ = pm.attention_block(x.double(), {"p." + n: t.double() for n, t in w.items()}, "p", cfg, list(range(T)),
+                                sin, cos, window)
+    pages = 8
+    kp = torch.full((pages, nkv, ps, hd), float("nan"), dtype=dtype, device=dev())
+    vp = torch.full((pages, nkv, ps, hd), float("nan"), dtype=dtype, device=dev())
+    table = [5, 2, 7, 0, 3, 6]
+    outs = []
+    for a, b in ((0, 20), (20, 22), (22, 45)):
+        n = b - a
+        p = np.arange(a, b)
+        slots = torch.tensor(np.asarray(table)[p // ps] * ps + p % ps, dtype=torch.int64, device=dev())
+        view = KVView(kp, vp, torch.tensor([table], dtype=torch.int32, device=dev()), slots, ps, True)
+        step = StepContext(token_ids=None, positions=torch.tensor(p, dtype=torch.int32, device=dev()),
+                           token_entry=torch.zeros(n, dtype=torch.int32, device=dev()),
+                           cu_tokens=torch.tensor([0, n], dtype=torch.int32, device=dev()),
+                           q_start=torch.tensor([a], dtype=torch.int32, device=dev()),
+                           logit_rows=None, num_tokens=n, num_entries=1, host_q_start=[a], host_q_len=[n],
+                           caches=[view], extra={})
+        outs.append(part.forward(x[a:b].to(dev()), step, view))
+    close(torch.cat(outs), ref, tol)
+
+
+# ----------------------------------------------------------------------------- generality of the assembly
+
+def _register_toy():
+    """A toy architecture defined here, in the test: blocks whose mixer keeps a running sum of its
+    inputs per request (state of fixed size, no pages) between blocks with attention, a layer that runs
+    twice and a run that reads another run's keys and values."""
+    from ginfer_amd.config import register_architecture, PartSpec, LayerSpec, ScheduleEntry, ModelSpec
+    from ginfer_amd.parts import register_mixer, Part, StateSpec
+    from ginfer_amd.weights import WeightSpec
+
+    @register_mixer("toy_running_mean")
+    class RunningMean(Part):
+        """out[t] = W . mean(x[0..t]) of the request; the state is (sum, count)."""
+
+        def __init__(self, hidden_size, dtype, device):
+            self.H, self.dtype, self.device = hidden_size, dtype, device
+
+        def cache_spec(self):
+            return StateSpec((self.H + 1,), torch.float32)
+
+        def weight_specs(self):
+            return {"mix.weight": WeightSpec((self.H, self.H))}
+
+        def bind_weights(self, t):
+            self.w = t["mix.weight"]
+
+        def forward(self, x, step, cache):
+            out = torch.empty_like(x)
+            o = 0
+            for e in range(step.num_entries):
+                n, start = step.host_q_len[e], step.host_q_start[e]
+                slot = cache.slots[e]
+                if start == 0:
+                    cache.state[slot] = 0
+                st = cache.state[slot]
+                sums = st[:self.H] + torch.cumsum(x[o:o + n].float(), dim=0)
+                counts = st[self.H] + torch.arange(1, n + 1, device=x.device, dtype=torch.float32)
+                out[o:o + n] = ((sums / counts[:, None]).to(self.dtype) @ self.w.t())
+                cache.state[slot, :self.H] = sums[-1]
+                cache.state[slot, self.H] = counts[-1]
+                o += n
+            return out
+
+    @register_architecture("ToyStateLM")
+    @dataclass
+    class ToyConfig:
+        hidden_size: int = 48
+        vocab_size: int = 211
+        architecture = "ToyStateLM"
+
+        @classmethod
+        def from_dict(cls, d):
+            return cls(d["hidden_size"], d["vocab_size"])
+
+        def to_dict(self):
+            return dict(architectures=["ToyStateLM"], hidden_size=self.hidden_size, vocab_size=self.vocab_size)
+
+        def model_spec(self):
+            Hd = self.hidden_size
+            norm = PartSpec("rmsnorm", dict(size=Hd, eps=1e-5))
+            pos = PartSpec("rope_neox", dict(theta=1e4, rotary_dim=16, max_positions=256))
+            attn = PartSpec("attention", dict(hidden_size=Hd, num_heads=3, num_kv_heads=1, head_dim=16, qkv_bias=True,
+                                              out_bias=False, window=None, position=pos, scale=None))
+            toy = PartSpec("toy_running_mean", dict(hidden_size=Hd))
+            ffn = PartSpec("swiglu", dict(hidden_size=Hd, intermediate_size=80))
+            layers = [LayerSpec("model.layers.%d" % i, m, ffn, norm, norm) for i, m in enumerate([attn, toy, attn])]
+            # layer 0, the toy layer, layer 2 reading run 0's cache, the toy layer again (a second state)
+            schedule = [ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(2, cache_of=0), ScheduleEntry(1)]
+            return ModelSpec(hidden_size=Hd, vocab_size=self.vocab_size, layers=layers, schedule=schedule,
+                             embedding=PartSpec("embedding", dict(vocab_size=self.vocab_size, hidden_size=Hd)),
+                             final_norm=norm, head=PartSpec("lm_head", dict(vocab_size=self.vocab_size, hidden_size=Hd,
+                                                                            tied=True)),
+                             max_positions=256, eos_token_ids=[0])
+    return ToyConfig
+
+
+def _toy_plain(folder, ids):
+    """The toy model on a whole sequence, written out plainly in 64-bit."""
+    w = pm.read_weights(folder)
+    T = len(ids)
+    cfg = dict(num_attention_heads=3, num_key_value_heads=1, head_dim=16)
+    sin, cos = pm.rope_tables(1e4, 16, T)
+    x = pm.embedding(w["model.embed_tokens.weight"], ids)
+    kept = {}
+    for run, (layer, cache_of) in enumerate([(0, None), (1, None), (2, 0), (1, None)]):
+        p = "model.layers.%d" % layer
+        n = pm.rms_norm(x, w[p + ".input_layernorm.weight"], 1e-5)
+        if layer == 1:
+            mean = torch.cumsum(n, dim=0) / torch.arange(1, T + 1, dtype=n.dtype)[:, None]
+            a = mean @ w[p + ".self_attn.mix.weight"].t()
+        else:
+            a, kv = pm.attention_block(n, w, p + ".self_attn", cfg, list(range(T)), sin, cos, None,
+                                       kv_from=None if cache_of is None else kept[cache_of])
+            kept[run] = kv
+        h = x + a
+        n = pm.rms_norm(h, w[p + ".post_attention_layernorm.weight"], 1e-5)
+        x = h + pm.feed_forward(n, w, p + ".mlp")
+    return pm.linear(pm.rms_norm(x, w["model.norm.weight"], 1e-5), w["model.embed_tokens.weight"]).float().numpy()
+
+
+def test_toy_mixer_with_state_is_registered_built_and_stepped(tmp_path):
+    from ginfer_amd import ModelRunner, write_random_model, config_from_folder
+    Toy = _register_toy()
+    folder = write_random_model(str(tmp_path / "toy"), Toy(), seed=4, dtype="float32")
+    assert type(config_from_folder(folder)).__name__ == "ToyConfig"
+    reqs = {"a": H.random_tokens(50, 211, 1), "b": H.random_tokens(23, 211, 2), "c": H.random_tokens(37, 211, 3)}
+    runner = ModelRunner(folder, dtype="float32", page_size=8, num_pages=16, max_requests=3)
+    specs = runner.cache.cache_specs
+    assert [type(s).__name__ for s in specs] == ["KVCacheSpec", "StateSpec", "NoneType", "StateSpec"]
+    assert len(runner.cache.groups) == 1 and runner.cache.groups[0].entries == [0]
+    for steps in (H.steps_whole(reqs), H.steps_portions(reqs, sizes=(5, 2, 11)), H.steps_mixed(reqs, max_live=3, seed=1)):
+        got = H.run_steps(runner, steps)
+        runner.cache.check()
+        for (rid, p), row in got.items():
+            ref = _toy_plain(folder, reqs[rid])
+            err = np.abs(row - ref[p]).max() / np.abs(ref).max()
+            assert err < 1e-4, "request %s position %d: %.3g" % (rid, p, err)
+
+
+def test_schedule_names_a_layer_twice_and_shares_a_cache(tmp_path):
+    """The order of layers is data: a Qwen2 folder run with another schedule."""
+    from ginfer_amd import ModelRunner, config_from_folder
+    from ginfer_amd.config import ScheduleEntry
+    folder = H.make_model_folder(tmp_path / "m", H.TINY_B, 1)
+    cfg = config_from_folder(folder)
+    base_spec = cfg.model_spec
+
+    def spec_with_schedule():
+        s = base_spec()
+        s.schedule = [ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(1), ScheduleEntry(2, cache_of=0)]
+        return s
+    cfg.model_spec = spec_with_schedule
+    runner = ModelRunner(folder, dtype="float32", page_size=8, num_pages=32, config=cfg)
+    assert len(runner.cache.groups[0].entries) == 3           # runs 0, 1, 2 own caches; run 3 reads run 0's
+    ids = H.random_tokens(60, 1000, 8)
+    pc, w = pm.read_config(folder), pm.read_weights(folder)
+    ref = pm.forward(pc, w, ids, schedule=[(0, None), (1, None), (1, None), (2, 0)]).float().numpy()
+    for steps in (H.steps_whole({"x": ids}), H.steps_portions({"x": ids}, sizes=(9, 2, 30))):
+        got = H.run_steps(runner, steps)
+        for (rid, p), row in got.items():
+            assert np.abs(row - ref[p]).max() / np.abs(ref).max() < 1e-4

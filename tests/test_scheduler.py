@@ -1,0 +1,176 @@
+"""The scheduler's decisions on the CPU, with a stand-in for the model (the next token is a function
+of the tokens so far, so recomputation after an eviction must give the same continuation)."""
+import random
+
+import pytest
+
+from ginfer_amd.cache import CacheManager, OutOfPages
+from ginfer_amd.engine.scheduler import Scheduler
+from ginfer_amd.engine.sequence import Sequence, State
+from ginfer_amd.parts import KVCacheSpec
+from ginfer_amd.sampling import SamplingParams, uniform
+
+
+def make(num_pages, page_size=4, max_num_seqs=4, budget=16, eos=(999,), max_model_len=256, window=None):
+    cache = CacheManager([KVCacheSpec(1, 16, window)], page_size, num_pages, max_num_seqs)
+    return Scheduler(cache, max_num_seqs, budget, eos, max_model_len), cache
+
+
+def fake_token(ids):
+    return (sum(ids) * 31 + len(ids)) % 900
+
+
+def run(sched, cache, seqs, check=None, max_steps=10000):
+    for s in seqs:
+        sched.add(s)
+    done, steps = [], []
+    while not sched.is_finished():
+        batch = sched.schedule()
+        assert batch, "an empty step"
+        assert sum(b.num_tokens for b in batch) <= sched.max_num_batched_tokens
+        assert len({id(b.seq) for b in batch}) == len(batch)
+        cache.check()
+        toks = []
+        for b in batch:
+            assert cache.pending(b.seq.request_id) == b.num_tokens
+            assert cache.length(b.seq.request_id) == b.seq.num_computed
+            assert b.samples == (b.seq.num_computed + b.num_tokens == b.seq.num_tokens)
+            if b.samples:
+                toks.append(fake_token(b.seq.token_ids))
+        if check:
+            check(batch)
+        steps.append([(b.seq.request_id, b.num_tokens) for b in batch])
+        done += sched.postprocess(batch, toks, now=float(len(steps)))
+        cache.check()
+        assert len(steps) < max_steps
+    return done, steps
+
+
+def seq(i, prompt_len, max_tokens=8, **kw):
+    return Sequence(i, [(i * 7 + j) % 900 for j in range(prompt_len)], prompt_len, SamplingParams(max_tokens=max_tokens, **kw))
+
+
+def expected(s0):
+    ids = list(s0.token_ids[:s0.num_prompt_tokens])
+    for _ in range(s0.params.max_tokens):
+        ids.append(fake_token(ids))
+    return ids
+
+
+def test_prompts_are_cut_under_the_budget_and_decoding_goes_on_beside_them():
+    sched, cache = make(num_pages=64, budget=16)
+    a, b = seq(0, 5, max_tokens=12), seq(1, 40, max_tokens=4)
+    done, steps = run(sched, cache, [a, b])
+    assert steps[0] == [(0, 5), (1, 11)]                       # arrival order, the second prompt cut to the budget
+    assert steps[1] == [(0, 1), (1, 15)]                       # a decoded token beside a portion
+    assert steps[2] == [(0, 1), (1, 14)]                       # the prompt ends: this portion samples
+    assert steps[3] == [(0, 1), (1, 1)]
+    assert {s.request_id: s.token_ids for s in done} == {0: expected(a), 1: expected(b)}
+    assert all(s.finish_reason == "max_tokens" for s in done) and not cache.requests
+
+
+def test_admission_is_in_arrival_order_and_bounded():
+    sched, cache = make(num_pages=64, max_num_seqs=2, budget=64)
+    seqs = [seq(i, 6, max_tokens=3) for i in range(5)]
+    done, steps = run(sched, cache, seqs)
+    assert steps[0] == [(0, 6), (1, 6)]                        # two at a time
+    assert all(len(st) <= 2 for st in steps)
+    assert [s.request_id for s in done] == [0, 1, 2, 3, 4]
+    first_step = {}
+    for i, st in enumerate(steps):
+        for rid, _ in st:
+            first_step.setdefault(rid, i)
+    assert [first_step[i] for i in range(5)] == sorted(first_step[i] for i in range(5))
+
+
+def test_finishing_rules():
+    sched, cache = make(num_pages=64)
+    a = seq(0, 4, max_tokens=50)
+    stop_tok = expected(a)[4 + 2]
+    a.params.stop_token_ids = [stop_tok]
+    b = seq(1, 4, max_tokens=50, ignore_eos=True)
+    b.params.stop_token_ids = [expected(b)[4]]
+    c = seq(2, 250, max_tokens=50)
+    sched.max_num_batched_tokens = 300
+    done, _ = run(sched, cache, [a, b, c])
+    by = {s.request_id: s for s in done}
+    assert by[0].finish_reason == "eos" and by[0].num_output_tokens == 3 and by[0].token_ids[-1] == stop_tok
+    assert by[1].finish_reason == "max_tokens" and by[1].num_output_tokens == 50
+    assert by[2].finish_reason == "max_model_len" and by[2].num_tokens == 256
+    # the configuration's ids apply when the request names none
+    sched2, cache2 = make(num_pages=64, eos=(expected(seq(0, 4))[5],))
+    d = seq(0, 4, max_tokens=50)
+    done, _ = run(sched2, cache2, [d])
+    assert done[0].finish_reason == "eos" and done[0].num_output_tokens == 2
+
+
+def test_out_of_pages_evicts_the_newest_and_recomputes_it():
+    # 3 requests of 10 + up to 14 tokens: 24 tokens = 6 pages each; 12 pages hold two of them
+    sched, cache = make(num_pages=12, budget=32)
+    seqs = [seq(i, 10, max_tokens=14) for i in range(3)]
+    evicted = []
+    real_evict = sched._evict
+    def spy(s):
+        evicted.append((s.request_id, [r.request_id for r in sched.running]))
+        real_evict(s)
+    sched._evict = spy
+    done, steps = run(sched, cache, seqs)
+    assert evicted, "the pool was large enough: nothing was evicted"
+    for victim, running in evicted:
+        assert victim == running[-1]                            # the newest running request goes
+    assert sched.num_evictions == len(evicted)
+    # recomputation feeds prompt and output again and continues where it stopped
+    assert {s.request_id: s.token_ids for s in done} == {i: expected(seqs[i]) for i in range(3)}
+    assert max(s.evictions for s in done) >= 1 and done[0].request_id == 0
+    assert not cache.requests and cache.groups[0].pool.num_free == 12
+
+
+def test_a_request_that_could_never_fit_is_refused():
+    sched, cache = make(num_pages=4, page_size=4)
+    with pytest.raises(ValueError, match="could never finish"):
+        sched.add(seq(0, 10, max_tokens=10))
+    sched.add(seq(1, 10, max_tokens=6))                        # 16 tokens: exactly the pool
+    with pytest.raises(ValueError, match="empty prompt"):
+        sched.add(Sequence(2, [], 0, SamplingParams()))
+    with pytest.raises(ValueError, match="max_model_len"):
+        sched.add(seq(3, 256))
+
+
+def test_lone_request_fills_the_pool_and_finishes():
+    sched, cache = make(num_pages=4, page_size=4, budget=5)
+    a = seq(0, 10, max_tokens=6)
+    done, steps = run(sched, cache, [a])
+    assert steps[:2] == [[(0, 5)], [(0, 5)]] and done[0].token_ids == expected(a)
+
+
+def test_portions_shrink_to_the_free_pages():
+    sched, cache = make(num_pages=8, page_size=4, budget=64, max_num_seqs=3)
+    a, b = seq(0, 20, max_tokens=4), seq(1, 30, max_tokens=2)
+    done, steps = run(sched, cache, [a, b])
+    assert steps[0] == [(0, 20), (1, 12)]                      # 5 pages for a, the 3 left hold 12 tokens of b
+    assert {s.request_id: s.token_ids for s in done} == {0: expected(a), 1: expected(b)}
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_workloads_finish_with_the_same_tokens(seed):
+    rng = random.Random(seed)
+    window = rng.choice([None, 12])
+    sched, cache = make(num_pages=rng.choice([16, 24, 40]), page_size=rng.choice([4, 8]), max_num_seqs=rng.choice([2, 4]),
+                        budget=rng.choice([8, 24, 64]), window=window)
+    cap = min(g.pool.num_pages for g in cache.groups) * cache.page_size
+    seqs = []
+    for i in range(12):
+        n = rng.randint(1, min(40, cap - 12))
+        seqs.append(seq(i, n, max_tokens=rng.randint(1, 12)))
+    done, steps = run(sched, cache, seqs)
+    assert {s.request_id: s.token_ids for s in done} == {s.request_id: expected(s) for s in seqs}
+    assert not cache.requests and all(g.pool.num_free == g.pool.num_pages for g in cache.groups)
+
+
+def test_uniform_numbers_are_a_function_of_seed_and_place():
+    us = [uniform(3, n) for n in range(1000)]
+    assert all(0.0 <= u < 1.0 for u in us) and len(set(us)) > 990
+    assert us == [uniform(3, n) for n in range(1000)] and uniform(4, 0) != uniform(3, 0)
+    assert abs(sum(us) / 1000 - 0.5) < 0.05
+    import numpy as np
+    assert all(float(np.float32(u)) == u for u in us)          # exact in 32-bit
