@@ -10,7 +10,9 @@ next token to be computed; its table keeps a -1 there.  Pages return to the pool
 released and are used again by later requests.  The reference has one pool, one table per sequence,
 no window and no state (ginfer/engine/block_manager.cc:63-148, ginfer/engine/model_runner.cc:52-87).
 
-Device layout of one group: tensor [entries_in_group, 2 (k, v), pages, nkv, page_size, hd].
+Device layout of one group: one allocation [entries_in_group, 2 (k, v), pages, nkv * page_size * hd]; an
+entry's keys are viewed [pages, nkv, page_size, hd] and its values [pages, nkv, hd, page_size]
+(transposed inside a page, which is what the matrix-core attention kernels read fastest).
 """
 from dataclasses import dataclass, field
 from typing import Dict, List, Optional
@@ -75,11 +77,18 @@ class CacheManager:
     def allocate_device(self, dtype, device):
         import torch
         for g in self.groups:
-            g.tensor = torch.zeros((len(g.entries), 2, g.pool.num_pages, g.spec.num_kv_heads, self.page_size,
-                                    g.spec.head_dim), dtype=dtype, device=device)
+            g.tensor = torch.zeros((len(g.entries), 2, g.pool.num_pages,
+                                    g.spec.num_kv_heads * self.page_size * g.spec.head_dim), dtype=dtype, device=device)
         for e in self.state_entries:
             s = self.cache_specs[e]
             self.state_tensors[e] = torch.zeros((self.max_requests,) + tuple(s.shape), dtype=s.dtype, device=device)
+
+    def kv_views(self, entry):
+        """(k_pages [pages, nkv, page_size, hd], v_pages [pages, nkv, hd, page_size]) of a schedule entry."""
+        gi, j = self.group_of[entry]
+        g = self.groups[gi]
+        n, nkv, hd = g.pool.num_pages, g.spec.num_kv_heads, g.spec.head_dim
+        return (g.tensor[j, 0].view(n, nkv, self.page_size, hd), g.tensor[j, 1].view(n, nkv, hd, self.page_size))
 
     # ---- requests
     def has(self, rid):

@@ -71,8 +71,8 @@ __global__ void paged_attention_generic_kernel(
         for (int j = j0; j <= j1; ++j) {
           const int cc = tile + j;
           const int64_t page = bt[cc / page_size];
-          const T* vp = v_pages + ((page * nkv + g) * page_size + (cc % page_size)) * hd;
-          a += p_s[j] * Num<T>::ld(vp + d);
+          const T* vp = v_pages + ((page * nkv + g) * hd + d) * page_size + (cc % page_size);
+          a += p_s[j] * Num<T>::ld(vp);
         }
         acc[i] = a;
       }
@@ -88,7 +88,7 @@ __global__ void paged_attention_generic_kernel(
 }
 
 // out: [T, nh*hd] (row stride out_stride elements); q: rows of stride q_stride (the fused q|k|v
-// buffer); k_pages, v_pages: [pages, nkv, page_size, hd]; block_table: [entries, table_width];
+// buffer); k_pages: [pages, nkv, page_size, hd]; v_pages: [pages, nkv, hd, page_size]; block_table: [entries, table_width];
 // token_entry, positions: [T].
 extern "C" int ga_paged_attention_generic(void* out, int64_t out_stride, const void* q,
                                           int64_t q_stride, const void* k_pages,

@@ -1,0 +1,353 @@
+// Paged attention on the matrix cores (bfloat16 storage; 32-bit scores, softmax and accumulators),
+// compiled for one head size: -DHEAD_DIM=<multiple of 16, at most 256>.
+//
+// Both kernels here share one inner loop.  A wavefront owns up to 16*NB "columns"; a column is one
+// (token, query head) pair, all columns of a wavefront reading the same kv head of the same request.
+//   decode kernel : columns = the query heads of one kv-head group for ONE token; the keys are split
+//                   over blockIdx.z, partial (max, sum, output) go to a workspace and a second kernel
+//                   combines the splits in ascending order.  Replaces the reference's unsplit,
+//                   one-head-per-block kernel (ginfer/core/op/kernels/cuda/page_attn_kernel/
+//                   flash_gqa_varlen_decode_kvcache.cu:272-335), in which every head of a group re-reads
+//                   the same keys.
+//   prefill kernel: columns = 16*NB consecutive tokens of one request's portion, one head per
+//                   wavefront, the heads of a kv-head group side by side in a workgroup so that they
+//                   stream the same keys together (flash_gqa_varlen_kernel.cu:420-512 is the reference's).
+// Mask: column with position p sees keys c in [max(0, p - window + 1), p]  (flash_gqa_varlen_kernel.cu:
+// 202-222 in absolute positions).  score = (q . k) * scale on the 32-bit product; online softmax over
+// tiles of 32 keys at absolute multiples of 32.
+//
+// Matrix-core mapping (v_mfma_f32_16x16x32_bf16: D[m][n] += sum_k A[m][k] B[n][k]; lane l supplies row
+// l%16 and k-slots (l/16)*8..+7 of both operands and receives D[(l/16)*4+i][l%16], i = 0..3):
+//   S^T = K Q^T : A = 16 keys x 32 dims of K (one 16-byte load per lane straight from the page),
+//                 B = 16 columns x 32 dims of Q (kept in registers); two such products per tile.
+//                 Row m of product t holds key 8*(m/4) + 4*t + m%4 of the tile, so a lane ends up with
+//                 the scores of the 8 CONSECUTIVE keys 8*(l/16)..+7 of its column,
+//   O^T += V^T P: which is exactly the k-slot layout of operand B for P, with no shuffle; operand A is
+//                 16 dims x 8 consecutive keys of V^T: one 16-byte load per lane because the cache keeps
+//                 values transposed inside a page ([page][kv_head][dim][slot]).
+// Nothing is staged through LDS: each operand element is loaded once per wavefront, and the heads of a
+// group that run side by side hit the same lines in the vector cache.
+#include "common.cuh"
+
+#ifndef HEAD_DIM
+#error "compile with -DHEAD_DIM=<head size>"
+#endif
+static_assert(HEAD_DIM % 16 == 0 && HEAD_DIM >= 16 && HEAD_DIM <= 256, "head size: multiples of 16 up to 256");
+
+constexpr int HD = HEAD_DIM;
+constexpr int KB = (HD + 31) / 32;   // 32-dim blocks of the q.k product (the last may be half empty)
+constexpr int DB = HD / 16;          // 16-dim blocks of the output
+constexpr int PREFILL_NB = HD <= 128 ? 2 : 1;
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+__device__ __forceinline__ bf16x8 zero8() {
+  uint4 z = {0u, 0u, 0u, 0u};
+  return __builtin_bit_cast(bf16x8, z);
+}
+__device__ __forceinline__ bf16x8 load8(const bf16_t* p) {
+  return __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(p));
+}
+
+// Attends columns to the key tiles [tile_begin, tile_end) (multiples of 32).  kv_min..kv_max is the
+// inclusive range of keys that any column of the wavefront may see: keys outside it are never loaded
+// (their pages may be gone) and count as zero.
+template <int NB>
+__device__ __forceinline__ void attend_tiles(f32x4 (&o)[NB][DB], float (&m)[NB], float (&l)[NB],
+                                             const bf16x8 (&q)[NB][KB], const int (&cpos)[NB],
+                                             const int (&clo)[NB], const bf16_t* __restrict__ k_pages,
+                                             const bf16_t* __restrict__ v_pages,
+                                             const int32_t* __restrict__ bt, int kvh, int nkv, int ps_shift,
+                                             int kv_min, int kv_max, int tile_begin, int tile_end,
+                                             float scale) {
+  const int lane = threadIdx.x & 63, c = lane & 15, g = lane >> 4;
+  const int ps = 1 << ps_shift;
+  for (int k0 = tile_begin; k0 < tile_end; k0 += 32) {
+    // ---- scores: S^T = K Q^T
+    f32x4 s[NB][2];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+      s[nb][0] = f32x4{0.f, 0.f, 0.f, 0.f};
+      s[nb][1] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      const int key = k0 + 8 * (c >> 2) + 4 * t + (c & 3);
+      const bool ok = key >= kv_min && key <= kv_max;
+      const bf16_t* kp = k_pages;
+      if (ok) {
+        const int64_t page = bt[key >> ps_shift];
+        kp = k_pages + ((page * nkv + kvh) * ps + (key & (ps - 1))) * HD + g * 8;
+      }
+#pragma unroll
+      for (int kb = 0; kb < KB; ++kb) {
+        bf16x8 a = zero8();
+        if (ok && kb * 32 + g * 8 < HD) a = load8(kp + kb * 32);
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+          s[nb][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, q[nb][kb], s[nb][t], 0, 0, 0);
+      }
+    }
+    // ---- mask and online softmax; the lane holds keys k0 + 8g + j, j = 0..7, of column c
+    bf16x8 pb[NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+      float sv[8];
+      float mx = -INFINITY;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int key = k0 + 8 * g + j;
+        const bool valid = key >= clo[nb] && key <= cpos[nb];
+        sv[j] = valid ? s[nb][j >> 2][j & 3] * scale : -INFINITY;
+        mx = fmaxf(mx, sv[j]);
+      }
+      mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+      const float m_new = fmaxf(m[nb], mx);
+      float alpha = 1.f, sum = 0.f;
+      float p[8];
+      if (m_new == -INFINITY) {            // the column has seen no key yet
+#pragma unroll
+        for (int j = 0; j < 8; ++j) p[j] = 0.f;
+      } else {
+        alpha = __expf(m[nb] - m_new);     // exp(-inf) = 0 the first time
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          p[j] = __expf(sv[j] - m_new);
+          sum += p[j];
+        }
+      }
+      sum += __shfl_xor(sum, 16, WAVE);
+      sum += __shfl_xor(sum, 32, WAVE);
+      l[nb] = l[nb] * alpha + sum;
+      m[nb] = m_new;
+#pragma unroll
+      for (int db = 0; db < DB; ++db) o[nb][db] *= alpha;
+      union { bf16x8 v; bf16_t e[8]; } pk;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) pk.e[j] = f32_to_bf16(p[j]);
+      pb[nb] = pk.v;
+    }
+    // ---- output: O^T += V^T P; the lane loads dims db*16 + c, keys k0 + 8g .. + 7
+    const int kbase = k0 + 8 * g;
+    const bool any_ok = kbase + 7 >= kv_min && kbase <= kv_max;
+    const bool all_ok = kbase >= kv_min && kbase + 7 <= kv_max;
+    const bf16_t* vp = v_pages;
+    if (any_ok) {
+      const int64_t page = bt[kbase >> ps_shift];
+      vp = v_pages + ((page * nkv + kvh) * HD + c) * ps + (kbase & (ps - 1));
+    }
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+      bf16x8 a = zero8();
+      if (any_ok) {
+        a = load8(vp + (int64_t)db * 16 * ps);
+        if (!all_ok) {                     // slots past the request's last key hold anything: clear them
+          union { bf16x8 v; bf16_t e[8]; } u;
+          u.v = a;
+#pragma unroll
+          for (int j = 0; j < 8; ++j)
+            if (kbase + j < kv_min || kbase + j > kv_max) u.e[j] = 0;
+          a = u.v;
+        }
+      }
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+        o[nb][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb[nb], o[nb][db], 0, 0, 0);
+    }
+  }
+}
+
+template <int NB>
+__device__ __forceinline__ void init_state(f32x4 (&o)[NB][DB], float (&m)[NB], float (&l)[NB]) {
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) {
+    m[nb] = -INFINITY;
+    l[nb] = 0.f;
+#pragma unroll
+    for (int db = 0; db < DB; ++db) o[nb][db] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+}
+
+// q operand of one column: 32-dim blocks of the column's query row, this lane's 8 dims
+__device__ __forceinline__ void load_q(bf16x8 (&q)[KB], const bf16_t* row /* null: empty column */, int g) {
+#pragma unroll
+  for (int kb = 0; kb < KB; ++kb) {
+    q[kb] = zero8();
+    if (row && kb * 32 + g * 8 < HD) q[kb] = load8(row + kb * 32 + g * 8);
+  }
+}
+
+// ----------------------------------------------------------------------------- decode
+// grid (decode tokens, nkv * head_blocks, splits), one wavefront each.
+// part_o: [n_tokens][nh][splits][HD] float; part_ml: [n_tokens][nh][splits][2] float (max, sum).
+__global__ __launch_bounds__(64) void attn_decode_split_kernel(
+    float* __restrict__ part_o, float* __restrict__ part_ml, const bf16_t* __restrict__ q, int64_t q_stride,
+    const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
+    const int32_t* __restrict__ block_table, int table_width, const int32_t* __restrict__ token_entry,
+    const int32_t* __restrict__ positions, const int32_t* __restrict__ token_list, int nh, int nkv,
+    int head_blocks, int ps_shift, int window, float scale, int split_keys, int num_splits) {
+  const int lane = threadIdx.x, c = lane & 15, g = lane >> 4;
+  const int ti = blockIdx.x, split = blockIdx.z;
+  const int kvh = blockIdx.y / head_blocks, hb = blockIdx.y % head_blocks;
+  const int group = nh / nkv;
+  const int t = token_list[ti];
+  const int pos = positions[t];
+  const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  const bool col_ok = hb * 16 + c < group;
+  const int head = kvh * group + hb * 16 + c;
+
+  f32x4 o[1][DB];
+  float m[1], l[1];
+  init_state<1>(o, m, l);
+  const int begin = (lo / 32) * 32 + split * split_keys;
+  if (begin <= pos) {
+    int end = begin + split_keys;
+    if (end > pos + 1) end = ((pos + 32) / 32) * 32;
+    bf16x8 qr[1][KB];
+    load_q(qr[0], col_ok ? q + (int64_t)t * q_stride + (int64_t)head * HD : nullptr, g);
+    const int cpos[1] = {col_ok ? pos : -1}, clo[1] = {lo};
+    attend_tiles<1>(o, m, l, qr, cpos, clo, k_pages, v_pages,
+                    block_table + (int64_t)token_entry[t] * table_width, kvh, nkv, ps_shift, lo, pos, begin,
+                    end, scale);
+  }
+  if (!col_ok) return;
+  const int64_t slot = ((int64_t)ti * nh + head) * num_splits + split;
+  float* po = part_o + slot * HD;
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+    *reinterpret_cast<f32x4*>(po + db * 16 + g * 4) = o[0][db];
+  if (g == 0) {
+    part_ml[slot * 2] = m[0];
+    part_ml[slot * 2 + 1] = l[0];
+  }
+}
+
+// grid (decode tokens, nh), 64 threads: merges the splits of one (token, head) in ascending order.
+__global__ __launch_bounds__(64) void attn_decode_combine_kernel(
+    bf16_t* __restrict__ out, int64_t out_stride, const float* __restrict__ part_o,
+    const float* __restrict__ part_ml, const int32_t* __restrict__ token_list, int nh, int num_splits) {
+  const int ti = blockIdx.x, head = blockIdx.y;
+  const int64_t base = ((int64_t)ti * nh + head) * num_splits;
+  float mx = -INFINITY;
+  for (int s = 0; s < num_splits; ++s) mx = fmaxf(mx, part_ml[(base + s) * 2]);
+  float total = 0.f;
+  for (int s = 0; s < num_splits; ++s) {
+    const float ms = part_ml[(base + s) * 2];
+    if (ms != -INFINITY) total += part_ml[(base + s) * 2 + 1] * __expf(ms - mx);
+  }
+  const float inv = 1.f / total;
+  bf16_t* op = out + (int64_t)token_list[ti] * out_stride + (int64_t)head * HD;
+  for (int d = threadIdx.x; d < HD; d += 64) {
+    float acc = 0.f;
+    for (int s = 0; s < num_splits; ++s) {
+      const float ms = part_ml[(base + s) * 2];
+      if (ms != -INFINITY) acc += part_o[(base + s) * HD + d] * __expf(ms - mx);
+    }
+    op[d] = f32_to_bf16(acc * inv);
+  }
+}
+
+// ----------------------------------------------------------------------------- prefill
+// grid (tiles, nkv * head_blocks); a workgroup holds `waves` wavefronts, one query head each.
+// tiles: int32 [n][4] = (entry, first token row of the step, rows (<= 16*PREFILL_NB), first position).
+__global__ __launch_bounds__(512) void attn_prefill_kernel(
+    bf16_t* __restrict__ out, int64_t out_stride, const bf16_t* __restrict__ q, int64_t q_stride,
+    const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
+    const int32_t* __restrict__ block_table, int table_width, const int32_t* __restrict__ tiles, int nh,
+    int nkv, int head_blocks, int waves, int ps_shift, int window, float scale) {
+  constexpr int NB = PREFILL_NB;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c = lane & 15, g = lane >> 4;
+  const int kvh = blockIdx.y / head_blocks, hb = blockIdx.y % head_blocks;
+  const int group = nh / nkv;
+  if (hb * waves + wave >= group) return;          // the whole wavefront leaves; nothing is shared
+  const int head = kvh * group + hb * waves + wave;
+  const int32_t* tile = tiles + (int64_t)blockIdx.x * 4;
+  const int entry = tile[0], row0 = tile[1], rows = tile[2], pos0 = tile[3];
+
+  f32x4 o[NB][DB];
+  float m[NB], l[NB];
+  init_state<NB>(o, m, l);
+  bf16x8 qr[NB][KB];
+  int cpos[NB], clo[NB];
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) {
+    const int j = nb * 16 + c;
+    const bool ok = j < rows;
+    cpos[nb] = ok ? pos0 + j : -1;
+    clo[nb] = (window > 0 && pos0 + j - window + 1 > 0) ? pos0 + j - window + 1 : 0;
+    load_q(qr[nb], ok ? q + (int64_t)(row0 + j) * q_stride + (int64_t)head * HD : nullptr, g);
+  }
+  const int kv_min = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;
+  const int kv_max = pos0 + rows - 1;
+  attend_tiles<NB>(o, m, l, qr, cpos, clo, k_pages, v_pages, block_table + (int64_t)entry * table_width, kvh,
+                   nkv, ps_shift, kv_min, kv_max, (kv_min / 32) * 32, (kv_max / 32 + 1) * 32, scale);
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) {
+    const int j = nb * 16 + c;
+    if (j >= rows) continue;
+    const float inv = 1.f / l[nb];
+    bf16_t* op = out + (int64_t)(row0 + j) * out_stride + (int64_t)head * HD + g * 4;
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+      union { uint2 u; bf16_t e[4]; } pk;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) pk.e[i] = f32_to_bf16(o[nb][db][i] * inv);
+      *reinterpret_cast<uint2*>(op + db * 16) = pk.u;
+    }
+  }
+}
+
+extern "C" int ga_attn_head_dim() { return HD; }
+extern "C" int ga_attn_prefill_tile_rows() { return 16 * PREFILL_NB; }
+
+// Decode tokens: token_list names the rows of the step that are single new tokens.  workspace_o must
+// hold n_tokens*nh*num_splits*HD floats and workspace_ml n_tokens*nh*num_splits*2.
+extern "C" int ga_attn_decode(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* k_pages,
+                              const void* v_pages, const void* block_table, int table_width,
+                              const void* token_entry, const void* positions, const void* token_list,
+                              int n_tokens, int nh, int nkv, int page_size, int window, float scale,
+                              int split_keys, int num_splits, void* workspace_o, void* workspace_ml,
+                              hipStream_t stream) {
+  if (n_tokens <= 0) return 0;
+  if (nkv <= 0 || nh % nkv) return -1;
+  int ps_shift = 0;
+  while ((1 << ps_shift) < page_size) ++ps_shift;
+  if ((1 << ps_shift) != page_size || page_size < 8) return -2;
+  if (split_keys <= 0 || split_keys % 32 || num_splits <= 0 || num_splits > 65535) return -3;
+  const int group = nh / nkv, head_blocks = (group + 15) / 16;
+  if ((int64_t)nkv * head_blocks > 65535) return -4;
+  dim3 grid(n_tokens, nkv * head_blocks, num_splits);
+  hipLaunchKernelGGL(attn_decode_split_kernel, grid, dim3(64), 0, stream, (float*)workspace_o,
+                     (float*)workspace_ml, (const bf16_t*)q, q_stride, (const bf16_t*)k_pages,
+                     (const bf16_t*)v_pages, (const int32_t*)block_table, table_width,
+                     (const int32_t*)token_entry, (const int32_t*)positions, (const int32_t*)token_list, nh, nkv,
+                     head_blocks, ps_shift, window, scale, split_keys, num_splits);
+  int rc = GA_CHECK_LAUNCH();
+  if (rc) return rc;
+  hipLaunchKernelGGL(attn_decode_combine_kernel, dim3(n_tokens, nh), dim3(64), 0, stream, (bf16_t*)out,
+                     out_stride, (const float*)workspace_o, (const float*)workspace_ml,
+                     (const int32_t*)token_list, nh, num_splits);
+  return GA_CHECK_LAUNCH();
+}
+
+extern "C" int ga_attn_prefill(void* out, int64_t out_stride, const void* q, int64_t q_stride,
+                               const void* k_pages, const void* v_pages, const void* block_table,
+                               int table_width, const void* tiles, int n_tiles, int nh, int nkv, int page_size,
+                               int window, float scale, hipStream_t stream) {
+  if (n_tiles <= 0) return 0;
+  if (nkv <= 0 || nh % nkv) return -1;
+  int ps_shift = 0;
+  while ((1 << ps_shift) < page_size) ++ps_shift;
+  if ((1 << ps_shift) != page_size || page_size < 8) return -2;
+  const int group = nh / nkv;
+  const int waves = group < 8 ? group : 8;
+  const int head_blocks = (group + waves - 1) / waves;
+  if ((int64_t)nkv * head_blocks > 65535) return -4;
+  hipLaunchKernelGGL(attn_prefill_kernel, dim3(n_tiles, nkv * head_blocks), dim3(64 * waves), 0, stream,
+                     (bf16_t*)out, out_stride, (const bf16_t*)q, q_stride, (const bf16_t*)k_pages,
+                     (const bf16_t*)v_pages, (const int32_t*)block_table, table_width, (const int32_t*)tiles,
+                     nh, nkv, head_blocks, waves, ps_shift, window, scale);
+  return GA_CHECK_LAUNCH();
+}

@@ -6,8 +6,11 @@
 // tables, one rounding.  Formula: ginfer/core/op/kernels/cuda/rope_kernel.cu:83-102; cache write:
 // ginfer/core/op/kernels/cuda/store_kvcache_kernel.cu:19-30 (which indexes with 32-bit ints; the
 // offsets here are 64-bit).
-// Cache layout of one layer: pages[page][kv_head][slot_in_page][head_dim]; the slot of token t is
-// slot_mapping[t] = page * page_size + slot_in_page, or -1 to write nothing for that token.
+// Cache layout of one layer: keys  k_pages[page][kv_head][slot_in_page][head_dim],
+//                            values v_pages[page][kv_head][head_dim][slot_in_page]  (transposed, so
+// that the matrix-core attention kernels read 8 consecutive keys of one dimension in one 16-byte
+// load).  The slot of token t is slot_mapping[t] = page * page_size + slot_in_page, or -1 to write
+// nothing for that token.
 #include "common.cuh"
 
 template <typename T>
@@ -22,13 +25,14 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, const int32_t* __restr
   T* x = qkv + (t * (nh + 2 * nkv) + head) * (int64_t)hd;
   const int p = positions[t];
   const bool is_q = head < nh, is_k = !is_q && head < nh + nkv;
-  T* dst = nullptr;
+  T* dst = nullptr;   // k: the slot's row of head_dim; v: the slot's column, elements page_size apart
   if (!is_q && write_kv) {
     const int64_t slot = slot_mapping[t];
     if (slot >= 0) {
       const int g = is_k ? head - nh : head - nh - nkv;
       const int64_t page = slot / page_size, off = slot - page * page_size;
-      dst = (is_k ? k_pages : v_pages) + ((page * nkv + g) * page_size + off) * hd;
+      dst = is_k ? k_pages + ((page * nkv + g) * page_size + off) * hd
+                 : v_pages + (page * nkv + g) * (int64_t)hd * page_size + off;
     }
   }
   if (is_q || is_k) {
@@ -48,7 +52,7 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, const int32_t* __restr
     if (dst)
       for (int j = rotary_dim + threadIdx.x; j < hd; j += blockDim.x) dst[j] = x[j];
   } else if (dst) {
-    for (int j = threadIdx.x; j < hd; j += blockDim.x) dst[j] = x[j];
+    for (int j = threadIdx.x; j < hd; j += blockDim.x) dst[(int64_t)j * page_size] = x[j];
   }
 }
 

@@ -50,7 +50,7 @@ class ModelRunner:
         for p in self.model.position_parts():
             p.limit_positions(self.max_model_len)
         # compile what this model needs, all at once, before anything runs
-        build.build_all(modules=[m for m in self.model.kernel_modules() if m in build.available_modules()])
+        build.build_all(modules=self.model.kernel_modules())
         load_weights(self.model, model_path, self.device)
         self.page_size = int(page_size)
         specs = self.model.cache_specs()
@@ -176,8 +176,8 @@ class ModelRunner:
             if isinstance(spec, KVCacheSpec):
                 gi, j = cache.group_of[owner]
                 bt, slots = group_views[gi]
-                t = cache.groups[gi].tensor
-                caches.append(KVView(t[j, 0], t[j, 1], bt, slots, ps, owner == i))
+                kp, vp = cache.kv_views(owner)
+                caches.append(KVView(kp, vp, bt, slots, ps, owner == i))
             elif isinstance(spec, StateSpec):
                 caches.append(StateView(cache.state_tensors[owner], state_slots, owner == i))
             else:

@@ -23,8 +23,11 @@ ARCH = "gfx950"
 # packed 32-bit float instructions are switched off for all device code
 FLAGS = ["--offload-arch=" + ARCH, "-O3", "-std=c++17", "-shared", "-fPIC",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
-MODULES = ("embedding", "norm", "rope_kv", "attention_generic", "attention_decode",
-           "attention_prefill", "gemm", "gemm_skinny", "activation", "sampling")
+MODULES = ("embedding", "norm", "rope_kv", "attention_generic", "attention_mfma", "gemm", "gemm_skinny",
+           "activation", "sampling")
+# Modules that are compiled for one value of a parameter (a macro) at a time; build_all() without a
+# list compiles these values, and any other value a model needs is compiled when it is first asked for.
+VARIANTS = {"attention_mfma": [{"HEAD_DIM": hd} for hd in (16, 32, 48, 64, 80, 128, 256)]}
 
 _loaded = {}
 _lock = threading.Lock()
@@ -45,12 +48,24 @@ def _hipcc():
     return None
 
 
+def _split(module):
+    """A module is named "source" or ("source", {macro: value}); returns (source, defines, library stem)."""
+    if isinstance(module, str):
+        return module, {}, module
+    src, defines = module
+    defines = dict(defines or {})
+    stem = src + "".join("_%s%s" % (k, defines[k]) for k in sorted(defines))
+    return src, defines, stem
+
+
 def _digest(module):
+    src, defines, _ = _split(module)
     h = hashlib.sha256()
-    for name in (module + ".hip", "common.cuh"):
+    for name in (src + ".hip", "common.cuh"):
         with open(os.path.join(CSRC, name), "rb") as f:
             h.update(f.read())
     h.update(" ".join(FLAGS).encode())
+    h.update(repr(sorted(defines.items())).encode())
     return h.hexdigest()[:16]
 
 
@@ -76,9 +91,10 @@ def _writable_dir():
 
 
 def _find_built(module, digest):
+    stem = _split(module)[2]
     for d in _build_dirs():
-        so = os.path.join(d, "lib%s.so" % module)
-        stamp = os.path.join(d, "%s.stamp" % module)
+        so = os.path.join(d, "lib%s.so" % stem)
+        stamp = os.path.join(d, "%s.stamp" % stem)
         try:
             with open(stamp) as f:
                 if f.read().strip() == digest and os.path.isfile(so):
@@ -99,9 +115,12 @@ def compile_module(module, out_dir=None, quiet=False):
     if hipcc is None:
         raise KernelBuildError("hipcc not found: cannot build kernel library %r" % module)
     out_dir = out_dir or _writable_dir()
-    so = os.path.join(out_dir, "lib%s.so" % module)
+    src, defines, stem = _split(module)
+    so = os.path.join(out_dir, "lib%s.so" % stem)
     tmp = so + ".%d.tmp" % os.getpid()
-    cmd = [hipcc] + FLAGS + ["-I", CSRC, "-o", tmp, os.path.join(CSRC, module + ".hip")]
+    cmd = ([hipcc] + FLAGS + ["-D%s=%s" % kv for kv in sorted(defines.items())]
+           + ["-I", CSRC, "-o", tmp, os.path.join(CSRC, src + ".hip")])
+    module = stem
     env = dict(os.environ)
     env.setdefault("HOME", tempfile.gettempdir())   # hipcc wants a home for its caches
     t0 = time.time()
@@ -123,51 +142,59 @@ def compile_module(module, out_dir=None, quiet=False):
             os.remove(tmp)
         raise KernelBuildError("hipcc failed for %s:\n%s" % (module, log))
     os.replace(tmp, so)
-    with open(os.path.join(out_dir, "%s.stamp" % module), "w") as f:
-        f.write(_digest(module))
+    with open(os.path.join(out_dir, "%s.stamp" % stem), "w") as f:
+        f.write(_digest((src, defines) if defines else src))
     return so
 
 
 def build_all(force=False, modules=None, quiet=False):
     """Builds every module (in parallel); with force, also those already built."""
     from concurrent.futures import ThreadPoolExecutor
-    modules = list(modules or available_modules())
+    if modules is None:
+        modules = []
+        for m in available_modules():
+            modules.extend([(m, v) for v in VARIANTS[m]] if m in VARIANTS else [m])
+    modules = [m for m in modules if os.path.isfile(os.path.join(CSRC, _split(m)[0] + ".hip"))]
     todo = [m for m in modules if force or _find_built(m, _digest(m)) is None]
     if not todo:
         return
     out_dir = _writable_dir()
     if not quiet:
         _say("compiling %d kernel librar%s for %s: %s" % (len(todo), "y" if len(todo) == 1 else "ies",
-                                                        ARCH, ", ".join(todo)))
+                                                        ARCH, ", ".join(_split(m)[2] for m in todo)))
     done = []
 
     def one(m):
         compile_module(m, out_dir, quiet=quiet)
         done.append(m)
         if not quiet:
-            _say("compiled %s (%d/%d)" % (m, len(done), len(todo)))
+            _say("compiled %s (%d/%d)" % (_split(m)[2], len(done), len(todo)))
     workers = max(1, min(len(todo), (os.cpu_count() or 4), 8))
     with ThreadPoolExecutor(workers) as ex:
         list(ex.map(one, todo))
 
 
-def load(module):
-    """The ctypes library of a module, building it first if it is missing or stale."""
+def load(module, defines=None):
+    """The ctypes library of a module (for one set of macro values), building it first if it is
+    missing or stale."""
+    if defines:
+        module = (module, dict(defines))
+    src, _, stem = _split(module)
     with _lock:
-        if module in _loaded:
-            return _loaded[module]
-        if not os.path.isfile(os.path.join(CSRC, module + ".hip")):
-            raise KernelBuildError("no kernel source for module %r in %s" % (module, CSRC))
+        if stem in _loaded:
+            return _loaded[stem]
+        if not os.path.isfile(os.path.join(CSRC, src + ".hip")):
+            raise KernelBuildError("no kernel source for module %r in %s" % (src, CSRC))
         digest = _digest(module)
         so = _find_built(module, digest)
         if so is None:
-            _say("kernel library %r is not built yet; compiling it for %s" % (module, ARCH))
+            _say("kernel library %r is not built yet; compiling it for %s" % (stem, ARCH))
             so = compile_module(module)
-            _say("compiled %s" % module)
+            _say("compiled %s" % stem)
         import torch  # noqa: F401  the HIP runtime that torch loaded is the one the library binds to
         try:
             lib = ctypes.CDLL(so)
         except OSError as e:
             raise KernelBuildError("cannot load kernel library %s: %s" % (so, e))
-        _loaded[module] = lib
+        _loaded[stem] = lib
         return lib

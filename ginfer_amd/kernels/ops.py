@@ -114,7 +114,7 @@ def silu_mul(gate_up, out=None):
 def rope_kv_write(qkv, positions, cos, sin, slot_mapping, k_pages, v_pages, num_heads, num_kv_heads,
                   head_dim, write_kv=True):
     """Rotates q and k inside qkv [T, (nh + 2 nkv) hd] in place and writes k, v to the paged cache
-    [pages, nkv, page_size, hd] at slot_mapping [T] int64 (-1: skip).  cos, sin: float32
+    (k [pages, nkv, page_size, hd], v [pages, nkv, hd, page_size]) at slot_mapping [T] int64 (-1: skip).  cos, sin: float32
     [positions, rotary_dim / 2]."""
     _dev(qkv, positions, cos, sin, slot_mapping, k_pages, v_pages)
     T = qkv.shape[0]
@@ -130,12 +130,7 @@ def rope_kv_write(qkv, positions, cos, sin, slot_mapping, k_pages, v_pages, num_
     if write_kv:
         _need(slot_mapping is not None and slot_mapping.dtype == torch.int64 and slot_mapping.shape == (T,)
               and slot_mapping.is_contiguous(), "slot_mapping must be contiguous int64 [T]")
-        for p in (k_pages, v_pages):
-            _need(p is not None and p.dtype == qkv.dtype and p.dim() == 4 and p.is_contiguous()
-                  and p.shape[1] == num_kv_heads and p.shape[3] == head_dim,
-                  "cache pages must be contiguous %s [pages, %d, page_size, %d]" % (qkv.dtype, num_kv_heads, head_dim))
-        _need(k_pages.shape == v_pages.shape, "k and v pages differ in shape")
-        page_size = k_pages.shape[2]
+        page_size = _check_pages(k_pages, v_pages, qkv.dtype, num_kv_heads, head_dim)
     lib = build.load("rope_kv")
     _check(lib.ga_rope_kv_write(_ptr(qkv), _ptr(positions), _ptr(cos), _ptr(sin), _ptr(slot_mapping),
                                 _ptr(k_pages), _ptr(v_pages), _i(T), _i(num_heads), _i(num_kv_heads),
@@ -143,15 +138,25 @@ def rope_kv_write(qkv, positions, cos, sin, slot_mapping, k_pages, v_pages, num_
                                 _i(_is_bf16(qkv.dtype)), _stream()), "rope_kv_write")
 
 
+def _check_pages(k_pages, v_pages, dtype, nkv, hd):
+    """k_pages [pages, nkv, page_size, hd], v_pages [pages, nkv, hd, page_size] (values transposed)."""
+    _need(k_pages is not None and v_pages is not None, "cache pages are missing")
+    for p in (k_pages, v_pages):
+        _need(p.dtype == dtype and p.dim() == 4 and p.is_contiguous() and p.shape[1] == nkv,
+              "cache pages must be contiguous %s with %d kv heads" % (dtype, nkv))
+    ps = k_pages.shape[2]
+    _need(k_pages.shape[3] == hd and tuple(v_pages.shape) == (k_pages.shape[0], nkv, hd, ps),
+          "cache pages must be k [pages, %d, page_size, %d] and v [pages, %d, %d, page_size], got %s and %s"
+          % (nkv, hd, nkv, hd, tuple(k_pages.shape), tuple(v_pages.shape)))
+    return ps
+
+
 def _check_attention_operands(q, k_pages, v_pages, block_table, token_entry, positions, nh, nkv, hd):
     _dev(q, k_pages, v_pages, block_table, token_entry, positions)
     T = q.shape[0]
     _need(q.dim() == 2 and q.stride(1) == 1 and q.shape[1] >= nh * hd, "q must be [T, >= nh*hd] with unit inner stride")
     _need(nkv > 0 and nh % nkv == 0, "num_heads %d is not a multiple of num_kv_heads %d" % (nh, nkv))
-    for p in (k_pages, v_pages):
-        _need(p.dtype == q.dtype and p.dim() == 4 and p.is_contiguous() and p.shape[1] == nkv and p.shape[3] == hd,
-              "cache pages must be contiguous %s [pages, %d, page_size, %d]" % (q.dtype, nkv, hd))
-    _need(k_pages.shape == v_pages.shape, "k and v pages differ in shape")
+    _check_pages(k_pages, v_pages, q.dtype, nkv, hd)
     _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous(),
           "block_table must be contiguous int32 [entries, width]")
     for name, x in (("token_entry", token_entry), ("positions", positions)):
@@ -228,8 +233,101 @@ def gemm_skinny_supported(a, w):
     return False
 
 
+# ----------------------------------------------------------------------------- attention on the matrix cores
+
+MFMA_HEAD_DIMS = tuple(range(16, 257, 16))
+_DECODE_TARGET_WAVEFRONTS = 1024      # enough single-wavefront workgroups to fill 256 compute units
+_MIN_SPLIT_KEYS = 64
+
+
+def attention_mfma_supported(dtype, head_dim, page_size):
+    return (dtype == torch.bfloat16 and head_dim in MFMA_HEAD_DIMS and page_size >= 8
+            and page_size & (page_size - 1) == 0)
+
+
+def _attention_plan(step, tile_rows, device):
+    """Which rows of the step are single new tokens and how the rows of prompt portions fall into tiles;
+    made once per step and shared by all layers."""
+    key = ("attention_plan", tile_rows)
+    plan = step.extra.get(key)
+    if plan is not None:
+        return plan
+    import numpy as np
+    decode_rows, decode_pos, tiles = [], [], []
+    o = 0
+    for e in range(step.num_entries):
+        n, start = step.host_q_len[e], step.host_q_start[e]
+        if n == 1:
+            decode_rows.append(o)
+            decode_pos.append(start)
+        else:
+            for r in range(0, n, tile_rows):
+                tiles.append((e, o + r, min(tile_rows, n - r), start + r))
+        o += n
+    tiles.sort(key=lambda t: -(t[3] + t[2]))      # the tiles with the most keys first
+    plan = dict(
+        n_decode=len(decode_rows), decode_pos=decode_pos, n_tiles=len(tiles),
+        token_list=(torch.tensor(decode_rows, dtype=torch.int32, device=device) if decode_rows else None),
+        tiles=(torch.tensor(np.asarray(tiles, dtype=np.int32).reshape(-1, 4), device=device) if tiles else None))
+    step.extra[key] = plan
+    return plan
+
+
+def _decode_splits(plan, window, nkv, head_blocks):
+    span = 0
+    for pos in plan["decode_pos"]:
+        lo = max(0, pos - window + 1) if window else 0
+        span = max(span, pos + 1 - (lo // 32) * 32)
+    per_split = plan["n_decode"] * nkv * head_blocks
+    splits = max(1, min(_DECODE_TARGET_WAVEFRONTS // max(per_split, 1), -(-span // _MIN_SPLIT_KEYS)))
+    split_keys = -(-(-(-span // splits)) // 32) * 32
+    return split_keys, -(-span // split_keys)
+
+
+def paged_attention_mfma(q, k_pages, v_pages, block_table, step, num_heads, num_kv_heads, head_dim, scale,
+                         window=None, out=None):
+    """bfloat16 attention of every token of the step on the matrix cores: single new tokens through the
+    split-key kernel, rows of prompt portions through the tiled kernel."""
+    T = _check_attention_operands(q, k_pages, v_pages, block_table, step.token_entry, step.positions, num_heads,
+                                  num_kv_heads, head_dim)
+    page_size = k_pages.shape[2]
+    _need(attention_mfma_supported(q.dtype, head_dim, page_size),
+          "the matrix-core attention kernels take bfloat16, head sizes in steps of 16 up to 256 and page sizes that "
+          "are powers of two from 8; got %s, head %d, page %d" % (q.dtype, head_dim, page_size))
+    _need(q.stride(0) % 8 == 0 and q.data_ptr() % 16 == 0, "q rows must be 16-byte aligned")
+    lib = build.load("attention_mfma", {"HEAD_DIM": head_dim})
+    _need(lib.ga_attn_head_dim() == head_dim, "attention library was built for another head size")
+    plan = _attention_plan(step, lib.ga_attn_prefill_tile_rows(), q.device)
+    _need(sum(step.host_q_len) == T, "the step's entries do not add up to its tokens")
+    if out is None:
+        out = torch.empty((T, num_heads * head_dim), dtype=q.dtype, device=q.device)
+    _need(out.dtype == q.dtype and out.shape == (T, num_heads * head_dim) and out.is_contiguous(), "out must be [T, nh*hd]")
+    w = int(window) if window else 0
+    if plan["n_decode"]:
+        group = num_heads // num_kv_heads
+        split_keys, num_splits = _decode_splits(plan, w, num_kv_heads, -(-group // 16))
+        n = plan["n_decode"] * num_heads * num_splits
+        ws_o = torch.empty((n * head_dim,), dtype=torch.float32, device=q.device)
+        ws_ml = torch.empty((n * 2,), dtype=torch.float32, device=q.device)
+        _check(lib.ga_attn_decode(
+            _ptr(out), _i64(out.stride(0)), _ptr(q), _i64(q.stride(0)), _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
+            _i(block_table.shape[1]), _ptr(step.token_entry), _ptr(step.positions), _ptr(plan["token_list"]),
+            _i(plan["n_decode"]), _i(num_heads), _i(num_kv_heads), _i(page_size), _i(w), _f(scale), _i(split_keys),
+            _i(num_splits), _ptr(ws_o), _ptr(ws_ml), _stream()), "attn_decode")
+    if plan["n_tiles"]:
+        _check(lib.ga_attn_prefill(
+            _ptr(out), _i64(out.stride(0)), _ptr(q), _i64(q.stride(0)), _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
+            _i(block_table.shape[1]), _ptr(plan["tiles"]), _i(plan["n_tiles"]), _i(num_heads), _i(num_kv_heads),
+            _i(page_size), _i(w), _f(scale), _stream()), "attn_prefill")
+    return out
+
+
 def paged_attention(q, k_pages, v_pages, block_table, step, num_heads, num_kv_heads, head_dim, scale, window=None):
     """Attention of every token of the step over its request's pages.  Chooses the kernel: the general
-    one in 32-bit; in bfloat16 the matrix-core kernels where they take the shape."""
+    one in 32-bit (fixed order of every sum: bit-identical however the work is cut); in bfloat16 the
+    matrix-core kernels where they take the shape."""
+    if attention_mfma_supported(q.dtype, head_dim, k_pages.shape[2]):
+        return paged_attention_mfma(q, k_pages, v_pages, block_table, step, num_heads, num_kv_heads, head_dim, scale,
+                                    window)
     return paged_attention_generic(q, k_pages, v_pages, block_table, step.token_entry, step.positions, num_heads,
                                    num_kv_heads, head_dim, scale, window)

@@ -54,7 +54,10 @@ class Attention(Part):
         self.b_o = t.get("o_proj.bias") if self.out_bias else None
 
     def kernel_modules(self):
-        return ["rope_kv", "attention_generic", "attention_decode", "attention_prefill", "gemm", "gemm_skinny"]
+        mods = ["rope_kv", "attention_generic", "gemm"]
+        if self.dtype == torch.bfloat16:
+            mods += [("attention_mfma", {"HEAD_DIM": self.hd}), "gemm_skinny"]
+        return mods
 
     def forward(self, x, step, cache):
         qkv = linear(x, self.w_qkv, self.b_qkv)

@@ -52,7 +52,7 @@ class LMHead(Part):
         self.weight = embedding_weight
 
     def kernel_modules(self):
-        return ["gemm", "gemm_skinny"]
+        return ["gemm"] + (["gemm_skinny"] if self.dtype == torch.bfloat16 else [])
 
     def forward(self, x):
         return linear(x, self.weight, None, out_dtype=torch.float32)

@@ -28,7 +28,7 @@ class SwiGLU(Part):
         self.w_down = t["down_proj.weight"]
 
     def kernel_modules(self):
-        return ["activation", "gemm", "gemm_skinny"]
+        return ["activation", "gemm"] + (["gemm_skinny"] if self.dtype == torch.bfloat16 else [])
 
     def forward(self, x):
         gu = linear(x, self.w_gate_up)

@@ -12,7 +12,7 @@ from .base import KVCacheSpec, StateSpec
 class KVView:
     """What an attention-like mixer sees of the cache for the schedule entry that is running."""
     k_pages: torch.Tensor          # [pages, nkv, page_size, hd]
-    v_pages: torch.Tensor
+    v_pages: torch.Tensor          # [pages, nkv, hd, page_size]: values are kept transposed
     block_table: torch.Tensor      # int32 [entries, width]; -1 where a page was given back
     slot_mapping: torch.Tensor     # int64 [T]: page * page_size + offset for every token of the step
     page_size: int
@@ -113,7 +113,7 @@ class DecoderModel:
     def kernel_modules(self):
         mods = []
         for _, part in self._named_parts():
-            for m in part.kernel_modules():
+            for m in part.kernel_modules():     # a name, or (name, {macro: value})
                 if m not in mods:
                     mods.append(m)
         return mods

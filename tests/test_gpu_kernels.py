@@ -122,7 +122,7 @@ def test_rope_and_cache_write(dtype, tol, T, nh, nkv, hd, rd, theta):
     slots = torch.randperm(pages * ps)[:T].to(torch.int64)
     slots[1] = -1 if T > 1 else slots[1]
     kp = rnd((pages, nkv, ps, hd), dtype, 13)
-    vp = rnd((pages, nkv, ps, hd), dtype, 14)
+    vp = rnd((pages, nkv, hd, ps), dtype, 14)
     kp0, vp0 = kp.clone(), vp.clone()
     x = qkv.clone()
     ops.rope_kv_write(x, positions, cos.to(dev()), sin.to(dev()), slots.to(dev()), kp, vp, nh, nkv, hd)
@@ -143,7 +143,7 @@ def test_rope_and_cache_write(dtype, tol, T, nh, nkv, hd, rd, theta):
         if s < 0:
             continue
         kexp[s // ps, :, s % ps, :] = xk[t]
-        vexp[s // ps, :, s % ps, :] = v[t]
+        vexp[s // ps, :, :, s % ps] = v[t]
     assert torch.equal(kp.cpu(), kexp) and torch.equal(vp.cpu(), vexp)
     # a run that reads another layer's cache writes nothing
     kp1, vp1 = kp0.clone(), vp0.clone()
@@ -165,7 +165,7 @@ def _paged_case(seqs, nh, nkv, hd, ps, dtype, seed, window=None, spike=None):
     width = max(blocks) + 1
     bt = torch.full((E, width), -1, dtype=torch.int32)
     kp = torch.full((num_pages, nkv, ps, hd), float("nan"))
-    vp = torch.full((num_pages, nkv, ps, hd), float("nan"))
+    vp = torch.full((num_pages, nkv, hd, ps), float("nan"))
     T = sum(q for q, _ in seqs)
     q = torch.randn((T, nh, hd), generator=g)
     ent, pos = [], []
@@ -189,7 +189,7 @@ def _paged_case(seqs, nh, nkv, hd, ps, dtype, seed, window=None, spike=None):
         bt[e, :len(pages)] = torch.tensor(pages, dtype=torch.int32)
         for c in range(kv):
             kp[pages[c // ps], :, c % ps, :] = k[c]
-            vp[pages[c // ps], :, c % ps, :] = v[c]
+            vp[pages[c // ps], :, :, c % ps] = v[c]
         qe = q[o:o + ql].to(dtype).float()
         refs.append(pm.attention(qe.double(), k.double(), v.double(), qpos, window))
         ent += [e] * ql
@@ -307,3 +307,65 @@ def test_kernels_refuse_what_they_cannot_take():
         ops.silu_mul(rnd((4, 7), torch.float32, 1))
     with pytest.raises(KernelError):
         ops.add_rmsnorm(torch.zeros(4, 8), None, torch.ones(8), 1e-6, torch.float32)      # CPU tensors
+
+
+# ----------------------------------------------------------------------------- matrix-core attention
+
+class _Step:
+    """The few fields of a step that the attention dispatcher reads."""
+
+    def __init__(self, seqs, a):
+        self.num_entries = len(seqs)
+        self.host_q_len = [q for q, _ in seqs]
+        self.host_q_start = [kv - q for q, kv in seqs]
+        self.token_entry, self.positions = a["token_entry"], a["positions"]
+        self.extra = {}
+
+
+MFMA_SEQS = ATTN_SEQS + [[(1, 31), (1, 32), (1, 33), (1, 64), (1, 65)], [(31, 31), (33, 95), (2, 2), (17, 100)],
+                         [(1, 5000)], [(300, 700)]]
+
+
+@pytest.mark.parametrize("nh,nkv,hd", ATTN_HEADS + [(40, 2, 64), (3, 1, 256), (18, 1, 16)])
+@pytest.mark.parametrize("seqs", MFMA_SEQS)
+def test_paged_attention_mfma(nh, nkv, hd, seqs):
+    from ginfer_amd.kernels import ops
+    if sum(kv for _, kv in seqs) * nkv * hd > 3e6 and (nh, nkv, hd) not in ((12, 2, 128), (6, 1, 32)):
+        pytest.skip("large case kept for two head shapes")
+    for ps in (16, 8, 64) if hd <= 48 else (16,):
+        a, ref, _ = _paged_case(seqs, nh, nkv, hd, ps, torch.bfloat16, seed=hd + ps)
+        out = ops.paged_attention_mfma(a["q"], a["k_pages"], a["v_pages"], a["block_table"], _Step(seqs, a), nh, nkv, hd,
+                                       1.0 / math.sqrt(hd))
+        close(out, ref, 2e-2)
+
+
+@pytest.mark.parametrize("window", [1, 5, 16, 40, 64, 100])
+def test_paged_attention_mfma_window(window):
+    from ginfer_amd.kernels import ops
+    nh, nkv, hd, ps = 6, 3, 48, 16
+    seqs = [(1, 200), (30, 90), (7, 7), (1, window), (1, window + 1), (50, 130), (1, 2000)]
+    a, ref, _ = _paged_case(seqs, nh, nkv, hd, ps, torch.bfloat16, seed=window, window=window)
+    out = ops.paged_attention_mfma(a["q"], a["k_pages"], a["v_pages"], a["block_table"], _Step(seqs, a), nh, nkv, hd,
+                                   1.0 / math.sqrt(hd), window=window)
+    close(out, ref, 2e-2)
+
+
+@pytest.mark.parametrize("where", ["first", "page_edge", "before_page_edge", "tile_edge", "before_tile_edge", "split_edge",
+                                   "last", "window_edge", "behind_window"])
+def test_paged_attention_mfma_finds_one_far_key(where):
+    from ginfer_amd.kernels import ops
+    nh, nkv, hd, ps = 4, 2, 32, 16
+    kv = 300
+    window = 100 if "window" in where else None
+    place = {"first": 0, "page_edge": 16 * 9, "before_page_edge": 16 * 9 - 1, "tile_edge": 32 * 3, "before_tile_edge": 95,
+             "split_edge": 64, "last": kv - 1, "window_edge": kv - 100, "behind_window": kv - 101}[where]
+    seqs = [(1, kv), (20, kv)]
+    a, ref, _ = _paged_case(seqs, nh, nkv, hd, ps, torch.bfloat16, seed=5, window=window, spike=lambda e, ql, n: place)
+    out = ops.paged_attention_mfma(a["q"], a["k_pages"], a["v_pages"], a["block_table"], _Step(seqs, a), nh, nkv, hd,
+                                   1.0 / math.sqrt(hd), window=window)
+    close(out, ref, 2e-2)
+    last_rows = out.float().cpu()[[0, 20]]
+    if where == "behind_window":
+        assert (last_rows.abs() < 3).all()
+    else:
+        assert (last_rows - 7.0).abs().max() < 0.1

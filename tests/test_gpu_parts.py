@@ -104,7 +104,7 @@ def test_attention_part_in_portions(dtype, tol, window):
                                 sin, cos, window)
     pages = 8
     kp = torch.full((pages, nkv, ps, hd), float("nan"), dtype=dtype, device=dev())
-    vp = torch.full((pages, nkv, ps, hd), float("nan"), dtype=dtype, device=dev())
+    vp = torch.full((pages, nkv, hd, ps), float("nan"), dtype=dtype, device=dev())
     table = [5, 2, 7, 0, 3, 6]
     outs = []
     for a, b in ((0, 20), (20, 22), (22, 45)):
