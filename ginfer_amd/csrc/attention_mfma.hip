@@ -180,15 +180,22 @@ __device__ __forceinline__ void load_q(bf16x8 (&q)[KB], const bf16_t* row /* nul
 }
 
 // ----------------------------------------------------------------------------- decode
-// grid (decode tokens, nkv * head_blocks, splits), one wavefront each.
+// grid (decode tokens, nkv * head_blocks, splits); a workgroup of DEC_WAVES wavefronts shares one split:
+// wavefront w takes the key tiles w, w + DEC_WAVES, ... of the split, and the states meet in LDS.
 // part_o: [n_tokens][nh][splits][HD] float; part_ml: [n_tokens][nh][splits][2] float (max, sum).
-__global__ __launch_bounds__(64) void attn_decode_split_kernel(
-    float* __restrict__ part_o, float* __restrict__ part_ml, const bf16_t* __restrict__ q, int64_t q_stride,
-    const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
-    const int32_t* __restrict__ block_table, int table_width, const int32_t* __restrict__ token_entry,
-    const int32_t* __restrict__ positions, const int32_t* __restrict__ token_list, int nh, int nkv,
-    int head_blocks, int ps_shift, int window, float scale, int split_keys, int num_splits) {
-  const int lane = threadIdx.x, c = lane & 15, g = lane >> 4;
+// With one split the normalised result goes straight to `out`.
+#define DEC_WAVES 4
+
+__global__ __launch_bounds__(64 * DEC_WAVES) void attn_decode_split_kernel(
+    bf16_t* __restrict__ out, int64_t out_stride, float* __restrict__ part_o, float* __restrict__ part_ml,
+    const bf16_t* __restrict__ q, int64_t q_stride, const bf16_t* __restrict__ k_pages,
+    const bf16_t* __restrict__ v_pages, const int32_t* __restrict__ block_table, int table_width,
+    const int32_t* __restrict__ token_entry, const int32_t* __restrict__ positions,
+    const int32_t* __restrict__ token_list, int nh, int nkv, int head_blocks, int ps_shift, int window,
+    float scale, int split_keys, int num_splits) {
+  __shared__ float o_s[DEC_WAVES][HD][17];
+  __shared__ float m_s[DEC_WAVES][16], l_s[DEC_WAVES][16];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c = lane & 15, g = lane >> 4;
   const int ti = blockIdx.x, split = blockIdx.z;
   const int kvh = blockIdx.y / head_blocks, hb = blockIdx.y % head_blocks;
   const int group = nh / nkv;
@@ -208,43 +215,80 @@ __global__ __launch_bounds__(64) void attn_decode_split_kernel(
     bf16x8 qr[1][KB];
     load_q(qr[0], col_ok ? q + (int64_t)t * q_stride + (int64_t)head * HD : nullptr, g);
     const int cpos[1] = {col_ok ? pos : -1}, clo[1] = {lo};
-    attend_tiles<1>(o, m, l, qr, cpos, clo, k_pages, v_pages,
-                    block_table + (int64_t)token_entry[t] * table_width, kvh, nkv, ps_shift, lo, pos, begin,
-                    end, scale);
+    const int32_t* bt = block_table + (int64_t)token_entry[t] * table_width;
+    for (int k0 = begin + 32 * wave; k0 < end; k0 += 32 * DEC_WAVES)
+      attend_tiles<1>(o, m, l, qr, cpos, clo, k_pages, v_pages, bt, kvh, nkv, ps_shift, lo, pos, k0, k0 + 32,
+                      scale);
   }
-  if (!col_ok) return;
-  const int64_t slot = ((int64_t)ti * nh + head) * num_splits + split;
-  float* po = part_o + slot * HD;
+  // the wavefronts' states meet: common max, rescaled sums and outputs added in wavefront order
+  if (g == 0) {
+    m_s[wave][c] = m[0];
+    l_s[wave][c] = l[0];
+  }
+  __syncthreads();
+  float mx = -INFINITY;
+#pragma unroll
+  for (int w = 0; w < DEC_WAVES; ++w) mx = fmaxf(mx, m_s[w][c]);
+  const float f = (m[0] == -INFINITY) ? 0.f : __expf(m[0] - mx);
 #pragma unroll
   for (int db = 0; db < DB; ++db)
-    *reinterpret_cast<f32x4*>(po + db * 16 + g * 4) = o[0][db];
-  if (g == 0) {
-    part_ml[slot * 2] = m[0];
-    part_ml[slot * 2 + 1] = l[0];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o_s[wave][db * 16 + g * 4 + i][c] = o[0][db][i] * f;
+  __syncthreads();
+  const int64_t slot_base = ((int64_t)ti * nh + kvh * group + hb * 16) * num_splits + split;
+  for (int idx = threadIdx.x; idx < 16 * HD; idx += 64 * DEC_WAVES) {
+    const int cc = idx / HD, d = idx % HD;
+    if (hb * 16 + cc >= group) continue;
+    // the thread's column cc is not the lane's own column c: its max is read again
+    float mcc = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < DEC_WAVES; ++w) mcc = fmaxf(mcc, m_s[w][cc]);
+    float lsum = 0.f, acc = 0.f;
+#pragma unroll
+    for (int w = 0; w < DEC_WAVES; ++w) {
+      const float mw = m_s[w][cc];
+      if (mw != -INFINITY) lsum += l_s[w][cc] * __expf(mw - mcc);
+      acc += o_s[w][d][cc];
+    }
+    if (num_splits == 1) {
+      out[(int64_t)t * out_stride + (int64_t)(kvh * group + hb * 16 + cc) * HD + d] = f32_to_bf16(acc / lsum);
+    } else {
+      const int64_t slot = slot_base + (int64_t)cc * num_splits;
+      part_o[slot * HD + d] = acc;
+      if (d == 0) {
+        part_ml[slot * 2] = mcc;
+        part_ml[slot * 2 + 1] = lsum;
+      }
+    }
   }
 }
 
 // grid (decode tokens, nh), 64 threads: merges the splits of one (token, head) in ascending order.
+#define MAX_SPLITS 256
 __global__ __launch_bounds__(64) void attn_decode_combine_kernel(
     bf16_t* __restrict__ out, int64_t out_stride, const float* __restrict__ part_o,
     const float* __restrict__ part_ml, const int32_t* __restrict__ token_list, int nh, int num_splits) {
-  const int ti = blockIdx.x, head = blockIdx.y;
+  __shared__ float w_s[MAX_SPLITS];
+  const int ti = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
   const int64_t base = ((int64_t)ti * nh + head) * num_splits;
   float mx = -INFINITY;
-  for (int s = 0; s < num_splits; ++s) mx = fmaxf(mx, part_ml[(base + s) * 2]);
+  for (int s = lane; s < num_splits; s += 64) mx = fmaxf(mx, part_ml[(base + s) * 2]);
+  mx = wave_max(mx);
   float total = 0.f;
-  for (int s = 0; s < num_splits; ++s) {
+  for (int s = lane; s < num_splits; s += 64) {
     const float ms = part_ml[(base + s) * 2];
-    if (ms != -INFINITY) total += part_ml[(base + s) * 2 + 1] * __expf(ms - mx);
+    const float w = ms == -INFINITY ? 0.f : __expf(ms - mx);
+    w_s[s] = w;
+    total += w * part_ml[(base + s) * 2 + 1];
   }
+  total = wave_sum(total);
+  __syncthreads();
   const float inv = 1.f / total;
   bf16_t* op = out + (int64_t)token_list[ti] * out_stride + (int64_t)head * HD;
-  for (int d = threadIdx.x; d < HD; d += 64) {
+  for (int d = lane; d < HD; d += 64) {
     float acc = 0.f;
-    for (int s = 0; s < num_splits; ++s) {
-      const float ms = part_ml[(base + s) * 2];
-      if (ms != -INFINITY) acc += part_o[(base + s) * HD + d] * __expf(ms - mx);
-    }
+#pragma unroll 8
+    for (int s = 0; s < num_splits; ++s) acc += part_o[(base + s) * HD + d] * w_s[s];
     op[d] = f32_to_bf16(acc * inv);
   }
 }
@@ -315,17 +359,18 @@ extern "C" int ga_attn_decode(void* out, int64_t out_stride, const void* q, int6
   int ps_shift = 0;
   while ((1 << ps_shift) < page_size) ++ps_shift;
   if ((1 << ps_shift) != page_size || page_size < 8) return -2;
-  if (split_keys <= 0 || split_keys % 32 || num_splits <= 0 || num_splits > 65535) return -3;
+  if (split_keys <= 0 || split_keys % 32 || num_splits <= 0) return -3;
   const int group = nh / nkv, head_blocks = (group + 15) / 16;
   if ((int64_t)nkv * head_blocks > 65535) return -4;
+  if (num_splits > MAX_SPLITS) return -5;
   dim3 grid(n_tokens, nkv * head_blocks, num_splits);
-  hipLaunchKernelGGL(attn_decode_split_kernel, grid, dim3(64), 0, stream, (float*)workspace_o,
-                     (float*)workspace_ml, (const bf16_t*)q, q_stride, (const bf16_t*)k_pages,
-                     (const bf16_t*)v_pages, (const int32_t*)block_table, table_width,
+  hipLaunchKernelGGL(attn_decode_split_kernel, grid, dim3(64 * DEC_WAVES), 0, stream, (bf16_t*)out, out_stride,
+                     (float*)workspace_o, (float*)workspace_ml, (const bf16_t*)q, q_stride,
+                     (const bf16_t*)k_pages, (const bf16_t*)v_pages, (const int32_t*)block_table, table_width,
                      (const int32_t*)token_entry, (const int32_t*)positions, (const int32_t*)token_list, nh, nkv,
                      head_blocks, ps_shift, window, scale, split_keys, num_splits);
   int rc = GA_CHECK_LAUNCH();
-  if (rc) return rc;
+  if (rc || num_splits == 1) return rc;
   hipLaunchKernelGGL(attn_decode_combine_kernel, dim3(n_tokens, nh), dim3(64), 0, stream, (bf16_t*)out,
                      out_stride, (const float*)workspace_o, (const float*)workspace_ml,
                      (const int32_t*)token_list, nh, num_splits);

@@ -9,86 +9,94 @@
 #include "common.cuh"
 
 #define SAMPLE_THREADS 1024
+#define SAMPLE_WAVES (SAMPLE_THREADS / WAVE)
 
 __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(
     int32_t* __restrict__ out, const float* __restrict__ logits, int64_t row_stride, int vocab,
     const float* __restrict__ temperature, const float* __restrict__ uniform) {
-  __shared__ float part_f[SAMPLE_THREADS];
-  __shared__ int part_i[SAMPLE_THREADS];
-  __shared__ int chosen;
-  const int r = blockIdx.x, tid = threadIdx.x;
+  __shared__ float part_f[SAMPLE_WAVES];
+  __shared__ int part_i[SAMPLE_WAVES];
+  __shared__ float seg_sum[SAMPLE_WAVES];
+  __shared__ float walk[2];
+  __shared__ int owner_s;
+  const int r = blockIdx.x, tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE;
   const float* x = logits + (int64_t)r * row_stride;
-  // contiguous chunk per thread, so that index order is thread order
-  const int chunk = (vocab + SAMPLE_THREADS - 1) / SAMPLE_THREADS;
-  const int begin = tid * chunk < vocab ? tid * chunk : vocab;
-  const int end = begin + chunk < vocab ? begin + chunk : vocab;
 
+  // ---- max and its lowest index: strided (coalesced) reads; a thread meets its indices in ascending order
   float best = -INFINITY;
   int best_i = 0x7fffffff;
-  for (int i = begin; i < end; ++i) {
+  for (int i = tid; i < vocab; i += SAMPLE_THREADS) {
     const float v = x[i];
-    if (best_i == 0x7fffffff || v > best) { best = v; best_i = i; }   // strictly greater: lowest index wins
+    if (best_i == 0x7fffffff || v > best) { best = v; best_i = i; }
   }
-  part_f[tid] = best;
-  part_i[tid] = best_i;
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const float b = __shfl_xor(best, o, WAVE);
+    const int bi = __shfl_xor(best_i, o, WAVE);
+    if (bi != 0x7fffffff && (best_i == 0x7fffffff || b > best || (b == best && bi < best_i))) { best = b; best_i = bi; }
+  }
+  if (lane == 0) { part_f[wave] = best; part_i[wave] = best_i; }
   __syncthreads();
-  for (int s = SAMPLE_THREADS / 2; s > 0; s >>= 1) {
-    if (tid < s) {
-      const float a = part_f[tid], b = part_f[tid + s];
-      const int ai = part_i[tid], bi = part_i[tid + s];
-      // among equal values the lower index wins (the two halves interleave index ranges)
-      if (bi != 0x7fffffff && (ai == 0x7fffffff || b > a || (b == a && bi < ai))) {
-        part_f[tid] = b;
-        part_i[tid] = bi;
-      }
-    }
-    __syncthreads();
+  float mx = part_f[0];
+  int arg = part_i[0];
+#pragma unroll
+  for (int w = 1; w < SAMPLE_WAVES; ++w) {
+    const float b = part_f[w];
+    const int bi = part_i[w];
+    if (bi != 0x7fffffff && (arg == 0x7fffffff || b > mx || (b == mx && bi < arg))) { mx = b; arg = bi; }
   }
-  const float mx = part_f[0];
-  const int arg = part_i[0];
   const float temp = temperature ? temperature[r] : 0.f;
   if (!(temp > 0.f)) {
     if (tid == 0) out[r] = arg;
     return;
   }
-  __syncthreads();
+  // ---- mass of each wavefront's contiguous segment of the vocabulary
   const float inv_t = 1.0f / temp;
+  const int seg = ((vocab + SAMPLE_WAVES - 1) / SAMPLE_WAVES + WAVE - 1) / WAVE * WAVE;
+  const int sb = wave * seg < vocab ? wave * seg : vocab;
+  const int se = sb + seg < vocab ? sb + seg : vocab;
   float sum = 0.f;
-  for (int i = begin; i < end; ++i) sum += expf((x[i] - mx) * inv_t);
-  part_f[tid] = sum;
-  if (tid == 0) chosen = -1;
+  for (int i = sb + lane; i < se; i += WAVE) sum += __expf((x[i] - mx) * inv_t);
+  sum = wave_sum(sum);
+  if (lane == 0) seg_sum[wave] = sum;
   __syncthreads();
   if (tid == 0) {
-    // serial scan over the thread sums: 1024 additions, in index order
     float total = 0.f;
-    for (int i = 0; i < SAMPLE_THREADS; ++i) total += part_f[i];
+    for (int w = 0; w < SAMPLE_WAVES; ++w) total += seg_sum[w];
     const float target = uniform[r] * total;
     float run = 0.f;
-    int owner = -1;
-    for (int i = 0; i < SAMPLE_THREADS; ++i) {
-      if (run + part_f[i] > target) { owner = i; break; }
-      run += part_f[i];
+    int owner = SAMPLE_WAVES - 1;
+    for (int w = 0; w < SAMPLE_WAVES; ++w) {
+      if (run + seg_sum[w] > target) { owner = w; break; }
+      if (w < SAMPLE_WAVES - 1) run += seg_sum[w];
     }
-    part_i[0] = owner;
-    part_f[0] = run;          // mass before the owner's chunk (the owner's own sum is not needed)
-    part_f[1] = target;
+    while (owner > 0 && owner * seg >= vocab) --owner;    // never an empty segment
+    owner_s = owner;
+    walk[0] = run;
+    walk[1] = target;
   }
   __syncthreads();
-  const int owner = part_i[0];
-  if (owner < 0) {            // rounding pushed the target past the end: the last index with mass
-    if (tid == 0) out[r] = vocab - 1;
-    return;
-  }
-  if (tid == owner) {
-    float run = part_f[0];
-    const float target = part_f[1];
-    int pick = end - 1;
-    for (int i = begin; i < end; ++i) {
-      run += expf((x[i] - mx) * inv_t);
-      if (run > target) { pick = i; break; }
+  if (wave != owner_s) return;
+  // ---- the owner walks its segment in index order, 64 tokens at a time, with a prefix sum over lanes
+  float run = walk[0];
+  const float target = walk[1];
+  int pick = se - 1;                       // if rounding leaves the target just past the segment's mass
+  for (int base = sb; base < se; base += WAVE) {
+    const int i = base + lane;
+    float e = i < se ? __expf((x[i] - mx) * inv_t) : 0.f;
+#pragma unroll
+    for (int o = 1; o < WAVE; o <<= 1) {   // inclusive prefix sum
+      const float up = __shfl_up(e, o, WAVE);
+      if (lane >= o) e += up;
     }
-    out[r] = pick;
+    const unsigned long long hit = __ballot(run + e > target && i < se);
+    if (hit) {
+      pick = base + __ffsll((long long)hit) - 1;
+      break;
+    }
+    run += __shfl(e, WAVE - 1, WAVE);
   }
+  if (lane == 0) out[r] = pick;
 }
 
 // out: [R] int32; logits: [R, vocab] float with row stride; temperature, uniform: [R] float

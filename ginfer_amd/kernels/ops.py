@@ -228,16 +228,45 @@ def sample_rows(logits, temperature=None, uniform=None, out=None):
     return out
 
 
+SKINNY_MAX_ROWS = 64
+
+
 def gemm_skinny_supported(a, w):
     """Whether the matrix-core kernel for few rows takes these operands."""
-    return False
+    return (a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and a.dim() == 2 and 0 < a.shape[0] <= SKINNY_MAX_ROWS
+            and a.shape[1] % 8 == 0 and a.stride(1) == 1 and a.stride(0) % 8 == 0 and a.data_ptr() % 16 == 0
+            and w.is_contiguous() and w.data_ptr() % 16 == 0)
+
+
+def gemm_skinny(a, w, bias=None, out=None, out_dtype=None):
+    """a [M <= 64, K] . w [N, K]^T (+ bias) -> [M, N] in bfloat16 (or float32): the decode step's products,
+    weights streamed once through the matrix cores."""
+    _dev(a, w, bias, out)
+    _need(a.dim() == 2 and w.dim() == 2 and a.shape[1] == w.shape[1], "gemm_skinny: a [M, K] and w [N, K] do not agree: %s, %s"
+          % (tuple(a.shape), tuple(w.shape)))
+    _need(gemm_skinny_supported(a, w), "gemm_skinny takes bfloat16, at most %d rows, K a multiple of 8 and 16-byte "
+          "aligned rows; got a %s %s, w %s %s" % (SKINNY_MAX_ROWS, a.dtype, tuple(a.shape), w.dtype, tuple(w.shape)))
+    M, K = a.shape
+    N = w.shape[0]
+    if bias is not None:
+        _need(bias.dtype == torch.bfloat16 and bias.shape == (N,) and bias.is_contiguous(), "gemm_skinny: bias must be bfloat16 [N]")
+    out_dtype = out_dtype or (out.dtype if out is not None else torch.bfloat16)
+    _need(out_dtype in (torch.bfloat16, torch.float32), "gemm_skinny: out dtype must be bfloat16 or float32")
+    if out is None:
+        out = torch.empty((M, N), dtype=out_dtype, device=a.device)
+    _need(out.shape == (M, N) and out.dtype == out_dtype and out.stride(1) == 1, "gemm_skinny: out must be [M, N]")
+    lib = build.load("gemm_skinny")
+    _check(lib.ga_gemm_skinny(_ptr(out), _i64(out.stride(0)), _ptr(a), _i64(a.stride(0)), _ptr(w), _ptr(bias), _i(M), _i(N),
+                              _i(K), _i(1 if out_dtype == torch.float32 else 0), _stream()), "gemm_skinny")
+    return out
 
 
 # ----------------------------------------------------------------------------- attention on the matrix cores
 
 MFMA_HEAD_DIMS = tuple(range(16, 257, 16))
-_DECODE_TARGET_WAVEFRONTS = 1024      # enough single-wavefront workgroups to fill 256 compute units
-_MIN_SPLIT_KEYS = 64
+_DECODE_TARGET_WORKGROUPS = 512       # four wavefronts each: enough to fill 256 compute units
+_MIN_SPLIT_KEYS = 128                 # one tile of 32 keys for each wavefront of a workgroup
+_MAX_SPLITS = 256
 
 
 def attention_mfma_supported(dtype, head_dim, page_size):
@@ -279,7 +308,7 @@ def _decode_splits(plan, window, nkv, head_blocks):
         lo = max(0, pos - window + 1) if window else 0
         span = max(span, pos + 1 - (lo // 32) * 32)
     per_split = plan["n_decode"] * nkv * head_blocks
-    splits = max(1, min(_DECODE_TARGET_WAVEFRONTS // max(per_split, 1), -(-span // _MIN_SPLIT_KEYS)))
+    splits = max(1, min(_DECODE_TARGET_WORKGROUPS // max(per_split, 1), -(-span // _MIN_SPLIT_KEYS), _MAX_SPLITS))
     split_keys = -(-(-(-span // splits)) // 32) * 32
     return split_keys, -(-span // split_keys)
 

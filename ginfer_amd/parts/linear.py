@@ -8,15 +8,12 @@ import torch
 
 from ..kernels import ops
 
-# up to this many rows the weight-streaming kernel is used in bfloat16
-SKINNY_MAX_ROWS = 64
-
 
 def linear(x, weight, bias=None, out_dtype=None):
     """x [M, K], weight [N, K], bias [N] | None -> [M, N] in x's dtype (or float32 on request)."""
     if x.dtype == torch.float32:
         return ops.gemm_nt(x, weight, bias)
-    if x.shape[0] <= SKINNY_MAX_ROWS and ops.gemm_skinny_supported(x, weight):
+    if ops.gemm_skinny_supported(x, weight):
         return ops.gemm_skinny(x, weight, bias, out_dtype=out_dtype)
     if out_dtype == torch.float32:
         y = torch.mm(x, weight.t(), out_dtype=torch.float32)

@@ -369,3 +369,36 @@ def test_paged_attention_mfma_finds_one_far_key(where):
         assert (last_rows.abs() < 3).all()
     else:
         assert (last_rows - 7.0).abs().max() < 0.1
+
+
+@pytest.mark.parametrize("M", [1, 2, 8, 16, 17, 33, 64])
+@pytest.mark.parametrize("N,K,bias", [(2048, 1536, True), (1536, 1536, False), (17920, 1536, False), (1536, 8960, False),
+                                      (1000, 192, True), (197, 4216, False), (33, 8, True), (777, 88, False), (5000, 72, True)])
+def test_gemm_skinny(M, N, K, bias):
+    from ginfer_amd.kernels import ops
+    a, w = rnd((M, K), torch.bfloat16, 30), rnd((N, K), torch.bfloat16, 31)
+    b = rnd((N,), torch.bfloat16, 32) if bias else None
+    assert ops.gemm_skinny_supported(a, w)
+    ref = a.double() @ w.double().t() + (b.double() if bias else 0)
+    close(ops.gemm_skinny(a, w, b), ref, 1e-2)
+    out = ops.gemm_skinny(a, w, b, out_dtype=torch.float32)
+    assert out.dtype == torch.float32
+    close(out, ref, 1e-5)
+    # a row does not depend on how many rows stand beside it
+    if M > 1:
+        one = ops.gemm_skinny(a[M - 1:M], w, b, out_dtype=torch.float32)
+        assert torch.equal(one[0], out[M - 1])
+    # rows of a wider buffer (a view with a row stride), as the fused projections hand them on
+    wide = rnd((M, K + 64), torch.bfloat16, 33)
+    view = wide[:, :K]
+    if ops.gemm_skinny_supported(view, w):
+        close(ops.gemm_skinny(view, w, b, out_dtype=torch.float32), view.double() @ w.double().t() + (b.double() if bias else 0), 1e-5)
+
+
+def test_gemm_skinny_refuses_other_shapes():
+    from ginfer_amd.kernels import ops, KernelError
+    assert not ops.gemm_skinny_supported(rnd((65, 64), torch.bfloat16, 1), rnd((8, 64), torch.bfloat16, 2))
+    assert not ops.gemm_skinny_supported(rnd((4, 12), torch.bfloat16, 1), rnd((8, 12), torch.bfloat16, 2))
+    assert not ops.gemm_skinny_supported(rnd((4, 64), torch.float32, 1), rnd((8, 64), torch.float32, 2))
+    with pytest.raises(KernelError):
+        ops.gemm_skinny(rnd((65, 64), torch.bfloat16, 1), rnd((8, 64), torch.bfloat16, 2))
