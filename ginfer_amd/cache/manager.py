@@ -17,6 +17,8 @@ entry's keys are viewed [pages, nkv, page_size, hd] and its values [pages, nkv, 
 from dataclasses import dataclass, field
 from typing import Dict, List, Optional
 
+import numpy as np
+
 from ..parts.base import KVCacheSpec, StateSpec
 from .pages import PagePool, SlotPool, OutOfPages
 
@@ -68,6 +70,11 @@ class CacheManager:
         self.slots = SlotPool(self.max_requests)
         self.state_tensors = {}          # schedule entry -> device tensor [max_requests, *shape]
         self.requests: Dict[object, _Request] = {}
+        # host mirrors for building a step without a Python loop per request: per group the block tables
+        # by state slot (int32, -1 where there is no page), and the lengths by state slot
+        self._table_np = [np.full((self.max_requests, 16), -1, dtype=np.int32) for _ in self.groups]
+        self._length_np = np.zeros(self.max_requests, dtype=np.int64)
+        self._any_window = any(g.window is not None for g in self.groups)
 
     # ---- device memory
     def bytes_per_page(self, element_size):
@@ -101,7 +108,11 @@ class CacheManager:
         if rid in self.requests:
             raise ValueError("request %r is already in the cache" % (rid,))
         self.requests[rid] = _Request(slot=self.slots.take(), tables=[[] for _ in self.groups])
-        return self.requests[rid].slot
+        slot = self.requests[rid].slot
+        for t in self._table_np:
+            t[slot, :] = -1
+        self._length_np[slot] = 0
+        return slot
 
     def length(self, rid):
         return self.requests[rid].length
@@ -167,6 +178,9 @@ class CacheManager:
             raise ValueError("request %r has %d reserved tokens that were not committed" % (rid, req.pending))
         if n_new < 1:
             raise ValueError("append needs at least one token")
+        if n_new == 1 and not self._any_window and req.length % self.page_size:
+            req.pending = 1              # the common decode step: room is left in the last page
+            return req.length
         plan = self._plan(req, n_new)
         for gi, (give, take, _, _) in enumerate(plan):
             if take > self.groups[gi].pool.num_free + len(give):
@@ -183,13 +197,32 @@ class CacheManager:
             for i in range(max(first, 0), need_blocks):
                 if table[i] < 0:
                     table[i] = next(new_pages)
+            mirror = self._table_np[gi]
+            if len(table) > mirror.shape[1]:
+                wider = np.full((self.max_requests, max(len(table), 2 * mirror.shape[1])), -1, dtype=np.int32)
+                wider[:, :mirror.shape[1]] = mirror
+                self._table_np[gi] = mirror = wider
+            mirror[req.slot, :len(table)] = table
         req.pending = n_new
         return req.length
+
+    def tables_array(self, group, slots, width):
+        """int32 [len(slots), width]: the block tables of the requests in these state slots."""
+        mirror = self._table_np[group]
+        if width > mirror.shape[1]:
+            out = np.full((len(slots), width), -1, dtype=np.int32)
+            out[:, :mirror.shape[1]] = mirror[slots]
+            return out
+        return mirror[slots, :width]
+
+    def lengths_array(self, slots):
+        return self._length_np[slots]
 
     def commit(self, rid):
         req = self.requests[rid]
         req.length += req.pending
         req.pending = 0
+        self._length_np[req.slot] = req.length
 
     def release(self, rid):
         """The request ends (or is evicted): every page and its slot go back."""
@@ -212,6 +245,13 @@ class CacheManager:
             held = set(g.pool.held())
             if held != set(seen):
                 raise AssertionError("group %d: pool holds %s, tables hold %s" % (gi, sorted(held), sorted(seen)))
+            for rid, req in self.requests.items():
+                row = self._table_np[gi][req.slot]
+                t = req.tables[gi]
+                if list(row[:len(t)]) != t or (row[len(t):] >= 0).any():
+                    raise AssertionError("group %d: the host mirror of %r's table differs from the table" % (gi, rid))
+                if self._length_np[req.slot] != req.length:
+                    raise AssertionError("the host mirror of %r's length differs" % (rid,))
             if len(held) + g.pool.num_free != g.pool.num_pages:
                 raise AssertionError("group %d: %d held + %d free != %d pages"
                                      % (gi, len(held), g.pool.num_free, g.pool.num_pages))

@@ -71,7 +71,7 @@ class Engine:
             s = sc.seq
             toks = s.token_ids[s.num_computed:s.num_computed + sc.num_tokens]
             entries.append(StepEntry(s.request_id, toks, [sc.num_tokens - 1] if sc.samples else []))
-        logits = self.runner.step(entries)
+        logits = self.runner.step(entries, borrow=True)
         sampling = [sc.seq for sc in scheduled if sc.samples]
         tokens = self.sampler.sample(logits, [s.params for s in sampling],
                                      [s.num_output_tokens for s in sampling])

@@ -38,7 +38,7 @@ def require_gpu():
 
 class ModelRunner:
     def __init__(self, model_path, dtype="bfloat16", page_size=16, num_pages=None, max_requests=64,
-                 max_model_len=None, gpu_memory_utilization=0.9, device=None, config=None):
+                 max_model_len=None, gpu_memory_utilization=0.9, device=None, config=None, use_graphs=True):
         self.device = device or require_gpu()
         if dtype not in DTYPES:
             raise ValueError("dtype must be one of %s, got %r" % (sorted(DTYPES), dtype))
@@ -59,6 +59,9 @@ class ModelRunner:
         self.cache = CacheManager(specs, self.page_size, int(num_pages), int(max_requests))
         self.cache.allocate_device(self.dtype, self.device)
         self._owner_of = [i if e.cache_of is None else e.cache_of for i, e in enumerate(self.model.schedule)]
+        self._buffers = _BufferCache(len(self.cache.groups), self.device)
+        self.use_graphs = bool(use_graphs) and self.model.capturable()
+        self._graphs, self._graph_seen = {}, {}
 
     def _pages_from_free_memory(self, specs, utilization):
         """Pages = free device memory (after the weights are resident) * utilization / bytes per page, the
@@ -78,9 +81,10 @@ class ModelRunner:
         return self.spec.vocab_size
 
     # ---- the step
-    def step(self, entries: List[StepEntry]):
+    def step(self, entries: List[StepEntry], borrow=False):
         """Returns float32 logits [R, V] on the device: the wanted places in the order of the entries
-        and of each entry's `want`."""
+        and of each entry's `want`.  With borrow=True the result may be a buffer that the next step
+        overwrites (the engine samples from it at once)."""
         if not entries:
             return torch.empty((0, self.vocab_size), dtype=torch.float32, device=self.device)
         cache = self.cache
@@ -110,12 +114,12 @@ class ModelRunner:
                 elif cache.pending(e.request_id) != len(e.tokens):
                     raise ValueError("request %r has %d tokens reserved but brings %d"
                                      % (e.request_id, cache.pending(e.request_id), len(e.tokens)))
-            ctx = self._build_context(entries)
+            host = self._host_arrays(entries)
         except Exception:
             for rid in reserved_here:       # leave the cache as it was
                 cache.requests[rid].pending = 0
             raise
-        logits = self.model.forward(ctx)
+        logits = self._run(host, borrow)
         for e in entries:
             cache.commit(e.request_id)
         return logits
@@ -124,66 +128,202 @@ class ModelRunner:
         if self.cache.has(request_id):
             self.cache.release(request_id)
 
-    def _build_context(self, entries):
+    # ---- the step's side inputs
+    def _host_arrays(self, entries):
+        """Everything the kernels need to know about the batch, as numpy arrays (no device work)."""
         cache, ps = self.cache, self.page_size
         E = len(entries)
-        q_len = [len(e.tokens) for e in entries]
-        q_start = [cache.length(e.request_id) for e in entries]
-        T = sum(q_len)
-        ids = np.empty(T, dtype=np.int32)
-        pos = np.empty(T, dtype=np.int32)
-        ent = np.empty(T, dtype=np.int32)
+        slots = np.fromiter((cache.slot(e.request_id) for e in entries), dtype=np.int64, count=E)
+        q_len = np.fromiter((len(e.tokens) for e in entries), dtype=np.int64, count=E)
+        q_start = cache.lengths_array(slots)
+        T = int(q_len.sum())
         cu = np.zeros(E + 1, dtype=np.int32)
-        rows = []
-        o = 0
-        for i, e in enumerate(entries):
-            n = q_len[i]
-            ids[o:o + n] = np.asarray(e.tokens, dtype=np.int64)
-            pos[o:o + n] = np.arange(q_start[i], q_start[i] + n, dtype=np.int32)
-            ent[o:o + n] = i
-            rows.extend(o + w for w in e.want)
-            o += n
-            cu[i + 1] = o
+        np.cumsum(q_len, out=cu[1:])
+        if T == E:                          # every request brings one token: no loop over tokens
+            ids = np.fromiter((e.tokens[0] for e in entries), dtype=np.int64, count=E)
+            ent = np.arange(E, dtype=np.int32)
+            pos = q_start.astype(np.int32)
+        else:
+            ids = np.concatenate([np.asarray(e.tokens, dtype=np.int64) for e in entries])
+            ent = np.repeat(np.arange(E, dtype=np.int32), q_len)
+            pos = (np.arange(T, dtype=np.int64) - np.repeat(cu[:-1].astype(np.int64), q_len)
+                   + np.repeat(q_start, q_len)).astype(np.int32)
         if ids.min() < 0 or ids.max() >= self.vocab_size:
             raise ValueError("token id outside [0, %d)" % self.vocab_size)
-        dev = self.device
+        if int(pos.max()) >= self.max_model_len:
+            raise ValueError("a token at position %d lies beyond max_model_len %d" % (int(pos.max()), self.max_model_len))
+        rows = [int(cu[i]) + w for i, e in enumerate(entries) for w in e.want]
+        max_kv = int((q_start + q_len).max())
+        width = -(-max_kv // ps)
+        tables, slot_maps = [], []
+        for gi in range(len(cache.groups)):
+            bt = cache.tables_array(gi, slots, width)
+            pages = bt[ent, pos // ps].astype(np.int64)
+            if (pages < 0).any():
+                raise AssertionError("a new token has no page in cache group %d" % gi)
+            tables.append(bt)
+            slot_maps.append(pages * ps + pos % ps)
+        return dict(E=E, T=T, ids=ids.astype(np.int32), pos=pos, ent=ent, cu=cu, q_start=q_start.astype(np.int32),
+                    q_len=q_len, rows=np.asarray(rows, dtype=np.int32), width=width, tables=tables,
+                    slot_maps=slot_maps, state_slots=slots, max_kv=max_kv,
+                    decode_rows=cu[:-1][q_len == 1].astype(np.int32) if T != E else ent)
 
-        def up(a):
-            return torch.from_numpy(a).to(dev, non_blocking=False)
-
-        # per group: block tables [E, W] and slot mapping [T]
-        group_views = []
-        for gi, g in enumerate(cache.groups):
-            width = max(1, max(len(cache.table(e.request_id, gi)) for e in entries))
-            bt = np.full((E, width), -1, dtype=np.int32)
-            slots = np.empty(T, dtype=np.int64)
-            o = 0
-            for i, e in enumerate(entries):
-                table = cache.table(e.request_id, gi)
-                bt[i, :len(table)] = table
-                p = np.arange(q_start[i], q_start[i] + q_len[i])
-                pages = np.asarray(table, dtype=np.int64)[p // ps]
-                if (pages < 0).any():
-                    raise AssertionError("request %r: a new token has no page in group %d" % (e.request_id, gi))
-                slots[o:o + q_len[i]] = pages * ps + p % ps
-                o += q_len[i]
-            group_views.append((up(bt), up(slots)))
-        state_slots = up(np.asarray([cache.slot(e.request_id) for e in entries], dtype=np.int64))
+    def _context(self, host, buf):
+        """Uploads the host arrays through one packed buffer and wraps the device views."""
+        buf.fill(host)
+        cache, ps = self.cache, self.page_size
         caches = []
         for i, sched in enumerate(self.model.schedule):
             owner = self._owner_of[i]
             spec = cache.cache_specs[owner]
             if isinstance(spec, KVCacheSpec):
-                gi, j = cache.group_of[owner]
-                bt, slots = group_views[gi]
+                gi, _ = cache.group_of[owner]
                 kp, vp = cache.kv_views(owner)
-                caches.append(KVView(kp, vp, bt, slots, ps, owner == i))
+                caches.append(KVView(kp, vp, buf.dev["table%d" % gi], buf.dev["slots%d" % gi], ps, owner == i))
             elif isinstance(spec, StateSpec):
-                caches.append(StateView(cache.state_tensors[owner], state_slots, owner == i))
+                caches.append(StateView(cache.state_tensors[owner], buf.dev["state_slots"], owner == i))
             else:
                 caches.append(None)
+        # decode rows come first in cu order only when every entry is a single token; the list is general
         return StepContext(
-            token_ids=up(ids), positions=up(pos), token_entry=up(ent), cu_tokens=up(cu),
-            q_start=up(np.asarray(q_start, dtype=np.int32)),
-            logit_rows=up(np.asarray(rows, dtype=np.int32)),
-            num_tokens=T, num_entries=E, host_q_start=q_start, host_q_len=q_len, caches=caches, extra={})
+            token_ids=buf.dev["ids"], positions=buf.dev["pos"], token_entry=buf.dev["ent"], cu_tokens=buf.dev["cu"],
+            q_start=buf.dev["q_start"], logit_rows=buf.dev["rows"], num_tokens=host["T"], num_entries=host["E"],
+            host_q_start=host["q_start"].tolist(), host_q_len=host["q_len"].tolist(), caches=caches,
+            extra={"decode_rows": buf.dev["decode_rows"]})
+
+    def _run(self, host, borrow):
+        E, T = host["E"], host["T"]
+        ngroups = len(self.cache.groups)
+        graphable = self.use_graphs and T == E and E <= GRAPH_MAX_ROWS and len(host["rows"]) == E and \
+            bool((host["rows"] == np.arange(E)).all())
+        if graphable:
+            bucket = 256
+            while bucket < host["max_kv"]:
+                bucket *= 2
+            key = (E, bucket)
+            g = self._graphs.get(key)
+            if g is None:
+                self._graph_seen[key] = self._graph_seen.get(key, 0) + 1
+                if self._graph_seen[key] >= GRAPH_AFTER:
+                    g = self._capture(key, host)
+            if g is not None:
+                g["buf"].fill(host)
+                g["graph"].replay()
+                return g["logits"] if borrow else g["logits"].clone()
+        buf = self._buffers.get(T, E, len(host["rows"]), host["width"], len(host["decode_rows"]))
+        ctx = self._context(host, buf)
+        return self.model.forward(ctx)
+
+    def _capture(self, key, host):
+        """Records the decode step of E single tokens (contexts up to `bucket`) into a HIP graph.  All
+        side inputs live in one static buffer that later steps refill; the attention kernels split the
+        keys for the bucket's longest context, so the grid does not depend on the step."""
+        E, bucket = key
+        width = bucket // self.page_size
+        buf = _StepBuffers(E, E, E, width, E, len(self.cache.groups), self.device)
+        padded = dict(host, width=width, tables=[self._widen(t, width) for t in host["tables"]])
+        ctx = self._context(padded, buf)
+        ctx.extra["decode_span"] = bucket
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            self.model.forward(ctx)          # warm-up outside the graph: libraries load, allocator settles
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        ctx.extra = {"decode_rows": buf.dev["decode_rows"], "decode_span": bucket}
+        with torch.cuda.graph(graph):
+            logits = self.model.forward(ctx)
+        g = dict(graph=graph, buf=_GraphBuffers(buf, width, self._widen), logits=logits, ctx=ctx)
+        self._graphs[key] = g
+        return g
+
+    @staticmethod
+    def _widen(table, width):
+        if table.shape[1] == width:
+            return table
+        out = np.full((table.shape[0], width), -1, dtype=np.int32)
+        out[:, :table.shape[1]] = table
+        return out
+
+
+GRAPH_MAX_ROWS = 64      # the decode step's own kernels take up to this many rows; beyond it library calls come in
+GRAPH_AFTER = 2          # a batch shape is recorded the second time it is seen
+
+
+class _StepBuffers:
+    """One pinned host buffer and one device buffer that hold all side inputs of a step; `fill` copies the
+    host arrays in and uploads them in one transfer."""
+
+    def __init__(self, T, E, R, width, n_decode, ngroups, device):
+        self.shape = (T, E, R, width, n_decode)
+        fields = [("slots%d" % g, np.int64, (T,)) for g in range(ngroups)]
+        fields += [("state_slots", np.int64, (E,))]
+        fields += [("ids", np.int32, (T,)), ("pos", np.int32, (T,)), ("ent", np.int32, (T,)), ("cu", np.int32, (E + 1,)),
+                   ("q_start", np.int32, (E,)), ("rows", np.int32, (R,)), ("decode_rows", np.int32, (n_decode,))]
+        fields += [("table%d" % g, np.int32, (E, max(width, 1))) for g in range(ngroups)]
+        offset, self.layout = 0, {}
+        for name, dt, shape in fields:
+            n = int(np.prod(shape)) * np.dtype(dt).itemsize
+            self.layout[name] = (offset, dt, shape)
+            offset += -(-max(n, 1) // 16) * 16
+        self.nbytes = offset
+        self.host_t = torch.empty(self.nbytes, dtype=torch.uint8, pin_memory=True)
+        self.dev_t = torch.empty(self.nbytes, dtype=torch.uint8, device=device)
+        host_np = self.host_t.numpy()
+        self.host, self.dev = {}, {}
+        tdt = {np.int64: torch.int64, np.int32: torch.int32}
+        for name, (off, dt, shape) in self.layout.items():
+            n = int(np.prod(shape))
+            nb = n * np.dtype(dt).itemsize
+            self.host[name] = host_np[off:off + nb].view(dt).reshape(shape)
+            self.dev[name] = self.dev_t[off:off + nb].view(tdt[dt]).view(shape)
+        self.event = torch.cuda.Event()
+        self.used = False
+
+    def fill(self, host):
+        if self.used:
+            self.event.synchronize()     # the last upload from this pinned buffer is through
+        h = self.host
+        h["ids"][:] = host["ids"]
+        h["pos"][:] = host["pos"]
+        h["ent"][:] = host["ent"]
+        h["cu"][:] = host["cu"]
+        h["q_start"][:] = host["q_start"]
+        h["rows"][:] = host["rows"]
+        h["decode_rows"][:] = host["decode_rows"]
+        h["state_slots"][:] = host["state_slots"]
+        for g, (bt, sm) in enumerate(zip(host["tables"], host["slot_maps"])):
+            h["table%d" % g][:, :bt.shape[1]] = bt
+            h["slots%d" % g][:] = sm
+        self.dev_t.copy_(self.host_t, non_blocking=True)
+        self.event.record()
+        self.used = True
+
+
+class _GraphBuffers:
+    """The static buffers of a recorded step: tables are padded to the bucket's width on the way in."""
+
+    def __init__(self, buf, width, widen):
+        self.buf, self.width, self.widen = buf, width, widen
+
+    def fill(self, host):
+        self.buf.fill(dict(host, tables=[self.widen(t, self.width) for t in host["tables"]]))
+
+
+class _BufferCache:
+    """Step buffers by (rounded) sizes, so that pinned memory is not allocated step after step."""
+
+    def __init__(self, ngroups, device, keep=24):
+        self.ngroups, self.device, self.keep = ngroups, device, keep
+        self.items = {}
+
+    def get(self, T, E, R, width, n_decode):
+        key = (T, E, R, width, n_decode)
+        buf = self.items.pop(key, None)
+        if buf is None:
+            buf = _StepBuffers(T, E, R, width, n_decode, self.ngroups, self.device)
+            while len(self.items) >= self.keep:
+                self.items.pop(next(iter(self.items)))
+        self.items[key] = buf            # most recently used last
+        return buf

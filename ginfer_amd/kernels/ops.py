@@ -294,9 +294,12 @@ def _attention_plan(step, tile_rows, device):
                 tiles.append((e, o + r, min(tile_rows, n - r), start + r))
         o += n
     tiles.sort(key=lambda t: -(t[3] + t[2]))      # the tiles with the most keys first
+    token_list = step.extra.get("decode_rows")      # the runner uploads the list with the step's other side inputs
+    if token_list is None and decode_rows:
+        token_list = torch.tensor(decode_rows, dtype=torch.int32, device=device)
     plan = dict(
-        n_decode=len(decode_rows), decode_pos=decode_pos, n_tiles=len(tiles),
-        token_list=(torch.tensor(decode_rows, dtype=torch.int32, device=device) if decode_rows else None),
+        n_decode=len(decode_rows), decode_pos=decode_pos, n_tiles=len(tiles), decode_span=step.extra.get("decode_span"),
+        token_list=token_list,
         tiles=(torch.tensor(np.asarray(tiles, dtype=np.int32).reshape(-1, 4), device=device) if tiles else None))
     step.extra[key] = plan
     return plan
@@ -304,9 +307,12 @@ def _attention_plan(step, tile_rows, device):
 
 def _decode_splits(plan, window, nkv, head_blocks):
     span = 0
-    for pos in plan["decode_pos"]:
-        lo = max(0, pos - window + 1) if window else 0
-        span = max(span, pos + 1 - (lo // 32) * 32)
+    if plan.get("decode_span"):             # a recorded step: the split must fit every context of its bucket
+        span = plan["decode_span"] if not window else min(plan["decode_span"], (window + 62) // 32 * 32)
+    else:
+        for pos in plan["decode_pos"]:
+            lo = max(0, pos - window + 1) if window else 0
+            span = max(span, pos + 1 - (lo // 32) * 32)
     per_split = plan["n_decode"] * nkv * head_blocks
     splits = max(1, min(_DECODE_TARGET_WORKGROUPS // max(per_split, 1), -(-span // _MIN_SPLIT_KEYS), _MAX_SPLITS))
     split_keys = -(-(-(-span // splits)) // 32) * 32

@@ -17,6 +17,8 @@ class Attention(Part):
     (:69-72, :32-33), attention over the request's pages (:34), output projection (:80-81).
     score scale 1/sqrt(head_dim) unless `scale` is given; `window` None attends to all earlier keys."""
 
+    capturable = True
+
     def __init__(self, hidden_size, num_heads, num_kv_heads, head_dim, qkv_bias, out_bias, window, position,
                  scale, dtype, device):
         if num_heads % num_kv_heads:

@@ -6,7 +6,11 @@ Every part
   * says which tensors it needs: `weight_specs() -> {local name: WeightSpec}`; local names are joined
     to the part's prefix by the model, e.g. "model.layers.3.self_attn" + "." + "q_proj.weight";
   * receives them, already on the device and in the right dtype: `bind_weights({local name: tensor})`;
-  * names the kernel libraries it launches: `kernel_modules() -> [module, ...]`.
+  * names the kernel libraries it launches: `kernel_modules() -> [module, ...]`;
+  * says whether its forward may be recorded into a HIP graph: `capturable` (False unless the part sets
+    it).  A capturable forward launches the same kernels with the same arguments whatever the step's
+    host-side numbers are: it reads sizes only from tensor shapes, does nothing that waits for the device,
+    and takes everything that changes from step to step from the step's device arrays.
 
 Mixer         forward(x [T, H], step, cache) -> [T, H]
               cache_spec() -> KVCacheSpec | StateSpec | None: what one run of this mixer keeps per
@@ -44,6 +48,8 @@ class StateSpec:
 
 
 class Part:
+    capturable = False
+
     def weight_specs(self):
         return {}
 

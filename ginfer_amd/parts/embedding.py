@@ -13,6 +13,8 @@ class Embedding(Part):
     """x[t, :] = E[ids[t], :], no scaling (ginfer/core/layer/embedding.cc:5-21); widened to the 32-bit
     residual stream as it is gathered."""
 
+    capturable = True
+
     def __init__(self, vocab_size, hidden_size, dtype, device):
         self.vocab_size, self.hidden_size, self.dtype, self.device = int(vocab_size), int(hidden_size), dtype, device
         self.weight = None
@@ -35,6 +37,8 @@ class LMHead(Part):
     """logits = x . W^T, no bias, returned in 32-bit; W is the embedding table when tied
     (ginfer/core/layer/transformer/lmhead.cc:15-27, ginfer/model/qwen2.cc:42-46).  One device copy serves
     both uses when tied (the reference uploads it twice)."""
+
+    capturable = True
 
     def __init__(self, vocab_size, hidden_size, tied, dtype, device):
         self.vocab_size, self.hidden_size, self.tied = int(vocab_size), int(hidden_size), bool(tied)

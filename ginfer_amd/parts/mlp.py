@@ -13,6 +13,8 @@ class SwiGLU(Part):
     """down(silu(gate(x)) * up(x)), no biases (ginfer/core/layer/transformer/feedforward.cc:22-25); gate and
     up are one product over the stacked weights, which equals the two separate ones."""
 
+    capturable = True
+
     def __init__(self, hidden_size, intermediate_size, dtype, device):
         self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)
         self.dtype, self.device = dtype, device

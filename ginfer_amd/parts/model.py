@@ -118,6 +118,10 @@ class DecoderModel:
                     mods.append(m)
         return mods
 
+    def capturable(self):
+        """Whether a step of this model may be recorded into a HIP graph: every part must allow it."""
+        return all(getattr(part, "capturable", False) for _, part in self._named_parts())
+
     def position_parts(self):
         return list(self._positions.values())
 

@@ -12,6 +12,8 @@ class RMSNorm(Part):
     """y = (h * g) / sqrt(mean(h^2) + eps) with h = residual + delta; plain gain, no bias, no mean
     subtraction (ginfer/core/op/kernels/cuda/rmsnorm_kernel.cu:27-66, ginfer/core/layer/rmsnorm.cc:6-22)."""
 
+    capturable = True
+
     def __init__(self, size, eps, dtype, device):
         self.size, self.eps, self.dtype, self.device = int(size), float(eps), dtype, device
         self.weight = None

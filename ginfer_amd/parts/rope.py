@@ -12,6 +12,8 @@ class RotaryNeoX(Part):
     computed once on the host and uploaded.  The rotation itself is part of the mixer's kernel
     (ginfer/core/op/kernels/cuda/rope_kernel.cu:83-102)."""
 
+    capturable = True
+
     style = "neox"
 
     def __init__(self, theta, rotary_dim, max_positions, dtype=None, device=None):

@@ -153,3 +153,43 @@ def test_temperature_sampling_matches_plain_with_same_uniforms(folders):
     # the inverse CDF is a step function of the uniform number; only a draw within rounding of a step may differ
     assert agree >= total - 1, "%d of %d sampled tokens agree with the plain sampler" % (agree, total)
     assert len({tuple(o.token_ids) for o in outs}) > 1
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["B", "C"])
+def test_recorded_decode_steps_equal_eager_ones(folders, name, dtype):
+    """Decode steps replayed from a HIP graph give the bits of the same steps launched one kernel at a
+    time: many replays, with eager steps (a prompt portion, another batch size) and synchronisations
+    between them, each replay checked."""
+    from ginfer_amd import ModelRunner, StepEntry
+    vocab = H.TINY[name][0]["vocab_size"]
+    ps = H.TINY[name][2]
+    runners = [ModelRunner(folders[name], dtype=dtype, page_size=ps, num_pages=160, max_requests=8, use_graphs=g)
+               for g in (True, False)]
+    prompts = {i: H.random_tokens(n, vocab, 500 + i) for i, n in enumerate((20, 45, 70))}
+    late = H.random_tokens(90, vocab, 600)
+    stream = H.random_tokens(400, vocab, 601)
+    outs = [[], []]
+    for k, r in enumerate(runners):
+        for i, p in prompts.items():
+            r.step([StepEntry(i, p, [])])
+        at = 0
+        for stepno in range(60):
+            batch = [StepEntry(i, [stream[at + i]], [0]) for i in prompts]
+            at += 3
+            outs[k].append(r.step(batch).cpu())
+            if stepno == 20:                       # an eager step between replays: a prompt portion of a newcomer
+                outs[k].append(r.step([StepEntry("late", late[:50], [49])]).cpu())
+            if stepno == 30:                       # and the newcomer joins the batch beside a portion of itself
+                outs[k].append(r.step([StepEntry("late", late[50:], [39])] + [StepEntry(0, [stream[at]], [0])]).cpu())
+                r.release(0)
+                prompts_now = [1, 2]
+                for _ in range(4):                 # another batch size gets a graph of its own
+                    outs[k].append(r.step([StepEntry(i, [stream[at + i]], [0]) for i in prompts_now]).cpu())
+                    at += 3
+                r.step([StepEntry(0, prompts[0] + stream[:31], [])])      # request 0 comes back, on other pages
+        r.cache.check()
+    assert runners[0]._graphs and not runners[1]._graphs
+    assert len(outs[0]) == len(outs[1])
+    for n, (a, b) in enumerate(zip(*outs)):
+        assert torch.equal(a, b), "step %d: a replayed step differs from the eager step" % n
