@@ -50,20 +50,81 @@ __device__ __forceinline__ bf16x8 load8(const bf16_t* p) {
   return __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(p));
 }
 
-// Attends columns to the key tiles [tile_begin, tile_end) (multiples of 32).  kv_min..kv_max is the
-// inclusive range of keys that any column of the wavefront may see: keys outside it are never loaded
-// (their pages may be gone) and count as zero.
+// K operands of one tile of 32 keys: [product t][32-dim block]; keys outside kv_min..kv_max are never
+// loaded (their pages may be gone) and count as zero.
+__device__ __forceinline__ void load_k_tile(bf16x8 (&kr)[2][KB], const bf16_t* __restrict__ k_pages,
+                                            const int32_t* __restrict__ bt, int kvh, int nkv, int ps_shift,
+                                            int kv_min, int kv_max, int k0, int c, int g) {
+  const int ps = 1 << ps_shift;
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+    const int key = k0 + 8 * (c >> 2) + 4 * t + (c & 3);
+    const bool ok = key >= kv_min && key <= kv_max;
+    const bf16_t* kp = k_pages;
+    if (ok) {
+      const int64_t page = bt[key >> ps_shift];
+      kp = k_pages + ((page * nkv + kvh) * ps + (key & (ps - 1))) * HD + g * 8;
+    }
+#pragma unroll
+    for (int kb = 0; kb < KB; ++kb) {
+      kr[t][kb] = zero8();
+      if (ok && kb * 32 + g * 8 < HD) kr[t][kb] = load8(kp + kb * 32);
+    }
+  }
+}
+
+// V^T operands of one tile: [16-dim block]; the lane loads dims db*16 + c, keys k0 + 8g .. + 7.
+__device__ __forceinline__ void load_v_tile(bf16x8 (&vr)[DB], const bf16_t* __restrict__ v_pages,
+                                            const int32_t* __restrict__ bt, int kvh, int nkv, int ps_shift,
+                                            int kv_min, int kv_max, int k0, int c, int g) {
+  const int ps = 1 << ps_shift;
+  const int kbase = k0 + 8 * g;
+  const bool any_ok = kbase + 7 >= kv_min && kbase <= kv_max;
+  const bool all_ok = kbase >= kv_min && kbase + 7 <= kv_max;
+  const bf16_t* vp = v_pages;
+  if (any_ok) {
+    const int64_t page = bt[kbase >> ps_shift];
+    vp = v_pages + ((page * nkv + kvh) * HD + c) * ps + (kbase & (ps - 1));
+  }
+#pragma unroll
+  for (int db = 0; db < DB; ++db) {
+    vr[db] = zero8();
+    if (any_ok) {
+      vr[db] = load8(vp + (int64_t)db * 16 * ps);
+      if (!all_ok) {                       // slots past the request's last key hold anything: clear them
+        union { bf16x8 v; bf16_t e[8]; } u;
+        u.v = vr[db];
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+          if (kbase + j < kv_min || kbase + j > kv_max) u.e[j] = 0;
+        vr[db] = u.v;
+      }
+    }
+  }
+}
+
+// Attends columns to the key tiles tile_begin, tile_begin + tile_stride, ... < tile_end (multiples of 32).
+// kv_min..kv_max is the inclusive range of keys that any column of the wavefront may see; full_lo..full_hi
+// the range that EVERY live column sees (tiles inside it need no mask).  The loop is software-pipelined:
+// the values of a tile and the keys of the next are requested before the tile's scores are computed, so
+// that their way from memory overlaps the matrix products and the softmax.
 template <int NB>
 __device__ __forceinline__ void attend_tiles(f32x4 (&o)[NB][DB], float (&m)[NB], float (&l)[NB],
                                              const bf16x8 (&q)[NB][KB], const int (&cpos)[NB],
                                              const int (&clo)[NB], const bf16_t* __restrict__ k_pages,
                                              const bf16_t* __restrict__ v_pages,
                                              const int32_t* __restrict__ bt, int kvh, int nkv, int ps_shift,
-                                             int kv_min, int kv_max, int tile_begin, int tile_end,
-                                             float scale) {
+                                             int kv_min, int kv_max, int full_lo, int full_hi, int tile_begin,
+                                             int tile_end, int tile_stride, float scale) {
   const int lane = threadIdx.x & 63, c = lane & 15, g = lane >> 4;
-  const int ps = 1 << ps_shift;
-  for (int k0 = tile_begin; k0 < tile_end; k0 += 32) {
+  if (tile_begin >= tile_end) return;
+  bf16x8 kr[2][KB];
+  load_k_tile(kr, k_pages, bt, kvh, nkv, ps_shift, kv_min, kv_max, tile_begin, c, g);
+  for (int k0 = tile_begin; k0 < tile_end; k0 += tile_stride) {
+    bf16x8 vr[DB], kn[2][KB];
+    load_v_tile(vr, v_pages, bt, kvh, nkv, ps_shift, kv_min, kv_max, k0, c, g);
+    const bool more = k0 + tile_stride < tile_end;
+    if (more) load_k_tile(kn, k_pages, bt, kvh, nkv, ps_shift, kv_min, kv_max, k0 + tile_stride, c, g);
     // ---- scores: S^T = K Q^T
     f32x4 s[NB][2];
 #pragma unroll
@@ -72,35 +133,33 @@ __device__ __forceinline__ void attend_tiles(f32x4 (&o)[NB][DB], float (&m)[NB],
       s[nb][1] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
-      const int key = k0 + 8 * (c >> 2) + 4 * t + (c & 3);
-      const bool ok = key >= kv_min && key <= kv_max;
-      const bf16_t* kp = k_pages;
-      if (ok) {
-        const int64_t page = bt[key >> ps_shift];
-        kp = k_pages + ((page * nkv + kvh) * ps + (key & (ps - 1))) * HD + g * 8;
-      }
+    for (int t = 0; t < 2; ++t)
 #pragma unroll
-      for (int kb = 0; kb < KB; ++kb) {
-        bf16x8 a = zero8();
-        if (ok && kb * 32 + g * 8 < HD) a = load8(kp + kb * 32);
+      for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb)
-          s[nb][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, q[nb][kb], s[nb][t], 0, 0, 0);
-      }
-    }
+          s[nb][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kr[t][kb], q[nb][kb], s[nb][t], 0, 0, 0);
     // ---- mask and online softmax; the lane holds keys k0 + 8g + j, j = 0..7, of column c
+    const bool interior = k0 >= full_lo && k0 + 31 <= full_hi;      // the same for the whole wavefront
     bf16x8 pb[NB];
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) {
       float sv[8];
       float mx = -INFINITY;
+      if (interior && cpos[nb] >= 0) {
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const int key = k0 + 8 * g + j;
-        const bool valid = key >= clo[nb] && key <= cpos[nb];
-        sv[j] = valid ? s[nb][j >> 2][j & 3] * scale : -INFINITY;
-        mx = fmaxf(mx, sv[j]);
+        for (int j = 0; j < 8; ++j) {
+          sv[j] = s[nb][j >> 2][j & 3] * scale;
+          mx = fmaxf(mx, sv[j]);
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int key = k0 + 8 * g + j;
+          const bool valid = key >= clo[nb] && key <= cpos[nb];
+          sv[j] = valid ? s[nb][j >> 2][j & 3] * scale : -INFINITY;
+          mx = fmaxf(mx, sv[j]);
+        }
       }
       mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
       mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
@@ -122,39 +181,24 @@ __device__ __forceinline__ void attend_tiles(f32x4 (&o)[NB][DB], float (&m)[NB],
       sum += __shfl_xor(sum, 32, WAVE);
       l[nb] = l[nb] * alpha + sum;
       m[nb] = m_new;
+      if (__any(alpha != 1.f)) {           // once the running max has settled nothing is rescaled
 #pragma unroll
-      for (int db = 0; db < DB; ++db) o[nb][db] *= alpha;
-      union { bf16x8 v; bf16_t e[8]; } pk;
-#pragma unroll
-      for (int j = 0; j < 8; ++j) pk.e[j] = f32_to_bf16(p[j]);
-      pb[nb] = pk.v;
-    }
-    // ---- output: O^T += V^T P; the lane loads dims db*16 + c, keys k0 + 8g .. + 7
-    const int kbase = k0 + 8 * g;
-    const bool any_ok = kbase + 7 >= kv_min && kbase <= kv_max;
-    const bool all_ok = kbase >= kv_min && kbase + 7 <= kv_max;
-    const bf16_t* vp = v_pages;
-    if (any_ok) {
-      const int64_t page = bt[kbase >> ps_shift];
-      vp = v_pages + ((page * nkv + kvh) * HD + c) * ps + (kbase & (ps - 1));
-    }
-#pragma unroll
-    for (int db = 0; db < DB; ++db) {
-      bf16x8 a = zero8();
-      if (any_ok) {
-        a = load8(vp + (int64_t)db * 16 * ps);
-        if (!all_ok) {                     // slots past the request's last key hold anything: clear them
-          union { bf16x8 v; bf16_t e[8]; } u;
-          u.v = a;
-#pragma unroll
-          for (int j = 0; j < 8; ++j)
-            if (kbase + j < kv_min || kbase + j > kv_max) u.e[j] = 0;
-          a = u.v;
-        }
+        for (int db = 0; db < DB; ++db) o[nb][db] *= alpha;
       }
 #pragma unroll
+      for (int j = 0; j < 8; ++j) pb[nb][j] = (__bf16)p[j];
+    }
+    // ---- output: O^T += V^T P
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
       for (int nb = 0; nb < NB; ++nb)
-        o[nb][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb[nb], o[nb][db], 0, 0, 0);
+        o[nb][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vr[db], pb[nb], o[nb][db], 0, 0, 0);
+    if (more) {
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb) kr[t][kb] = kn[t][kb];
     }
   }
 }
@@ -216,9 +260,9 @@ __global__ __launch_bounds__(64 * DEC_WAVES) void attn_decode_split_kernel(
     load_q(qr[0], col_ok ? q + (int64_t)t * q_stride + (int64_t)head * HD : nullptr, g);
     const int cpos[1] = {col_ok ? pos : -1}, clo[1] = {lo};
     const int32_t* bt = block_table + (int64_t)token_entry[t] * table_width;
-    for (int k0 = begin + 32 * wave; k0 < end; k0 += 32 * DEC_WAVES)
-      attend_tiles<1>(o, m, l, qr, cpos, clo, k_pages, v_pages, bt, kvh, nkv, ps_shift, lo, pos, k0, k0 + 32,
-                      scale);
+    // every live column of a decode wavefront sees the same keys: lo..pos
+    attend_tiles<1>(o, m, l, qr, cpos, clo, k_pages, v_pages, bt, kvh, nkv, ps_shift, lo, pos, lo, pos,
+                    begin + 32 * wave, end, 32 * DEC_WAVES, scale);
   }
   // the wavefronts' states meet: common max, rescaled sums and outputs added in wavefront order
   if (g == 0) {
@@ -294,39 +338,91 @@ __global__ __launch_bounds__(64) void attn_decode_combine_kernel(
 }
 
 // ----------------------------------------------------------------------------- prefill
-// grid (tiles, nkv * head_blocks); a workgroup holds `waves` wavefronts, one query head each.
-// tiles: int32 [n][4] = (entry, first token row of the step, rows (<= 16*PREFILL_NB), first position).
+// grid (tiles, nkv * head_blocks); a workgroup holds hpw * splits wavefronts: hpw query heads of one kv
+// head, and for each head `splits` wavefronts that take the key tiles s, s + splits, ... of the same
+// 16*NB rows, so that the longest rows of a causal prompt are not one wavefront's serial work.  The
+// states of a head's wavefronts meet in LDS: wavefront 0 of the head merges and writes the rows.
+// tiles: int32 [n][4] = (entry, first token row of the step, rows (<= 16*NB), first position).
+template <int NB>
 __global__ __launch_bounds__(512) void attn_prefill_kernel(
     bf16_t* __restrict__ out, int64_t out_stride, const bf16_t* __restrict__ q, int64_t q_stride,
     const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
     const int32_t* __restrict__ block_table, int table_width, const int32_t* __restrict__ tiles, int nh,
-    int nkv, int head_blocks, int waves, int ps_shift, int window, float scale) {
-  constexpr int NB = PREFILL_NB;
+    int nkv, int head_blocks, int hpw, int splits, int ps_shift, int window, float scale) {
+  extern __shared__ float lds[];          // [hpw][splits-1][NB] x { o[HD][17], m[16], l[16] }
+  constexpr int STATE = HD * 17 + 32;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c = lane & 15, g = lane >> 4;
   const int kvh = blockIdx.y / head_blocks, hb = blockIdx.y % head_blocks;
   const int group = nh / nkv;
-  if (hb * waves + wave >= group) return;          // the whole wavefront leaves; nothing is shared
-  const int head = kvh * group + hb * waves + wave;
+  const int hl = wave / splits, split = wave % splits;
+  const bool head_ok = hb * hpw + hl < group;
+  const int head = kvh * group + hb * hpw + hl;
   const int32_t* tile = tiles + (int64_t)blockIdx.x * 4;
   const int entry = tile[0], row0 = tile[1], rows = tile[2], pos0 = tile[3];
 
   f32x4 o[NB][DB];
   float m[NB], l[NB];
   init_state<NB>(o, m, l);
-  bf16x8 qr[NB][KB];
-  int cpos[NB], clo[NB];
+  if (head_ok) {
+    bf16x8 qr[NB][KB];
+    int cpos[NB], clo[NB];
 #pragma unroll
-  for (int nb = 0; nb < NB; ++nb) {
-    const int j = nb * 16 + c;
-    const bool ok = j < rows;
-    cpos[nb] = ok ? pos0 + j : -1;
-    clo[nb] = (window > 0 && pos0 + j - window + 1 > 0) ? pos0 + j - window + 1 : 0;
-    load_q(qr[nb], ok ? q + (int64_t)(row0 + j) * q_stride + (int64_t)head * HD : nullptr, g);
+    for (int nb = 0; nb < NB; ++nb) {
+      const int j = nb * 16 + c;
+      const bool ok = j < rows;
+      cpos[nb] = ok ? pos0 + j : -1;
+      clo[nb] = (window > 0 && pos0 + j - window + 1 > 0) ? pos0 + j - window + 1 : 0;
+      load_q(qr[nb], ok ? q + (int64_t)(row0 + j) * q_stride + (int64_t)head * HD : nullptr, g);
+    }
+    const int kv_min = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;
+    const int kv_max = pos0 + rows - 1;
+    // every row of the tile sees the keys from the last row's window start up to the first row's position
+    const int full_lo = (window > 0 && kv_max - window + 1 > 0) ? kv_max - window + 1 : 0;
+    attend_tiles<NB>(o, m, l, qr, cpos, clo, k_pages, v_pages, block_table + (int64_t)entry * table_width, kvh,
+                     nkv, ps_shift, kv_min, kv_max, full_lo, pos0, (kv_min / 32) * 32 + 32 * split,
+                     (kv_max / 32 + 1) * 32, 32 * splits, scale);
   }
-  const int kv_min = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;
-  const int kv_max = pos0 + rows - 1;
-  attend_tiles<NB>(o, m, l, qr, cpos, clo, k_pages, v_pages, block_table + (int64_t)entry * table_width, kvh,
-                   nkv, ps_shift, kv_min, kv_max, (kv_min / 32) * 32, (kv_max / 32 + 1) * 32, scale);
+  if (splits > 1) {
+    if (head_ok && split > 0) {
+      float* st = lds + (int64_t)((hl * (splits - 1) + split - 1) * NB) * STATE;
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) {
+        float* sn = st + nb * STATE;
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) sn[(db * 16 + g * 4 + i) * 17 + c] = o[nb][db][i];
+        if (g == 0) {
+          sn[HD * 17 + c] = m[nb];
+          sn[HD * 17 + 16 + c] = l[nb];
+        }
+      }
+    }
+    __syncthreads();
+    if (!head_ok || split > 0) return;
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+      float mx = m[nb];
+      for (int sp = 1; sp < splits; ++sp)
+        mx = fmaxf(mx, lds[(int64_t)((hl * (splits - 1) + sp - 1) * NB + nb) * STATE + HD * 17 + c]);
+      const float f0 = m[nb] == -INFINITY ? 0.f : __expf(m[nb] - mx);
+      l[nb] *= f0;
+#pragma unroll
+      for (int db = 0; db < DB; ++db) o[nb][db] *= f0;
+      for (int sp = 1; sp < splits; ++sp) {      // in split order
+        const float* sn = lds + (int64_t)((hl * (splits - 1) + sp - 1) * NB + nb) * STATE;
+        const float ms = sn[HD * 17 + c];
+        const float f = ms == -INFINITY ? 0.f : __expf(ms - mx);
+        l[nb] += sn[HD * 17 + 16 + c] * f;
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) o[nb][db][i] += sn[(db * 16 + g * 4 + i) * 17 + c] * f;
+      }
+    }
+  } else if (!head_ok) {
+    return;
+  }
 #pragma unroll
   for (int nb = 0; nb < NB; ++nb) {
     const int j = nb * 16 + c;
@@ -344,7 +440,8 @@ __global__ __launch_bounds__(512) void attn_prefill_kernel(
 }
 
 extern "C" int ga_attn_head_dim() { return HD; }
-extern "C" int ga_attn_prefill_tile_rows() { return 16 * PREFILL_NB; }
+// rows of a prefill tile: 16 or (head sizes up to 128) 32
+extern "C" int ga_attn_prefill_max_tile_rows() { return 16 * PREFILL_NB; }
 
 // Decode tokens: token_list names the rows of the step that are single new tokens.  workspace_o must
 // hold n_tokens*nh*num_splits*HD floats and workspace_ml n_tokens*nh*num_splits*2.
@@ -379,20 +476,35 @@ extern "C" int ga_attn_decode(void* out, int64_t out_stride, const void* q, int6
 
 extern "C" int ga_attn_prefill(void* out, int64_t out_stride, const void* q, int64_t q_stride,
                                const void* k_pages, const void* v_pages, const void* block_table,
-                               int table_width, const void* tiles, int n_tiles, int nh, int nkv, int page_size,
-                               int window, float scale, hipStream_t stream) {
+                               int table_width, const void* tiles, int n_tiles, int tile_rows, int nh, int nkv,
+                               int page_size, int window, float scale, hipStream_t stream) {
   if (n_tiles <= 0) return 0;
   if (nkv <= 0 || nh % nkv) return -1;
+  if (tile_rows != 16 && tile_rows != 16 * PREFILL_NB) return -6;
   int ps_shift = 0;
   while ((1 << ps_shift) < page_size) ++ps_shift;
   if ((1 << ps_shift) != page_size || page_size < 8) return -2;
   const int group = nh / nkv;
-  const int waves = group < 8 ? group : 8;
-  const int head_blocks = (group + waves - 1) / waves;
+  int hpw = 1;                               // heads of a group that share a workgroup: a divisor of the group, at most 4
+  for (int d = 2; d <= 4; ++d)
+    if (group % d == 0) hpw = d;
+  int splits = 8 / hpw;
+  if (splits > 4) splits = 4;
+  const int head_blocks = group / hpw;
   if ((int64_t)nkv * head_blocks > 65535) return -4;
-  hipLaunchKernelGGL(attn_prefill_kernel, dim3(n_tiles, nkv * head_blocks), dim3(64 * waves), 0, stream,
-                     (bf16_t*)out, out_stride, (const bf16_t*)q, q_stride, (const bf16_t*)k_pages,
-                     (const bf16_t*)v_pages, (const int32_t*)block_table, table_width, (const int32_t*)tiles,
-                     nh, nkv, head_blocks, waves, ps_shift, window, scale);
+  const int nb = tile_rows / 16;
+  const size_t lds = (size_t)hpw * (splits - 1) * nb * (HD * 17 + 32) * sizeof(float);
+  dim3 grid(n_tiles, nkv * head_blocks), block(64 * hpw * splits);
+#define LAUNCH(NB)                                                                                        \
+  hipLaunchKernelGGL(attn_prefill_kernel<NB>, grid, block, lds, stream, (bf16_t*)out, out_stride,         \
+                     (const bf16_t*)q, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages,           \
+                     (const int32_t*)block_table, table_width, (const int32_t*)tiles, nh, nkv, head_blocks, \
+                     hpw, splits, ps_shift, window, scale)
+  if (lds > 48 * 1024) {                     // more dynamic LDS than the default limit: ask for it
+    const void* fn = nb == 1 ? (const void*)attn_prefill_kernel<1> : (const void*)attn_prefill_kernel<PREFILL_NB>;
+    if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) return -7;
+  }
+  if (nb == 1) LAUNCH(1); else LAUNCH(PREFILL_NB);
+#undef LAUNCH
   return GA_CHECK_LAUNCH();
 }

@@ -267,6 +267,7 @@ MFMA_HEAD_DIMS = tuple(range(16, 257, 16))
 _DECODE_TARGET_WORKGROUPS = 512       # four wavefronts each: enough to fill 256 compute units
 _MIN_SPLIT_KEYS = 128                 # one tile of 32 keys for each wavefront of a workgroup
 _MAX_SPLITS = 256
+PREFILL_WIDE_TILES_FROM = 1 << 30     # tokens in a step from which prompt rows go 32 to a wavefront
 
 
 def attention_mfma_supported(dtype, head_dim, page_size):
@@ -332,7 +333,9 @@ def paged_attention_mfma(q, k_pages, v_pages, block_table, step, num_heads, num_
     _need(q.stride(0) % 8 == 0 and q.data_ptr() % 16 == 0, "q rows must be 16-byte aligned")
     lib = build.load("attention_mfma", {"HEAD_DIM": head_dim})
     _need(lib.ga_attn_head_dim() == head_dim, "attention library was built for another head size")
-    plan = _attention_plan(step, lib.ga_attn_prefill_tile_rows(), q.device)
+    # rows of a prompt portion per wavefront: 32 where the kernel has it and the step is long, else 16
+    tile_rows = lib.ga_attn_prefill_max_tile_rows() if T >= PREFILL_WIDE_TILES_FROM else 16
+    plan = _attention_plan(step, tile_rows, q.device)
     _need(sum(step.host_q_len) == T, "the step's entries do not add up to its tokens")
     if out is None:
         out = torch.empty((T, num_heads * head_dim), dtype=q.dtype, device=q.device)
@@ -352,7 +355,7 @@ def paged_attention_mfma(q, k_pages, v_pages, block_table, step, num_heads, num_
     if plan["n_tiles"]:
         _check(lib.ga_attn_prefill(
             _ptr(out), _i64(out.stride(0)), _ptr(q), _i64(q.stride(0)), _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
-            _i(block_table.shape[1]), _ptr(plan["tiles"]), _i(plan["n_tiles"]), _i(num_heads), _i(num_kv_heads),
+            _i(block_table.shape[1]), _ptr(plan["tiles"]), _i(plan["n_tiles"]), _i(tile_rows), _i(num_heads), _i(num_kv_heads),
             _i(page_size), _i(w), _f(scale), _stream()), "attn_prefill")
     return out
 

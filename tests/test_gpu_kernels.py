@@ -326,10 +326,14 @@ MFMA_SEQS = ATTN_SEQS + [[(1, 31), (1, 32), (1, 33), (1, 64), (1, 65)], [(31, 31
                          [(1, 5000)], [(300, 700)]]
 
 
-@pytest.mark.parametrize("nh,nkv,hd", ATTN_HEADS + [(40, 2, 64), (3, 1, 256), (18, 1, 16)])
+@pytest.mark.parametrize("wide", [False, True])
+@pytest.mark.parametrize("nh,nkv,hd", ATTN_HEADS + [(40, 2, 64), (3, 1, 256), (18, 1, 16), (7, 1, 64), (8, 4, 256)])
 @pytest.mark.parametrize("seqs", MFMA_SEQS)
-def test_paged_attention_mfma(nh, nkv, hd, seqs):
+def test_paged_attention_mfma(nh, nkv, hd, seqs, wide, monkeypatch):
     from ginfer_amd.kernels import ops
+    monkeypatch.setattr(ops, "PREFILL_WIDE_TILES_FROM", 0 if wide else 1 << 30)    # 32 or 16 rows to a wavefront
+    if wide and max(q for q, _ in seqs) == 1:
+        pytest.skip("no prompt rows in this case")
     if sum(kv for _, kv in seqs) * nkv * hd > 3e6 and (nh, nkv, hd) not in ((12, 2, 128), (6, 1, 32)):
         pytest.skip("large case kept for two head shapes")
     for ps in (16, 8, 64) if hd <= 48 else (16,):
