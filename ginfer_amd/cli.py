@@ -1,0 +1,137 @@
+"""Command line of the engine, in the manner of the reference's test_engine binary
+(ginfer/test/test_engine.cc:14-111): the model folder comes from --model-path or the MODEL_PATH
+environment variable, the engine settings carry the names of its `engine::Config` fields
+(ginfer/engine/config.h:8-21) and the sampling settings those of `SamplingParams`
+(ginfer/engine/sampling_params.h:5-8).  There is no tokenizer: prompts are token ids.
+
+    python -m ginfer_amd generate  --model-path DIR --prompt-ids 1,2,3 --prompt-ids 4,5 --max-tokens 16
+    python -m ginfer_amd benchmark --model-path DIR --num-prompts 256 --prompt-len 512 --max-tokens 128
+    python -m ginfer_amd random-weights --config config.json --seed 0 --out DIR
+"""
+import argparse
+import json
+import os
+import random
+import sys
+import time
+
+
+def _engine_args(p):
+    p.add_argument("--model-path", default=os.environ.get("MODEL_PATH"),
+                   help="folder with config.json and model.safetensors (default: $MODEL_PATH)")
+    p.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"],
+                   help="bfloat16: the serving kernels; float32: everything in true 32-bit")
+    p.add_argument("--max-num-batched-tokens", type=int, default=2048, help="token budget of one step")
+    p.add_argument("--max-num-seqs", type=int, default=64, help="requests running at a time")
+    p.add_argument("--max-seq-len", type=int, default=4096, help="longest sequence (prompt + output)")
+    p.add_argument("--gpu-memory-utilization", type=float, default=0.9,
+                   help="share of the free device memory that becomes cache pages")
+    p.add_argument("--kvcache-block-size", type=int, default=16, help="tokens per cache page")
+    p.add_argument("--num-kvcache-blocks", type=int, default=None, help="cache pages (default: from free memory)")
+    p.add_argument("--max-tokens", type=int, default=64, help="output tokens per request")
+    p.add_argument("--ignore-eos", action="store_true", help="do not stop at an end-of-sequence token")
+    p.add_argument("--temperature", type=float, default=0.0, help="0: greedy")
+    p.add_argument("--seed", type=int, default=0, help="seed of the sampler's random stream")
+
+
+def _engine(args):
+    from . import Engine, EngineConfig
+    if not args.model_path:
+        sys.exit("no model: give --model-path or set MODEL_PATH")
+    return Engine(EngineConfig(
+        model_path=args.model_path, dtype=args.dtype, max_num_batched_tokens=args.max_num_batched_tokens,
+        max_num_seqs=args.max_num_seqs, max_seq_len=args.max_seq_len,
+        gpu_memory_utilization=args.gpu_memory_utilization, kvcache_block_size=args.kvcache_block_size,
+        num_kvcache_blocks=args.num_kvcache_blocks))
+
+
+def _params(args, n):
+    from . import SamplingParams
+    return [SamplingParams(max_tokens=args.max_tokens, ignore_eos=args.ignore_eos, temperature=args.temperature,
+                           seed=args.seed + i) for i in range(n)]
+
+
+def _report(engine, outs, wall):
+    st = engine.stats
+    for o in outs:
+        sys.stderr.write("request %d: prompt_tokens=%d output_tokens=%d finish=%s ttft=%.2f ms tpot=%s evictions=%d\n" % (
+            o.request_id, len(o.prompt_token_ids), len(o.token_ids), o.finish_reason, (o.ttft or 0) * 1e3,
+            "%.3f ms" % (o.tpot * 1e3) if o.tpot else "-", o.evictions))
+    pf = st["prefill_tokens"] / st["prefill_time"] if st["prefill_time"] else 0.0
+    dc = st["decode_tokens"] / st["decode_time"] if st["decode_time"] else 0.0
+    sys.stderr.write("steps=%d prefill=%.1f tok/s decode=%.1f tok/s wall=%.3f s evictions=%d\n"
+                     % (st["steps"], pf, dc, wall, engine.scheduler.num_evictions))
+    return dict(steps=st["steps"], prefill_tok_s=pf, decode_tok_s=dc, wall_s=wall)
+
+
+def cmd_generate(args):
+    prompts = [[int(t) for t in p.replace(",", " ").split()] for p in args.prompt_ids or []]
+    if args.prompt_file:
+        with open(args.prompt_file) as f:
+            for line in f:
+                line = line.strip()
+                if line:
+                    prompts.append(json.loads(line) if line.startswith("[") else [int(t) for t in line.replace(",", " ").split()])
+    if not prompts:
+        sys.exit("no prompts: give --prompt-ids 1,2,3 (repeatable) or --prompt-file FILE (one list of ids a line)")
+    engine = _engine(args)
+    t0 = time.perf_counter()
+    outs = engine.generate(prompts, _params(args, len(prompts)))
+    _report(engine, outs, time.perf_counter() - t0)
+    for o in outs:
+        print(json.dumps({"request_id": o.request_id, "token_ids": o.token_ids, "finish_reason": o.finish_reason}))
+
+
+def cmd_benchmark(args):
+    """The reference's EngineTest.Benchmark (ginfer/test/test_engine.cc:57-111): random prompts of one
+    length, a warm-up generate, then the timed one."""
+    engine = _engine(args)
+    rng = random.Random(0)
+    vocab = min(engine.runner.vocab_size, 10001)
+    prompts = [[rng.randrange(vocab) for _ in range(args.prompt_len)] for _ in range(args.num_prompts)]
+    args.ignore_eos = True
+    engine.generate(prompts[:2], _params(args, 2))
+    for k in engine.stats:
+        engine.stats[k] = 0 if isinstance(engine.stats[k], int) else 0.0
+    t0 = time.perf_counter()
+    outs = engine.generate(prompts, _params(args, len(prompts)))
+    wall = time.perf_counter() - t0
+    rep = _report(engine, [], wall)
+    total = sum(len(o.prompt_token_ids) + len(o.token_ids) for o in outs)
+    rep.update(total_tokens=total, total_tok_s=total / wall, output_tok_s=sum(len(o.token_ids) for o in outs) / wall)
+    print(json.dumps(rep))
+
+
+def cmd_random_weights(args):
+    from . import config_from_dict, write_random_model
+    with open(args.config) as f:
+        cfg = config_from_dict(json.load(f))
+    write_random_model(args.out, cfg, args.seed, args.storage_dtype)
+    print(args.out)
+
+
+def main(argv=None):
+    ap = argparse.ArgumentParser(prog="ginfer_amd", description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    sub = ap.add_subparsers(dest="command", required=True)
+    g = sub.add_parser("generate", help="generate token ids for prompts given as token ids")
+    _engine_args(g)
+    g.add_argument("--prompt-ids", action="append", help="one prompt as comma-separated token ids (repeatable)")
+    g.add_argument("--prompt-file", help="file with one prompt a line (JSON list or comma-separated ids)")
+    g.set_defaults(fn=cmd_generate)
+    b = sub.add_parser("benchmark", help="throughput with random prompts")
+    _engine_args(b)
+    b.add_argument("--num-prompts", type=int, default=256)
+    b.add_argument("--prompt-len", type=int, default=512)
+    b.set_defaults(fn=cmd_benchmark, max_num_batched_tokens=16384, max_num_seqs=256, max_tokens=128)
+    r = sub.add_parser("random-weights", help="write a model folder with random weights")
+    r.add_argument("--config", required=True, help="a config.json of a registered architecture")
+    r.add_argument("--seed", type=int, default=0)
+    r.add_argument("--out", required=True)
+    r.add_argument("--storage-dtype", default="bfloat16", choices=["bfloat16", "float32", "float16"])
+    r.set_defaults(fn=cmd_random_weights)
+    args = ap.parse_args(argv)
+    args.fn(args)
+
+
+if __name__ == "__main__":
+    main()

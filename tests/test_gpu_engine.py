@@ -193,3 +193,44 @@ def test_recorded_decode_steps_equal_eager_ones(folders, name, dtype):
     assert len(outs[0]) == len(outs[1])
     for n, (a, b) in enumerate(zip(*outs)):
         assert torch.equal(a, b), "step %d: a replayed step differs from the eager step" % n
+
+
+def test_eviction_and_recomputation_keep_the_tokens(folders):
+    """When pages run out the newest request is evicted and later fed again from its first token; in
+    32-bit its continuation is the same as with room for everybody."""
+    from ginfer_amd import Engine, EngineConfig, SamplingParams
+    name = "B"
+    vocab = H.TINY[name][0]["vocab_size"]
+    prompts = [H.random_tokens(n, vocab, 700 + n) for n in (30, 41, 52, 25)]
+    results = []
+    for blocks in (64, 14):                       # 14 pages of 8: two requests of ~80 tokens do not fit beside a third
+        eng = Engine(EngineConfig(model_path=folders[name], dtype="float32", max_num_batched_tokens=48, max_num_seqs=4,
+                                  max_seq_len=128, kvcache_block_size=8, num_kvcache_blocks=blocks))
+        outs = eng.generate(prompts, [SamplingParams(max_tokens=30, ignore_eos=True, temperature=t, seed=5)
+                                      for t in (0.0, 0.0, 0.7, 0.7)])
+        eng.runner.cache.check()
+        assert not eng.runner.cache.requests
+        results.append((outs, eng.scheduler.num_evictions))
+    (big, ev_big), (small, ev_small) = results
+    assert ev_big == 0 and ev_small > 0
+    for a, b in zip(big, small):
+        assert a.token_ids == b.token_ids and len(a.token_ids) == 30
+    assert max(o.evictions for o in small) >= 1
+
+
+def test_command_line(folders, tmp_path):
+    import json
+    import subprocess
+    import sys
+    import os
+    name = "A"
+    env = dict(os.environ, MODEL_PATH=str(folders[name]))
+    cmd = [sys.executable, os.path.join(H.ROOT, "bin", "ginfer"), "generate", "--dtype", "float32", "--prompt-ids", "5,17,3",
+           "--prompt-ids", "9 8 7 6", "--max-tokens", "6", "--ignore-eos", "--max-num-seqs", "2", "--max-seq-len", "64",
+           "--num-kvcache-blocks", "16"]
+    out = subprocess.run(cmd, env=env, capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stderr
+    lines = [json.loads(l) for l in out.stdout.strip().splitlines()]
+    cfg, w = pm.read_config(folders[name]), pm.read_weights(folders[name])
+    assert [l["token_ids"] for l in lines] == [pm.generate(cfg, w, p, 6, ignore_eos=True) for p in ([5, 17, 3], [9, 8, 7, 6])]
+    assert "decode=" in out.stderr and "ttft=" in out.stderr
