@@ -28,25 +28,38 @@ __device__ __forceinline__ bf16x8 load8(const bf16_t* p) {
   return __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(p));
 }
 
-template <int NT, int MB, typename TC>
+// NT: 16-row tiles of W per wavefront; MB: 16-row blocks of A; KS: wavefronts of a workgroup that split K
+// for the same rows (the workgroup's SK_WAVES / KS groups own different rows of W).  The grid's y
+// dimension splits K further: then every workgroup writes its part in 32-bit to P[y][M][N] and the
+// consumer adds the parts in order (the bias rides on part 0).
+// GATED (NT == 2): W holds two stacked matrices of N rows each (gate over up); the wavefront's two tiles
+// are rows n0.. of the gate and the same rows of the up matrix, and the epilogue writes
+// silu(gate) * up = (g * (1 / (1 + exp(-g)))) * u (ginfer/core/op/kernels/cuda/swiglu_kernel.cu:24-27) for N
+// columns: the activation of the feed-forward without a pass over memory of its own.
+template <int NT, int MB, int KS, typename TC, bool GATED>
 __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(TC* __restrict__ C, int64_t ldc,
                                                                  const bf16_t* __restrict__ A, int64_t lda,
                                                                  const bf16_t* __restrict__ W,
                                                                  const bf16_t* __restrict__ bias, int M, int N,
-                                                                 int K, int kchunk) {
+                                                                 int K, int kchunk_wg, int kchunk_wave) {
   __shared__ float red[SK_WAVES][NT * 16][MB * 16 + 1];
+  constexpr int GROUPS = SK_WAVES / KS;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r = lane & 15, g = lane >> 4;
-  const int n0 = blockIdx.x * NT * 16;
-  const int kb = wave * kchunk;
-  const int ke = kb + kchunk < K ? kb + kchunk : K;
+  const int grp = wave / KS, ks = wave % KS;
+  constexpr int NCOL = GATED ? 16 : NT * 16;       // output columns of a group
+  const int n0 = (blockIdx.x * GROUPS + grp) * NCOL;
+  const int kwg = blockIdx.y * kchunk_wg;
+  const int kwg_end = kwg + kchunk_wg < K ? kwg + kchunk_wg : K;
+  const int kb = kwg + ks * kchunk_wave;
+  const int ke = kb + kchunk_wave < kwg_end ? kb + kchunk_wave : kwg_end;
 
   const bf16_t* wp[NT];
   bool wok[NT];
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) {
-    const int n = n0 + nt * 16 + r;
+    const int n = GATED ? n0 + r : n0 + nt * 16 + r;
     wok[nt] = n < N;
-    wp[nt] = W + (int64_t)(wok[nt] ? n : 0) * K;
+    wp[nt] = W + ((int64_t)(wok[nt] ? n : 0) + (GATED ? (int64_t)nt * N : 0)) * K;
   }
   const bf16_t* ap[MB];
   bool aok[MB];
@@ -62,25 +75,33 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(TC* __restrict_
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) acc[nt][mb] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-#pragma unroll 2
-  for (int k = kb; k < ke; k += 64) {
+  // UNROLL steps of 64 elements per trip, all loads of a trip issued before its products; the guard on
+  // every 8-element piece makes the tail of the range safe
+  constexpr int UNROLL = (NT * MB <= 4) ? 4 : 2;
+  for (int k = kb; k < ke; k += 64 * UNROLL) {
+    bf16x8 a[UNROLL][2][NT], b[UNROLL][2][MB];
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int kk = k + g * 16 + j * 8;
-      const bool ok = kk < ke;
-      bf16x8 a[NT], b[MB];
+    for (int u = 0; u < UNROLL; ++u)
 #pragma unroll
-      for (int nt = 0; nt < NT; ++nt) a[nt] = (ok && wok[nt]) ? load8(wp[nt] + kk) : zero8();
+      for (int j = 0; j < 2; ++j) {
+        const int kk = k + u * 64 + g * 16 + j * 8;
+        const bool ok = kk < ke;
 #pragma unroll
-      for (int mb = 0; mb < MB; ++mb) b[mb] = (ok && aok[mb]) ? load8(ap[mb] + kk) : zero8();
+        for (int nt = 0; nt < NT; ++nt) a[u][j][nt] = (ok && wok[nt]) ? load8(wp[nt] + kk) : zero8();
 #pragma unroll
-      for (int nt = 0; nt < NT; ++nt)
+        for (int mb = 0; mb < MB; ++mb) b[u][j][mb] = (ok && aok[mb]) ? load8(ap[mb] + kk) : zero8();
+      }
 #pragma unroll
-        for (int mb = 0; mb < MB; ++mb)
-          acc[nt][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[nt], b[mb], acc[nt][mb], 0, 0, 0);
-    }
+    for (int u = 0; u < UNROLL; ++u)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+          for (int mb = 0; mb < MB; ++mb)
+            acc[nt][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][j][nt], b[u][j][mb], acc[nt][mb], 0, 0, 0);
   }
-  // parts of the K-split meet in LDS and are added in wavefront order
+  // the KS parts of a group meet in LDS and are added in wavefront order
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
@@ -88,44 +109,85 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(TC* __restrict_
 #pragma unroll
       for (int i = 0; i < 4; ++i) red[wave][nt * 16 + g * 4 + i][mb * 16 + r] = acc[nt][mb][i];
   __syncthreads();
-  for (int idx = threadIdx.x; idx < NT * 16 * MB * 16; idx += SK_THREADS) {
-    const int nl = idx % (NT * 16), m = idx / (NT * 16);
-    const int n = n0 + nl;
+  const bool partial = gridDim.y > 1;
+  float* P = reinterpret_cast<float*>(C) + (int64_t)blockIdx.y * M * N;      // parts are [y][M][N], dense
+  for (int idx = threadIdx.x; idx < GROUPS * NCOL * MB * 16; idx += SK_THREADS) {
+    const int nl = idx % NCOL, rest = idx / NCOL;
+    const int gi = rest % GROUPS, m = rest / GROUPS;
+    const int n = (blockIdx.x * GROUPS + gi) * NCOL + nl;
     if (m >= M || n >= N) continue;
     float v = 0.f;
 #pragma unroll
-    for (int w = 0; w < SK_WAVES; ++w) v += red[w][nl][m];
-    if (bias) v += bf16_to_f32(bias[n]);
-    Num<TC>::st(C + (int64_t)m * ldc + n, v);
+    for (int w = 0; w < KS; ++w) v += red[gi * KS + w][nl][m];
+    if (GATED) {
+      float u = 0.f;
+#pragma unroll
+      for (int w = 0; w < KS; ++w) u += red[gi * KS + w][16 + nl][m];
+      v = (v * (1.0f / (1.0f + expf(-v)))) * u;
+    }
+    if (bias && blockIdx.y == 0) v += bf16_to_f32(bias[n]);
+    if (partial) P[(int64_t)m * N + n] = v;
+    else Num<TC>::st(C + (int64_t)m * ldc + n, v);
   }
 }
 
-// A [M, K] (row stride lda), W [N, K] contiguous, bias [N] or null, C [M, N] (row stride ldc) in
-// bfloat16 or float.  M <= 64, K a multiple of 8, rows 16-byte aligned.
+// A [M, K] (row stride lda), W [N, K] contiguous, bias [N] or null.  grid_splits == 1: C [M, N] (row
+// stride ldc) in bfloat16 or float.  grid_splits > 1: C is float [grid_splits][M][N], parts to be added
+// by the consumer.  gated: W is [2N, K] (gate over up), C [M, N] = silu(A.gate^T) * (A.up^T), no bias, no
+// grid split.  M <= 64, K a multiple of 8, rows 16-byte aligned.  nt in {1,2,4}, ks in {1,2,4,8}; 0 lets
+// the library choose.
 extern "C" int ga_gemm_skinny(void* C, int64_t ldc, const void* A, int64_t lda, const void* W, const void* bias,
-                              int M, int N, int K, int out_f32, hipStream_t stream) {
+                              int M, int N, int K, int out_f32, int nt, int ks, int grid_splits, int gated,
+                              hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
-  if (M > 64 || K <= 0 || K % 8 || lda % 8) return -1;
+  if (M > 64 || K <= 0 || K % 8 || lda % 8 || grid_splits < 1) return -1;
   const int mb = (M + 15) / 16;
-  const int nt = N >= 4096 ? 2 : 1;
-  int kchunk = ((K + SK_WAVES - 1) / SK_WAVES + 63) / 64 * 64;
-  dim3 grid((N + nt * 16 - 1) / (nt * 16)), block(SK_THREADS);
-#define LAUNCH(NT, MB, TC)                                                                              \
-  hipLaunchKernelGGL((gemm_skinny_kernel<NT, MB, TC>), grid, block, 0, stream, (TC*)C, ldc,            \
-                     (const bf16_t*)A, lda, (const bf16_t*)W, (const bf16_t*)bias, M, N, K, kchunk)
-#define PICK_MB(NT, TC)                                                                                 \
+  if (gated) nt = 2;
+  if (nt == 0) nt = (N >= 4096 && mb > 1) ? 4 : 1;
+  if (ks == 0) ks = 8;
+  if ((nt != 1 && nt != 2 && nt != 4) || (ks != 1 && ks != 2 && ks != 4 && ks != 8)) return -2;
+  if (nt == 4 && mb > 2 && ks < 2) return -2;      // LDS of the reduction
+  if (grid_splits > 1 && !out_f32) return -3;
+  if (gated && (grid_splits > 1 || bias)) return -4;
+  const int groups = SK_WAVES / ks;
+  const int ncol = gated ? 16 : nt * 16;
+  const int kchunk_wg = ((K + grid_splits - 1) / grid_splits + 63) / 64 * 64;
+  const int kchunk_wave = ((kchunk_wg + ks - 1) / ks + 63) / 64 * 64;
+  dim3 grid((N + groups * ncol - 1) / (groups * ncol), grid_splits), block(SK_THREADS);
+#define LAUNCH(NT, MB, KS, TC, G)                                                                       \
+  hipLaunchKernelGGL((gemm_skinny_kernel<NT, MB, KS, TC, G>), grid, block, 0, stream, (TC*)C, ldc,     \
+                     (const bf16_t*)A, lda, (const bf16_t*)W, (const bf16_t*)bias, M, N, K, kchunk_wg, \
+                     kchunk_wave)
+#define PICK_KS(NT, MB, TC, G)                                                                          \
+  switch (ks) {                                                                                         \
+    case 1: LAUNCH(NT, MB, 1, TC, G); break;                                                            \
+    case 2: LAUNCH(NT, MB, 2, TC, G); break;                                                            \
+    case 4: LAUNCH(NT, MB, 4, TC, G); break;                                                            \
+    default: LAUNCH(NT, MB, 8, TC, G); break;                                                           \
+  }
+#define PICK_MB(NT, TC, G)                                                                              \
   switch (mb) {                                                                                         \
-    case 1: LAUNCH(NT, 1, TC); break;                                                                   \
-    case 2: LAUNCH(NT, 2, TC); break;                                                                   \
-    case 3: LAUNCH(NT, 3, TC); break;                                                                   \
-    default: LAUNCH(NT, 4, TC); break;                                                                  \
+    case 1: PICK_KS(NT, 1, TC, G) break;                                                                \
+    case 2: PICK_KS(NT, 2, TC, G) break;                                                                \
+    case 3: PICK_KS(NT, 3, TC, G) break;                                                                \
+    default: PICK_KS(NT, 4, TC, G) break;                                                               \
   }
-  if (out_f32) {
-    if (nt == 2) { PICK_MB(2, float) } else { PICK_MB(1, float) }
+#define PICK_NT(TC)                                                                                     \
+  switch (nt) {                                                                                         \
+    case 1: PICK_MB(1, TC, false) break;                                                                \
+    case 2: PICK_MB(2, TC, false) break;                                                                \
+    default: PICK_MB(4, TC, false) break;                                                               \
+  }
+  if (gated) {
+    if (out_f32) { PICK_MB(2, float, true) } else { PICK_MB(2, bf16_t, true) }
+  } else if (out_f32) {
+    PICK_NT(float)
   } else {
-    if (nt == 2) { PICK_MB(2, bf16_t) } else { PICK_MB(1, bf16_t) }
+    PICK_NT(bf16_t)
   }
+#undef PICK_NT
 #undef PICK_MB
+#undef PICK_KS
 #undef LAUNCH
   return GA_CHECK_LAUNCH();
 }

@@ -12,20 +12,27 @@
 
 #define NORM_THREADS 256
 
-template <typename T, typename G>
+// D is the type of delta: the compute dtype, or float when delta holds `parts` partial sums of a
+// K-split matrix product ([parts][T][H]); the parts are added in order, after one another.
+template <typename T, typename G, typename D>
 __global__ void add_rmsnorm_kernel(T* __restrict__ out, float* __restrict__ residual,
-                                   const T* __restrict__ delta, const G* __restrict__ gain,
-                                   const int32_t* __restrict__ rows, int hidden, float eps) {
+                                   const D* __restrict__ delta, int parts, int64_t part_stride,
+                                   const G* __restrict__ gain, const int32_t* __restrict__ rows, int hidden,
+                                   float eps) {
   __shared__ float scratch[NORM_THREADS / WAVE];
   const int64_t r = blockIdx.x;
   const int64_t t = rows ? (int64_t)rows[r] : r;
   float* res = residual + t * hidden;
-  const T* d = delta ? delta + t * hidden : nullptr;
+  const D* d = delta ? delta + t * hidden : nullptr;
   const bool write_back = (rows == nullptr) && (d != nullptr);
   float ss = 0.f;
   for (int i = threadIdx.x; i < hidden; i += NORM_THREADS) {
     float h = res[i];
-    if (d) h += Num<T>::ld(d + i);
+    if (d) {
+      float add = Num<D>::ld(d + i);
+      for (int p = 1; p < parts; ++p) add += Num<D>::ld(d + p * part_stride + i);
+      h += add;
+    }
     if (write_back) res[i] = h;
     ss += h * h;
   }
@@ -34,26 +41,38 @@ __global__ void add_rmsnorm_kernel(T* __restrict__ out, float* __restrict__ resi
   T* o = out + r * hidden;
   for (int i = threadIdx.x; i < hidden; i += NORM_THREADS) {
     float h = res[i];                       // own write of the first pass when write_back
-    if (d && !write_back) h += Num<T>::ld(d + i);
+    if (d && !write_back) {
+      float add = Num<D>::ld(d + i);
+      for (int p = 1; p < parts; ++p) add += Num<D>::ld(d + p * part_stride + i);
+      h += add;
+    }
     Num<T>::st(o + i, (h * Num<G>::ld(gain + i)) / rms);
   }
 }
 
-// out: [R, H] in the compute dtype; residual: [T, H] float; delta: [T, H] compute dtype or null;
-// gain: [H] compute dtype, or float when gain_is_f32; rows: [R] int32 or null (then R == T).
-extern "C" int ga_add_rmsnorm(void* out, void* residual, const void* delta, const void* gain,
-                              const void* rows, int num_rows, int hidden, float eps, int is_bf16,
-                              int gain_is_f32, hipStream_t stream) {
+// out: [R, H] in the compute dtype; residual: [T, H] float; delta: [T, H] compute dtype or null, or, with
+// delta_parts > 0, float [delta_parts][T][H] partial sums; gain: [H] compute dtype, or float when
+// gain_is_f32; rows: [R] int32 or null (then R == T); num_tokens = T.
+extern "C" int ga_add_rmsnorm(void* out, void* residual, const void* delta, int delta_parts, int num_tokens,
+                              const void* gain, const void* rows, int num_rows, int hidden, float eps,
+                              int is_bf16, int gain_is_f32, hipStream_t stream) {
   if (num_rows <= 0) return 0;
   dim3 grid(num_rows), block(NORM_THREADS);
-#define LAUNCH(T, G)                                                                              \
-  hipLaunchKernelGGL((add_rmsnorm_kernel<T, G>), grid, block, 0, stream, (T*)out,                \
-                     (float*)residual, (const T*)delta, (const G*)gain, (const int32_t*)rows,     \
-                     hidden, eps)
-  if (is_bf16) {
-    if (gain_is_f32) LAUNCH(bf16_t, float); else LAUNCH(bf16_t, bf16_t);
+  const int64_t stride = (int64_t)num_tokens * hidden;
+#define LAUNCH(T, G, D, PARTS)                                                                    \
+  hipLaunchKernelGGL((add_rmsnorm_kernel<T, G, D>), grid, block, 0, stream, (T*)out,             \
+                     (float*)residual, (const D*)delta, PARTS, stride, (const G*)gain,            \
+                     (const int32_t*)rows, hidden, eps)
+  if (delta_parts > 0) {
+    if (is_bf16) {
+      if (gain_is_f32) LAUNCH(bf16_t, float, float, delta_parts); else LAUNCH(bf16_t, bf16_t, float, delta_parts);
+    } else {
+      LAUNCH(float, float, float, delta_parts);
+    }
+  } else if (is_bf16) {
+    if (gain_is_f32) LAUNCH(bf16_t, float, bf16_t, 1); else LAUNCH(bf16_t, bf16_t, bf16_t, 1);
   } else {
-    LAUNCH(float, float);
+    LAUNCH(float, float, float, 1);
   }
 #undef LAUNCH
   return GA_CHECK_LAUNCH();

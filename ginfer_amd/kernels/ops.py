@@ -71,12 +71,18 @@ def embedding_gather(table, ids, out=None):
 
 def add_rmsnorm(residual, delta, gain, eps, dtype, rows=None, out=None):
     """residual float32 [T, H] (updated in place with + delta unless rows is given); delta [T, H] in
-    `dtype` or None; gain [H] in `dtype` (or float32); rows int32 [R] or None -> normed [R or T, H]."""
+    `dtype`, or float32 [parts, T, H] (partial sums of a K-split product, added in order), or None;
+    gain [H] in `dtype` (or float32); rows int32 [R] or None -> normed [R or T, H]."""
     _dev(residual, delta, gain, rows, out)
     _need(residual.dtype == torch.float32 and residual.dim() == 2 and residual.is_contiguous(),
           "residual must be contiguous float32 [T, H]")
     T, H = residual.shape
-    if delta is not None:
+    parts = 0
+    if delta is not None and delta.dim() == 3:
+        _need(delta.dtype == torch.float32 and delta.shape[1:] == (T, H) and delta.is_contiguous() and delta.shape[0] >= 1,
+              "partial sums must be contiguous float32 [parts, %d, %d], got %s %s" % (T, H, delta.dtype, tuple(delta.shape)))
+        parts = delta.shape[0]
+    elif delta is not None:
         _need(delta.dtype == dtype and delta.shape == (T, H) and delta.is_contiguous(),
               "delta must be contiguous %s [%d, %d], got %s %s" % (dtype, T, H, delta.dtype, tuple(delta.shape)))
     _need(gain.shape == (H,) and gain.is_contiguous() and gain.dtype in (dtype, torch.float32),
@@ -89,7 +95,7 @@ def add_rmsnorm(residual, delta, gain, eps, dtype, rows=None, out=None):
         out = torch.empty((R, H), dtype=dtype, device=residual.device)
     _need(out.dtype == dtype and out.shape == (R, H) and out.is_contiguous(), "out must be contiguous [R, H]")
     lib = build.load("norm")
-    _check(lib.ga_add_rmsnorm(_ptr(out), _ptr(residual), _ptr(delta), _ptr(gain), _ptr(rows), _i(R), _i(H),
+    _check(lib.ga_add_rmsnorm(_ptr(out), _ptr(residual), _ptr(delta), _i(parts), _i(T), _ptr(gain), _ptr(rows), _i(R), _i(H),
                               _f(eps), _i(_is_bf16(dtype)),
                               _i(1 if (gain.dtype == torch.float32 and dtype != torch.float32) else 0),
                               _stream()), "add_rmsnorm")
@@ -238,9 +244,11 @@ def gemm_skinny_supported(a, w):
             and w.is_contiguous() and w.data_ptr() % 16 == 0)
 
 
-def gemm_skinny(a, w, bias=None, out=None, out_dtype=None):
+def gemm_skinny(a, w, bias=None, out=None, out_dtype=None, nt=0, ks=0, grid_splits=1, gated=False):
     """a [M <= 64, K] . w [N, K]^T (+ bias) -> [M, N] in bfloat16 (or float32): the decode step's products,
-    weights streamed once through the matrix cores."""
+    weights streamed once through the matrix cores.  grid_splits > 1: K is split over workgroups too and
+    the result is float32 [grid_splits, M, N], parts for the consumer to add.  gated: w is [2N, K] (gate
+    over up) and the result is silu(a.gate^T) * (a.up^T)."""
     _dev(a, w, bias, out)
     _need(a.dim() == 2 and w.dim() == 2 and a.shape[1] == w.shape[1], "gemm_skinny: a [M, K] and w [N, K] do not agree: %s, %s"
           % (tuple(a.shape), tuple(w.shape)))
@@ -248,16 +256,29 @@ def gemm_skinny(a, w, bias=None, out=None, out_dtype=None):
           "aligned rows; got a %s %s, w %s %s" % (SKINNY_MAX_ROWS, a.dtype, tuple(a.shape), w.dtype, tuple(w.shape)))
     M, K = a.shape
     N = w.shape[0]
+    if gated:       # w stacks gate over up: the result has half as many columns
+        _need(N % 2 == 0 and bias is None and grid_splits == 1, "gated product: w must be [2N, K], without bias or split")
+        N //= 2
     if bias is not None:
         _need(bias.dtype == torch.bfloat16 and bias.shape == (N,) and bias.is_contiguous(), "gemm_skinny: bias must be bfloat16 [N]")
     out_dtype = out_dtype or (out.dtype if out is not None else torch.bfloat16)
     _need(out_dtype in (torch.bfloat16, torch.float32), "gemm_skinny: out dtype must be bfloat16 or float32")
-    if out is None:
-        out = torch.empty((M, N), dtype=out_dtype, device=a.device)
-    _need(out.shape == (M, N) and out.dtype == out_dtype and out.stride(1) == 1, "gemm_skinny: out must be [M, N]")
+    if grid_splits > 1:
+        _need(out_dtype == torch.float32, "gemm_skinny: parts of a split product are float32")
+        if out is None:
+            out = torch.empty((grid_splits, M, N), dtype=torch.float32, device=a.device)
+        _need(out.shape == (grid_splits, M, N) and out.dtype == torch.float32 and out.is_contiguous(),
+              "gemm_skinny: parts must be contiguous float32 [splits, M, N]")
+        ldc = N
+    else:
+        if out is None:
+            out = torch.empty((M, N), dtype=out_dtype, device=a.device)
+        _need(out.shape == (M, N) and out.dtype == out_dtype and out.stride(1) == 1, "gemm_skinny: out must be [M, N]")
+        ldc = out.stride(0)
     lib = build.load("gemm_skinny")
-    _check(lib.ga_gemm_skinny(_ptr(out), _i64(out.stride(0)), _ptr(a), _i64(a.stride(0)), _ptr(w), _ptr(bias), _i(M), _i(N),
-                              _i(K), _i(1 if out_dtype == torch.float32 else 0), _stream()), "gemm_skinny")
+    _check(lib.ga_gemm_skinny(_ptr(out), _i64(ldc), _ptr(a), _i64(a.stride(0)), _ptr(w), _ptr(bias), _i(M), _i(N),
+                              _i(K), _i(1 if out_dtype == torch.float32 else 0), _i(nt), _i(ks), _i(grid_splits),
+                              _i(1 if gated else 0), _stream()), "gemm_skinny")
     return out
 
 

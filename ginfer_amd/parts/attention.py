@@ -68,4 +68,4 @@ class Attention(Part):
                           self.nh, self.nkv, self.hd, write_kv=cache.owner)
         a = ops.paged_attention(qkv, cache.k_pages, cache.v_pages, cache.block_table, step, self.nh, self.nkv,
                                 self.hd, self.scale, self.window)
-        return linear(a, self.w_o, self.b_o)
+        return linear(a, self.w_o, self.b_o, parts_ok=True)

@@ -12,12 +12,13 @@ Every part
     host-side numbers are: it reads sizes only from tensor shapes, does nothing that waits for the device,
     and takes everything that changes from step to step from the step's device arrays.
 
-Mixer         forward(x [T, H], step, cache) -> [T, H]
+Mixer         forward(x [T, H], step, cache) -> [T, H], or float32 [parts, T, H]: partial sums that the
+              norm which follows adds up in order (what a K-split matrix product leaves)
               cache_spec() -> KVCacheSpec | StateSpec | None: what one run of this mixer keeps per
               request; `cache` in forward is the matching view (`KVView`, `StateView` or None) of the
               schedule entry that is running.  `step` is the `StepContext` of the batch.
-FeedForward   forward(x [T, H]) -> [T, H]
-Norm          forward(residual float32 [T, H], delta [T, H] | None, rows=None) -> [R or T, H]
+FeedForward   forward(x [T, H]) -> [T, H] (or partial sums, as a mixer)
+Norm          forward(residual float32 [T, H], delta [T, H] | [parts, T, H] | None, rows=None) -> [R or T, H]
               adds delta into the 32-bit residual stream and returns the normalised rows; with `rows`
               (int32 indices) only those rows are returned and the residual is left as it is.
 Position      what the mixer's kernel needs to encode positions (for rotary kinds: `tables()`).

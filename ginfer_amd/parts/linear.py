@@ -9,11 +9,20 @@ import torch
 from ..kernels import ops
 
 
-def linear(x, weight, bias=None, out_dtype=None):
-    """x [M, K], weight [N, K], bias [N] | None -> [M, N] in x's dtype (or float32 on request)."""
+# a product with at least this many input features whose consumer adds partial sums is split over K
+SPLIT_K_FROM = 4096
+SPLIT_K_PARTS = 4
+
+
+def linear(x, weight, bias=None, out_dtype=None, parts_ok=False):
+    """x [M, K], weight [N, K], bias [N] | None -> [M, N] in x's dtype (or float32 on request).
+    With parts_ok the result may instead be float32 [parts, M, N]: partial sums of a K-split product,
+    which the norm that follows adds up in order."""
     if x.dtype == torch.float32:
         return ops.gemm_nt(x, weight, bias)
     if ops.gemm_skinny_supported(x, weight):
+        if parts_ok and out_dtype is None and x.shape[1] >= SPLIT_K_FROM:
+            return ops.gemm_skinny(x, weight, bias, out_dtype=torch.float32, grid_splits=SPLIT_K_PARTS)
         return ops.gemm_skinny(x, weight, bias, out_dtype=out_dtype)
     if out_dtype == torch.float32:
         y = torch.mm(x, weight.t(), out_dtype=torch.float32)
@@ -23,3 +32,10 @@ def linear(x, weight, bias=None, out_dtype=None):
     if bias is not None:
         return torch.addmm(bias, x, weight.t())
     return torch.mm(x, weight.t())
+
+
+def gated_linear(x, weight_gate_up):
+    """silu(x . Wg^T) * (x . Wu^T) with Wg over Wu stacked in one matrix [2I, K] -> [M, I]."""
+    if x.dtype == torch.bfloat16 and ops.gemm_skinny_supported(x, weight_gate_up):
+        return ops.gemm_skinny(x, weight_gate_up, gated=True)
+    return ops.silu_mul(linear(x, weight_gate_up))

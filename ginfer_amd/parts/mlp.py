@@ -4,7 +4,7 @@ import torch
 from ..kernels import ops
 from ..weights.loader import WeightSpec
 from .base import Part
-from .linear import linear
+from .linear import linear, gated_linear
 from .registry import register_feed_forward
 
 
@@ -33,5 +33,5 @@ class SwiGLU(Part):
         return ["activation", "gemm"] + (["gemm_skinny"] if self.dtype == torch.bfloat16 else [])
 
     def forward(self, x):
-        gu = linear(x, self.w_gate_up)
-        return linear(ops.silu_mul(gu), self.w_down)
+        # the result may be partial sums of a K-split product: the norm that follows adds them up
+        return linear(gated_linear(x, self.w_gate_up), self.w_down, parts_ok=True)

@@ -406,3 +406,37 @@ def test_gemm_skinny_refuses_other_shapes():
     assert not ops.gemm_skinny_supported(rnd((4, 64), torch.float32, 1), rnd((8, 64), torch.float32, 2))
     with pytest.raises(KernelError):
         ops.gemm_skinny(rnd((65, 64), torch.bfloat16, 1), rnd((8, 64), torch.bfloat16, 2))
+
+
+@pytest.mark.parametrize("M", [1, 8, 33, 64])
+@pytest.mark.parametrize("N,K", [(1536, 8960), (1536, 1536), (200, 4096), (777, 88)])
+@pytest.mark.parametrize("nt,ks,gs", [(1, 8, 4), (2, 4, 2), (4, 8, 8), (1, 1, 3), (4, 2, 1), (2, 8, 1)])
+def test_gemm_skinny_tilings_and_split_parts(M, N, K, nt, ks, gs):
+    from ginfer_amd.kernels import ops
+    if K // (gs * ks) < 8:
+        pytest.skip("K too small for this split")
+    a, w, b = rnd((M, K), torch.bfloat16, 40), rnd((N, K), torch.bfloat16, 41), rnd((N,), torch.bfloat16, 42)
+    ref = a.double() @ w.double().t() + b.double()
+    out = ops.gemm_skinny(a, w, b, out_dtype=torch.float32, nt=nt, ks=ks, grid_splits=gs)
+    if gs > 1:
+        assert out.shape == (gs, M, N)
+        # the norm that follows adds the parts to the residual stream
+        res = rnd((M, N), torch.float32, 43)
+        gain = torch.ones(N, dtype=torch.bfloat16, device=dev())
+        r2 = res.clone()
+        normed = ops.add_rmsnorm(r2, out, gain, 1e-6, torch.bfloat16)
+        close(r2, res.double() + ref, 1e-5)
+        close(normed, pm.rms_norm(res.double() + ref, gain.double(), 1e-6), 1e-2)
+        out = out.sum(0)
+    close(out, ref, 1e-5)
+
+
+@pytest.mark.parametrize("M", [1, 8, 17, 64])
+@pytest.mark.parametrize("I,K", [(8960, 1536), (160, 64), (136, 88), (448, 192)])
+def test_gemm_skinny_gated(M, I, K):
+    from ginfer_amd.kernels import ops
+    a, w = rnd((M, K), torch.bfloat16, 50), rnd((2 * I, K), torch.bfloat16, 51, scale=0.3)
+    g, u = a.double() @ w[:I].double().t(), a.double() @ w[I:].double().t()
+    ref = pm.swiglu(g, u)
+    close(ops.gemm_skinny(a, w, gated=True, out_dtype=torch.float32), ref, 1e-5)
+    close(ops.gemm_skinny(a, w, gated=True), ref, 1e-2)
