@@ -288,7 +288,7 @@ MFMA_HEAD_DIMS = tuple(range(16, 257, 16))
 _DECODE_TARGET_WORKGROUPS = 512       # four wavefronts each: enough to fill 256 compute units
 _MIN_SPLIT_KEYS = 128                 # one tile of 32 keys for each wavefront of a workgroup
 _MAX_SPLITS = 256
-PREFILL_WIDE_TILES_FROM = 1 << 30     # tokens in a step from which prompt rows go 32 to a wavefront
+PREFILL_WIDE_TILES_FROM = 512         # tokens in a step from which prompt rows go 32 to a wavefront
 
 
 def attention_mfma_supported(dtype, head_dim, page_size):

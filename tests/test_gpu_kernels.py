@@ -43,7 +43,8 @@ def test_embedding(dtype, tol, T, V, H):
 
 
 @pytest.mark.parametrize("dtype,tol", DTYPES)
-@pytest.mark.parametrize("T,H,eps", [(3 * 127, 128, 1e-5), (5, 1536, 1e-6), (17, 88, 3e-6), (2, 8192, 1e-6)])
+@pytest.mark.parametrize("T,H,eps", [(3 * 127, 128, 1e-5), (5, 1536, 1e-6), (17, 88, 3e-6), (2, 8192, 1e-6), (3, 8200, 1e-6),
+                                     (4, 77, 1e-5), (2, 3584, 1e-6)])
 def test_add_rmsnorm(dtype, tol, T, H, eps):
     from ginfer_amd.kernels import ops
     res = rnd((T, H), torch.float32, 2)
@@ -73,7 +74,7 @@ def test_add_rmsnorm(dtype, tol, T, H, eps):
 
 
 @pytest.mark.parametrize("dtype,tol", DTYPES)
-@pytest.mark.parametrize("T,I", [(4 * 128, 256), (2 * 511, 1024), (1023, 2048), (3, 136), (1, 8960)])
+@pytest.mark.parametrize("T,I", [(4 * 128, 256), (2 * 511, 1024), (1023, 2048), (3, 136), (1, 8960), (5, 77), (2049, 8960)])
 def test_silu_mul(dtype, tol, T, I):
     from ginfer_amd.kernels import ops
     gu = rnd((T, 2 * I), dtype, 5, scale=3.0)
@@ -111,7 +112,8 @@ def test_gemm_nt_rows_do_not_depend_on_the_batch():
 
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-4), (torch.bfloat16, 1e-2)])
 @pytest.mark.parametrize("T,nh,nkv,hd,rd,theta", [(128, 32, 8, 128, 128, 1e4), (64, 12, 12, 64, 64, 1e4),
-                                                  (9, 6, 3, 48, 48, 5e5), (5, 4, 2, 32, 16, 1e6)])
+                                                  (9, 6, 3, 48, 48, 5e5), (5, 4, 2, 32, 16, 1e6), (7, 3, 1, 24, 20, 1e4),
+                                                  (300, 12, 2, 128, 128, 1e4)])
 def test_rope_and_cache_write(dtype, tol, T, nh, nkv, hd, rd, theta):
     from ginfer_amd.kernels import ops
     ps, pages = 8, 64
