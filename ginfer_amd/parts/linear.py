@@ -21,9 +21,16 @@ def linear(x, weight, bias=None, out_dtype=None, parts_ok=False):
     if x.dtype == torch.float32:
         return ops.gemm_nt(x, weight, bias)
     if ops.gemm_skinny_supported(x, weight):
+        # tilings measured on MI355X (graph replays, weights not cache-resident): up to 16 rows one
+        # 16-row tile of W per wavefront streams best; beyond, four tiles halve the re-reading of x; a
+        # long K is split over workgroups where the consumer can add the parts
+        many = x.shape[0] > 16
         if parts_ok and out_dtype is None and x.shape[1] >= SPLIT_K_FROM:
-            return ops.gemm_skinny(x, weight, bias, out_dtype=torch.float32, grid_splits=SPLIT_K_PARTS)
-        return ops.gemm_skinny(x, weight, bias, out_dtype=out_dtype)
+            return ops.gemm_skinny(x, weight, bias, out_dtype=torch.float32, nt=4 if many else 1,
+                                   grid_splits=2 * SPLIT_K_PARTS if many else SPLIT_K_PARTS)
+        if parts_ok and out_dtype is None and x.shape[1] >= 1024:
+            return ops.gemm_skinny(x, weight, bias, out_dtype=torch.float32, nt=1, grid_splits=2)
+        return ops.gemm_skinny(x, weight, bias, out_dtype=out_dtype, nt=4 if (many and weight.shape[0] >= 4096) else 1)
     if out_dtype == torch.float32:
         y = torch.mm(x, weight.t(), out_dtype=torch.float32)
         if bias is not None:

@@ -234,3 +234,40 @@ def test_command_line(folders, tmp_path):
     cfg, w = pm.read_config(folders[name]), pm.read_weights(folders[name])
     assert [l["token_ids"] for l in lines] == [pm.generate(cfg, w, p, 6, ignore_eos=True) for p in ([5, 17, 3], [9, 8, 7, 6])]
     assert "decode=" in out.stderr and "ttft=" in out.stderr
+
+
+def test_real_layer_sizes(tmp_path):
+    """Two layers of the 1.5B shape (width 1536, 12 heads in 2 groups of head size 128, feed-forward 8960,
+    vocabulary 151,936): the sizes the kernels serve, cut and batched in every way, in both dtypes."""
+    from ginfer_amd import ModelRunner
+    cfg = dict(architectures=["Qwen2ForCausalLM"], num_hidden_layers=2, hidden_size=1536, num_attention_heads=12,
+               num_key_value_heads=2, intermediate_size=8960, vocab_size=151936, rope_theta=10000.0, rms_norm_eps=1e-6,
+               tie_word_embeddings=False, max_position_embeddings=4096, use_sliding_window=False, sliding_window=4096,
+               max_window_layers=21)
+    folder = H.make_model_folder(tmp_path / "real", cfg, 3, "float32")
+    reqs = {"a": H.random_tokens(150, 151936, 1), "b": H.random_tokens(70, 151936, 2), "c": H.random_tokens(40, 151936, 3)}
+    pcfg, w = pm.read_config(folder), pm.read_weights(folder, torch.float32)
+    refs = {rid: pm.forward(pcfg, w, ids).numpy() for rid, ids in reqs.items()}
+    del w
+    want_last = 34          # logits of the last places only: the vocabulary is wide
+    for dtype in ("float32", "bfloat16"):
+        runner = ModelRunner(folder, dtype=dtype, page_size=16, num_pages=24, max_requests=4)
+        for what, steps in (("whole", H.steps_whole(reqs)), ("last 32 decoded", H.steps_last_decoded(reqs)),
+                            ("mixed", H.steps_mixed(reqs, max_live=3, seed=2))):
+            at = {}
+            for st in steps:                # keep only the wanted places that lie near the end of a request
+                for e in st["entries"]:
+                    base = at.get(e["id"], 0)
+                    e["want"] = [i for i in range(len(e["tokens"])) if base + i >= len(reqs[e["id"]]) - want_last]
+                    at[e["id"]] = base + len(e["tokens"])
+            got = H.run_steps(runner, steps)
+            runner.cache.check()
+            assert len(got) == 3 * want_last
+            for (rid, p), row in got.items():
+                ref = refs[rid]
+                err = np.abs(row - ref[p]).max() / np.abs(ref).max()
+                # the plain run is itself 32-bit here: both sides round, so twice the 32-bit tolerance
+                assert err <= (2 * H.TOL[dtype] if dtype == "float32" else H.TOL[dtype]), \
+                    "%s %s: request %s position %d: %.3g" % (dtype, what, rid, p, err)
+        del runner
+        torch.cuda.empty_cache()
