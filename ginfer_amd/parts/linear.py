@@ -1,9 +1,11 @@
 """y = x . W^T (+ b), W stored [out, in] as in the checkpoint (ginfer/core/layer/linear.cc:9-20).
 
 32-bit: the package's own FMA kernel (no matrix unit, no reduced-precision mode).  bfloat16: the
-package's matrix-core kernel for few rows (decode), the BLAS library for many rows (prefill), which
+package's matrix-core kernel for up to 64 rows (decode), the BLAS library for more rows (prefill), which
 is where the reference calls its library (ginfer/core/op/kernels/cuda/gemm_kernel/gemm_kernel.cu:42-164);
-both accumulate in 32-bit and add the bias before the one rounding."""
+both accumulate in 32-bit and add the bias before the one rounding.  Steps that are recorded into HIP
+graphs (decode, up to 64 rows) run the package's own kernels only: replays of a graph that holds the
+library's products were measured to differ, by a rounding, from the same step launched eagerly."""
 import torch
 
 from ..kernels import ops
