@@ -299,7 +299,7 @@ __global__ __launch_bounds__(64 * DEC_WAVES) void attn_decode_split_kernel(
       acc += o_s[w][d][cc];
     }
     if (num_splits == 1) {
-      out[(int64_t)t * out_stride + (int64_t)(kvh * group + hb * 16 + cc) * HD + d] = f32_to_bf16(acc / lsum);
+      out[(int64_t)t * out_stride + (int64_t)(kvh * group + hb * 16 + cc) * HD + d] = f32_to_bf16(acc * (1.f / lsum));
     } else {
       const int64_t slot = slot_base + (int64_t)cc * num_splits;
       part_o[slot * HD + d] = acc;

@@ -189,7 +189,7 @@ class ModelRunner:
             token_ids=buf.dev["ids"], positions=buf.dev["pos"], token_entry=buf.dev["ent"], cu_tokens=buf.dev["cu"],
             q_start=buf.dev["q_start"], logit_rows=buf.dev["rows"], num_tokens=host["T"], num_entries=host["E"],
             host_q_start=host["q_start"].tolist(), host_q_len=host["q_len"].tolist(), caches=caches,
-            extra={"decode_rows": buf.dev["decode_rows"]})
+            extra={"decode_rows": buf.dev["decode_rows"], "decode_span": _context_bucket(host["max_kv"])})
 
     def _run(self, host, borrow):
         E, T = host["E"], host["T"]
@@ -197,9 +197,7 @@ class ModelRunner:
         graphable = self.use_graphs and T == E and E <= GRAPH_MAX_ROWS and len(host["rows"]) == E and \
             bool((host["rows"] == np.arange(E)).all())
         if graphable:
-            bucket = 256
-            while bucket < host["max_kv"]:
-                bucket *= 2
+            bucket = _context_bucket(host["max_kv"])
             key = (E, bucket)
             g = self._graphs.get(key)
             if g is None:
@@ -223,7 +221,6 @@ class ModelRunner:
         buf = _StepBuffers(E, E, E, width, E, len(self.cache.groups), self.device)
         padded = dict(host, width=width, tables=[self._widen(t, width) for t in host["tables"]])
         ctx = self._context(padded, buf)
-        ctx.extra["decode_span"] = bucket
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
@@ -245,6 +242,15 @@ class ModelRunner:
         out = np.full((table.shape[0], width), -1, dtype=np.int32)
         out[:, :table.shape[1]] = table
         return out
+
+
+def _context_bucket(max_kv):
+    """Contexts are rounded up to a power of two (at least 256): the attention kernels split the keys for
+    the bucket's longest context, in recorded and in eager steps alike, so that both do the same sums."""
+    bucket = 256
+    while bucket < max_kv:
+        bucket *= 2
+    return bucket
 
 
 GRAPH_MAX_ROWS = 64      # the decode step's own kernels take up to this many rows; beyond it library calls come in
