@@ -3,9 +3,9 @@
 32-bit: the package's own FMA kernel (no matrix unit, no reduced-precision mode).  bfloat16: the
 package's matrix-core kernel for up to 64 rows (decode), the BLAS library for more rows (prefill), which
 is where the reference calls its library (ginfer/core/op/kernels/cuda/gemm_kernel/gemm_kernel.cu:42-164);
-both accumulate in 32-bit and add the bias before the one rounding.  Steps that are recorded into HIP
-graphs (decode, up to 64 rows) run the package's own kernels only: replays of a graph that holds the
-library's products were measured to differ, by a rounding, from the same step launched eagerly."""
+both accumulate in 32-bit and add the bias before the one rounding.  From 17 rows on the library also takes
+the products with a wide output, where it was measured faster; replays of recorded steps that hold
+these calls are checked bit for bit against eager steps in the tests."""
 import torch
 
 from ..kernels import ops
@@ -22,7 +22,7 @@ def linear(x, weight, bias=None, out_dtype=None, parts_ok=False):
     which the norm that follows adds up in order."""
     if x.dtype == torch.float32:
         return ops.gemm_nt(x, weight, bias)
-    if ops.gemm_skinny_supported(x, weight):
+    if ops.gemm_skinny_supported(x, weight) and not _library_is_faster(x.shape[0], weight.shape[0]):
         # tilings measured on MI355X (graph replays, weights not cache-resident): up to 16 rows one
         # 16-row tile of W per wavefront streams best; beyond, four tiles halve the re-reading of x; a
         # long K is split over workgroups where the consumer can add the parts
@@ -43,8 +43,18 @@ def linear(x, weight, bias=None, out_dtype=None, parts_ok=False):
     return torch.mm(x, weight.t())
 
 
+def _library_is_faster(rows, out_features):
+    """Measured on MI355X: from 17 rows on, products with a wide output (the gate-up product, the head) run
+    faster in the BLAS library than in the weight-streaming kernel, which re-reads x once per 64 outputs."""
+    return rows > LIBRARY_FROM_ROWS and out_features >= 4096
+
+
+LIBRARY_FROM_ROWS = 16
+
+
 def gated_linear(x, weight_gate_up):
     """silu(x . Wg^T) * (x . Wu^T) with Wg over Wu stacked in one matrix [2I, K] -> [M, I]."""
-    if x.dtype == torch.bfloat16 and ops.gemm_skinny_supported(x, weight_gate_up):
+    if (x.dtype == torch.bfloat16 and ops.gemm_skinny_supported(x, weight_gate_up)
+            and not _library_is_faster(x.shape[0], weight_gate_up.shape[0])):
         return ops.gemm_skinny(x, weight_gate_up, gated=True)
     return ops.silu_mul(linear(x, weight_gate_up))

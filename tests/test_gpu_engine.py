@@ -302,3 +302,22 @@ def test_real_layer_sizes(tmp_path):
                     "%s %s: request %s position %d: %.3g" % (dtype, what, rid, p, err)
         del runner
         torch.cuda.empty_cache()
+    # recorded decode steps at these sizes (40 rows: the wide products go to the BLAS library) against the
+    # same steps launched eagerly, several replays with eager steps between them
+    from ginfer_amd import StepEntry
+    outs = [[], []]
+    stream = H.random_tokens(40 * 12, 151936, 77)
+    for k, graphs in enumerate((True, False)):
+        r = ModelRunner(folder, dtype="bfloat16", page_size=16, num_pages=120, max_requests=41, use_graphs=graphs)
+        r.step([StepEntry(i, H.random_tokens(3 + i % 9, 151936, 100 + i), []) for i in range(40)])
+        for stepno in range(10):
+            outs[k].append(r.step([StepEntry(i, [stream[stepno * 40 + i]], [0]) for i in range(40)]).cpu())
+            if stepno in (3, 6):
+                outs[k].append(r.step([StepEntry("p", H.random_tokens(70, 151936, stepno), [69])]).cpu())
+                r.release("p")
+        assert bool(r._graphs) == graphs
+        del r
+        torch.cuda.empty_cache()
+    for n, (a, b) in enumerate(zip(*outs)):
+        assert torch.equal(a, b), "real sizes, step %d: a replayed step differs from the eager step by %.3g" % (
+            n, float((a - b).abs().max() / b.abs().max()))
