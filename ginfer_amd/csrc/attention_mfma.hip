@@ -238,8 +238,7 @@ __global__ __launch_bounds__(64 * DEC_WAVES) void attn_decode_split_kernel(
     bf16_t* __restrict__ out, int64_t out_stride, float* __restrict__ part_o, float* __restrict__ part_ml,
     const bf16_t* __restrict__ q, int64_t q_stride, const bf16_t* __restrict__ k_pages,
     const bf16_t* __restrict__ v_pages, const int32_t* __restrict__ block_table, int table_width,
-    const int32_t* __restrict__ token_entry, const int32_t* __restrict__ positions,
-    const int32_t* __restrict__ token_list, int nh, int nkv, int head_blocks, int ps_shift, int window,
+    const int4* __restrict__ decode_info, int nh, int nkv, int head_blocks, int ps_shift, int window,
     float scale, int split_keys, int num_splits) {
   __shared__ float o_s[DEC_WAVES][HD][17];
   __shared__ float m_s[DEC_WAVES][16], l_s[DEC_WAVES][16];
@@ -247,8 +246,8 @@ __global__ __launch_bounds__(64 * DEC_WAVES) void attn_decode_split_kernel(
   const int ti = blockIdx.x, split = blockIdx.z;
   const int kvh = blockIdx.y / head_blocks, hb = blockIdx.y % head_blocks;
   const int group = nh / nkv;
-  const int t = token_list[ti];
-  const int pos = positions[t];
+  const int4 info = decode_info[ti];       // (row of the step, position, entry of the block table, -): one load
+  const int t = info.x, pos = info.y;
   const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
   const bool col_ok = hb * 16 + c < group;
   const int head = kvh * group + hb * 16 + c;
@@ -263,7 +262,7 @@ __global__ __launch_bounds__(64 * DEC_WAVES) void attn_decode_split_kernel(
     bf16x8 qr[1][KB];
     load_q(qr[0], col_ok ? q + (int64_t)t * q_stride + (int64_t)head * HD : nullptr, g);
     const int cpos[1] = {col_ok ? pos : -1}, clo[1] = {lo};
-    const int32_t* bt = block_table + (int64_t)token_entry[t] * table_width;
+    const int32_t* bt = block_table + (int64_t)info.z * table_width;
     // every live column of a decode wavefront sees the same keys: lo..pos
     attend_tiles<1>(o, m, l, qr, cpos, clo, k_pages, v_pages, bt, kvh, nkv, ps_shift, lo, pos, lo, pos,
                     begin + 32 * wave, end, 32 * DEC_WAVES, scale);
@@ -315,7 +314,7 @@ __global__ __launch_bounds__(64 * DEC_WAVES) void attn_decode_split_kernel(
 #define MAX_SPLITS 256
 __global__ __launch_bounds__(64) void attn_decode_combine_kernel(
     bf16_t* __restrict__ out, int64_t out_stride, const float* __restrict__ part_o,
-    const float* __restrict__ part_ml, const int32_t* __restrict__ token_list, int nh, int num_splits) {
+    const float* __restrict__ part_ml, const int4* __restrict__ decode_info, int nh, int num_splits) {
   __shared__ float w_s[MAX_SPLITS];
   const int ti = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
   const int64_t base = ((int64_t)ti * nh + head) * num_splits;
@@ -332,7 +331,7 @@ __global__ __launch_bounds__(64) void attn_decode_combine_kernel(
   total = wave_sum(total);
   __syncthreads();
   const float inv = 1.f / total;
-  bf16_t* op = out + (int64_t)token_list[ti] * out_stride + (int64_t)head * HD;
+  bf16_t* op = out + (int64_t)decode_info[ti].x * out_stride + (int64_t)head * HD;
   for (int d = lane; d < HD; d += 64) {
     float acc = 0.f;
 #pragma unroll 8
@@ -771,12 +770,12 @@ extern "C" int ga_attn_head_dim() { return HD; }
 // rows of a prefill tile: 16 or (head sizes up to 128) 32
 extern "C" int ga_attn_prefill_max_tile_rows() { return 16 * PREFILL_NB; }
 
-// Decode tokens: token_list names the rows of the step that are single new tokens.  workspace_o must
-// hold n_tokens*nh*num_splits*HD floats and workspace_ml n_tokens*nh*num_splits*2.
+// Decode tokens: decode_info holds, for every single new token of the step, int32 x 4 = (its row in the
+// step, its position, its entry of the block table, unused).  workspace_o must hold
+// n_tokens*nh*num_splits*HD floats and workspace_ml n_tokens*nh*num_splits*2.
 extern "C" int ga_attn_decode(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* k_pages,
                               const void* v_pages, const void* block_table, int table_width,
-                              const void* token_entry, const void* positions, const void* token_list,
-                              int n_tokens, int nh, int nkv, int page_size, int window, float scale,
+                              const void* decode_info, int n_tokens, int nh, int nkv, int page_size, int window, float scale,
                               int split_keys, int num_splits, void* workspace_o, void* workspace_ml,
                               hipStream_t stream) {
   if (n_tokens <= 0) return 0;
@@ -792,13 +791,13 @@ extern "C" int ga_attn_decode(void* out, int64_t out_stride, const void* q, int6
   hipLaunchKernelGGL(attn_decode_split_kernel, grid, dim3(64 * DEC_WAVES), 0, stream, (bf16_t*)out, out_stride,
                      (float*)workspace_o, (float*)workspace_ml, (const bf16_t*)q, q_stride,
                      (const bf16_t*)k_pages, (const bf16_t*)v_pages, (const int32_t*)block_table, table_width,
-                     (const int32_t*)token_entry, (const int32_t*)positions, (const int32_t*)token_list, nh, nkv,
-                     head_blocks, ps_shift, window, scale * LOG2E, split_keys, num_splits);
+                     (const int4*)decode_info, nh, nkv, head_blocks, ps_shift, window, scale * LOG2E, split_keys,
+                     num_splits);
   int rc = GA_CHECK_LAUNCH();
   if (rc || num_splits == 1) return rc;
   hipLaunchKernelGGL(attn_decode_combine_kernel, dim3(n_tokens, nh), dim3(64), 0, stream, (bf16_t*)out,
                      out_stride, (const float*)workspace_o, (const float*)workspace_ml,
-                     (const int32_t*)token_list, nh, num_splits);
+                     (const int4*)decode_info, nh, num_splits);
   return GA_CHECK_LAUNCH();
 }
 

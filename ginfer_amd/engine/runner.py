@@ -166,7 +166,19 @@ class ModelRunner:
         return dict(E=E, T=T, ids=ids.astype(np.int32), pos=pos, ent=ent, cu=cu, q_start=q_start.astype(np.int32),
                     q_len=q_len, rows=np.asarray(rows, dtype=np.int32), width=width, tables=tables,
                     slot_maps=slot_maps, state_slots=slots, max_kv=max_kv,
-                    decode_rows=cu[:-1][q_len == 1].astype(np.int32) if T != E else ent)
+                    decode_info=self._decode_info(cu, q_len, q_start, ent, T == E))
+
+    @staticmethod
+    def _decode_info(cu, q_len, q_start, ent, all_single):
+        """int32 [n, 4]: (row in the step, position, entry, 0) of every entry that brings a single token."""
+        if all_single:
+            rows, pos, entries = ent, q_start, ent
+        else:
+            mask = q_len == 1
+            rows, pos, entries = cu[:-1][mask], q_start[mask], np.flatnonzero(mask)
+        info = np.zeros((len(rows), 4), dtype=np.int32)
+        info[:, 0], info[:, 1], info[:, 2] = rows, pos, entries
+        return info
 
     def _context(self, host, buf):
         """Uploads the host arrays through one packed buffer and wraps the device views."""
@@ -189,7 +201,7 @@ class ModelRunner:
             token_ids=buf.dev["ids"], positions=buf.dev["pos"], token_entry=buf.dev["ent"], cu_tokens=buf.dev["cu"],
             q_start=buf.dev["q_start"], logit_rows=buf.dev["rows"], num_tokens=host["T"], num_entries=host["E"],
             host_q_start=host["q_start"].tolist(), host_q_len=host["q_len"].tolist(), caches=caches,
-            extra={"decode_rows": buf.dev["decode_rows"], "decode_span": _context_bucket(host["max_kv"])})
+            extra={"decode_info": buf.dev["decode_info"], "decode_span": _context_bucket(host["max_kv"])})
 
     def _run(self, host, borrow):
         E, T = host["E"], host["T"]
@@ -208,7 +220,7 @@ class ModelRunner:
                 g["buf"].fill(host)
                 g["graph"].replay()
                 return g["logits"] if borrow else g["logits"].clone()
-        buf = self._buffers.get(T, E, len(host["rows"]), host["width"], len(host["decode_rows"]))
+        buf = self._buffers.get(T, E, len(host["rows"]), host["width"], len(host["decode_info"]))
         ctx = self._context(host, buf)
         return self.model.forward(ctx)
 
@@ -228,7 +240,7 @@ class ModelRunner:
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
-        ctx.extra = {"decode_rows": buf.dev["decode_rows"], "decode_span": bucket}
+        ctx.extra = {"decode_info": buf.dev["decode_info"], "decode_span": bucket}
         with torch.cuda.graph(graph):
             logits = self.model.forward(ctx)
         g = dict(graph=graph, buf=_GraphBuffers(buf, width, self._widen), logits=logits, ctx=ctx)
@@ -266,7 +278,7 @@ class _StepBuffers:
         fields = [("slots%d" % g, np.int64, (T,)) for g in range(ngroups)]
         fields += [("state_slots", np.int64, (E,))]
         fields += [("ids", np.int32, (T,)), ("pos", np.int32, (T,)), ("ent", np.int32, (T,)), ("cu", np.int32, (E + 1,)),
-                   ("q_start", np.int32, (E,)), ("rows", np.int32, (R,)), ("decode_rows", np.int32, (n_decode,))]
+                   ("q_start", np.int32, (E,)), ("rows", np.int32, (R,)), ("decode_info", np.int32, (n_decode, 4))]
         fields += [("table%d" % g, np.int32, (E, max(width, 1))) for g in range(ngroups)]
         offset, self.layout = 0, {}
         for name, dt, shape in fields:
@@ -297,7 +309,7 @@ class _StepBuffers:
         h["cu"][:] = host["cu"]
         h["q_start"][:] = host["q_start"]
         h["rows"][:] = host["rows"]
-        h["decode_rows"][:] = host["decode_rows"]
+        h["decode_info"][:] = host["decode_info"]
         h["state_slots"][:] = host["state_slots"]
         for g, (bt, sm) in enumerate(zip(host["tables"], host["slot_maps"])):
             h["table%d" % g][:, :bt.shape[1]] = bt

@@ -319,12 +319,15 @@ def _attention_plan(step, tile_rows, device):
                 tiles.append((e, o + r, min(tile_rows, n - r), start + r))
         o += n
     tiles.sort(key=lambda t: -(t[3] + t[2]))      # the tiles with the most keys first
-    token_list = step.extra.get("decode_rows")      # the runner uploads the list with the step's other side inputs
-    if token_list is None and decode_rows:
-        token_list = torch.tensor(decode_rows, dtype=torch.int32, device=device)
+    # (row, position, entry, -) of every single new token; the runner uploads it with the step's other inputs
+    decode_info = step.extra.get("decode_info")
+    if decode_info is None and decode_rows:
+        entries = [e for e in range(step.num_entries) if step.host_q_len[e] == 1]
+        decode_info = torch.tensor([[r, p, e, 0] for r, p, e in zip(decode_rows, decode_pos, entries)], dtype=torch.int32,
+                                   device=device)
     plan = dict(
         n_decode=len(decode_rows), decode_pos=decode_pos, n_tiles=len(tiles), decode_span=step.extra.get("decode_span"),
-        token_list=token_list,
+        decode_info=decode_info,
         tiles=(torch.tensor(np.asarray(tiles, dtype=np.int32).reshape(-1, 4), device=device) if tiles else None))
     step.extra[key] = plan
     return plan
@@ -379,8 +382,7 @@ def paged_attention_mfma(q, k_pages, v_pages, block_table, step, num_heads, num_
         ws_ml = torch.empty((n * 2,), dtype=torch.float32, device=q.device)
         _check(lib.ga_attn_decode(
             _ptr(out), _i64(out.stride(0)), _ptr(q), _i64(q.stride(0)), _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
-            _i(block_table.shape[1]), _ptr(step.token_entry), _ptr(step.positions), _ptr(plan["token_list"]),
-            _i(plan["n_decode"]), _i(num_heads), _i(num_kv_heads), _i(page_size), _i(w), _f(scale), _i(split_keys),
+            _i(block_table.shape[1]), _ptr(plan["decode_info"]), _i(plan["n_decode"]), _i(num_heads), _i(num_kv_heads), _i(page_size), _i(w), _f(scale), _i(split_keys),
             _i(num_splits), _ptr(ws_o), _ptr(ws_ml), _stream()), "attn_decode")
     if plan["n_tiles"] and through_lds:
         _check(lib.ga_attn_prefill_lds(
