@@ -265,7 +265,7 @@ def _context_bucket(max_kv):
     return bucket
 
 
-GRAPH_MAX_ROWS = 64      # the decode step's own kernels take up to this many rows; beyond it library calls come in
+GRAPH_MAX_ROWS = 256     # decode batches up to this many requests are recorded
 GRAPH_AFTER = 2          # a batch shape is recorded the second time it is seen
 
 

@@ -155,8 +155,9 @@ def test_temperature_sampling_matches_plain_with_same_uniforms(folders):
     assert len({tuple(o.token_ids) for o in outs}) > 1
 
 
-def test_recorded_decode_steps_of_40_rows(folders):
-    """A decode batch of 40 rows with wide products (several row blocks and four-tile wavefronts in the
+@pytest.mark.parametrize("rows", [40, 150])
+def test_recorded_decode_steps_of_many_rows(folders, rows):
+    """Decode batches of 40 and 150 rows with wide products (several row blocks and four-tile wavefronts in the
     weight-streaming kernel); recorded into a graph and replayed many times, with eager steps between the
     replays, it must give the eager bits every time."""
     from ginfer_amd import ModelRunner, StepEntry
@@ -165,15 +166,15 @@ def test_recorded_decode_steps_of_40_rows(folders):
     cfgd = dict(H.TINY[name][0], vocab_size=4600, intermediate_size=2304)      # wide: the four-tile kernel variants
     import tempfile
     folder = H.make_model_folder(tempfile.mkdtemp(), cfgd, 9, "float32")
-    runners = [ModelRunner(folder, dtype="bfloat16", page_size=8, num_pages=600, max_requests=48, use_graphs=g)
+    runners = [ModelRunner(folder, dtype="bfloat16", page_size=8, num_pages=2000, max_requests=rows + 8, use_graphs=g)
                for g in (True, False)]
-    prompts = {i: H.random_tokens(5 + i % 7, 4600, 800 + i) for i in range(40)}
-    stream = H.random_tokens(40 * 30, 4600, 900)
+    prompts = {i: H.random_tokens(5 + i % 7, 4600, 800 + i) for i in range(rows)}
+    stream = H.random_tokens(rows * 30, 4600, 900)
     outs = [[], []]
     for k, r in enumerate(runners):
         r.step([StepEntry(i, p, []) for i, p in prompts.items()])
         for stepno in range(25):
-            outs[k].append(r.step([StepEntry(i, [stream[stepno * 40 + i]], [0]) for i in prompts]).cpu())
+            outs[k].append(r.step([StepEntry(i, [stream[stepno * rows + i]], [0]) for i in prompts]).cpu())
             if stepno % 6 == 2:                  # eager work between replays
                 outs[k].append(r.step([StepEntry("x%d" % stepno, H.random_tokens(30, 4600, stepno), [29])]).cpu())
                 r.release("x%d" % stepno)
