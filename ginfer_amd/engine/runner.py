@@ -211,10 +211,14 @@ class ModelRunner:
         if graphable:
             bucket = _context_bucket(host["max_kv"])
             key = (E, bucket)
-            g = self._graphs.get(key)
-            if g is None:
+            g = self._graphs.pop(key, None)
+            if g is not None:
+                self._graphs[key] = g        # most recently used last
+            else:
                 self._graph_seen[key] = self._graph_seen.get(key, 0) + 1
                 if self._graph_seen[key] >= GRAPH_AFTER:
+                    while len(self._graphs) >= GRAPH_KEEP:      # each graph holds its buffers: forget the oldest
+                        self._graphs.pop(next(iter(self._graphs)))
                     g = self._capture(key, host)
             if g is not None:
                 g["buf"].fill(host)
@@ -267,6 +271,7 @@ def _context_bucket(max_kv):
 
 GRAPH_MAX_ROWS = 256     # decode batches up to this many requests are recorded
 GRAPH_AFTER = 2          # a batch shape is recorded the second time it is seen
+GRAPH_KEEP = 32          # recorded shapes kept at a time (least recently used goes first)
 
 
 class _StepBuffers:

@@ -322,3 +322,21 @@ def test_real_layer_sizes(tmp_path):
     for n, (a, b) in enumerate(zip(*outs)):
         assert torch.equal(a, b), "real sizes, step %d: a replayed step differs from the eager step by %.3g" % (
             n, float((a - b).abs().max() / b.abs().max()))
+
+
+def test_recorded_shapes_are_bounded(folders, monkeypatch):
+    """Every batch size gets a graph of its own; only the most recently used are kept."""
+    from ginfer_amd import ModelRunner, StepEntry
+    from ginfer_amd.engine import runner as R
+    monkeypatch.setattr(R, "GRAPH_KEEP", 3)
+    r = ModelRunner(folders["A"], dtype="bfloat16", page_size=16, num_pages=64, max_requests=8)
+    ref = ModelRunner(folders["A"], dtype="bfloat16", page_size=16, num_pages=64, max_requests=8, use_graphs=False)
+    toks = H.random_tokens(400, 512, 5)
+    at = 0
+    for n in (1, 2, 3, 4, 5, 2, 1, 6):
+        for _ in range(3):
+            batch = [StepEntry(i, [toks[at + i]], [0]) for i in range(n)]
+            at += n
+            assert torch.equal(r.step(batch), ref.step(batch))
+        assert len(r._graphs) <= 3
+    assert len(r._graphs) == 3 and (6, 256) in r._graphs
