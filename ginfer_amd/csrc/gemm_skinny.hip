@@ -28,6 +28,38 @@ __device__ __forceinline__ bf16x8 load8(const bf16_t* p) {
   return __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(p));
 }
 
+// The wavefront's share of the sum over k in [kb, ke): UNROLL steps of 64 elements per trip, all loads of a
+// trip issued before its products; the guard on every 8-element piece makes the tail of the range safe.
+template <int NT, int MB>
+__device__ __forceinline__ void skinny_accumulate(f32x4 (&acc)[NT][MB], const bf16_t* const (&wp)[NT],
+                                                  const bool (&wok)[NT], const bf16_t* const (&ap)[MB],
+                                                  const bool (&aok)[MB], int kb, int ke, int g) {
+  constexpr int UNROLL = (NT * MB <= 4) ? 4 : 2;
+  for (int k = kb; k < ke; k += 64 * UNROLL) {
+    bf16x8 a[UNROLL][2][NT], b[UNROLL][2][MB];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const int kk = k + u * 64 + g * 16 + j * 8;
+        const bool ok = kk < ke;
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) a[u][j][nt] = (ok && wok[nt]) ? load8(wp[nt] + kk) : zero8();
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) b[u][j][mb] = (ok && aok[mb]) ? load8(ap[mb] + kk) : zero8();
+      }
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+          for (int mb = 0; mb < MB; ++mb)
+            acc[nt][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][j][nt], b[u][j][mb], acc[nt][mb], 0, 0, 0);
+  }
+}
+
 // NT: 16-row tiles of W per wavefront; MB: 16-row blocks of A; KS: wavefronts of a workgroup that split K
 // for the same rows (the workgroup's SK_WAVES / KS groups own different rows of W).  The grid's y
 // dimension splits K further: then every workgroup writes its part in 32-bit to P[y][M][N] and the
@@ -75,32 +107,7 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(TC* __restrict_
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) acc[nt][mb] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  // UNROLL steps of 64 elements per trip, all loads of a trip issued before its products; the guard on
-  // every 8-element piece makes the tail of the range safe
-  constexpr int UNROLL = (NT * MB <= 4) ? 4 : 2;
-  for (int k = kb; k < ke; k += 64 * UNROLL) {
-    bf16x8 a[UNROLL][2][NT], b[UNROLL][2][MB];
-#pragma unroll
-    for (int u = 0; u < UNROLL; ++u)
-#pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        const int kk = k + u * 64 + g * 16 + j * 8;
-        const bool ok = kk < ke;
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt) a[u][j][nt] = (ok && wok[nt]) ? load8(wp[nt] + kk) : zero8();
-#pragma unroll
-        for (int mb = 0; mb < MB; ++mb) b[u][j][mb] = (ok && aok[mb]) ? load8(ap[mb] + kk) : zero8();
-      }
-#pragma unroll
-    for (int u = 0; u < UNROLL; ++u)
-#pragma unroll
-      for (int j = 0; j < 2; ++j)
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-          for (int mb = 0; mb < MB; ++mb)
-            acc[nt][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][j][nt], b[u][j][mb], acc[nt][mb], 0, 0, 0);
-  }
+  skinny_accumulate<NT, MB>(acc, wp, wok, ap, aok, kb, ke, g);
   // the KS parts of a group meet in LDS and are added in wavefront order
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt)
@@ -188,6 +195,138 @@ extern "C" int ga_gemm_skinny(void* C, int64_t ldc, const void* A, int64_t lda, 
 #undef PICK_NT
 #undef PICK_MB
 #undef PICK_KS
+#undef LAUNCH
+  return GA_CHECK_LAUNCH();
+}
+
+// The fused q|k|v projection of a decode step with its epilogue: bias, NeoX rotation of q and k
+// (ginfer/core/op/kernels/cuda/rope_kernel.cu:83-102, on the 32-bit sums: one rounding fewer than rotating
+// the rounded projection), q to its own buffer, k and v straight into the paged cache (v transposed;
+// ginfer/core/op/kernels/cuda/store_kvcache_kernel.cu:19-30).  A wavefront group owns a UNIT of 32 output
+// columns as two tiles of 16: for a q or k head the columns j0..j0+15 and their rotation partners
+// j0+half..; for a v head 32 consecutive columns.  head_dim a multiple of 32, rotary_dim == head_dim.
+template <int MB, int KS>
+__global__ __launch_bounds__(SK_THREADS) void qkv_rope_skinny_kernel(
+    bf16_t* __restrict__ q_out, const bf16_t* __restrict__ A, int64_t lda, const bf16_t* __restrict__ W,
+    const bf16_t* __restrict__ bias, const int32_t* __restrict__ positions, const float* __restrict__ cos_t,
+    const float* __restrict__ sin_t, const int64_t* __restrict__ slot_mapping, bf16_t* __restrict__ k_pages,
+    bf16_t* __restrict__ v_pages, int M, int K, int nh, int nkv, int hd, int page_size, int write_kv,
+    int kchunk_wave) {
+  __shared__ float red[SK_WAVES][32][MB * 16 + 1];
+  constexpr int GROUPS = SK_WAVES / KS;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r = lane & 15, g = lane >> 4;
+  const int grp = wave / KS, ks = wave % KS;
+  const int half = hd >> 1, upq = half / 16;            // units per q or k head
+  const int qk_units = (nh + nkv) * upq, units = qk_units + nkv * (hd / 32);
+  const int unit = blockIdx.x * GROUPS + grp;
+  const bool unit_ok = unit < units;
+  // first rows of the unit's two tiles
+  int row0 = 0, row1 = 0;
+  if (unit_ok) {
+    if (unit < qk_units) {
+      row0 = (unit / upq) * hd + (unit % upq) * 16;
+      row1 = row0 + half;
+    } else {
+      const int u = unit - qk_units;
+      row0 = (nh + nkv) * hd + u * 32;
+      row1 = row0 + 16;
+    }
+  }
+  const int kb = ks * kchunk_wave;
+  const int ke = kb + kchunk_wave < K ? kb + kchunk_wave : K;
+  const bf16_t* wp[2] = {W + (int64_t)(row0 + r) * K, W + (int64_t)(row1 + r) * K};
+  const bool wok[2] = {unit_ok, unit_ok};
+  const bf16_t* ap[MB];
+  bool aok[MB];
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) {
+    const int m = mb * 16 + r;
+    aok[mb] = m < M;
+    ap[mb] = A + (int64_t)(aok[mb] ? m : 0) * lda;
+  }
+  f32x4 acc[2][MB];
+#pragma unroll
+  for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) acc[nt][mb] = f32x4{0.f, 0.f, 0.f, 0.f};
+  skinny_accumulate<2, MB>(acc, wp, wok, ap, aok, kb, ke, g);
+#pragma unroll
+  for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) red[wave][nt * 16 + g * 4 + i][mb * 16 + r] = acc[nt][mb][i];
+  __syncthreads();
+  for (int idx = threadIdx.x; idx < GROUPS * 16 * MB * 16; idx += SK_THREADS) {
+    const int nl = idx % 16, rest = idx / 16;
+    const int gi = rest % GROUPS, m = rest / GROUPS;
+    const int u = blockIdx.x * GROUPS + gi;
+    if (m >= M || u >= units) continue;
+    float lo = 0.f, hi = 0.f;
+#pragma unroll
+    for (int w = 0; w < KS; ++w) {
+      lo += red[gi * KS + w][nl][m];
+      hi += red[gi * KS + w][16 + nl][m];
+    }
+    const int64_t slot = write_kv ? slot_mapping[m] : -1;
+    const int64_t page = slot >= 0 ? slot / page_size : 0, off = slot >= 0 ? slot - page * page_size : 0;
+    if (u < qk_units) {
+      const int head = u / upq, j = (u % upq) * 16 + nl;
+      if (bias) {
+        lo += bf16_to_f32(bias[head * hd + j]);
+        hi += bf16_to_f32(bias[head * hd + j + half]);
+      }
+      const int p = positions[m];
+      const float c = cos_t[(int64_t)p * half + j], sn = sin_t[(int64_t)p * half + j];
+      const bf16_t olo = f32_to_bf16(lo * c - hi * sn), ohi = f32_to_bf16(lo * sn + hi * c);
+      if (head < nh) {
+        bf16_t* o = q_out + (int64_t)m * nh * hd + (int64_t)head * hd + j;
+        o[0] = olo;
+        o[half] = ohi;
+      } else if (slot >= 0) {
+        bf16_t* o = k_pages + ((page * nkv + (head - nh)) * page_size + off) * hd + j;
+        o[0] = olo;
+        o[half] = ohi;
+      }
+    } else if (slot >= 0) {
+      const int v = u - qk_units;
+      const int gh = v / (hd / 32), d = (v % (hd / 32)) * 32 + nl;
+      if (bias) {
+        lo += bf16_to_f32(bias[(nh + nkv + gh) * hd + d]);
+        hi += bf16_to_f32(bias[(nh + nkv + gh) * hd + d + 16]);
+      }
+      bf16_t* o = v_pages + ((page * nkv + gh) * (int64_t)hd + d) * page_size + off;
+      o[0] = f32_to_bf16(lo);
+      o[(int64_t)16 * page_size] = f32_to_bf16(hi);
+    }
+  }
+}
+
+// q_out [M, nh*hd]; A [M, K] (row stride lda); W [(nh + 2 nkv) hd, K]; bias [(nh + 2 nkv) hd] or null;
+// positions int32 [M]; cos_t, sin_t float [positions, hd/2]; slot_mapping int64 [M] (-1: no cache write);
+// k_pages [pages, nkv, page_size, hd], v_pages [pages, nkv, hd, page_size].
+extern "C" int ga_qkv_rope_skinny(void* q_out, const void* A, int64_t lda, const void* W, const void* bias,
+                                  const void* positions, const void* cos_t, const void* sin_t,
+                                  const void* slot_mapping, void* k_pages, void* v_pages, int M, int K, int nh,
+                                  int nkv, int hd, int page_size, int write_kv, hipStream_t stream) {
+  if (M <= 0) return 0;
+  if (M > 64 || K <= 0 || K % 8 || lda % 8 || hd % 32 || nh <= 0 || nkv <= 0) return -1;
+  const int mb = (M + 15) / 16;
+  const int ks = 8, groups = SK_WAVES / ks;
+  const int units = (nh + 2 * nkv) * hd / 32;
+  const int kchunk_wave = ((K + ks - 1) / ks + 63) / 64 * 64;
+  dim3 grid((units + groups - 1) / groups), block(SK_THREADS);
+#define LAUNCH(MB)                                                                                        \
+  hipLaunchKernelGGL((qkv_rope_skinny_kernel<MB, 8>), grid, block, 0, stream, (bf16_t*)q_out,            \
+                     (const bf16_t*)A, lda, (const bf16_t*)W, (const bf16_t*)bias, (const int32_t*)positions, \
+                     (const float*)cos_t, (const float*)sin_t, (const int64_t*)slot_mapping, (bf16_t*)k_pages, \
+                     (bf16_t*)v_pages, M, K, nh, nkv, hd, page_size, write_kv, kchunk_wave)
+  switch (mb) {
+    case 1: LAUNCH(1); break;
+    case 2: LAUNCH(2); break;
+    case 3: LAUNCH(3); break;
+    default: LAUNCH(4); break;
+  }
 #undef LAUNCH
   return GA_CHECK_LAUNCH();
 }

@@ -282,6 +282,40 @@ def gemm_skinny(a, w, bias=None, out=None, out_dtype=None, nt=0, ks=0, grid_spli
     return out
 
 
+def qkv_rope_skinny_supported(x, w, head_dim, rotary_dim):
+    """Whether the fused projection + rotation + cache-write kernel takes these operands."""
+    return gemm_skinny_supported(x, w) and head_dim % 32 == 0 and rotary_dim == head_dim
+
+
+def qkv_rope_skinny(x, w, bias, positions, cos, sin, slot_mapping, k_pages, v_pages, num_heads, num_kv_heads, head_dim,
+                    write_kv=True):
+    """The decode step's q|k|v projection with its epilogue in one kernel: x [M <= 64, K] . w^T + bias, NeoX
+    rotation of q and k, q returned as [M, nh*hd], k and v written into the paged cache at slot_mapping."""
+    _dev(x, w, bias, positions, cos, sin, slot_mapping, k_pages, v_pages)
+    M, K = x.shape
+    width = (num_heads + 2 * num_kv_heads) * head_dim
+    _need(w.shape == (width, K), "qkv weight must be [%d, %d], got %s" % (width, K, tuple(w.shape)))
+    _need(qkv_rope_skinny_supported(x, w, head_dim, 2 * cos.shape[1]), "the fused q|k|v kernel takes bfloat16, at most %d "
+          "rows, head sizes that are multiples of 32 and a rotation of the whole head" % SKINNY_MAX_ROWS)
+    if bias is not None:
+        _need(bias.dtype == torch.bfloat16 and bias.shape == (width,) and bias.is_contiguous(), "qkv bias must be bfloat16 [%d]" % width)
+    _need(positions.dtype == torch.int32 and positions.shape == (M,) and positions.is_contiguous(), "positions must be int32 [M]")
+    _need(cos.dtype == torch.float32 and sin.dtype == torch.float32 and cos.shape == sin.shape and cos.is_contiguous()
+          and sin.is_contiguous(), "cos and sin must be contiguous float32 [P, head_dim/2]")
+    page_size = 1
+    if write_kv:
+        _need(slot_mapping is not None and slot_mapping.dtype == torch.int64 and slot_mapping.shape == (M,)
+              and slot_mapping.is_contiguous(), "slot_mapping must be contiguous int64 [M]")
+        page_size = _check_pages(k_pages, v_pages, torch.bfloat16, num_kv_heads, head_dim)
+    q = torch.empty((M, num_heads * head_dim), dtype=torch.bfloat16, device=x.device)
+    lib = build.load("gemm_skinny")
+    _check(lib.ga_qkv_rope_skinny(_ptr(q), _ptr(x), _i64(x.stride(0)), _ptr(w), _ptr(bias), _ptr(positions), _ptr(cos),
+                                  _ptr(sin), _ptr(slot_mapping), _ptr(k_pages), _ptr(v_pages), _i(M), _i(K), _i(num_heads),
+                                  _i(num_kv_heads), _i(head_dim), _i(page_size), _i(1 if write_kv else 0), _stream()),
+           "qkv_rope_skinny")
+    return q
+
+
 # ----------------------------------------------------------------------------- attention on the matrix cores
 
 MFMA_HEAD_DIMS = tuple(range(16, 257, 16))

@@ -62,10 +62,15 @@ class Attention(Part):
         return mods
 
     def forward(self, x, step, cache):
-        qkv = linear(x, self.w_qkv, self.b_qkv)
         cos, sin = self.position.tables()
-        ops.rope_kv_write(qkv, step.positions, cos, sin, cache.slot_mapping, cache.k_pages, cache.v_pages,
-                          self.nh, self.nkv, self.hd, write_kv=cache.owner)
+        if ops.qkv_rope_skinny_supported(x, self.w_qkv, self.hd, self.position.rotary_dim):
+            # few rows (decode): projection, rotation and cache write in one kernel
+            qkv = ops.qkv_rope_skinny(x, self.w_qkv, self.b_qkv, step.positions, cos, sin, cache.slot_mapping,
+                                      cache.k_pages, cache.v_pages, self.nh, self.nkv, self.hd, write_kv=cache.owner)
+        else:
+            qkv = linear(x, self.w_qkv, self.b_qkv)
+            ops.rope_kv_write(qkv, step.positions, cos, sin, cache.slot_mapping, cache.k_pages, cache.v_pages,
+                              self.nh, self.nkv, self.hd, write_kv=cache.owner)
         a = ops.paged_attention(qkv, cache.k_pages, cache.v_pages, cache.block_table, step, self.nh, self.nkv,
                                 self.hd, self.scale, self.window)
         return linear(a, self.w_o, self.b_o, parts_ok=True)

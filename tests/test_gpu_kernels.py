@@ -447,3 +447,44 @@ def test_gemm_skinny_gated(M, I, K):
     ref = pm.swiglu(g, u)
     close(ops.gemm_skinny(a, w, gated=True, out_dtype=torch.float32), ref, 1e-5)
     close(ops.gemm_skinny(a, w, gated=True), ref, 1e-2)
+
+
+@pytest.mark.parametrize("M", [1, 8, 33, 64])
+@pytest.mark.parametrize("nh,nkv,hd,K,theta", [(12, 2, 128, 1536, 1e4), (6, 1, 32, 192, 1e6), (4, 4, 64, 88, 1e4), (5, 1, 96, 72, 5e5)])
+def test_qkv_rope_skinny(M, nh, nkv, hd, K, theta):
+    """The fused decode kernel equals projection, then rotation and cache write."""
+    from ginfer_amd.kernels import ops
+    ps, pages = 8, 40
+    width = (nh + 2 * nkv) * hd
+    x, w, b = rnd((M, K), torch.bfloat16, 60), rnd((width, K), torch.bfloat16, 61, scale=0.2), rnd((width,), torch.bfloat16, 62)
+    positions = torch.randint(0, 300, (M,), dtype=torch.int32, device=dev())
+    sin, cos = pm.rope_tables(theta, hd, 300)
+    slots = torch.randperm(pages * ps)[:M].to(torch.int64)
+    if M > 1:
+        slots[1] = -1
+    kp, vp = rnd((pages, nkv, ps, hd), torch.bfloat16, 63), rnd((pages, nkv, hd, ps), torch.bfloat16, 64)
+    kp0, vp0 = kp.clone().cpu(), vp.clone().cpu()
+    assert ops.qkv_rope_skinny_supported(x, w, hd, hd)
+    q = ops.qkv_rope_skinny(x, w, b, positions, cos.to(dev()), sin.to(dev()), slots.to(dev()), kp, vp, nh, nkv, hd)
+    y = x.double().cpu() @ w.double().cpu().t() + b.double().cpu()
+    pos = positions.cpu().tolist()
+    qr = pm.apply_rope(y[:, :nh * hd].view(M, nh, hd), pos, sin.double(), cos.double()).reshape(M, -1)
+    kr = pm.apply_rope(y[:, nh * hd:(nh + nkv) * hd].view(M, nkv, hd), pos, sin.double(), cos.double())
+    v = y[:, (nh + nkv) * hd:].view(M, nkv, hd)
+    close(q, qr, 1e-2)
+    kpc, vpc = kp.float().cpu(), vp.float().cpu()
+    touched_k, touched_v = torch.zeros_like(kpc, dtype=torch.bool), torch.zeros_like(vpc, dtype=torch.bool)
+    for t in range(M):
+        s = int(slots[t])
+        if s < 0:
+            continue
+        close(kpc[s // ps, :, s % ps, :], kr[t], 1e-2)
+        close(vpc[s // ps, :, :, s % ps], v[t], 1e-2)
+        touched_k[s // ps, :, s % ps, :] = True
+        touched_v[s // ps, :, :, s % ps] = True
+    assert torch.equal(kp.cpu()[~touched_k], kp0[~touched_k]) and torch.equal(vp.cpu()[~touched_v], vp0[~touched_v])
+    # a run that reads another layer's cache writes nothing
+    kp1, vp1 = kp0.clone().to(dev()), vp0.clone().to(dev())
+    q2 = ops.qkv_rope_skinny(x, w, b, positions, cos.to(dev()), sin.to(dev()), slots.to(dev()), kp1, vp1, nh, nkv, hd,
+                             write_kv=False)
+    assert torch.equal(q2, q) and torch.equal(kp1.cpu(), kp0) and torch.equal(vp1.cpu(), vp0)
