@@ -16,7 +16,8 @@ import time
 
 sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
 
-# BASELINE.json configs[2]: Qwen2 1.5B shape (DeepSeek-R1-Distill-Qwen-1.5B layout)
+# The benchmark's model: the Qwen2 1.5B shape (the layout of DeepSeek-R1-Distill-Qwen-1.5B, the checkpoint the
+# reference publishes its numbers on: README.md:31-32 of 11Aln0/ginfer)
 SHAPE = dict(architectures=["Qwen2ForCausalLM"], model_type="qwen2", num_hidden_layers=28, hidden_size=1536,
              num_attention_heads=12, num_key_value_heads=2, head_dim=128, intermediate_size=8960, vocab_size=151936,
              rope_theta=10000.0, rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=131072,

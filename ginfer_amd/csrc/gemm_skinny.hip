@@ -244,6 +244,39 @@ __global__ __launch_bounds__(SK_THREADS) void qkv_rope_skinny_kernel(
     aok[mb] = m < M;
     ap[mb] = A + (int64_t)(aok[mb] ? m : 0) * lda;
   }
+  // What the epilogue needs from memory (position, slot, cosine and sine, bias) is asked for now, so that
+  // it arrives while the weights stream: an epilogue item is (unit of the workgroup, column, row of A).
+  constexpr int ITEMS = (GROUPS * 16 * MB * 16 + SK_THREADS - 1) / SK_THREADS;
+  int64_t e_slot[ITEMS];
+  float e_cos[ITEMS], e_sin[ITEMS], e_blo[ITEMS], e_bhi[ITEMS];
+#pragma unroll
+  for (int it = 0; it < ITEMS; ++it) {
+    const int idx = threadIdx.x + it * SK_THREADS;
+    const int nl = idx % 16, rest = idx / 16;
+    const int gi = rest % GROUPS, m = rest / GROUPS;
+    const int u = blockIdx.x * GROUPS + gi;
+    e_slot[it] = -1;
+    e_cos[it] = 1.f;
+    e_sin[it] = e_blo[it] = e_bhi[it] = 0.f;
+    if (m < M && u < units) {
+      if (write_kv) e_slot[it] = slot_mapping[m];
+      if (u < qk_units) {
+        const int head = u / upq, j = (u % upq) * 16 + nl;
+        const int p = positions[m];
+        e_cos[it] = cos_t[(int64_t)p * half + j];
+        e_sin[it] = sin_t[(int64_t)p * half + j];
+        if (bias) {
+          e_blo[it] = bf16_to_f32(bias[head * hd + j]);
+          e_bhi[it] = bf16_to_f32(bias[head * hd + j + half]);
+        }
+      } else if (bias) {
+        const int v = u - qk_units;
+        const int at = (nh + nkv + v / (hd / 32)) * hd + (v % (hd / 32)) * 32 + nl;
+        e_blo[it] = bf16_to_f32(bias[at]);
+        e_bhi[it] = bf16_to_f32(bias[at + 16]);
+      }
+    }
+  }
   f32x4 acc[2][MB];
 #pragma unroll
   for (int nt = 0; nt < 2; ++nt)
@@ -257,27 +290,24 @@ __global__ __launch_bounds__(SK_THREADS) void qkv_rope_skinny_kernel(
 #pragma unroll
       for (int i = 0; i < 4; ++i) red[wave][nt * 16 + g * 4 + i][mb * 16 + r] = acc[nt][mb][i];
   __syncthreads();
-  for (int idx = threadIdx.x; idx < GROUPS * 16 * MB * 16; idx += SK_THREADS) {
+#pragma unroll
+  for (int it = 0; it < ITEMS; ++it) {
+    const int idx = threadIdx.x + it * SK_THREADS;
     const int nl = idx % 16, rest = idx / 16;
     const int gi = rest % GROUPS, m = rest / GROUPS;
     const int u = blockIdx.x * GROUPS + gi;
     if (m >= M || u >= units) continue;
-    float lo = 0.f, hi = 0.f;
+    float lo = e_blo[it], hi = e_bhi[it];
 #pragma unroll
     for (int w = 0; w < KS; ++w) {
       lo += red[gi * KS + w][nl][m];
       hi += red[gi * KS + w][16 + nl][m];
     }
-    const int64_t slot = write_kv ? slot_mapping[m] : -1;
+    const int64_t slot = e_slot[it];
     const int64_t page = slot >= 0 ? slot / page_size : 0, off = slot >= 0 ? slot - page * page_size : 0;
     if (u < qk_units) {
       const int head = u / upq, j = (u % upq) * 16 + nl;
-      if (bias) {
-        lo += bf16_to_f32(bias[head * hd + j]);
-        hi += bf16_to_f32(bias[head * hd + j + half]);
-      }
-      const int p = positions[m];
-      const float c = cos_t[(int64_t)p * half + j], sn = sin_t[(int64_t)p * half + j];
+      const float c = e_cos[it], sn = e_sin[it];
       const bf16_t olo = f32_to_bf16(lo * c - hi * sn), ohi = f32_to_bf16(lo * sn + hi * c);
       if (head < nh) {
         bf16_t* o = q_out + (int64_t)m * nh * hd + (int64_t)head * hd + j;
@@ -291,10 +321,6 @@ __global__ __launch_bounds__(SK_THREADS) void qkv_rope_skinny_kernel(
     } else if (slot >= 0) {
       const int v = u - qk_units;
       const int gh = v / (hd / 32), d = (v % (hd / 32)) * 32 + nl;
-      if (bias) {
-        lo += bf16_to_f32(bias[(nh + nkv + gh) * hd + d]);
-        hi += bf16_to_f32(bias[(nh + nkv + gh) * hd + d + 16]);
-      }
       bf16_t* o = v_pages + ((page * nkv + gh) * (int64_t)hd + d) * page_size + off;
       o[0] = f32_to_bf16(lo);
       o[(int64_t)16 * page_size] = f32_to_bf16(hi);
