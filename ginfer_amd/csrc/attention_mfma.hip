@@ -241,7 +241,7 @@ __global__ __launch_bounds__(64 * DEC_WAVES) void attn_decode_split_kernel(
     const int4* __restrict__ decode_info, int nh, int nkv, int head_blocks, int ps_shift, int window,
     float scale, int split_keys, int num_splits) {
   __shared__ float o_s[DEC_WAVES][HD][17];
-  __shared__ float m_s[DEC_WAVES][16], l_s[DEC_WAVES][16];
+  __shared__ float m_s[DEC_WAVES][16], l_s[DEC_WAVES][16], mx_s[16], lsum_s[16];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c = lane & 15, g = lane >> 4;
   const int ti = blockIdx.x, split = blockIdx.z;
   const int kvh = blockIdx.y / head_blocks, hb = blockIdx.y % head_blocks;
@@ -282,29 +282,37 @@ __global__ __launch_bounds__(64 * DEC_WAVES) void attn_decode_split_kernel(
 #pragma unroll
     for (int i = 0; i < 4; ++i) o_s[wave][db * 16 + g * 4 + i][c] = o[0][db][i] * f;
   __syncthreads();
-  const int64_t slot_base = ((int64_t)ti * nh + kvh * group + hb * 16) * num_splits + split;
-  for (int idx = threadIdx.x; idx < 16 * HD; idx += 64 * DEC_WAVES) {
-    const int cc = idx / HD, d = idx % HD;
-    if (hb * 16 + cc >= group) continue;
-    // the thread's column cc is not the lane's own column c: its max is read again
+  // per column: the common max and the sum of the rescaled sums, once (the outputs in o_s are rescaled already)
+  if (threadIdx.x < 16) {
+    const int cc = threadIdx.x;
     float mcc = -INFINITY;
 #pragma unroll
     for (int w = 0; w < DEC_WAVES; ++w) mcc = fmaxf(mcc, m_s[w][cc]);
-    float lsum = 0.f, acc = 0.f;
+    float lsum = 0.f;
 #pragma unroll
     for (int w = 0; w < DEC_WAVES; ++w) {
       const float mw = m_s[w][cc];
       if (mw != -INFINITY) lsum += l_s[w][cc] * exp2f(mw - mcc);
-      acc += o_s[w][d][cc];
     }
+    mx_s[cc] = mcc;
+    lsum_s[cc] = lsum;
+  }
+  __syncthreads();
+  const int64_t slot_base = ((int64_t)ti * nh + kvh * group + hb * 16) * num_splits + split;
+  for (int idx = threadIdx.x; idx < 16 * HD; idx += 64 * DEC_WAVES) {
+    const int cc = idx / HD, d = idx % HD;
+    if (hb * 16 + cc >= group) continue;
+    float acc = 0.f;
+#pragma unroll
+    for (int w = 0; w < DEC_WAVES; ++w) acc += o_s[w][d][cc];
     if (num_splits == 1) {
-      out[(int64_t)t * out_stride + (int64_t)(kvh * group + hb * 16 + cc) * HD + d] = f32_to_bf16(acc * (1.f / lsum));
+      out[(int64_t)t * out_stride + (int64_t)(kvh * group + hb * 16 + cc) * HD + d] = f32_to_bf16(acc * (1.f / lsum_s[cc]));
     } else {
       const int64_t slot = slot_base + (int64_t)cc * num_splits;
       part_o[slot * HD + d] = acc;
       if (d == 0) {
-        part_ml[slot * 2] = mcc;
-        part_ml[slot * 2 + 1] = lsum;
+        part_ml[slot * 2] = mx_s[cc];
+        part_ml[slot * 2 + 1] = lsum_s[cc];
       }
     }
   }
