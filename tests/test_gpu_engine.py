@@ -340,3 +340,34 @@ def test_recorded_shapes_are_bounded(folders, monkeypatch):
             assert torch.equal(r.step(batch), ref.step(batch))
         assert len(r._graphs) <= 3
     assert len(r._graphs) == 3 and (6, 256) in r._graphs
+
+
+@pytest.mark.parametrize("name,seed", [("C", 1), ("A", 2)])
+def test_random_workload_through_the_engine(folders, name, seed):
+    """A dozen requests of random lengths and sampling settings through scheduler, cache and kernels with a
+    pool that forces evictions (and, for C, windows that give pages back): in 32-bit every request's tokens
+    are the plain implementation's."""
+    import random
+    from ginfer_amd import Engine, EngineConfig, SamplingParams
+    from ginfer_amd.sampling import uniform
+    rng = random.Random(seed)
+    cfgd, _, ps = H.TINY[name]
+    vocab = cfgd["vocab_size"]
+    prompts = [H.random_tokens(rng.randint(1, 60), vocab, 1000 + i) for i in range(12)]
+    params = [SamplingParams(max_tokens=rng.randint(1, 20), ignore_eos=True, temperature=rng.choice([0.0, 0.0, 0.9]),
+                             seed=rng.randint(0, 99)) for _ in prompts]
+    eng = Engine(EngineConfig(model_path=folders[name], dtype="float32", max_num_batched_tokens=40, max_num_seqs=4,
+                              max_seq_len=96, kvcache_block_size=ps, num_kvcache_blocks=(96 // ps) * 2 + 1))
+    outs = eng.generate(prompts, params)
+    eng.runner.cache.check()
+    assert not eng.runner.cache.requests
+    cfg, w = pm.read_config(folders[name]), pm.read_weights(folders[name])
+    disagreements = 0
+    for p, sp, o in zip(prompts, params, outs):
+        assert len(o.token_ids) == sp.max_tokens
+        logits = pm.forward(cfg, w, (p + o.token_ids)[:-1])
+        for k, tok in enumerate(o.token_ids):
+            want = pm.sample_token(logits[len(p) - 1 + k], sp.temperature, uniform(sp.seed, k))
+            disagreements += int(want != tok)
+    assert disagreements <= 1, "%d tokens differ from the plain implementation" % disagreements
+    assert eng.scheduler.num_evictions > 0, "the pool was meant to be too small"
