@@ -54,64 +54,57 @@ __device__ __forceinline__ bf16x8 load8(const bf16_t* p) {
   return __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(p));
 }
 
-// K operands of one tile of 32 keys: [product t][32-dim block]; keys outside kv_min..kv_max are never
-// loaded (their pages may be gone) and count as zero.
+// The pages of a tile's keys as this lane needs them: for its two K rows and for its 8-key piece of V^T.
+// Keys outside kv_min..kv_max (their pages may be gone, or lie past the table) take page 0, which is
+// always there; what is read for them is masked (scores) or cleared (values) in the edge tiles.
+struct TilePages {
+  int k[2], v;
+};
+__device__ __forceinline__ void lookup_pages(TilePages& tp, const int32_t* __restrict__ bt, int ps_shift,
+                                             int kv_min, int kv_max, int k0, int c, int g) {
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+    const int key = k0 + 8 * (c >> 2) + 4 * t + (c & 3);
+    tp.k[t] = (key >= kv_min && key <= kv_max) ? bt[key >> ps_shift] : 0;
+  }
+  const int kbase = k0 + 8 * g;
+  const int kv = kbase < kv_min ? kv_min : kbase;       // a piece that straddles an end of the range has a live key
+  tp.v = (kbase + 7 >= kv_min && kbase <= kv_max) ? bt[kv >> ps_shift] : 0;
+}
+
+// K operands of one tile of 32 keys: [product t][32-dim block]
 __device__ __forceinline__ void load_k_tile(bf16x8 (&kr)[2][KB], const bf16_t* __restrict__ k_pages,
-                                            const int32_t* __restrict__ bt, int kvh, int nkv, int ps_shift,
-                                            int kv_min, int kv_max, int k0, int c, int g) {
+                                            const TilePages& tp, int kvh, int nkv, int ps_shift, int k0, int c,
+                                            int g) {
   const int ps = 1 << ps_shift;
 #pragma unroll
   for (int t = 0; t < 2; ++t) {
     const int key = k0 + 8 * (c >> 2) + 4 * t + (c & 3);
-    const bool ok = key >= kv_min && key <= kv_max;
-    const bf16_t* kp = k_pages;
-    if (ok) {
-      const int64_t page = bt[key >> ps_shift];
-      kp = k_pages + ((page * nkv + kvh) * ps + (key & (ps - 1))) * HD + g * 8;
-    }
+    const bf16_t* kp = k_pages + (((int64_t)tp.k[t] * nkv + kvh) * ps + (key & (ps - 1))) * HD + g * 8;
 #pragma unroll
     for (int kb = 0; kb < KB; ++kb) {
-      kr[t][kb] = zero8();
-      if (ok && kb * 32 + g * 8 < HD) kr[t][kb] = load8(kp + kb * 32);
+      if (HD % 32 == 0 || kb * 32 + g * 8 < HD) kr[t][kb] = load8(kp + kb * 32);
+      else kr[t][kb] = zero8();
     }
   }
 }
 
 // V^T operands of one tile: [16-dim block]; the lane loads dims db*16 + c, keys k0 + 8g .. + 7.
 __device__ __forceinline__ void load_v_tile(bf16x8 (&vr)[DB], const bf16_t* __restrict__ v_pages,
-                                            const int32_t* __restrict__ bt, int kvh, int nkv, int ps_shift,
-                                            int kv_min, int kv_max, int k0, int c, int g) {
+                                            const TilePages& tp, int kvh, int nkv, int ps_shift, int k0, int c,
+                                            int g) {
   const int ps = 1 << ps_shift;
-  const int kbase = k0 + 8 * g;
-  const bool any_ok = kbase + 7 >= kv_min && kbase <= kv_max;
-  const bool all_ok = kbase >= kv_min && kbase + 7 <= kv_max;
-  const bf16_t* vp = v_pages;
-  if (any_ok) {
-    const int64_t page = bt[kbase >> ps_shift];
-    vp = v_pages + ((page * nkv + kvh) * HD + c) * ps + (kbase & (ps - 1));
-  }
+  const bf16_t* vp = v_pages + (((int64_t)tp.v * nkv + kvh) * HD + c) * ps + ((k0 + 8 * g) & (ps - 1));
 #pragma unroll
-  for (int db = 0; db < DB; ++db) {
-    vr[db] = zero8();
-    if (any_ok) {
-      vr[db] = load8(vp + (int64_t)db * 16 * ps);
-      if (!all_ok) {                       // slots past the request's last key hold anything: clear them
-        union { bf16x8 v; bf16_t e[8]; } u;
-        u.v = vr[db];
-#pragma unroll
-        for (int j = 0; j < 8; ++j)
-          if (kbase + j < kv_min || kbase + j > kv_max) u.e[j] = 0;
-        vr[db] = u.v;
-      }
-    }
-  }
+  for (int db = 0; db < DB; ++db) vr[db] = load8(vp + (int64_t)db * 16 * ps);
 }
 
 // Attends columns to the key tiles tile_begin, tile_begin + tile_stride, ... < tile_end (multiples of 32).
 // kv_min..kv_max is the inclusive range of keys that any column of the wavefront may see; full_lo..full_hi
-// the range that EVERY live column sees (tiles inside it need no mask).  The loop is software-pipelined:
-// the values of a tile and the keys of the next are requested before the tile's scores are computed, so
-// that their way from memory overlaps the matrix products and the softmax.
+// the range that EVERY live column sees (tiles inside it need no mask).  The loop is software-pipelined
+// two deep: the page ids of tile i+2, the keys of tile i+1 and the values of tile i are requested before
+// the scores of tile i are computed, so that no load waits for a look-up and their way from memory
+// overlaps the matrix products and the softmax.
 template <int NB>
 __device__ __forceinline__ void attend_tiles(f32x4 (&o)[NB][DB], float (&m)[NB], float (&l)[NB],
                                              const bf16x8 (&q)[NB][KB], const int (&cpos)[NB],
@@ -122,13 +115,21 @@ __device__ __forceinline__ void attend_tiles(f32x4 (&o)[NB][DB], float (&m)[NB],
                                              int tile_end, int tile_stride, float scale) {
   const int lane = threadIdx.x & 63, c = lane & 15, g = lane >> 4;
   if (tile_begin >= tile_end) return;
+  TilePages pg_cur, pg_nxt, pg_nn;
+  lookup_pages(pg_cur, bt, ps_shift, kv_min, kv_max, tile_begin, c, g);
+  pg_nxt = pg_cur;
+  if (tile_begin + tile_stride < tile_end)
+    lookup_pages(pg_nxt, bt, ps_shift, kv_min, kv_max, tile_begin + tile_stride, c, g);
+  pg_nn = pg_nxt;
   bf16x8 kr[2][KB];
-  load_k_tile(kr, k_pages, bt, kvh, nkv, ps_shift, kv_min, kv_max, tile_begin, c, g);
+  load_k_tile(kr, k_pages, pg_cur, kvh, nkv, ps_shift, tile_begin, c, g);
   for (int k0 = tile_begin; k0 < tile_end; k0 += tile_stride) {
     bf16x8 vr[DB], kn[2][KB];
-    load_v_tile(vr, v_pages, bt, kvh, nkv, ps_shift, kv_min, kv_max, k0, c, g);
+    if (k0 + 2 * tile_stride < tile_end)
+      lookup_pages(pg_nn, bt, ps_shift, kv_min, kv_max, k0 + 2 * tile_stride, c, g);
+    load_v_tile(vr, v_pages, pg_cur, kvh, nkv, ps_shift, k0, c, g);
     const bool more = k0 + tile_stride < tile_end;
-    if (more) load_k_tile(kn, k_pages, bt, kvh, nkv, ps_shift, kv_min, kv_max, k0 + tile_stride, c, g);
+    if (more) load_k_tile(kn, k_pages, pg_nxt, kvh, nkv, ps_shift, k0 + tile_stride, c, g);
     // ---- scores: S^T = K Q^T
     f32x4 s[NB][2];
 #pragma unroll
@@ -143,7 +144,8 @@ __device__ __forceinline__ void attend_tiles(f32x4 (&o)[NB][DB], float (&m)[NB],
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb)
           s[nb][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kr[t][kb], q[nb][kb], s[nb][t], 0, 0, 0);
-    // ---- mask and online softmax; the lane holds keys k0 + 8g + j, j = 0..7, of column c
+    // ---- mask and online softmax; the lane holds keys k0 + 8g + j, j = 0..7, of column c.  The running
+    // max is kept in scaled units; the scale rides on the exponent's multiply-add.
     const bool interior = k0 >= full_lo && k0 + 31 <= full_hi;      // the same for the whole wavefront
     bf16x8 pb[NB];
 #pragma unroll
@@ -153,7 +155,7 @@ __device__ __forceinline__ void attend_tiles(f32x4 (&o)[NB][DB], float (&m)[NB],
       if (interior && cpos[nb] >= 0) {
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-          sv[j] = s[nb][j >> 2][j & 3] * scale;
+          sv[j] = s[nb][j >> 2][j & 3];
           mx = fmaxf(mx, sv[j]);
         }
       } else {
@@ -161,23 +163,23 @@ __device__ __forceinline__ void attend_tiles(f32x4 (&o)[NB][DB], float (&m)[NB],
         for (int j = 0; j < 8; ++j) {
           const int key = k0 + 8 * g + j;
           const bool valid = key >= clo[nb] && key <= cpos[nb];
-          sv[j] = valid ? s[nb][j >> 2][j & 3] * scale : -INFINITY;
+          sv[j] = valid ? s[nb][j >> 2][j & 3] : -INFINITY;      // a select: what was read for a dead key is dropped
           mx = fmaxf(mx, sv[j]);
         }
       }
       mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
       mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
-      const float m_new = fmaxf(m[nb], mx);
+      const float m_new = fmaxf(m[nb], mx * scale);
       float alpha = 1.f, sum = 0.f;
       float p[8];
       if (m_new == -INFINITY) {            // the column has seen no key yet
 #pragma unroll
         for (int j = 0; j < 8; ++j) p[j] = 0.f;
       } else {
-        alpha = exp2f(m[nb] - m_new);     // exp(-inf) = 0 the first time
+        alpha = exp2f(m[nb] - m_new);      // exp2(-inf) = 0 the first time
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-          p[j] = exp2f(sv[j] - m_new);
+          p[j] = exp2f(__builtin_fmaf(sv[j], scale, -m_new));
           sum += p[j];
         }
       }
@@ -192,7 +194,20 @@ __device__ __forceinline__ void attend_tiles(f32x4 (&o)[NB][DB], float (&m)[NB],
 #pragma unroll
       for (int j = 0; j < 8; ++j) pb[nb][j] = (__bf16)p[j];
     }
-    // ---- output: O^T += V^T P
+    // ---- output: O^T += V^T P.  In a tile that reaches past the ends of the key range the values read
+    // for dead keys (anything: the slot may never have been written) are cleared: 0 * NaN is not 0.
+    if (k0 < kv_min || k0 + 31 > kv_max) {
+      const int kbase = k0 + 8 * g;
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        union { bf16x8 v; bf16_t e[8]; } u;
+        u.v = vr[db];
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+          if (kbase + j < kv_min || kbase + j > kv_max) u.e[j] = 0;
+        vr[db] = u.v;
+      }
+    }
 #pragma unroll
     for (int db = 0; db < DB; ++db)
 #pragma unroll
@@ -204,6 +219,8 @@ __device__ __forceinline__ void attend_tiles(f32x4 (&o)[NB][DB], float (&m)[NB],
 #pragma unroll
         for (int kb = 0; kb < KB; ++kb) kr[t][kb] = kn[t][kb];
     }
+    pg_cur = pg_nxt;
+    pg_nxt = pg_nn;
   }
 }
 

@@ -319,7 +319,7 @@ def qkv_rope_skinny(x, w, bias, positions, cos, sin, slot_mapping, k_pages, v_pa
 # ----------------------------------------------------------------------------- attention on the matrix cores
 
 MFMA_HEAD_DIMS = tuple(range(16, 257, 16))
-_DECODE_TARGET_WORKGROUPS = 512       # four wavefronts each: enough to fill 256 compute units
+_DECODE_TARGET_WORKGROUPS = 256       # four wavefronts each, one workgroup per compute unit: measured best on MI355X
 _MIN_SPLIT_KEYS = 128                 # one tile of 32 keys for each wavefront of a workgroup
 _MAX_SPLITS = 256
 PREFILL_WIDE_TILES_FROM = 512         # tokens in a step from which prompt rows go 32 to a wavefront
