@@ -45,6 +45,11 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 // The kernels keep scores, running maxima and the maxima of partial results in units of log2(e): the
 // launchers multiply the score scale by LOG2E once, and every exponential is a bare exp2.
 #define LOG2E 1.4426950408889634f
+#define LAZY_MAX 8.0f
+
+// the bare v_exp_f32: arguments here are differences to a running maximum (<= 0, or -inf), for which the
+// library routine's extra steps for denormal results buy nothing
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 __device__ __forceinline__ bf16x8 zero8() {
   uint4 z = {0u, 0u, 0u, 0u};
@@ -101,10 +106,10 @@ __device__ __forceinline__ void load_v_tile(bf16x8 (&vr)[DB], const bf16_t* __re
 
 // Attends columns to the key tiles tile_begin, tile_begin + tile_stride, ... < tile_end (multiples of 32).
 // kv_min..kv_max is the inclusive range of keys that any column of the wavefront may see; full_lo..full_hi
-// the range that EVERY live column sees (tiles inside it need no mask).  The loop is software-pipelined
-// two deep: the page ids of tile i+2, the keys of tile i+1 and the values of tile i are requested before
-// the scores of tile i are computed, so that no load waits for a look-up and their way from memory
-// overlaps the matrix products and the softmax.
+// the range that EVERY live column sees (tiles inside it need no mask).  The loop is software-pipelined:
+// page ids are looked up a tile before they are needed, and the keys and values of tile i+1 are requested
+// right after the products of tile i that free their registers, so that no load waits for a look-up and
+// each has most of a tile's matrix products and softmax to arrive in.
 template <int NB>
 __device__ __forceinline__ void attend_tiles(f32x4 (&o)[NB][DB], float (&m)[NB], float (&l)[NB],
                                              const bf16x8 (&q)[NB][KB], const int (&cpos)[NB],
@@ -115,21 +120,23 @@ __device__ __forceinline__ void attend_tiles(f32x4 (&o)[NB][DB], float (&m)[NB],
                                              int tile_end, int tile_stride, float scale) {
   const int lane = threadIdx.x & 63, c = lane & 15, g = lane >> 4;
   if (tile_begin >= tile_end) return;
-  TilePages pg_cur, pg_nxt, pg_nn;
-  lookup_pages(pg_cur, bt, ps_shift, kv_min, kv_max, tile_begin, c, g);
-  pg_nxt = pg_cur;
-  if (tile_begin + tile_stride < tile_end)
-    lookup_pages(pg_nxt, bt, ps_shift, kv_min, kv_max, tile_begin + tile_stride, c, g);
-  pg_nn = pg_nxt;
-  bf16x8 kr[2][KB];
-  load_k_tile(kr, k_pages, pg_cur, kvh, nkv, ps_shift, tile_begin, c, g);
+  // pg_nxt: pages of the tile after the current one; they are looked up a whole tile before the loads
+  // that need them are issued.  kr and vr hold the operands of the CURRENT tile at the top of the loop;
+  // each is refilled with the next tile's as soon as its matrix products have been issued, so every load
+  // has most of a tile's work to arrive in, and no operand is held twice.
+  TilePages pg_nxt;
+  bf16x8 kr[2][KB], vr[DB];
+  {
+    TilePages pg;
+    lookup_pages(pg, bt, ps_shift, kv_min, kv_max, tile_begin, c, g);
+    load_k_tile(kr, k_pages, pg, kvh, nkv, ps_shift, tile_begin, c, g);
+    load_v_tile(vr, v_pages, pg, kvh, nkv, ps_shift, tile_begin, c, g);
+    pg_nxt = pg;
+    if (tile_begin + tile_stride < tile_end)
+      lookup_pages(pg_nxt, bt, ps_shift, kv_min, kv_max, tile_begin + tile_stride, c, g);
+  }
   for (int k0 = tile_begin; k0 < tile_end; k0 += tile_stride) {
-    bf16x8 vr[DB], kn[2][KB];
-    if (k0 + 2 * tile_stride < tile_end)
-      lookup_pages(pg_nn, bt, ps_shift, kv_min, kv_max, k0 + 2 * tile_stride, c, g);
-    load_v_tile(vr, v_pages, pg_cur, kvh, nkv, ps_shift, k0, c, g);
     const bool more = k0 + tile_stride < tile_end;
-    if (more) load_k_tile(kn, k_pages, pg_nxt, kvh, nkv, ps_shift, k0 + tile_stride, c, g);
     // ---- scores: S^T = K Q^T
     f32x4 s[NB][2];
 #pragma unroll
@@ -144,6 +151,7 @@ __device__ __forceinline__ void attend_tiles(f32x4 (&o)[NB][DB], float (&m)[NB],
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb)
           s[nb][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kr[t][kb], q[nb][kb], s[nb][t], 0, 0, 0);
+    if (more) load_k_tile(kr, k_pages, pg_nxt, kvh, nkv, ps_shift, k0 + tile_stride, c, g);
     // ---- mask and online softmax; the lane holds keys k0 + 8g + j, j = 0..7, of column c.  The running
     // max is kept in scaled units; the scale rides on the exponent's multiply-add.
     const bool interior = k0 >= full_lo && k0 + 31 <= full_hi;      // the same for the whole wavefront
@@ -167,30 +175,35 @@ __device__ __forceinline__ void attend_tiles(f32x4 (&o)[NB][DB], float (&m)[NB],
           mx = fmaxf(mx, sv[j]);
         }
       }
-      mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
-      mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
-      const float m_new = fmaxf(m[nb], mx * scale);
-      float alpha = 1.f, sum = 0.f;
+      // The running max is raised lazily: only when some score of the tile exceeds it by more than
+      // LAZY_MAX (in log2 units), which after the first tiles is rare.  Until then exponentials may reach
+      // 2^LAZY_MAX, harmless in 32-bit sums, and the tile costs no exchange between lanes: the four lanes
+      // of a column keep partial sums of their own keys (added up once, by finish_sums, after the loop).
+      if (__any(mx * scale > m[nb] + LAZY_MAX)) {
+        mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+        const float m_new = fmaxf(m[nb], mx * scale);
+        if (m_new != -INFINITY) {
+          const float alpha = fast_exp2(m[nb] - m_new);      // exp2(-inf) = 0 the first time
+          l[nb] *= alpha;
+#pragma unroll
+          for (int db = 0; db < DB; ++db) o[nb][db] *= alpha;
+        }
+        m[nb] = m_new;
+      }
+      float sum = 0.f;
       float p[8];
-      if (m_new == -INFINITY) {            // the column has seen no key yet
+      if (m[nb] == -INFINITY) {            // the column has seen no key yet
 #pragma unroll
         for (int j = 0; j < 8; ++j) p[j] = 0.f;
       } else {
-        alpha = exp2f(m[nb] - m_new);      // exp2(-inf) = 0 the first time
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-          p[j] = exp2f(__builtin_fmaf(sv[j], scale, -m_new));
+          p[j] = fast_exp2(__builtin_fmaf(sv[j], scale, -m[nb]));
           sum += p[j];
         }
       }
-      sum += __shfl_xor(sum, 16, WAVE);
-      sum += __shfl_xor(sum, 32, WAVE);
-      l[nb] = l[nb] * alpha + sum;
-      m[nb] = m_new;
-      if (__any(alpha != 1.f)) {           // once the running max has settled nothing is rescaled
-#pragma unroll
-        for (int db = 0; db < DB; ++db) o[nb][db] *= alpha;
-      }
+      l[nb] += sum;
 #pragma unroll
       for (int j = 0; j < 8; ++j) pb[nb][j] = (__bf16)p[j];
     }
@@ -214,13 +227,20 @@ __device__ __forceinline__ void attend_tiles(f32x4 (&o)[NB][DB], float (&m)[NB],
       for (int nb = 0; nb < NB; ++nb)
         o[nb][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vr[db], pb[nb], o[nb][db], 0, 0, 0);
     if (more) {
-#pragma unroll
-      for (int t = 0; t < 2; ++t)
-#pragma unroll
-        for (int kb = 0; kb < KB; ++kb) kr[t][kb] = kn[t][kb];
+      load_v_tile(vr, v_pages, pg_nxt, kvh, nkv, ps_shift, k0 + tile_stride, c, g);
+      if (k0 + 2 * tile_stride < tile_end)
+        lookup_pages(pg_nxt, bt, ps_shift, kv_min, kv_max, k0 + 2 * tile_stride, c, g);
     }
-    pg_cur = pg_nxt;
-    pg_nxt = pg_nn;
+  }
+}
+
+// after attend_tiles: the four lanes of a column add up their partial sums
+template <int NB>
+__device__ __forceinline__ void finish_sums(float (&l)[NB]) {
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) {
+    l[nb] += __shfl_xor(l[nb], 16, WAVE);
+    l[nb] += __shfl_xor(l[nb], 32, WAVE);
   }
 }
 
@@ -283,6 +303,7 @@ __global__ __launch_bounds__(64 * DEC_WAVES) void attn_decode_split_kernel(
     // every live column of a decode wavefront sees the same keys: lo..pos
     attend_tiles<1>(o, m, l, qr, cpos, clo, k_pages, v_pages, bt, kvh, nkv, ps_shift, lo, pos, lo, pos,
                     begin + 32 * wave, end, 32 * DEC_WAVES, scale);
+    finish_sums<1>(l);
   }
   // the wavefronts' states meet: common max, rescaled sums and outputs added in wavefront order
   if (g == 0) {
@@ -293,7 +314,7 @@ __global__ __launch_bounds__(64 * DEC_WAVES) void attn_decode_split_kernel(
   float mx = -INFINITY;
 #pragma unroll
   for (int w = 0; w < DEC_WAVES; ++w) mx = fmaxf(mx, m_s[w][c]);
-  const float f = (m[0] == -INFINITY) ? 0.f : exp2f(m[0] - mx);
+  const float f = (m[0] == -INFINITY) ? 0.f : fast_exp2(m[0] - mx);
 #pragma unroll
   for (int db = 0; db < DB; ++db)
 #pragma unroll
@@ -309,7 +330,7 @@ __global__ __launch_bounds__(64 * DEC_WAVES) void attn_decode_split_kernel(
 #pragma unroll
     for (int w = 0; w < DEC_WAVES; ++w) {
       const float mw = m_s[w][cc];
-      if (mw != -INFINITY) lsum += l_s[w][cc] * exp2f(mw - mcc);
+      if (mw != -INFINITY) lsum += l_s[w][cc] * fast_exp2(mw - mcc);
     }
     mx_s[cc] = mcc;
     lsum_s[cc] = lsum;
@@ -349,7 +370,7 @@ __global__ __launch_bounds__(64) void attn_decode_combine_kernel(
   float total = 0.f;
   for (int s = lane; s < num_splits; s += 64) {
     const float ms = part_ml[(base + s) * 2];
-    const float w = ms == -INFINITY ? 0.f : exp2f(ms - mx);
+    const float w = ms == -INFINITY ? 0.f : fast_exp2(ms - mx);
     w_s[s] = w;
     total += w * part_ml[(base + s) * 2 + 1];
   }
@@ -409,6 +430,7 @@ __global__ __launch_bounds__(512) void attn_prefill_kernel(
     attend_tiles<NB>(o, m, l, qr, cpos, clo, k_pages, v_pages, block_table + (int64_t)entry * table_width, kvh,
                      nkv, ps_shift, kv_min, kv_max, full_lo, pos0, (kv_min / 32) * 32 + 32 * split,
                      (kv_max / 32 + 1) * 32, 32 * splits, scale);
+    finish_sums<NB>(l);
   }
   if (splits > 1) {
     if (head_ok && split > 0) {
@@ -433,14 +455,14 @@ __global__ __launch_bounds__(512) void attn_prefill_kernel(
       float mx = m[nb];
       for (int sp = 1; sp < splits; ++sp)
         mx = fmaxf(mx, lds[(int64_t)((hl * (splits - 1) + sp - 1) * NB + nb) * STATE + HD * 17 + c]);
-      const float f0 = m[nb] == -INFINITY ? 0.f : exp2f(m[nb] - mx);
+      const float f0 = m[nb] == -INFINITY ? 0.f : fast_exp2(m[nb] - mx);
       l[nb] *= f0;
 #pragma unroll
       for (int db = 0; db < DB; ++db) o[nb][db] *= f0;
       for (int sp = 1; sp < splits; ++sp) {      // in split order
         const float* sn = lds + (int64_t)((hl * (splits - 1) + sp - 1) * NB + nb) * STATE;
         const float ms = sn[HD * 17 + c];
-        const float f = ms == -INFINITY ? 0.f : exp2f(ms - mx);
+        const float f = ms == -INFINITY ? 0.f : fast_exp2(ms - mx);
         l[nb] += sn[HD * 17 + 16 + c] * f;
 #pragma unroll
         for (int db = 0; db < DB; ++db)
@@ -691,10 +713,10 @@ __global__ __launch_bounds__(512) void attn_prefill_lds_kernel(
 #pragma unroll
             for (int j = 0; j < 8; ++j) p[j] = 0.f;
           } else {
-            alpha = exp2f(m[nb] - m_new);
+            alpha = fast_exp2(m[nb] - m_new);
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
-              p[j] = exp2f(sv[j] - m_new);
+              p[j] = fast_exp2(sv[j] - m_new);
               sum += p[j];
             }
           }
