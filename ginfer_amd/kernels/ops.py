@@ -322,7 +322,7 @@ MFMA_HEAD_DIMS = tuple(range(16, 257, 16))
 _DECODE_TARGET_WORKGROUPS = 256       # four wavefronts each, one workgroup per compute unit: measured best on MI355X
 _MIN_SPLIT_KEYS = 128                 # one tile of 32 keys for each wavefront of a workgroup
 _MAX_SPLITS = 256
-PREFILL_WIDE_TILES_FROM = 512         # tokens in a step from which prompt rows go 32 to a wavefront
+PREFILL_WIDE_TILES_FROM = 1024        # tokens in a step from which prompt rows go 32 to a wavefront
 # tokens in a step from which key tiles are shared through LDS: never, as measured on MI355X the
 # register kernel is as fast up to 8k-token prompts; the LDS kernel stays tested for longer ones
 PREFILL_LDS_FROM = 1 << 30
