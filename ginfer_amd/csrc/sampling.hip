@@ -23,12 +23,30 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(
   const float* x = logits + (int64_t)r * row_stride;
 
   // ---- max and its lowest index: strided (coalesced) reads; a thread meets its indices in ascending order
-  float best = -INFINITY;
-  int best_i = 0x7fffffff;
-  for (int i = tid; i < vocab; i += SAMPLE_THREADS) {
-    const float v = x[i];
-    if (best_i == 0x7fffffff || v > best) { best = v; best_i = i; }
+  // four independent candidates per thread, so that four loads are in flight; merged lowest index first
+  float bests[4] = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+  int bests_i[4] = {0x7fffffff, 0x7fffffff, 0x7fffffff, 0x7fffffff};
+  for (int i0 = tid; i0 < vocab; i0 += 4 * SAMPLE_THREADS) {
+    float v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int i = i0 + u * SAMPLE_THREADS;
+      v[u] = i < vocab ? x[i] : -INFINITY;
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int i = i0 + u * SAMPLE_THREADS;
+      if (i < vocab && (bests_i[u] == 0x7fffffff || v[u] > bests[u])) { bests[u] = v[u]; bests_i[u] = i; }
+    }
   }
+  float best = bests[0];
+  int best_i = bests_i[0];
+#pragma unroll
+  for (int u = 1; u < 4; ++u)
+    if (bests_i[u] != 0x7fffffff && (best_i == 0x7fffffff || bests[u] > best || (bests[u] == best && bests_i[u] < best_i))) {
+      best = bests[u];
+      best_i = bests_i[u];
+    }
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) {
     const float b = __shfl_xor(best, o, WAVE);
