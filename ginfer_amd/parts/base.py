@@ -18,7 +18,9 @@ Mixer         forward(x [T, H], step, cache) -> [T, H], or float32 [parts, T, H]
               request; `cache` in forward is the matching view (`KVView`, `StateView` or None) of the
               schedule entry that is running.  `step` is the `StepContext` of the batch.
 FeedForward   forward(x [T, H]) -> [T, H] (or partial sums, as a mixer)
-Norm          forward(residual float32 [T, H], delta [T, H] | [parts, T, H] | None, rows=None) -> [R or T, H]
+Norm          forward(residual float32 [T, H], delta [T, H] | None, rows=None) -> [R or T, H]; a norm that
+              sets `accepts_partial_sums` also takes delta as float32 [parts, T, H] (else the block adds
+              the parts up before it calls the norm); it keeps its compute dtype in `dtype`
               adds delta into the 32-bit residual stream and returns the normalised rows; with `rows`
               (int32 indices) only those rows are returned and the residual is left as it is.
 Position      what the mixer's kernel needs to encode positions (for rotary kinds: `tables()`).

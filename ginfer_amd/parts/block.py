@@ -19,7 +19,15 @@ class PreNormBlock:
                 ("feed_forward_norm", self.feed_forward_norm)]
 
     def forward(self, residual, delta, step, cache):
-        n = self.mixer_norm.forward(residual, delta)
+        n = self.mixer_norm.forward(residual, whole(delta, self.mixer_norm))
         a = self.mixer.forward(n, step, cache)
-        n = self.feed_forward_norm.forward(residual, a)
+        n = self.feed_forward_norm.forward(residual, whole(a, self.feed_forward_norm))
         return self.feed_forward.forward(n)
+
+
+def whole(delta, norm):
+    """A mixer or feed-forward may hand on float32 partial sums [parts, T, H] of a K-split product.  A norm
+    that says `accepts_partial_sums` adds them up itself; for any other they are added up here."""
+    if delta is not None and delta.dim() == 3 and not getattr(norm, "accepts_partial_sums", False):
+        return delta.sum(dim=0).to(norm.dtype)
+    return delta

@@ -6,6 +6,7 @@ import torch
 
 from . import registry
 from .base import KVCacheSpec, StateSpec
+from .block import whole
 
 
 @dataclass
@@ -142,7 +143,7 @@ class DecoderModel:
         for i, e in enumerate(self.schedule):
             cache = step.caches[i]
             delta = self.blocks[e.layer].forward(residual, delta, step, cache)
-        n = self.final_norm.forward(residual, delta, rows=step.logit_rows)
+        n = self.final_norm.forward(residual, whole(delta, self.final_norm), rows=step.logit_rows)
         return self.head.forward(n)
 
 

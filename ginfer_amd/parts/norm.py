@@ -13,6 +13,7 @@ class RMSNorm(Part):
     subtraction (ginfer/core/op/kernels/cuda/rmsnorm_kernel.cu:27-66, ginfer/core/layer/rmsnorm.cc:6-22)."""
 
     capturable = True
+    accepts_partial_sums = True
 
     def __init__(self, size, eps, dtype, device):
         self.size, self.eps, self.dtype, self.device = int(size), float(eps), dtype, device

@@ -87,3 +87,21 @@ def test_schedule_is_validated():
     spec.schedule = [ScheduleEntry(0), ScheduleEntry(1, cache_of=0), ScheduleEntry(2, cache_of=1)]
     with pytest.raises(ValueError, match="owns none"):
         spec.validate()
+
+
+def test_partial_sums_are_added_up_for_norms_that_do_not_take_them():
+    import torch
+    from ginfer_amd.parts.block import whole
+
+    class Plain:
+        dtype = torch.bfloat16
+
+    class Taking(Plain):
+        accepts_partial_sums = True
+    parts = torch.randn(4, 3, 8)
+    out = whole(parts, Plain())
+    assert out.shape == (3, 8) and out.dtype == torch.bfloat16
+    assert torch.allclose(out.float(), parts.sum(0), atol=2e-2)
+    assert whole(parts, Taking()) is parts
+    x = torch.randn(3, 8)
+    assert whole(x, Plain()) is x and whole(None, Plain()) is None
