@@ -115,11 +115,11 @@ class ModelRunner:
                     raise ValueError("request %r has %d tokens reserved but brings %d"
                                      % (e.request_id, cache.pending(e.request_id), len(e.tokens)))
             host = self._host_arrays(entries)
+            logits = self._run(host, borrow)
         except Exception:
-            for rid in reserved_here:       # leave the cache as it was
+            for rid in reserved_here:       # nothing is committed: the requests stay as long as they were
                 cache.requests[rid].pending = 0
             raise
-        logits = self._run(host, borrow)
         for e in entries:
             cache.commit(e.request_id)
         return logits
@@ -205,7 +205,6 @@ class ModelRunner:
 
     def _run(self, host, borrow):
         E, T = host["E"], host["T"]
-        ngroups = len(self.cache.groups)
         graphable = self.use_graphs and T == E and E <= GRAPH_MAX_ROWS and len(host["rows"]) == E and \
             bool((host["rows"] == np.arange(E)).all())
         if graphable:
@@ -233,7 +232,7 @@ class ModelRunner:
         side inputs live in one static buffer that later steps refill; the attention kernels split the
         keys for the bucket's longest context, so the grid does not depend on the step."""
         E, bucket = key
-        width = bucket // self.page_size
+        width = max(1, -(-bucket // self.page_size))
         buf = _StepBuffers(E, E, E, width, E, len(self.cache.groups), self.device)
         padded = dict(host, width=width, tables=[self._widen(t, width) for t in host["tables"]])
         ctx = self._context(padded, buf)

@@ -34,6 +34,9 @@ class Scheduler:
     def __init__(self, cache, max_num_seqs, max_num_batched_tokens, eos_token_ids, max_model_len):
         if max_num_batched_tokens < 1 or max_num_seqs < 1:
             raise ValueError("max_num_seqs and max_num_batched_tokens must be positive")
+        if max_num_batched_tokens < max_num_seqs:
+            raise ValueError("max_num_batched_tokens (%d) must be at least max_num_seqs (%d): every running "
+                             "request decodes one token a step" % (max_num_batched_tokens, max_num_seqs))
         self.cache = cache
         self.max_num_seqs, self.max_num_batched_tokens = int(max_num_seqs), int(max_num_batched_tokens)
         self.eos_token_ids = set(eos_token_ids)

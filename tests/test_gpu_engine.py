@@ -371,3 +371,21 @@ def test_random_workload_through_the_engine(folders, name, seed):
             disagreements += int(want != tok)
     assert disagreements <= 1, "%d tokens differ from the plain implementation" % disagreements
     assert eng.scheduler.num_evictions > 0, "the pool was meant to be too small"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_sizes_that_fit_no_vector_width(tmp_path, dtype):
+    """A width of 50, a feed-forward of 100 and a vocabulary of 333: nothing is a multiple of 8, so the
+    kernels' scalar paths and the fall-backs of the matrix products run."""
+    from ginfer_amd import ModelRunner
+    cfg = dict(architectures=["Qwen2ForCausalLM"], num_hidden_layers=2, hidden_size=50, num_attention_heads=3,
+               num_key_value_heads=1, head_dim=16, intermediate_size=100, vocab_size=333, rope_theta=1e4,
+               rms_norm_eps=1e-6, tie_word_embeddings=True, max_position_embeddings=128)
+    folder = H.make_model_folder(tmp_path / "odd", cfg, 5, "float32")
+    reqs = {"a": H.random_tokens(70, 333, 1), "b": H.random_tokens(33, 333, 2), "c": H.random_tokens(9, 333, 3)}
+    runner = ModelRunner(folder, dtype=dtype, page_size=16, num_pages=12, max_requests=4)
+    for what, steps in (("whole", H.steps_whole(reqs)), ("mixed", H.steps_mixed(reqs, max_live=3, seed=4)),
+                        ("last 32 decoded", H.steps_last_decoded(reqs))):
+        got = H.run_steps(runner, steps)
+        runner.cache.check()
+        H.compare_with_plain(got, reqs, folder, H.TOL[dtype], "odd sizes %s %s" % (dtype, what))
