@@ -27,7 +27,7 @@ MODULES = ("embedding", "norm", "rope_kv", "attention_generic", "attention_mfma"
            "activation", "sampling")
 # Modules that are compiled for one value of a parameter (a macro) at a time; build_all() without a
 # list compiles these values, and any other value a model needs is compiled when it is first asked for.
-VARIANTS = {"attention_mfma": [{"HEAD_DIM": hd} for hd in (16, 32, 48, 64, 80, 128, 256)]}
+VARIANTS = {"attention_mfma": [{"HEAD_DIM": hd} for hd in range(16, 257, 16)]}
 
 _loaded = {}
 _lock = threading.Lock()

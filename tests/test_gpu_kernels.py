@@ -346,6 +346,19 @@ def test_paged_attention_mfma(nh, nkv, hd, seqs, wide, lds, monkeypatch):
         close(out, ref, 2e-2)
 
 
+@pytest.mark.parametrize("wide", [False, True])
+@pytest.mark.parametrize("hd", list(range(16, 257, 16)))
+def test_paged_attention_mfma_every_head_size(hd, wide, monkeypatch):
+    """Head sizes in steps of 16 up to 256, each with a group of 3 heads: portions of prompts beside single tokens."""
+    from ginfer_amd.kernels import ops
+    monkeypatch.setattr(ops, "PREFILL_WIDE_TILES_FROM", 0 if wide else 1 << 30)
+    seqs = [(1, 130), (37, 101), (64, 64), (1, 17), (2, 300)]
+    a, ref, _ = _paged_case(seqs, 6, 2, hd, 16, torch.bfloat16, seed=hd)
+    out = ops.paged_attention_mfma(a["q"], a["k_pages"], a["v_pages"], a["block_table"], _Step(seqs, a), 6, 2, hd,
+                                   1.0 / math.sqrt(hd))
+    close(out, ref, 2e-2)
+
+
 @pytest.mark.parametrize("lds", [False, True])
 @pytest.mark.parametrize("window", [1, 5, 16, 40, 64, 100])
 def test_paged_attention_mfma_window(window, lds, monkeypatch):
