@@ -1,130 +1,187 @@
-// Choosing the next token from 32-bit logits, one workgroup per row.
+// Choosing the next token from 32-bit logits in two launches: every row's vocabulary is cut into
+// segments that workgroups scan side by side, then one workgroup per row picks.
 //   temperature == 0: argmax, the lowest index among equal maxima (the reference's reduction,
 //     ginfer/core/op/kernels/cuda/argmax_kernel.cu:52-98, keeps whichever equal value its tree meets
 //     first; ginfer/model/model.cc:219-220 is where it is used).
 //   temperature  > 0: p = softmax(logits / temperature) in 32-bit, and the first index whose running
 //     sum of exp((x - max) / temperature) exceeds uniform * total: an inverse-CDF draw from a uniform
-//     number the caller supplies, so the choice is a pure function of (logits, temperature, uniform).
+//     number the caller supplies, so the choice is a pure function of (logits, temperature, uniform):
+//     the cut into segments depends on the vocabulary alone, never on the rows beside it.
 // The reference samples greedily only (ginfer/engine/sampling_params.h:5-8).
 #include "common.cuh"
 
-#define SAMPLE_THREADS 1024
-#define SAMPLE_WAVES (SAMPLE_THREADS / WAVE)
+#define SCAN_THREADS 256
+#define SCAN_WAVES (SCAN_THREADS / WAVE)
+#define MAX_SEGMENTS 64
+#define NO_INDEX 0x7fffffff
 
-__global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(
-    int32_t* __restrict__ out, const float* __restrict__ logits, int64_t row_stride, int vocab,
-    const float* __restrict__ temperature, const float* __restrict__ uniform) {
-  __shared__ float part_f[SAMPLE_WAVES];
-  __shared__ int part_i[SAMPLE_WAVES];
-  __shared__ float seg_sum[SAMPLE_WAVES];
-  __shared__ float walk[2];
-  __shared__ int owner_s;
-  const int r = blockIdx.x, tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE;
+__device__ __forceinline__ bool better(float b, int bi, float best, int best_i) {
+  return bi != NO_INDEX && (best_i == NO_INDEX || b > best || (b == best && bi < best_i));
+}
+
+// Segment (blockIdx.x) of row (blockIdx.y): its maximum with the lowest index that holds it, and, for a
+// row with a temperature, the sum of exp((x - segment max) / temperature) over the segment.
+__global__ __launch_bounds__(SCAN_THREADS) void sample_scan_kernel(
+    float* __restrict__ seg_max, int32_t* __restrict__ seg_arg, float* __restrict__ seg_sum,
+    const float* __restrict__ logits, int64_t row_stride, int vocab, int seg, int segments,
+    const float* __restrict__ temperature) {
+  __shared__ float part_f[SCAN_WAVES];
+  __shared__ int part_i[SCAN_WAVES];
+  const int s = blockIdx.x, r = blockIdx.y, tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE;
   const float* x = logits + (int64_t)r * row_stride;
-
-  // ---- max and its lowest index: strided (coalesced) reads; a thread meets its indices in ascending order
-  // four independent candidates per thread, so that four loads are in flight; merged lowest index first
+  const int sb = s * seg < vocab ? s * seg : vocab;
+  const int se = sb + seg < vocab ? sb + seg : vocab;
+  // strided (coalesced) reads, four loads in flight; a thread meets its indices in ascending order
   float bests[4] = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
-  int bests_i[4] = {0x7fffffff, 0x7fffffff, 0x7fffffff, 0x7fffffff};
-  for (int i0 = tid; i0 < vocab; i0 += 4 * SAMPLE_THREADS) {
+  int bests_i[4] = {NO_INDEX, NO_INDEX, NO_INDEX, NO_INDEX};
+  for (int i0 = sb + tid; i0 < se; i0 += 4 * SCAN_THREADS) {
     float v[4];
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
-      const int i = i0 + u * SAMPLE_THREADS;
-      v[u] = i < vocab ? x[i] : -INFINITY;
+      const int i = i0 + u * SCAN_THREADS;
+      v[u] = i < se ? x[i] : -INFINITY;
     }
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
-      const int i = i0 + u * SAMPLE_THREADS;
-      if (i < vocab && (bests_i[u] == 0x7fffffff || v[u] > bests[u])) { bests[u] = v[u]; bests_i[u] = i; }
+      const int i = i0 + u * SCAN_THREADS;
+      if (i < se && (bests_i[u] == NO_INDEX || v[u] > bests[u])) { bests[u] = v[u]; bests_i[u] = i; }
     }
   }
   float best = bests[0];
   int best_i = bests_i[0];
 #pragma unroll
   for (int u = 1; u < 4; ++u)
-    if (bests_i[u] != 0x7fffffff && (best_i == 0x7fffffff || bests[u] > best || (bests[u] == best && bests_i[u] < best_i))) {
-      best = bests[u];
-      best_i = bests_i[u];
-    }
+    if (better(bests[u], bests_i[u], best, best_i)) { best = bests[u]; best_i = bests_i[u]; }
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) {
     const float b = __shfl_xor(best, o, WAVE);
     const int bi = __shfl_xor(best_i, o, WAVE);
-    if (bi != 0x7fffffff && (best_i == 0x7fffffff || b > best || (b == best && bi < best_i))) { best = b; best_i = bi; }
+    if (better(b, bi, best, best_i)) { best = b; best_i = bi; }
   }
   if (lane == 0) { part_f[wave] = best; part_i[wave] = best_i; }
   __syncthreads();
   float mx = part_f[0];
   int arg = part_i[0];
 #pragma unroll
-  for (int w = 1; w < SAMPLE_WAVES; ++w) {
-    const float b = part_f[w];
-    const int bi = part_i[w];
-    if (bi != 0x7fffffff && (arg == 0x7fffffff || b > mx || (b == mx && bi < arg))) { mx = b; arg = bi; }
-  }
+  for (int w = 1; w < SCAN_WAVES; ++w)
+    if (better(part_f[w], part_i[w], mx, arg)) { mx = part_f[w]; arg = part_i[w]; }
+  const int64_t o = (int64_t)r * segments + s;
+  if (tid == 0) { seg_max[o] = mx; seg_arg[o] = arg; }
+  const float temp = temperature ? temperature[r] : 0.f;
+  if (!(temp > 0.f)) return;
+  const float inv_t = 1.0f / temp;
+  float sum = 0.f;
+  for (int i = sb + tid; i < se; i += SCAN_THREADS) sum += __expf((x[i] - mx) * inv_t);
+  sum = block_sum<SCAN_WAVES>(sum, part_f);
+  if (tid == 0) seg_sum[o] = sum;
+}
+
+// One workgroup per row: the row's maximum from the segments' (lowest segment first, so the lowest index
+// wins among equals); with a temperature, the segments' masses brought to the row's maximum, added in
+// segment order, the segment that holds uniform * total, and inside it SCAN_THREADS runs of consecutive
+// tokens whose masses are added in order until the target is passed.
+__global__ __launch_bounds__(SCAN_THREADS) void sample_pick_kernel(
+    int32_t* __restrict__ out, const float* __restrict__ seg_max, const int32_t* __restrict__ seg_arg,
+    const float* __restrict__ seg_sum, const float* __restrict__ logits, int64_t row_stride, int vocab, int seg,
+    int segments, const float* __restrict__ temperature, const float* __restrict__ uniform) {
+  __shared__ float mass[MAX_SEGMENTS];
+  __shared__ float runs[SCAN_THREADS];
+  __shared__ float walk[3];
+  __shared__ int owner_s[2];
+  const int r = blockIdx.x, tid = threadIdx.x;
+  const float* x = logits + (int64_t)r * row_stride;
+  const int64_t o = (int64_t)r * segments;
+  float mx = seg_max[o];
+  int arg = seg_arg[o];
+  for (int s = 1; s < segments; ++s)
+    if (better(seg_max[o + s], seg_arg[o + s], mx, arg)) { mx = seg_max[o + s]; arg = seg_arg[o + s]; }
   const float temp = temperature ? temperature[r] : 0.f;
   if (!(temp > 0.f)) {
     if (tid == 0) out[r] = arg;
     return;
   }
-  // ---- mass of each wavefront's contiguous segment of the vocabulary
   const float inv_t = 1.0f / temp;
-  const int seg = ((vocab + SAMPLE_WAVES - 1) / SAMPLE_WAVES + WAVE - 1) / WAVE * WAVE;
-  const int sb = wave * seg < vocab ? wave * seg : vocab;
-  const int se = sb + seg < vocab ? sb + seg : vocab;
-  float sum = 0.f;
-  for (int i = sb + lane; i < se; i += WAVE) sum += __expf((x[i] - mx) * inv_t);
-  sum = wave_sum(sum);
-  if (lane == 0) seg_sum[wave] = sum;
+  if (tid < segments) mass[tid] = seg_sum[o + tid] * __expf((seg_max[o + tid] - mx) * inv_t);
   __syncthreads();
   if (tid == 0) {
     float total = 0.f;
-    for (int w = 0; w < SAMPLE_WAVES; ++w) total += seg_sum[w];
+    for (int s = 0; s < segments; ++s) total += mass[s];
     const float target = uniform[r] * total;
     float run = 0.f;
-    int owner = SAMPLE_WAVES - 1;
-    for (int w = 0; w < SAMPLE_WAVES; ++w) {
-      if (run + seg_sum[w] > target) { owner = w; break; }
-      if (w < SAMPLE_WAVES - 1) run += seg_sum[w];
+    int owner = segments - 1;
+    for (int s = 0; s < segments; ++s) {
+      if (run + mass[s] > target) { owner = s; break; }
+      if (s < segments - 1) run += mass[s];
     }
     while (owner > 0 && owner * seg >= vocab) --owner;    // never an empty segment
-    owner_s = owner;
+    owner_s[0] = owner;
     walk[0] = run;
     walk[1] = target;
   }
   __syncthreads();
-  if (wave != owner_s) return;
-  // ---- the owner walks its segment in index order, 64 tokens at a time, with a prefix sum over lanes
-  float run = walk[0];
+  const int owner = owner_s[0];
   const float target = walk[1];
-  int pick = se - 1;                       // if rounding leaves the target just past the segment's mass
-  for (int base = sb; base < se; base += WAVE) {
-    const int i = base + lane;
-    float e = i < se ? __expf((x[i] - mx) * inv_t) : 0.f;
-#pragma unroll
-    for (int o = 1; o < WAVE; o <<= 1) {   // inclusive prefix sum
-      const float up = __shfl_up(e, o, WAVE);
-      if (lane >= o) e += up;
+  const int sb = owner * seg, se = sb + seg < vocab ? sb + seg : vocab;
+  const int per = (se - sb + SCAN_THREADS - 1) / SCAN_THREADS;     // consecutive tokens of a thread
+  const int tb = sb + tid * per < se ? sb + tid * per : se;
+  const int te = tb + per < se ? tb + per : se;
+  float mine = 0.f;
+  for (int i = tb; i < te; ++i) mine += __expf((x[i] - mx) * inv_t);
+  runs[tid] = mine;
+  __syncthreads();
+  if (tid == 0) {
+    float run = walk[0];
+    int t = SCAN_THREADS - 1;
+    for (int k = 0; k < SCAN_THREADS; ++k) {
+      if (run + runs[k] > target) { t = k; break; }
+      if (k < SCAN_THREADS - 1) run += runs[k];
     }
-    const unsigned long long hit = __ballot(run + e > target && i < se);
-    if (hit) {
-      pick = base + __ffsll((long long)hit) - 1;
-      break;
-    }
-    run += __shfl(e, WAVE - 1, WAVE);
+    while (t > 0 && sb + t * per >= se) --t;                // never an empty run
+    owner_s[1] = t;
+    walk[2] = run;
   }
-  if (lane == 0) out[r] = pick;
+  __syncthreads();
+  if (tid != owner_s[1]) return;
+  float run = walk[2];
+  int pick = te - 1;                       // if rounding leaves the target just past the run's mass
+  for (int i = tb; i < te; ++i) {
+    run += __expf((x[i] - mx) * inv_t);
+    if (run > target) { pick = i; break; }
+  }
+  out[r] = pick;
+}
+
+// How the vocabulary is cut: a function of its size alone.
+static void segments_of(int vocab, int* seg, int* segments) {
+  int n = (vocab + 2047) / 2048;
+  if (n > MAX_SEGMENTS) n = MAX_SEGMENTS;
+  if (n < 1) n = 1;
+  *seg = (vocab + n - 1) / n;
+  *segments = (vocab + *seg - 1) / *seg;
+}
+
+// Floats of scratch memory that ga_sample_rows needs for these sizes.
+extern "C" int64_t ga_sample_scratch_floats(int rows, int vocab) {
+  int seg, segments;
+  segments_of(vocab > 0 ? vocab : 1, &seg, &segments);
+  return (int64_t)3 * (rows > 0 ? rows : 0) * segments;
 }
 
 // out: [R] int32; logits: [R, vocab] float with row stride; temperature, uniform: [R] float
-// (temperature may be null: all rows greedy).
+// (temperature may be null: all rows greedy); scratch: ga_sample_scratch_floats(rows, vocab) floats.
 extern "C" int ga_sample_rows(void* out, const void* logits, int64_t row_stride, int rows, int vocab,
-                              const void* temperature, const void* uniform, hipStream_t stream) {
+                              const void* temperature, const void* uniform, void* scratch, hipStream_t stream) {
   if (rows <= 0) return 0;
-  if (vocab <= 0) return -1;
-  hipLaunchKernelGGL(sample_rows_kernel, dim3(rows), dim3(SAMPLE_THREADS), 0, stream, (int32_t*)out,
-                     (const float*)logits, row_stride, vocab, (const float*)temperature,
-                     (const float*)uniform);
+  if (vocab <= 0 || !scratch) return -1;
+  int seg, segments;
+  segments_of(vocab, &seg, &segments);
+  float* seg_max = (float*)scratch;
+  int32_t* seg_arg = (int32_t*)(seg_max + (int64_t)rows * segments);
+  float* seg_sum = seg_max + (int64_t)2 * rows * segments;
+  hipLaunchKernelGGL(sample_scan_kernel, dim3(segments, rows), dim3(SCAN_THREADS), 0, stream, seg_max, seg_arg,
+                     seg_sum, (const float*)logits, row_stride, vocab, seg, segments, (const float*)temperature);
+  hipLaunchKernelGGL(sample_pick_kernel, dim3(rows), dim3(SCAN_THREADS), 0, stream, (int32_t*)out, seg_max,
+                     seg_arg, seg_sum, (const float*)logits, row_stride, vocab, seg, segments,
+                     (const float*)temperature, (const float*)uniform);
   return GA_CHECK_LAUNCH();
 }

@@ -228,9 +228,12 @@ def sample_rows(logits, temperature=None, uniform=None, out=None):
     if out is None:
         out = torch.empty((R,), dtype=torch.int32, device=logits.device)
     _need(out.dtype == torch.int32 and out.shape == (R,) and out.is_contiguous(), "out must be contiguous int32 [R]")
+    _need(R <= 65535, "at most 65535 rows a call")
     lib = build.load("sampling")
+    lib.ga_sample_scratch_floats.restype = ctypes.c_int64
+    scratch = torch.empty((max(1, lib.ga_sample_scratch_floats(_i(R), _i(V))),), dtype=torch.float32, device=logits.device)
     _check(lib.ga_sample_rows(_ptr(out), _ptr(logits), _i64(logits.stride(0)), _i(R), _i(V), _ptr(temperature),
-                              _ptr(uniform), _stream()), "sample_rows")
+                              _ptr(uniform), _ptr(scratch), _stream()), "sample_rows")
     return out
 
 

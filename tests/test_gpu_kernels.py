@@ -296,6 +296,23 @@ def test_temperature_sampling(V):
     assert ops.sample_rows(one, torch.ones(1, device=dev()), torch.full((1,), 0.9999999, device=dev())).item() == V - 1
 
 
+@pytest.mark.parametrize("V", [777, 5000, 151936])
+def test_sampling_does_not_depend_on_the_rows_beside(V):
+    """A row's token is a function of its logits, temperature and uniform number alone: the same row drawn alone,
+    among 7 and among 300 rows gives the same token, bit for bit in the sums behind it."""
+    from ginfer_amd.kernels import ops
+    R = 300
+    x = rnd((R, V), torch.float32, 33, scale=3.0)
+    temps = torch.full((R,), 1.3, device=dev())
+    temps[::5] = 0.0
+    uni = torch.rand((R,), generator=torch.Generator().manual_seed(4)).to(dev())
+    every = ops.sample_rows(x, temps, uni).cpu().tolist()
+    some = ops.sample_rows(x[10:17], temps[10:17].contiguous(), uni[10:17].contiguous()).cpu().tolist()
+    assert some == every[10:17]
+    for r in (0, 1, 151, 299):
+        assert ops.sample_rows(x[r:r + 1], temps[r:r + 1].contiguous(), uni[r:r + 1].contiguous()).item() == every[r]
+
+
 def test_kernels_refuse_what_they_cannot_take():
     from ginfer_amd.kernels import ops, KernelError
     with pytest.raises(KernelError):
