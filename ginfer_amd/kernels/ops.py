@@ -238,6 +238,59 @@ def sample_rows(logits, temperature=None, uniform=None, out=None):
 
 
 SKINNY_MAX_ROWS = 64
+FOLDED_NORM_MAX_ROWS = 16
+
+
+class ScaledRows:
+    """The rows of a root-mean-square norm in two factors, as the products around a folded norm hand them on:
+    `scaled` = h * g (bfloat16 [M, H]) and `sumsq` (float32 [M, parts]), partial sums of h^2 over the columns;
+    the normalised row is scaled / sqrt(sum(sumsq) / H + eps).  A product that takes them multiplies its
+    32-bit sums by the rows' factors, which gives what the normalised rows would."""
+
+    __slots__ = ("scaled", "sumsq", "eps")
+
+    def __init__(self, scaled, sumsq, eps):
+        self.scaled, self.sumsq, self.eps = scaled, sumsq, float(eps)
+
+    @property
+    def shape(self):
+        return self.scaled.shape
+
+    @property
+    def dtype(self):
+        return self.scaled.dtype
+
+    def rows(self):
+        """The normalised rows themselves (for checks; the kernels never build them)."""
+        rstd = torch.rsqrt(self.sumsq.double().sum(dim=1, keepdim=True) / self.scaled.shape[1] + self.eps)
+        return (self.scaled.double() * rstd).float()
+
+
+class _SkinnyNorm(ctypes.Structure):
+    _fields_ = [("in_sumsq", _vp), ("in_parts", _i), ("inv_width", _f), ("eps", _f), ("residual", _vp), ("ldr", _i64),
+                ("gain", _vp), ("gain_f32", _i), ("scaled", _vp), ("lds", _i64), ("out_sumsq", _vp)]
+
+
+def _norm_in(norm, a):
+    """Fills the in_ fields from ScaledRows; returns the rows the product runs on."""
+    _need(a.scaled.dtype == torch.bfloat16 and a.scaled.dim() == 2 and a.scaled.shape[0] <= FOLDED_NORM_MAX_ROWS,
+          "rows of a folded norm are bfloat16 [M <= %d, H]" % FOLDED_NORM_MAX_ROWS)
+    M, H = a.scaled.shape
+    _need(a.sumsq.dtype == torch.float32 and a.sumsq.dim() == 2 and a.sumsq.shape[0] == M and a.sumsq.is_contiguous()
+          and 1 <= a.sumsq.shape[1] <= 512, "partial sums of a folded norm are contiguous float32 [M, parts <= 512]")
+    norm.in_sumsq, norm.in_parts = a.sumsq.data_ptr(), a.sumsq.shape[1]
+    norm.inv_width, norm.eps = 1.0 / H, a.eps
+    return a.scaled
+
+
+def folded_norm_supported(a, w, residual, gain):
+    """Whether a [M, K] . w [N, K]^T can add itself to `residual` and hand on the rows of the norm with `gain`
+    in two factors (ScaledRows)."""
+    x = a.scaled if isinstance(a, ScaledRows) else a
+    N = w.shape[0]
+    return (gemm_skinny_supported(x, w) and x.shape[0] <= FOLDED_NORM_MAX_ROWS and N % 8 == 0 and N <= 16 * 512
+            and residual.dtype == torch.float32 and residual.shape == (x.shape[0], N) and residual.stride(1) == 1
+            and gain.dtype in (torch.bfloat16, torch.float32) and gain.shape == (N,) and gain.is_contiguous())
 
 
 def gemm_skinny_supported(a, w):
@@ -247,11 +300,32 @@ def gemm_skinny_supported(a, w):
             and w.is_contiguous() and w.data_ptr() % 16 == 0)
 
 
-def gemm_skinny(a, w, bias=None, out=None, out_dtype=None, nt=0, ks=0, grid_splits=1, gated=False):
+def gemm_skinny(a, w, bias=None, out=None, out_dtype=None, nt=0, ks=0, grid_splits=1, gated=False, into_norm=None):
     """a [M <= 64, K] . w [N, K]^T (+ bias) -> [M, N] in bfloat16 (or float32): the decode step's products,
     weights streamed once through the matrix cores.  grid_splits > 1: K is split over workgroups too and
     the result is float32 [grid_splits, M, N], parts for the consumer to add.  gated: w is [2N, K] (gate
-    over up) and the result is silu(a.gate^T) * (a.up^T)."""
+    over up) and the result is silu(a.gate^T) * (a.up^T).
+    a may be ScaledRows (at most 16 rows): the rows of a norm in two factors.  into_norm = (residual, gain, eps):
+    the product is added to the float32 residual [M, N] in place and the rows of the norm that follows come
+    back as ScaledRows instead of the product."""
+    norm = None
+    if isinstance(a, ScaledRows):
+        norm = _SkinnyNorm()
+        a = _norm_in(norm, a)
+    if into_norm is not None:
+        residual, gain, eps = into_norm
+        _need(folded_norm_supported(a, w, residual, gain) and not gated and grid_splits == 1 and out is None,
+              "a product folds the norm after it for at most %d bfloat16 rows, a float32 residual [M, N] and a "
+              "gain [N], N a multiple of 8 up to 8192" % FOLDED_NORM_MAX_ROWS)
+        _dev(residual, gain)
+        norm = norm or _SkinnyNorm()
+        M, N = residual.shape
+        lib = build.load("gemm_skinny")
+        scaled = torch.empty((M, N), dtype=torch.bfloat16, device=a.device)
+        sumsq = torch.empty((M, lib.ga_skinny_norm_parts(_i(N))), dtype=torch.float32, device=a.device)
+        norm.residual, norm.ldr = residual.data_ptr(), residual.stride(0)
+        norm.gain, norm.gain_f32 = gain.data_ptr(), 1 if gain.dtype == torch.float32 else 0
+        norm.scaled, norm.lds, norm.out_sumsq = scaled.data_ptr(), scaled.stride(0), sumsq.data_ptr()
     _dev(a, w, bias, out)
     _need(a.dim() == 2 and w.dim() == 2 and a.shape[1] == w.shape[1], "gemm_skinny: a [M, K] and w [N, K] do not agree: %s, %s"
           % (tuple(a.shape), tuple(w.shape)))
@@ -264,6 +338,10 @@ def gemm_skinny(a, w, bias=None, out=None, out_dtype=None, nt=0, ks=0, grid_spli
         N //= 2
     if bias is not None:
         _need(bias.dtype == torch.bfloat16 and bias.shape == (N,) and bias.is_contiguous(), "gemm_skinny: bias must be bfloat16 [N]")
+    if into_norm is not None:
+        _check(lib.ga_gemm_skinny(_vp(0), _i64(0), _ptr(a), _i64(a.stride(0)), _ptr(w), _ptr(bias), _i(M), _i(N), _i(K),
+                                  _i(0), _i(1), _i(8), _i(1), _i(0), ctypes.byref(norm), _stream()), "gemm_skinny")
+        return ScaledRows(scaled, sumsq, eps)
     out_dtype = out_dtype or (out.dtype if out is not None else torch.bfloat16)
     _need(out_dtype in (torch.bfloat16, torch.float32), "gemm_skinny: out dtype must be bfloat16 or float32")
     if grid_splits > 1:
@@ -281,19 +359,27 @@ def gemm_skinny(a, w, bias=None, out=None, out_dtype=None, nt=0, ks=0, grid_spli
     lib = build.load("gemm_skinny")
     _check(lib.ga_gemm_skinny(_ptr(out), _i64(ldc), _ptr(a), _i64(a.stride(0)), _ptr(w), _ptr(bias), _i(M), _i(N),
                               _i(K), _i(1 if out_dtype == torch.float32 else 0), _i(nt), _i(ks), _i(grid_splits),
-                              _i(1 if gated else 0), _stream()), "gemm_skinny")
+                              _i(1 if gated else 0), ctypes.byref(norm) if norm is not None else _vp(0), _stream()),
+           "gemm_skinny")
     return out
 
 
 def qkv_rope_skinny_supported(x, w, head_dim, rotary_dim):
     """Whether the fused projection + rotation + cache-write kernel takes these operands."""
+    if isinstance(x, ScaledRows):
+        x = x.scaled
     return gemm_skinny_supported(x, w) and head_dim % 32 == 0 and rotary_dim == head_dim
 
 
 def qkv_rope_skinny(x, w, bias, positions, cos, sin, slot_mapping, k_pages, v_pages, num_heads, num_kv_heads, head_dim,
                     write_kv=True):
     """The decode step's q|k|v projection with its epilogue in one kernel: x [M <= 64, K] . w^T + bias, NeoX
-    rotation of q and k, q returned as [M, nh*hd], k and v written into the paged cache at slot_mapping."""
+    rotation of q and k, q returned as [M, nh*hd], k and v written into the paged cache at slot_mapping.
+    x may be ScaledRows."""
+    norm = None
+    if isinstance(x, ScaledRows):
+        norm = _SkinnyNorm()
+        x = _norm_in(norm, x)
     _dev(x, w, bias, positions, cos, sin, slot_mapping, k_pages, v_pages)
     M, K = x.shape
     width = (num_heads + 2 * num_kv_heads) * head_dim
@@ -314,8 +400,8 @@ def qkv_rope_skinny(x, w, bias, positions, cos, sin, slot_mapping, k_pages, v_pa
     lib = build.load("gemm_skinny")
     _check(lib.ga_qkv_rope_skinny(_ptr(q), _ptr(x), _i64(x.stride(0)), _ptr(w), _ptr(bias), _ptr(positions), _ptr(cos),
                                   _ptr(sin), _ptr(slot_mapping), _ptr(k_pages), _ptr(v_pages), _i(M), _i(K), _i(num_heads),
-                                  _i(num_kv_heads), _i(head_dim), _i(page_size), _i(1 if write_kv else 0), _stream()),
-           "qkv_rope_skinny")
+                                  _i(num_kv_heads), _i(head_dim), _i(page_size), _i(1 if write_kv else 0),
+                                  ctypes.byref(norm) if norm is not None else _vp(0), _stream()), "qkv_rope_skinny")
     return q
 
 

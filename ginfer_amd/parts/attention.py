@@ -6,7 +6,7 @@ import torch
 from ..kernels import ops
 from ..weights.loader import WeightSpec
 from .base import Part, KVCacheSpec
-from .linear import linear
+from .linear import linear, linear_into_norm
 from .registry import register_mixer
 
 
@@ -18,6 +18,8 @@ class Attention(Part):
     score scale 1/sqrt(head_dim) unless `scale` is given; `window` None attends to all earlier keys."""
 
     capturable = True
+    takes_scaled_rows = True
+    folds_norm = True
 
     def __init__(self, hidden_size, num_heads, num_kv_heads, head_dim, qkv_bias, out_bias, window, position,
                  scale, dtype, device):
@@ -61,7 +63,9 @@ class Attention(Part):
             mods += [("attention_mfma", {"HEAD_DIM": self.hd}), "gemm_skinny"]
         return mods
 
-    def forward(self, x, step, cache):
+    def forward(self, x, step, cache, into_norm=None):
+        """into_norm = (residual, norm): where the output projection's kernel can, the result is added to the
+        residual here and the rows of `norm` come back as ops.ScaledRows; else the result comes back as ever."""
         cos, sin = self.position.tables()
         if ops.qkv_rope_skinny_supported(x, self.w_qkv, self.hd, self.position.rotary_dim):
             # few rows (decode): projection, rotation and cache write in one kernel
@@ -73,4 +77,8 @@ class Attention(Part):
                               self.nh, self.nkv, self.hd, write_kv=cache.owner)
         a = ops.paged_attention(qkv, cache.k_pages, cache.v_pages, cache.block_table, step, self.nh, self.nkv,
                                 self.hd, self.scale, self.window)
+        if into_norm is not None:
+            folded = linear_into_norm(a, self.w_o, self.b_o, *into_norm)
+            if folded is not None:
+                return folded
         return linear(a, self.w_o, self.b_o, parts_ok=True)

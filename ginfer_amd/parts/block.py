@@ -1,4 +1,5 @@
 """How a layer's parts are arranged around the residual stream."""
+from ..kernels import ops
 from .registry import register_arrangement
 
 
@@ -7,11 +8,16 @@ class PreNormBlock:
     """n = norm1(x); h = x + mixer(n); n = norm2(h); x = h + feed_forward(n)
     (ginfer/core/layer/transformer/encoder.cc:33-39).  The residual stream is kept in 32-bit and every add
     is fused into the norm that follows it, so a block takes the previous block's output as a pending
-    `delta` and returns its own feed-forward output as the next one."""
+    `delta` and returns its own feed-forward output as the next one.  Where the mixer says `folds_norm`, the
+    feed-forward `takes_scaled_rows` and the norm between them is `foldable`, the mixer may add its result to
+    the residual itself and hand the norm's rows on in two factors (ops.ScaledRows): then the second norm makes
+    no pass over memory of its own."""
 
     def __init__(self, mixer, feed_forward, mixer_norm, feed_forward_norm):
         self.mixer, self.feed_forward = mixer, feed_forward
         self.mixer_norm, self.feed_forward_norm = mixer_norm, feed_forward_norm
+        self.folds = (getattr(mixer, "folds_norm", False) and getattr(feed_forward, "takes_scaled_rows", False)
+                      and getattr(feed_forward_norm, "foldable", False))
 
     def parts(self):
         """(role, part): the roles are the keys of `LayerSpec.names`, which gives each its tensor prefix."""
@@ -20,7 +26,12 @@ class PreNormBlock:
 
     def forward(self, residual, delta, step, cache):
         n = self.mixer_norm.forward(residual, whole(delta, self.mixer_norm))
-        a = self.mixer.forward(n, step, cache)
+        if self.folds:
+            a = self.mixer.forward(n, step, cache, into_norm=(residual, self.feed_forward_norm))
+            if isinstance(a, ops.ScaledRows):
+                return self.feed_forward.forward(a)
+        else:
+            a = self.mixer.forward(n, step, cache)
         n = self.feed_forward_norm.forward(residual, whole(a, self.feed_forward_norm))
         return self.feed_forward.forward(n)
 

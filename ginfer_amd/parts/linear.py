@@ -19,7 +19,9 @@ SPLIT_K_PARTS = 4
 def linear(x, weight, bias=None, out_dtype=None, parts_ok=False):
     """x [M, K], weight [N, K], bias [N] | None -> [M, N] in x's dtype (or float32 on request).
     With parts_ok the result may instead be float32 [parts, M, N]: partial sums of a K-split product,
-    which the norm that follows adds up in order."""
+    which the norm that follows adds up in order.  x may be ops.ScaledRows, the rows of a folded norm."""
+    if isinstance(x, ops.ScaledRows):
+        return ops.gemm_skinny(x, weight, bias, out_dtype=out_dtype, nt=1)
     if x.dtype == torch.float32:
         return ops.gemm_nt(x, weight, bias)
     if ops.gemm_skinny_supported(x, weight) and not _library_is_faster(x.shape[0], weight.shape[0]):
@@ -52,8 +54,23 @@ def _library_is_faster(rows, out_features):
 LIBRARY_FROM_ROWS = 16
 
 
+def linear_into_norm(x, weight, bias, residual, norm):
+    """residual += x . W^T (+ b) in place, and the rows of `norm` over the new residual as ops.ScaledRows: the
+    product's kernel folds the add and the norm, so neither makes a pass over memory of its own.  None where
+    the kernel does not take these operands (more than 16 rows, 32-bit, odd sizes, a norm that is no plain
+    root-mean-square norm with a gain): the caller then takes the ordinary way."""
+    if not getattr(norm, "foldable", False) or x.dtype != torch.bfloat16 or residual is None:
+        return None
+    if not ops.folded_norm_supported(x, weight, residual, norm.weight):
+        return None
+    return ops.gemm_skinny(x, weight, bias, into_norm=(residual, norm.weight, norm.eps))
+
+
 def gated_linear(x, weight_gate_up):
-    """silu(x . Wg^T) * (x . Wu^T) with Wg over Wu stacked in one matrix [2I, K] -> [M, I]."""
+    """silu(x . Wg^T) * (x . Wu^T) with Wg over Wu stacked in one matrix [2I, K] -> [M, I].  x may be
+    ops.ScaledRows."""
+    if isinstance(x, ops.ScaledRows):
+        return ops.gemm_skinny(x, weight_gate_up, gated=True)
     if (x.dtype == torch.bfloat16 and ops.gemm_skinny_supported(x, weight_gate_up)
             and not _library_is_faster(x.shape[0], weight_gate_up.shape[0])):
         return ops.gemm_skinny(x, weight_gate_up, gated=True)

@@ -14,6 +14,7 @@ class SwiGLU(Part):
     up are one product over the stacked weights, which equals the two separate ones."""
 
     capturable = True
+    takes_scaled_rows = True
 
     def __init__(self, hidden_size, intermediate_size, dtype, device):
         self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)

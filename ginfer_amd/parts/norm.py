@@ -14,6 +14,7 @@ class RMSNorm(Part):
 
     capturable = True
     accepts_partial_sums = True
+    foldable = True          # a plain gain over the root mean square: the products around it can fold it
 
     def __init__(self, size, eps, dtype, device):
         self.size, self.eps, self.dtype, self.device = int(size), float(eps), dtype, device

@@ -479,6 +479,71 @@ def test_gemm_skinny_gated(M, I, K):
     close(ops.gemm_skinny(a, w, gated=True), ref, 1e-2)
 
 
+@pytest.mark.parametrize("M", [1, 3, 8, 16])
+@pytest.mark.parametrize("N,K,bias,gain_dtype", [(1536, 1536, False, torch.bfloat16), (1536, 8960, False, torch.float32),
+                                                 (88, 136, True, torch.bfloat16), (200, 64, True, torch.float32),
+                                                 (8192, 72, False, torch.bfloat16)])
+def test_gemm_skinny_folds_the_norm_after_it(M, N, K, bias, gain_dtype):
+    """The product that adds itself to the residual and hands on the norm's rows in two factors, and the
+    products that take such rows: together they equal add, norm, product."""
+    from ginfer_amd.kernels import ops
+    eps = 1e-5
+    a, w = rnd((M, K), torch.bfloat16, 70), rnd((N, K), torch.bfloat16, 71, scale=0.3)
+    b = rnd((N,), torch.bfloat16, 72) if bias else None
+    res0 = rnd((M, N), torch.float32, 73, scale=2.0)
+    gain = (1 + 0.1 * rnd((N,), torch.float32, 74)).to(gain_dtype)
+    assert ops.folded_norm_supported(a, w, res0, gain)
+    res = res0.clone()
+    rows = ops.gemm_skinny(a, w, b, into_norm=(res, gain, eps))
+    h = res0.double() + a.double() @ w.double().t() + (b.double() if bias else 0)
+    close(res, h, 1e-5)
+    close(rows.scaled, h * gain.double(), 1e-2)
+    close(rows.sumsq.sum(dim=1), (h * h).sum(dim=1), 1e-5)
+    normed = pm.rms_norm(h, gain.double(), eps)
+    close(rows.rows(), normed, 1e-2)
+    # the partial sums come from the 32-bit residual that was written, column block by column block
+    parts = torch.stack([(res[:, c:c + 16].double() ** 2).sum(dim=1) for c in range(0, N, 16)], dim=1)
+    close(rows.sumsq, parts, 1e-6)
+    # products that take the rows: plain, gated, and the fused q|k|v projection
+    w2 = rnd((72, N), torch.bfloat16, 75, scale=0.2)
+    b2 = rnd((72,), torch.bfloat16, 76)
+    given = rows.rows().double()          # what the rows stand for, from the rounded h * g
+    close(ops.gemm_skinny(rows, w2, b2, out_dtype=torch.float32), given @ w2.double().t() + b2.double(), 1e-5)
+    wg = rnd((2 * 40, N), torch.bfloat16, 77, scale=0.1)
+    close(ops.gemm_skinny(rows, wg, gated=True, out_dtype=torch.float32),
+          pm.swiglu(given @ wg[:40].double().t(), given @ wg[40:].double().t()), 1e-5)
+    nh, nkv, hd = 3, 1, 32
+    wq, bq = rnd(((nh + 2 * nkv) * hd, N), torch.bfloat16, 78, scale=0.1), rnd(((nh + 2 * nkv) * hd,), torch.bfloat16, 79)
+    positions = torch.arange(M, dtype=torch.int32, device=dev()) * 7
+    sin, cos = pm.rope_tables(1e4, hd, 200)
+    kp, vp = rnd((4, nkv, 8, hd), torch.bfloat16, 80), rnd((4, nkv, hd, 8), torch.bfloat16, 81)
+    slots = torch.arange(M, dtype=torch.int64, device=dev())
+    q = ops.qkv_rope_skinny(rows, wq, bq, positions, cos.to(dev()), sin.to(dev()), slots, kp, vp, nh, nkv, hd)
+    kp2, vp2 = kp.clone(), vp.clone()
+    q2 = ops.qkv_rope_skinny(rows.rows().to(torch.bfloat16), wq, bq, positions, cos.to(dev()), sin.to(dev()), slots, kp2, vp2,
+                             nh, nkv, hd)
+    close(q, q2, 2e-2)
+    close(kp, kp2, 2e-2)
+    close(vp, vp2, 2e-2)
+    # a row's factors do not depend on the rows beside it
+    if M > 1:
+        res1 = res0[M - 1:M].clone()
+        alone = ops.gemm_skinny(a[M - 1:M], w, b, into_norm=(res1, gain, eps))
+        assert torch.equal(alone.scaled[0], rows.scaled[M - 1]) and torch.equal(alone.sumsq[0], rows.sumsq[M - 1])
+        assert torch.equal(res1[0], res[M - 1])
+
+
+def test_folded_norm_refuses_what_it_cannot_take():
+    from ginfer_amd.kernels import ops, KernelError
+    a, w = rnd((17, 64), torch.bfloat16, 1), rnd((32, 64), torch.bfloat16, 2)
+    res, gain = rnd((17, 32), torch.float32, 3), rnd((32,), torch.bfloat16, 4)
+    assert not ops.folded_norm_supported(a, w, res, gain)                       # more than 16 rows
+    assert not ops.folded_norm_supported(a[:4], w, res[:4].bfloat16(), gain)    # residual not 32-bit
+    assert not ops.folded_norm_supported(a[:4], w[:28], res[:4, :28], gain[:28])  # width no multiple of 8
+    with pytest.raises(KernelError):
+        ops.gemm_skinny(a, w, into_norm=(res, gain, 1e-6))
+
+
 @pytest.mark.parametrize("M", [1, 8, 33, 64])
 @pytest.mark.parametrize("nh,nkv,hd,K,theta", [(12, 2, 128, 1536, 1e4), (6, 1, 32, 192, 1e6), (4, 4, 64, 88, 1e4), (5, 1, 96, 72, 5e5)])
 def test_qkv_rope_skinny(M, nh, nkv, hd, K, theta):

@@ -122,6 +122,55 @@ def test_attention_part_in_portions(dtype, tol, window):
     close(torch.cat(outs), ref, tol)
 
 
+@pytest.mark.parametrize("T", [1, 5, 16, 17])
+def test_block_folds_the_norm_between_mixer_and_feed_forward(T):
+    """With few rows the output projection adds itself to the residual and hands the second norm's rows on in
+    two factors; the block's result equals the one with the norm as a kernel of its own."""
+    from ginfer_amd.kernels import ops
+    from ginfer_amd.parts import lookup, KVView, StepContext
+    Hd, nh, nkv, hd, I, ps = 96, 3, 1, 32, 136, 8
+    dtype = torch.bfloat16
+    pos = lookup("position", "rope_neox")(theta=1e4, rotary_dim=hd, max_positions=64, device=dev())
+    mixer = lookup("mixer", "attention")(hidden_size=Hd, num_heads=nh, num_kv_heads=nkv, head_dim=hd, qkv_bias=True,
+                                         out_bias=False, window=None, position=pos, scale=None, dtype=dtype, device=dev())
+    ff = lookup("feed_forward", "swiglu")(hidden_size=Hd, intermediate_size=I, dtype=dtype, device=dev())
+    norms = [lookup("norm", "rmsnorm")(size=Hd, eps=1e-5, dtype=dtype, device=dev()) for _ in range(2)]
+    for k, part in enumerate([mixer, ff] + norms):
+        part.bind_weights({n: ((1 + rnd(sp.shape, 10 * k + i, 0.1)) if n == "weight" and part in norms
+                               else rnd(sp.shape, 10 * k + i, 0.15)).to(dtype).to(dev())
+                           for i, (n, sp) in enumerate(part.weight_specs().items())})
+    block = lookup("arrangement", "prenorm")(mixer, ff, norms[0], norms[1])
+    assert block.folds
+    seen = []
+    inner = mixer.forward
+    mixer.forward = lambda *a, **k: (seen.append(inner(*a, **k)), seen[-1])[1]
+    results = []
+    for folds in (True, False):
+        block.folds = folds
+        kp = torch.zeros((4, nkv, ps, hd), dtype=dtype, device=dev())
+        vp = torch.zeros((4, nkv, hd, ps), dtype=dtype, device=dev())
+        p = np.arange(T)
+        table = [2, 0, 3]
+        slots = torch.tensor(np.asarray(table)[p // ps] * ps + p % ps, dtype=torch.int64, device=dev())
+        view = KVView(kp, vp, torch.tensor([table], dtype=torch.int32, device=dev()), slots, ps, True)
+        step = StepContext(token_ids=None, positions=torch.tensor(p, dtype=torch.int32, device=dev()),
+                           token_entry=torch.zeros(T, dtype=torch.int32, device=dev()),
+                           cu_tokens=torch.tensor([0, T], dtype=torch.int32, device=dev()),
+                           q_start=torch.tensor([0], dtype=torch.int32, device=dev()),
+                           logit_rows=None, num_tokens=T, num_entries=1, host_q_start=[0], host_q_len=[T],
+                           caches=[view], extra={})
+        residual = rnd((T, Hd), 50).to(dev())
+        delta = block.forward(residual, rnd((T, Hd), 51, 0.3).to(dtype).to(dev()), step, view)
+        if delta.dim() == 3:
+            delta = delta.sum(dim=0)
+        results.append((residual, delta.float()))
+    assert isinstance(seen[0], ops.ScaledRows) == (T <= 16)        # folded up to 16 rows, else the ordinary way
+    assert not isinstance(seen[1], ops.ScaledRows)
+    # the ordinary way rounds the mixer's output to bfloat16 before the add, the folded one adds the 32-bit sums
+    close(results[0][0], results[1][0], 4e-3)
+    close(results[0][1], results[1][1], 2e-2)
+
+
 # ----------------------------------------------------------------------------- generality of the assembly
 
 def _register_toy():
