@@ -288,7 +288,8 @@ def folded_norm_supported(a, w, residual, gain):
     in two factors (ScaledRows)."""
     x = a.scaled if isinstance(a, ScaledRows) else a
     N = w.shape[0]
-    return (gemm_skinny_supported(x, w) and x.shape[0] <= FOLDED_NORM_MAX_ROWS and N % 8 == 0 and N <= 16 * 512
+    return (gemm_skinny_supported(x, w) and x.shape[0] <= FOLDED_NORM_MAX_ROWS and N % 8 == 0
+            and N <= (8 if x.shape[0] <= 8 else 16) * 512
             and residual.dtype == torch.float32 and residual.shape == (x.shape[0], N) and residual.stride(1) == 1
             and gain.dtype in (torch.bfloat16, torch.float32) and gain.shape == (N,) and gain.is_contiguous())
 
@@ -300,11 +301,14 @@ def gemm_skinny_supported(a, w):
             and w.is_contiguous() and w.data_ptr() % 16 == 0)
 
 
-def gemm_skinny(a, w, bias=None, out=None, out_dtype=None, nt=0, ks=0, grid_splits=1, gated=False, into_norm=None):
+def gemm_skinny(a, w, bias=None, out=None, out_dtype=None, nt=0, ks=0, grid_splits=1, gated=False, into_norm=None,
+                pack=0):
     """a [M <= 64, K] . w [N, K]^T (+ bias) -> [M, N] in bfloat16 (or float32): the decode step's products,
     weights streamed once through the matrix cores.  grid_splits > 1: K is split over workgroups too and
     the result is float32 [grid_splits, M, N], parts for the consumer to add.  gated: w is [2N, K] (gate
     over up) and the result is silu(a.gate^T) * (a.up^T).
+    pack = 2 (at most 8 rows): a tile of the matrix cores holds 8 rows of w twice, for the two halves of K,
+    so that twice the workgroups stream the weights.
     a may be ScaledRows (at most 16 rows): the rows of a norm in two factors.  into_norm = (residual, gain, eps):
     the product is added to the float32 residual [M, N] in place and the rows of the norm that follows come
     back as ScaledRows instead of the product."""
@@ -316,13 +320,13 @@ def gemm_skinny(a, w, bias=None, out=None, out_dtype=None, nt=0, ks=0, grid_spli
         residual, gain, eps = into_norm
         _need(folded_norm_supported(a, w, residual, gain) and not gated and grid_splits == 1 and out is None,
               "a product folds the norm after it for at most %d bfloat16 rows, a float32 residual [M, N] and a "
-              "gain [N], N a multiple of 8 up to 8192" % FOLDED_NORM_MAX_ROWS)
+              "gain [N], N a multiple of 8 up to 4096 (8192 from 9 rows on)" % FOLDED_NORM_MAX_ROWS)
         _dev(residual, gain)
         norm = norm or _SkinnyNorm()
         M, N = residual.shape
         lib = build.load("gemm_skinny")
         scaled = torch.empty((M, N), dtype=torch.bfloat16, device=a.device)
-        sumsq = torch.empty((M, lib.ga_skinny_norm_parts(_i(N))), dtype=torch.float32, device=a.device)
+        sumsq = torch.empty((M, lib.ga_skinny_norm_parts(_i(M), _i(N))), dtype=torch.float32, device=a.device)
         norm.residual, norm.ldr = residual.data_ptr(), residual.stride(0)
         norm.gain, norm.gain_f32 = gain.data_ptr(), 1 if gain.dtype == torch.float32 else 0
         norm.scaled, norm.lds, norm.out_sumsq = scaled.data_ptr(), scaled.stride(0), sumsq.data_ptr()
@@ -340,7 +344,7 @@ def gemm_skinny(a, w, bias=None, out=None, out_dtype=None, nt=0, ks=0, grid_spli
         _need(bias.dtype == torch.bfloat16 and bias.shape == (N,) and bias.is_contiguous(), "gemm_skinny: bias must be bfloat16 [N]")
     if into_norm is not None:
         _check(lib.ga_gemm_skinny(_vp(0), _i64(0), _ptr(a), _i64(a.stride(0)), _ptr(w), _ptr(bias), _i(M), _i(N), _i(K),
-                                  _i(0), _i(1), _i(8), _i(1), _i(0), ctypes.byref(norm), _stream()), "gemm_skinny")
+                                  _i(0), _i(1), _i(8), _i(1), _i(0), _i(0), ctypes.byref(norm), _stream()), "gemm_skinny")
         return ScaledRows(scaled, sumsq, eps)
     out_dtype = out_dtype or (out.dtype if out is not None else torch.bfloat16)
     _need(out_dtype in (torch.bfloat16, torch.float32), "gemm_skinny: out dtype must be bfloat16 or float32")
@@ -359,8 +363,8 @@ def gemm_skinny(a, w, bias=None, out=None, out_dtype=None, nt=0, ks=0, grid_spli
     lib = build.load("gemm_skinny")
     _check(lib.ga_gemm_skinny(_ptr(out), _i64(ldc), _ptr(a), _i64(a.stride(0)), _ptr(w), _ptr(bias), _i(M), _i(N),
                               _i(K), _i(1 if out_dtype == torch.float32 else 0), _i(nt), _i(ks), _i(grid_splits),
-                              _i(1 if gated else 0), ctypes.byref(norm) if norm is not None else _vp(0), _stream()),
-           "gemm_skinny")
+                              _i(1 if gated else 0), _i(pack), ctypes.byref(norm) if norm is not None else _vp(0),
+                              _stream()), "gemm_skinny")
     return out
 
 
@@ -372,7 +376,7 @@ def qkv_rope_skinny_supported(x, w, head_dim, rotary_dim):
 
 
 def qkv_rope_skinny(x, w, bias, positions, cos, sin, slot_mapping, k_pages, v_pages, num_heads, num_kv_heads, head_dim,
-                    write_kv=True):
+                    write_kv=True, pack=0):
     """The decode step's q|k|v projection with its epilogue in one kernel: x [M <= 64, K] . w^T + bias, NeoX
     rotation of q and k, q returned as [M, nh*hd], k and v written into the paged cache at slot_mapping.
     x may be ScaledRows."""
@@ -400,7 +404,7 @@ def qkv_rope_skinny(x, w, bias, positions, cos, sin, slot_mapping, k_pages, v_pa
     lib = build.load("gemm_skinny")
     _check(lib.ga_qkv_rope_skinny(_ptr(q), _ptr(x), _i64(x.stride(0)), _ptr(w), _ptr(bias), _ptr(positions), _ptr(cos),
                                   _ptr(sin), _ptr(slot_mapping), _ptr(k_pages), _ptr(v_pages), _i(M), _i(K), _i(num_heads),
-                                  _i(num_kv_heads), _i(head_dim), _i(page_size), _i(1 if write_kv else 0),
+                                  _i(num_kv_heads), _i(head_dim), _i(page_size), _i(1 if write_kv else 0), _i(pack),
                                   ctypes.byref(norm) if norm is not None else _vp(0), _stream()), "qkv_rope_skinny")
     return q
 

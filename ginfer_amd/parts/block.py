@@ -11,7 +11,9 @@ class PreNormBlock:
     `delta` and returns its own feed-forward output as the next one.  Where the mixer says `folds_norm`, the
     feed-forward `takes_scaled_rows` and the norm between them is `foldable`, the mixer may add its result to
     the residual itself and hand the norm's rows on in two factors (ops.ScaledRows): then the second norm makes
-    no pass over memory of its own."""
+    no pass over memory of its own.  The same holds across blocks: a block whose feed-forward `folds_norm` may be
+    given the first norm of the block that runs next (`into_norm`), if that block says `takes_folded_input()`;
+    it then returns ops.ScaledRows in place of its delta, and the next block skips its first norm."""
 
     def __init__(self, mixer, feed_forward, mixer_norm, feed_forward_norm):
         self.mixer, self.feed_forward = mixer, feed_forward
@@ -24,16 +26,31 @@ class PreNormBlock:
         return [("mixer", self.mixer), ("feed_forward", self.feed_forward), ("mixer_norm", self.mixer_norm),
                 ("feed_forward_norm", self.feed_forward_norm)]
 
-    def forward(self, residual, delta, step, cache):
-        n = self.mixer_norm.forward(residual, whole(delta, self.mixer_norm))
+    @property
+    def folds_output(self):
+        """Whether forward() takes `into_norm`."""
+        return bool(getattr(self.feed_forward, "folds_norm", False))
+
+    def takes_folded_input(self):
+        """The norm whose rows this block takes in two factors (ops.ScaledRows) in place of a delta, or None."""
+        if getattr(self.mixer, "takes_scaled_rows", False) and getattr(self.mixer_norm, "foldable", False):
+            return self.mixer_norm
+        return None
+
+    def forward(self, residual, delta, step, cache, into_norm=None):
+        if isinstance(delta, ops.ScaledRows):      # the block before has added its output and folded this norm
+            n = delta
+        else:
+            n = self.mixer_norm.forward(residual, whole(delta, self.mixer_norm))
         if self.folds:
             a = self.mixer.forward(n, step, cache, into_norm=(residual, self.feed_forward_norm))
-            if isinstance(a, ops.ScaledRows):
-                return self.feed_forward.forward(a)
         else:
             a = self.mixer.forward(n, step, cache)
-        n = self.feed_forward_norm.forward(residual, whole(a, self.feed_forward_norm))
-        return self.feed_forward.forward(n)
+        if not isinstance(a, ops.ScaledRows):
+            a = self.feed_forward_norm.forward(residual, whole(a, self.feed_forward_norm))
+        if into_norm is not None:
+            return self.feed_forward.forward(a, into_norm=(residual, into_norm))
+        return self.feed_forward.forward(a)
 
 
 def whole(delta, norm):

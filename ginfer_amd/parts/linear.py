@@ -14,6 +14,9 @@ from ..kernels import ops
 # a product with at least this many input features whose consumer adds partial sums is split over K
 SPLIT_K_FROM = 4096
 SPLIT_K_PARTS = 4
+# a folded norm keeps K within a workgroup; measured on MI355X, a product with a long K still gains from
+# folding while its tiles are packed (up to 8 rows)
+FOLD_LONG_K_UP_TO_ROWS = 8
 
 
 def linear(x, weight, bias=None, out_dtype=None, parts_ok=False):
@@ -61,6 +64,8 @@ def linear_into_norm(x, weight, bias, residual, norm):
     root-mean-square norm with a gain): the caller then takes the ordinary way."""
     if not getattr(norm, "foldable", False) or x.dtype != torch.bfloat16 or residual is None:
         return None
+    if x.shape[1] >= SPLIT_K_FROM and x.shape[0] > FOLD_LONG_K_UP_TO_ROWS:
+        return None      # a long K wants its split over workgroups more than it wants the norm folded
     if not ops.folded_norm_supported(x, weight, residual, norm.weight):
         return None
     return ops.gemm_skinny(x, weight, bias, into_norm=(residual, norm.weight, norm.eps))

@@ -4,7 +4,7 @@ import torch
 from ..kernels import ops
 from ..weights.loader import WeightSpec
 from .base import Part
-from .linear import linear, gated_linear
+from .linear import linear, gated_linear, linear_into_norm
 from .registry import register_feed_forward
 
 
@@ -15,6 +15,7 @@ class SwiGLU(Part):
 
     capturable = True
     takes_scaled_rows = True
+    folds_norm = True
 
     def __init__(self, hidden_size, intermediate_size, dtype, device):
         self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)
@@ -33,6 +34,13 @@ class SwiGLU(Part):
     def kernel_modules(self):
         return ["activation", "gemm"] + (["gemm_skinny"] if self.dtype == torch.bfloat16 else [])
 
-    def forward(self, x):
+    def forward(self, x, into_norm=None):
+        """into_norm = (residual, norm): where the down projection's kernel can, the result is added to the
+        residual here and the rows of `norm` come back as ops.ScaledRows."""
+        act = gated_linear(x, self.w_gate_up)
+        if into_norm is not None:
+            folded = linear_into_norm(act, self.w_down, None, *into_norm)
+            if folded is not None:
+                return folded
         # the result may be partial sums of a K-split product: the norm that follows adds them up
-        return linear(gated_linear(x, self.w_gate_up), self.w_down, parts_ok=True)
+        return linear(act, self.w_down, parts_ok=True)

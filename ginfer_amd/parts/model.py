@@ -75,6 +75,14 @@ class DecoderModel:
             n2 = self._build("norm", ls.feed_forward_norm)
             self.blocks.append(registry.lookup("arrangement", ls.arrangement)(mixer, ffn, n1, n2))
         self.schedule = list(spec.schedule)
+        # per run of the schedule: the first norm of the block that runs next, where this run's block can fold it
+        # into its own last product and that block takes its input so (a matter of speed only)
+        self._fold_into = []
+        for i, e in enumerate(self.schedule):
+            nxt = self.blocks[self.schedule[i + 1].layer] if i + 1 < len(self.schedule) else None
+            takes = getattr(nxt, "takes_folded_input", None)
+            norm = takes() if takes is not None else None
+            self._fold_into.append(norm if getattr(self.blocks[e.layer], "folds_output", False) else None)
 
     def _build(self, role, part_spec):
         params = dict(part_spec.params)
@@ -142,7 +150,10 @@ class DecoderModel:
         delta = None
         for i, e in enumerate(self.schedule):
             cache = step.caches[i]
-            delta = self.blocks[e.layer].forward(residual, delta, step, cache)
+            if self._fold_into[i] is not None:
+                delta = self.blocks[e.layer].forward(residual, delta, step, cache, into_norm=self._fold_into[i])
+            else:
+                delta = self.blocks[e.layer].forward(residual, delta, step, cache)
         n = self.final_norm.forward(residual, whole(delta, self.final_norm), rows=step.logit_rows)
         return self.head.forward(n)
 
