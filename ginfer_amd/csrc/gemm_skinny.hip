@@ -285,8 +285,8 @@ struct GaSkinnyNorm {
 };
 
 // Tiles of a product of M rows when the caller leaves the choice to the library: packed whenever they can be
-// (measured on MI355X: up to a third faster where a product has few columns; ga_gemm_skinny leaves a product
-// with thousands of workgroups, the head, as it is).
+// (measured on MI355X: up to a third faster where a product has few columns; ga_gemm_skinny leaves products
+// with many workgroups as they are: the head, and the gated product, which was measured slower packed).
 static int auto_pack(int M) { return M <= 8 ? 2 : 1; }
 
 // Partial sums a row gets from a product of M rows and N columns that feeds a norm.
@@ -328,7 +328,7 @@ extern "C" int ga_gemm_skinny(void* C, int64_t ldc, const void* A, int64_t lda, 
   if (grid_splits > 1 && !out_f32) return -3;
   if (gated && (grid_splits > 1 || bias)) return -4;
   const int groups = SK_WAVES / ks;
-  if (pack == 0) pack = (grid_splits == 1 && N / (groups * (gated ? 16 : nt * 16)) <= 1024) ? auto_pack(M) : 1;
+  if (pack == 0) pack = (grid_splits == 1 && !gated && N / (groups * nt * 16) <= 1024) ? auto_pack(M) : 1;
   if (pack != 1 && (pack != 2 || M > 8)) return -2;
   const int cp = 16 / pack;
   const int ncol = gated ? cp : nt * cp;
