@@ -140,6 +140,29 @@ struct Packed {
   static __device__ __forceinline__ int seg(int r) { return r / CP; }
 };
 
+// How K is dealt out: in steps of 64 elements, as evenly as whole steps allow, to `units` consumers (the
+// wavefronts that split K, over all workgroups of a column, times the halves of a packed tile).  Consumer u
+// takes the steps [u * steps / units, (u + 1) * steps / units).  A lane works in its own coordinates, starting
+// at 0 at its first element: `shift` is where that lies, `ke` its own end, `kend` the end of the wavefront's
+// trips (the longer of its halves).
+template <int PACK>
+struct KRange {
+  int shift, ke, kend;
+  __device__ __forceinline__ KRange(int first_unit, int seg, int steps, int units, int K) {
+    int longest = 0;
+#pragma unroll
+    for (int q = 0; q < PACK; ++q) {
+      const int b = (int)(((int64_t)(first_unit + q) * steps) / units), e = (int)(((int64_t)(first_unit + q + 1) * steps) / units);
+      longest = e - b > longest ? e - b : longest;
+      if (q == seg) {
+        shift = b * 64;
+        ke = (e * 64 < K ? e * 64 : K) - b * 64;
+      }
+    }
+    kend = longest * 64;
+  }
+};
+
 // NT: tiles of W per wavefront; MB: 16-row blocks of A; KS: wavefronts of a workgroup that split K
 // for the same rows (the workgroup's SK_WAVES / KS groups own different rows of W).  The grid's y
 // dimension splits K further: then every workgroup writes its part in 32-bit to P[y][M][N] and the
@@ -153,8 +176,8 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(TC* __restrict_
                                                                  const bf16_t* __restrict__ A, int64_t lda,
                                                                  const bf16_t* __restrict__ W,
                                                                  const bf16_t* __restrict__ bias, int M, int N,
-                                                                 int K, int kchunk_wg, int kchunk_wave, int kseg,
-                                                                 NormIn norm_in, NormOut norm_out) {
+                                                                 int K, int ksteps, NormIn norm_in,
+                                                                 NormOut norm_out) {
   static_assert(PACK == 1 || MB == 1, "a packed tile holds at most 8 rows of A");
   __shared__ float red[SK_WAVES][NT * 16][MB * 16 + 1];
   __shared__ float rstd[16];
@@ -165,14 +188,8 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(TC* __restrict_
   const int grp = wave / KS, ks = wave % KS;
   constexpr int NCOL = GATED ? CP : NT * CP;       // output columns of a group
   const int n0 = (blockIdx.x * GROUPS + grp) * NCOL;
-  const int kwg = blockIdx.y * kchunk_wg;
-  const int kwg_end = kwg + kchunk_wg < K ? kwg + kchunk_wg : K;
-  const int kb = kwg + ks * kchunk_wave;
-  const int kwave_end = kb + kchunk_wave < kwg_end ? kb + kchunk_wave : kwg_end;
-  // this lane's range in its own coordinates: its pointers are shifted by its half's offset
-  const int shift = P::seg(r) * kseg;
-  const int kend = kb + kseg < kwave_end ? kb + kseg : kwave_end;          // the trips' end, the same for all lanes
-  const int ke = kend < kwave_end - shift ? kend : kwave_end - shift;
+  const KRange<PACK> kr((blockIdx.y * KS + ks) * PACK, P::seg(r), ksteps, gridDim.y * KS * PACK, K);
+  const int shift = kr.shift;
 
   const bf16_t* wp[NT];
   bool wok[NT];
@@ -209,7 +226,7 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(TC* __restrict_
     }
   }
 
-  skinny_accumulate<NT, MB>(acc, wp, wok, ap, aok, kb, kend, ke, g);
+  skinny_accumulate<NT, MB>(acc, wp, wok, ap, aok, 0, kr.kend, kr.ke, g);
   if (MB == 1) in_loads.finish(norm_in, rstd, M, wave, lane);
   // the KS parts of a group meet in LDS and are added in wavefront order, the halves of a packed tile in theirs
 #pragma unroll
@@ -332,14 +349,12 @@ extern "C" int ga_gemm_skinny(void* C, int64_t ldc, const void* A, int64_t lda, 
   if (pack != 1 && (pack != 2 || M > 8)) return -2;
   const int cp = 16 / pack;
   const int ncol = gated ? cp : nt * cp;
-  const int kchunk_wg = ((K + grid_splits - 1) / grid_splits + 63) / 64 * 64;
-  const int kchunk_wave = ((kchunk_wg + ks - 1) / ks + 63) / 64 * 64;
-  const int kseg = ((kchunk_wave + pack - 1) / pack + 63) / 64 * 64;
+  const int ksteps = (K + 63) / 64;
   dim3 grid((N + groups * ncol - 1) / (groups * ncol), grid_splits), block(SK_THREADS);
 #define LAUNCH(NT, MB, KS, TC, G, PK)                                                                     \
   hipLaunchKernelGGL((gemm_skinny_kernel<NT, MB, KS, TC, G, PK>), grid, block, 0, stream, (TC*)C, ldc,   \
-                     (const bf16_t*)A, lda, (const bf16_t*)W, (const bf16_t*)bias, M, N, K, kchunk_wg,   \
-                     kchunk_wave, kseg, norm_in, norm_out)
+                     (const bf16_t*)A, lda, (const bf16_t*)W, (const bf16_t*)bias, M, N, K, ksteps,      \
+                     norm_in, norm_out)
 #define PICK_KS(NT, MB, TC, G, PK)                                                                        \
   switch (ks) {                                                                                           \
     case 1: LAUNCH(NT, MB, 1, TC, G, PK); break;                                                          \
@@ -389,7 +404,7 @@ __global__ __launch_bounds__(SK_THREADS) void qkv_rope_skinny_kernel(
     const bf16_t* __restrict__ bias, const int32_t* __restrict__ positions, const float* __restrict__ cos_t,
     const float* __restrict__ sin_t, const int64_t* __restrict__ slot_mapping, bf16_t* __restrict__ k_pages,
     bf16_t* __restrict__ v_pages, int M, int K, int nh, int nkv, int hd, int page_size, int write_kv,
-    int kchunk_wave, int kseg, NormIn norm_in) {
+    int ksteps, NormIn norm_in) {
   static_assert(PACK == 1 || MB == 1, "a packed tile holds at most 8 rows of A");
   __shared__ float red[SK_WAVES][32][MB * 16 + 1];
   __shared__ float rstd[16];
@@ -415,11 +430,8 @@ __global__ __launch_bounds__(SK_THREADS) void qkv_rope_skinny_kernel(
       row1 = row0 + CP;
     }
   }
-  const int kb = ks * kchunk_wave;
-  const int kwave_end = kb + kchunk_wave < K ? kb + kchunk_wave : K;
-  const int shift = P::seg(r) * kseg;
-  const int kend = kb + kseg < kwave_end ? kb + kseg : kwave_end;
-  const int ke = kend < kwave_end - shift ? kend : kwave_end - shift;
+  const KRange<PACK> kr(ks * PACK, P::seg(r), ksteps, KS * PACK, K);
+  const int shift = kr.shift;
   const bf16_t* wp[2] = {W + (int64_t)(row0 + P::col(r)) * K + shift, W + (int64_t)(row1 + P::col(r)) * K + shift};
   const bool wok[2] = {unit_ok, unit_ok};
   const bf16_t* ap[MB];
@@ -471,7 +483,7 @@ __global__ __launch_bounds__(SK_THREADS) void qkv_rope_skinny_kernel(
     for (int mb = 0; mb < MB; ++mb) acc[nt][mb] = f32x4{0.f, 0.f, 0.f, 0.f};
   NormInLoads in_loads;
   if (MB == 1) in_loads.load(norm_in, M, wave, lane);
-  skinny_accumulate<2, MB>(acc, wp, wok, ap, aok, kb, kend, ke, g);
+  skinny_accumulate<2, MB>(acc, wp, wok, ap, aok, 0, kr.kend, kr.ke, g);
   if (MB == 1) in_loads.finish(norm_in, rstd, M, wave, lane);
   const bool scale_rows = MB == 1 && norm_in.sumsq != nullptr;
 #pragma unroll
@@ -550,14 +562,13 @@ extern "C" int ga_qkv_rope_skinny(void* q_out, const void* A, int64_t lda, const
   if (pack != 1 && (pack != 2 || M > 8)) return -2;
   const int ks = 8, groups = SK_WAVES / ks;
   const int units = (nh + 2 * nkv) * hd / (2 * (16 / pack));
-  const int kchunk_wave = ((K + ks - 1) / ks + 63) / 64 * 64;
-  const int kseg = ((kchunk_wave + pack - 1) / pack + 63) / 64 * 64;
+  const int ksteps = (K + 63) / 64;
   dim3 grid((units + groups - 1) / groups), block(SK_THREADS);
 #define LAUNCH(MB, PK)                                                                                    \
   hipLaunchKernelGGL((qkv_rope_skinny_kernel<MB, 8, PK>), grid, block, 0, stream, (bf16_t*)q_out,        \
                      (const bf16_t*)A, lda, (const bf16_t*)W, (const bf16_t*)bias, (const int32_t*)positions, \
                      (const float*)cos_t, (const float*)sin_t, (const int64_t*)slot_mapping, (bf16_t*)k_pages, \
-                     (bf16_t*)v_pages, M, K, nh, nkv, hd, page_size, write_kv, kchunk_wave, kseg, norm_in)
+                     (bf16_t*)v_pages, M, K, nh, nkv, hd, page_size, write_kv, ksteps, norm_in)
   switch (mb) {
     case 1:
       if (pack == 2) LAUNCH(1, 2); else LAUNCH(1, 1);

@@ -26,7 +26,13 @@ def _ptr(t):
 
 
 def _stream():
-    return _vp(torch.cuda.current_stream().cuda_stream)
+    """The raw handle of torch's current stream on the current device (the recording stream while a step is
+    being recorded)."""
+    return _vp(_raw_stream(_current_device()))
+
+
+_raw_stream = torch._C._cuda_getCurrentRawStream
+_current_device = torch.cuda.current_device
 
 
 def _check(rc, name):
@@ -44,9 +50,12 @@ def _dev(*tensors):
     for t in tensors:
         if t is None:
             continue
-        _need(t.is_cuda, "kernel operands must live on the GPU (got a %s tensor)" % t.device)
-        dev = dev or t.device
-        _need(t.device == dev, "kernel operands lie on different devices")
+        if not t.is_cuda:
+            raise KernelError("kernel operands must live on the GPU (got a %s tensor)" % t.device)
+        if dev is None:
+            dev = t.device
+        elif t.device != dev:
+            raise KernelError("kernel operands lie on different devices")
 
 
 def _is_bf16(dtype):

@@ -13,7 +13,7 @@ from ..kernels import ops
 
 # a product with at least this many input features whose consumer adds partial sums is split over K
 SPLIT_K_FROM = 4096
-SPLIT_K_PARTS = 4
+MAX_SPLIT_K_PARTS = 16
 # a folded norm keeps K within a workgroup; measured on MI355X, a product with a long K still gains from
 # folding while its tiles are packed (up to 8 rows)
 FOLD_LONG_K_UP_TO_ROWS = 8
@@ -33,8 +33,12 @@ def linear(x, weight, bias=None, out_dtype=None, parts_ok=False):
         # long K is split over workgroups where the consumer can add the parts
         many = x.shape[0] > 16
         if parts_ok and out_dtype is None and x.shape[1] >= SPLIT_K_FROM:
-            return ops.gemm_skinny(x, weight, bias, out_dtype=torch.float32, nt=4 if many else 1,
-                                   grid_splits=2 * SPLIT_K_PARTS if many else SPLIT_K_PARTS)
+            # enough parts that a wavefront's share of K is one trip of loads (4 steps of 64 with one tile,
+            # 2 with four), and a tenth more, which was measured faster than an exact fit
+            per_trip = 2 if many else 4
+            steps = -(-x.shape[1] // 64)
+            splits = min(MAX_SPLIT_K_PARTS, max(2, -(-steps * 11 // (10 * 8 * per_trip))))
+            return ops.gemm_skinny(x, weight, bias, out_dtype=torch.float32, nt=4 if many else 1, grid_splits=splits)
         if parts_ok and out_dtype is None and x.shape[1] >= 1024:
             return ops.gemm_skinny(x, weight, bias, out_dtype=torch.float32, nt=1, grid_splits=2)
         return ops.gemm_skinny(x, weight, bias, out_dtype=out_dtype, nt=4 if (many and weight.shape[0] >= 4096) else 1)
