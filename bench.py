@@ -80,7 +80,7 @@ def main():
     ctx_pages = -(-(args.context + 1) // page)
     pages = max_b * ctx_pages + -(-args.prefill_tokens // page) + 8
     runner = ModelRunner(folder, dtype=args.dtype, page_size=page, num_pages=pages, max_requests=max_b + 1,
-                         max_model_len=args.context + 8)
+                         max_model_len=max(args.context, args.prefill_tokens) + 8)
     sampler = Sampler(runner.device)
     g = torch.Generator().manual_seed(0)
     vocab = cfg["vocab_size"]
