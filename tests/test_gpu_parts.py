@@ -83,6 +83,25 @@ def test_embedding_and_head_parts(dtype, tol, tied):
     close(logits, x.double() @ Wh.double().t(), 1e-5 if dtype == torch.float32 else 1e-4)
 
 
+@pytest.mark.parametrize("theta,rd,n", [(1e4, 16, 300), (1e6, 128, 70), (5e5, 96, 33)])
+def test_position_part(theta, rd, n):
+    """The position encoding alone: its 32-bit tables equal the plain formula's, bit for bit in the angles'
+    inputs (position cast to float before the multiply), and a limit cuts them without changing a value."""
+    from ginfer_amd.parts import lookup
+    part = lookup("position", "rope_neox")(theta=theta, rotary_dim=rd, max_positions=n, device=dev())
+    cos, sin = part.tables()
+    ref_sin, ref_cos = pm.rope_tables(theta, rd, n)
+    assert cos.dtype == torch.float32 and cos.shape == (n, rd // 2) and sin.shape == (n, rd // 2)
+    close(cos, ref_cos, 1e-6)
+    close(sin, ref_sin, 1e-6)
+    assert torch.equal(cos[0].cpu(), torch.ones(rd // 2)) and torch.equal(sin[0].cpu(), torch.zeros(rd // 2))
+    part.limit_positions(10)
+    cos10, sin10 = part.tables()
+    assert cos10.shape == (10, rd // 2) and torch.equal(cos10, cos[:10]) and torch.equal(sin10, sin[:10])
+    with pytest.raises(ValueError):
+        lookup("position", "rope_neox")(theta=theta, rotary_dim=15, max_positions=n, device=dev())
+
+
 @pytest.mark.parametrize("dtype,tol", PART_DTYPES)
 @pytest.mark.parametrize("window", [None, 12])
 def test_attention_part_in_portions(dtype, tol, window):
