@@ -389,3 +389,41 @@ def test_sizes_that_fit_no_vector_width(tmp_path, dtype):
         got = H.run_steps(runner, steps)
         runner.cache.check()
         H.compare_with_plain(got, reqs, folder, H.TOL[dtype], "odd sizes %s %s" % (dtype, what))
+
+
+def _drawn_configuration(seed):
+    """A configuration of the architecture drawn at random: every size and option varies."""
+    import random
+    rng = random.Random(seed)
+    nkv = rng.choice([1, 1, 2, 3, 4])
+    group = rng.choice([1, 2, 3, 4, 7])
+    hd = 16 * rng.randint(1, 6)
+    layers = rng.randint(1, 3)
+    cfg = dict(architectures=["Qwen2ForCausalLM"], num_hidden_layers=layers, hidden_size=rng.randint(17, 130),
+               num_attention_heads=nkv * group, num_key_value_heads=nkv, head_dim=hd,
+               intermediate_size=rng.randint(16, 200), vocab_size=rng.randint(50, 700),
+               rope_theta=rng.choice([1e4, 1e6, 5e5]), rms_norm_eps=rng.choice([1e-6, 1e-5, 1e-3]),
+               tie_word_embeddings=rng.random() < 0.5, max_position_embeddings=rng.choice([96, 128, 512]))
+    if rng.random() < 0.5:
+        cfg.update(use_sliding_window=True, sliding_window=rng.randint(3, 40), max_window_layers=rng.randint(0, layers))
+    return cfg, rng.choice([8, 16, 32])
+
+
+@pytest.mark.parametrize("seed", list(range(8)))
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_configurations_drawn_at_random(tmp_path, seed, dtype):
+    """Whole, mixed with so few pages that they are used again, and the last tokens one by one, for configurations
+    nobody chose: heads, groups, widths, windows, page sizes."""
+    from ginfer_amd import ModelRunner
+    cfg, page = _drawn_configuration(seed)
+    folder = H.make_model_folder(tmp_path / "drawn", cfg, seed, "float32")
+    V = cfg["vocab_size"]
+    reqs = {"a": H.random_tokens(90, V, 10 + seed), "b": H.random_tokens(41, V, 20 + seed),
+            "c": H.random_tokens(1 + seed, V, 30 + seed), "d": H.random_tokens(64, V, 40 + seed)}
+    mixed = H.steps_mixed(reqs, max_live=3, seed=seed)
+    pages = -(-H.max_live_tokens(mixed) // page)
+    runner = ModelRunner(folder, dtype=dtype, page_size=page, num_pages=pages, max_requests=4)
+    for what, steps in (("mixed", mixed), ("whole", H.steps_whole(reqs)), ("last decoded", H.steps_last_decoded(reqs))):
+        got = H.run_steps(runner, steps)
+        runner.cache.check()
+        H.compare_with_plain(got, reqs, folder, H.TOL[dtype], "drawn %d %s %s %s" % (seed, dtype, what, cfg))
