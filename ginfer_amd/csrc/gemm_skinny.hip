@@ -397,8 +397,10 @@ extern "C" int ga_gemm_skinny(void* C, int64_t ldc, const void* A, int64_t lda, 
 // ginfer/core/op/kernels/cuda/store_kvcache_kernel.cu:19-30).  A wavefront group owns a UNIT of 2 CP output
 // columns as two tiles of CP (16, or 8 when packed): for a q or k head the columns j0..j0+CP-1 and their
 // rotation partners j0+half..; for a v head 2 CP consecutive columns.  head_dim a multiple of 32,
-// rotary_dim == head_dim.
-template <int MB, int KS, int PACK>
+// rotary_dim == head_dim.  HALF (with more than 16 rows of A, where tiles cannot be packed): a tile holds 8 rows
+// of W and nothing in its other half, so that twice the workgroups share the product; this product has too few
+// columns to fill the chip otherwise, and its K cannot be split over workgroups (the epilogue needs whole sums).
+template <int MB, int KS, int PACK, bool HALF>
 __global__ __launch_bounds__(SK_THREADS) void qkv_rope_skinny_kernel(
     bf16_t* __restrict__ q_out, const bf16_t* __restrict__ A, int64_t lda, const bf16_t* __restrict__ W,
     const bf16_t* __restrict__ bias, const int32_t* __restrict__ positions, const float* __restrict__ cos_t,
@@ -406,10 +408,11 @@ __global__ __launch_bounds__(SK_THREADS) void qkv_rope_skinny_kernel(
     bf16_t* __restrict__ v_pages, int M, int K, int nh, int nkv, int hd, int page_size, int write_kv,
     int ksteps, NormIn norm_in) {
   static_assert(PACK == 1 || MB == 1, "a packed tile holds at most 8 rows of A");
+  static_assert(PACK == 1 || !HALF, "a tile is packed or half empty, not both");
   __shared__ float red[SK_WAVES][32][MB * 16 + 1];
   __shared__ float rstd[16];
   using P = Packed<PACK>;
-  constexpr int CP = P::CP;
+  constexpr int CP = HALF ? 8 : P::CP;
   constexpr int GROUPS = SK_WAVES / KS;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r = lane & 15, g = lane >> 4;
   const int grp = wave / KS, ks = wave % KS;
@@ -432,8 +435,10 @@ __global__ __launch_bounds__(SK_THREADS) void qkv_rope_skinny_kernel(
   }
   const KRange<PACK> kr(ks * PACK, P::seg(r), ksteps, KS * PACK, K);
   const int shift = kr.shift;
-  const bf16_t* wp[2] = {W + (int64_t)(row0 + P::col(r)) * K + shift, W + (int64_t)(row1 + P::col(r)) * K + shift};
-  const bool wok[2] = {unit_ok, unit_ok};
+  const int wrow = HALF ? (r & 7) : P::col(r);
+  const bool lane_ok = unit_ok && (!HALF || r < 8);
+  const bf16_t* wp[2] = {W + (int64_t)(row0 + wrow) * K + shift, W + (int64_t)(row1 + wrow) * K + shift};
+  const bool wok[2] = {lane_ok, lane_ok};
   const bf16_t* ap[MB];
   bool aok[MB];
 #pragma unroll
@@ -505,7 +510,7 @@ __global__ __launch_bounds__(SK_THREADS) void qkv_rope_skinny_kernel(
     for (int w = 0; w < KS; ++w)
 #pragma unroll
       for (int q = 0; q < PACK; ++q) {
-        const int col = (m / CP) * 16 + q * CP + m % CP;
+        const int col = PACK == 1 ? m : q * CP + m;
         lo += red[gi * KS + w][q * CP + nl][col];
         hi += red[gi * KS + w][16 + q * CP + nl][col];
       }
@@ -561,21 +566,30 @@ extern "C" int ga_qkv_rope_skinny(void* q_out, const void* A, int64_t lda, const
   if (pack == 0) pack = auto_pack(M);
   if (pack != 1 && (pack != 2 || M > 8)) return -2;
   const int ks = 8, groups = SK_WAVES / ks;
-  const int units = (nh + 2 * nkv) * hd / (2 * (16 / pack));
+  // with more than 8 rows and so few columns that full tiles leave most of the chip idle: half tiles (measured on
+  // MI355X: 64 rows 11.4 us against 15.9 with 64 workgroups of full tiles; with 144 of them, slower)
+  const bool half_tiles = pack == 1 && M > 8 && (nh + 2 * nkv) * hd / 32 < 128;
+  const int units = (nh + 2 * nkv) * hd / (2 * (half_tiles ? 8 : 16 / pack));
   const int ksteps = (K + 63) / 64;
   dim3 grid((units + groups - 1) / groups), block(SK_THREADS);
-#define LAUNCH(MB, PK)                                                                                    \
-  hipLaunchKernelGGL((qkv_rope_skinny_kernel<MB, 8, PK>), grid, block, 0, stream, (bf16_t*)q_out,        \
+#define LAUNCH(MB, PK, HF)                                                                                \
+  hipLaunchKernelGGL((qkv_rope_skinny_kernel<MB, 8, PK, HF>), grid, block, 0, stream, (bf16_t*)q_out,    \
                      (const bf16_t*)A, lda, (const bf16_t*)W, (const bf16_t*)bias, (const int32_t*)positions, \
                      (const float*)cos_t, (const float*)sin_t, (const int64_t*)slot_mapping, (bf16_t*)k_pages, \
                      (bf16_t*)v_pages, M, K, nh, nkv, hd, page_size, write_kv, ksteps, norm_in)
   switch (mb) {
     case 1:
-      if (pack == 2) LAUNCH(1, 2); else LAUNCH(1, 1);
+      if (pack == 2) LAUNCH(1, 2, false); else if (half_tiles) LAUNCH(1, 1, true); else LAUNCH(1, 1, false);
       break;
-    case 2: LAUNCH(2, 1); break;
-    case 3: LAUNCH(3, 1); break;
-    default: LAUNCH(4, 1); break;
+    case 2:
+      if (half_tiles) LAUNCH(2, 1, true); else LAUNCH(2, 1, false);
+      break;
+    case 3:
+      if (half_tiles) LAUNCH(3, 1, true); else LAUNCH(3, 1, false);
+      break;
+    default:
+      if (half_tiles) LAUNCH(4, 1, true); else LAUNCH(4, 1, false);
+      break;
   }
 #undef LAUNCH
   return GA_CHECK_LAUNCH();

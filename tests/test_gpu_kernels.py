@@ -557,8 +557,9 @@ def test_folded_norm_refuses_what_it_cannot_take():
         ops.gemm_skinny(a, w, into_norm=(res, gain, 1e-6))
 
 
-@pytest.mark.parametrize("M,pack", [(1, 1), (1, 2), (5, 2), (8, 1), (8, 2), (33, 1), (64, 1)])
-@pytest.mark.parametrize("nh,nkv,hd,K,theta", [(12, 2, 128, 1536, 1e4), (6, 1, 32, 192, 1e6), (4, 4, 64, 88, 1e4), (5, 1, 96, 72, 5e5)])
+@pytest.mark.parametrize("M,pack", [(1, 1), (1, 2), (5, 2), (8, 1), (8, 2), (12, 1), (33, 1), (64, 1)])
+@pytest.mark.parametrize("nh,nkv,hd,K,theta", [(12, 2, 128, 1536, 1e4), (6, 1, 32, 192, 1e6), (4, 4, 64, 88, 1e4), (5, 1, 96, 72, 5e5),
+                                               (28, 4, 128, 72, 1e4)])     # the last: so many columns that tiles stay full
 def test_qkv_rope_skinny(M, pack, nh, nkv, hd, K, theta):
     """The fused decode kernel equals projection, then rotation and cache write."""
     from ginfer_amd.kernels import ops
