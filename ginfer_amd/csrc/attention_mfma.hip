@@ -489,330 +489,6 @@ __global__ __launch_bounds__(512) void attn_prefill_kernel(
   }
 }
 
-// ----------------------------------------------------------------------------- prefill through LDS
-// The same arithmetic as attn_prefill_kernel, for long prompts: a workgroup of hpw * rbw wavefronts
-// (hpw query heads of one kv head, rbw blocks of 16*NB rows each) walks the keys in tiles of LBN = 64 and
-// ALL its wavefronts take their K and V^T operands from one copy of the tile in LDS.  The copy is
-// double-buffered: while the wavefronts compute on tile i, the loads of tile i+1 are in flight into
-// registers; they are stored to the other buffer after the computation and one barrier ends the step.
-// Rows of the K tile are stored in the order in which the matrix-core products read them (row t*16 + m of
-// a 32-key half holds key 8*(m/4) + 4t + m%4), and rows are padded by 16 bytes, so that the 16 lanes of a
-// 128-bit LDS read hit different banks.
-// tiles: int32 [n][4] = (entry, first token row of the step, rows (<= rbw*16*NB), first position).
-constexpr int LBN = 64;
-constexpr int KROW = HD + 8;       // elements per row of the K tile in LDS
-constexpr int VROW = LBN + 8;      // elements per row of the V^T tile in LDS
-constexpr int LDS_TILE = LBN * KROW + HD * VROW;     // elements of one stage
-constexpr int K_CHUNKS = LBN * HD / 8, V_CHUNKS = HD * LBN / 8;
-constexpr int LDS_MIN_THREADS = 256;
-constexpr int K_PER_THREAD = (K_CHUNKS + LDS_MIN_THREADS - 1) / LDS_MIN_THREADS;
-constexpr int V_PER_THREAD = (V_CHUNKS + LDS_MIN_THREADS - 1) / LDS_MIN_THREADS;
-
-template <int NB>
-__global__ __launch_bounds__(512) void attn_prefill_lds_kernel(
-    bf16_t* __restrict__ out, int64_t out_stride, const bf16_t* __restrict__ q, int64_t q_stride,
-    const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
-    const int32_t* __restrict__ block_table, int table_width, const int32_t* __restrict__ tiles, int nh,
-    int nkv, int head_blocks, int hpw, int rbw, int ps_shift, int window, float scale) {
-  extern __shared__ __attribute__((aligned(16))) bf16_t lds_kv[];     // [2 stages][K tile | V^T tile], then page ids
-  const int tid = threadIdx.x, nthreads = blockDim.x;
-  const int lane = tid & 63, wave = tid >> 6, c = lane & 15, g = lane >> 4;
-  const int kvh = blockIdx.y / head_blocks, hb = blockIdx.y % head_blocks;
-  const int group = nh / nkv;
-  const int hl = wave / rbw, rb = wave % rbw;
-  const int head = kvh * group + hb * hpw + hl;          // hpw divides the group: every wavefront has a head
-  const int32_t* tile = tiles + (int64_t)blockIdx.x * 4;
-  const int entry = tile[0], row0 = tile[1], rows = tile[2], pos0 = tile[3];
-  const int32_t* bt = block_table + (int64_t)entry * table_width;
-  const int ps = 1 << ps_shift;
-
-  // the wavefront's own rows
-  const int wrow = rb * 16 * NB;                         // first row of the wavefront inside the tile
-  f32x4 o[NB][DB];
-  float m[NB], l[NB];
-  init_state<NB>(o, m, l);
-  bf16x8 qr[NB][KB];
-  int cpos[NB], clo[NB];
-#pragma unroll
-  for (int nb = 0; nb < NB; ++nb) {
-    const int j = wrow + nb * 16 + c;
-    const bool ok = j < rows;
-    cpos[nb] = ok ? pos0 + j : -1;
-    clo[nb] = (window > 0 && pos0 + j - window + 1 > 0) ? pos0 + j - window + 1 : 0;
-    load_q(qr[nb], ok ? q + (int64_t)(row0 + j) * q_stride + (int64_t)head * HD : nullptr, g);
-  }
-  // keys the workgroup walks, and the ranges that need no mask for this wavefront
-  const int kv_min = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;
-  const int kv_max = pos0 + rows - 1;
-  const int wlast = wrow + 16 * NB - 1 < rows - 1 ? wrow + 16 * NB - 1 : rows - 1;   // last live row of the wavefront
-  const int full_lo = (window > 0 && pos0 + wlast - window + 1 > 0) ? pos0 + wlast - window + 1 : 0;
-  const int full_hi = pos0 + wrow;
-  const bool wave_live = wrow < rows;
-  const int wave_max = pos0 + wlast;                     // no key beyond this matters to the wavefront
-  const int t_begin = (kv_min / LBN) * LBN, t_end = (kv_max / LBN + 1) * LBN;
-
-  // the pages of the keys this workgroup walks, copied to LDS once: a tile's loads then do not wait for
-  // a look-up in global memory first
-  int32_t* pages_s = reinterpret_cast<int32_t*>(lds_kv + 2 * LDS_TILE);
-  const int first_page = kv_min >> ps_shift;
-  for (int i = tid; i <= (kv_max >> ps_shift) - first_page; i += nthreads) pages_s[i] = bt[first_page + i];
-  __syncthreads();
-  const int cpr_shift = ps >= LBN ? 3 : ps_shift - 3;    // log2 of the 8-key pieces per (page, dim) inside a tile
-
-  // What a thread copies does not change from tile to tile: chunk i of the K tile is (key k0 + kkey[i],
-  // 8 dims), chunk i of the V^T tile (dim, keys k0 + vkey[i] .. + 7).  Offsets inside a page and inside
-  // LDS are worked out once, here; a tile then costs a page look-up, a multiply-add and two compares per
-  // chunk.  (k0 is a multiple of 64; pages smaller than that start at multiples of their size, larger
-  // ones hold the whole tile.)
-  const int64_t page_stride = (int64_t)nkv * ps * HD;
-  int kkey[K_PER_THREAD], kin[K_PER_THREAD], kout[K_PER_THREAD];
-  int vkey[V_PER_THREAD], vin[V_PER_THREAD], vout[V_PER_THREAD];
-#pragma unroll
-  for (int i = 0; i < K_PER_THREAD; ++i) {
-    const int id = tid + i * nthreads;
-    const int idc = id < K_CHUNKS ? id : K_CHUNKS - 1;
-    const int kl = idc / (HD / 8), ch = idc % (HD / 8);
-    const int kk = kl & 31;
-    kkey[i] = kl;
-    kin[i] = (kvh * ps + (kl & (ps - 1))) * HD + ch * 8;
-    kout[i] = id < K_CHUNKS ? ((kl & 32) + (((kk >> 2) & 1) << 4) + (((kk >> 3) << 2) | (kk & 3))) * KROW + ch * 8 : -1;
-  }
-#pragma unroll
-  for (int i = 0; i < V_PER_THREAD; ++i) {
-    const int id = tid + i * nthreads;
-    const int idc = id < V_CHUNKS ? id : V_CHUNKS - 1;
-    // chunks ordered as memory is: page of the tile, dim, 8-key piece of the page's row
-    const int pg = (idc >> cpr_shift) / HD, rem = idc - ((pg * HD) << cpr_shift);
-    const int d = rem >> cpr_shift, pc = rem & ((1 << cpr_shift) - 1);
-    const int kl = ((pg << cpr_shift) + pc) * 8;
-    vkey[i] = kl;
-    vin[i] = (kvh * HD + d) * ps + (kl & (ps - 1));
-    vout[i] = id < V_CHUNKS ? d * VROW + kl : -1;
-  }
-  // fetch only ISSUES loads (every address is valid memory: a chunk outside the request's keys reads the
-  // start of the pool instead); what must count as zero is cleared in stash, after the computation, so
-  // that nothing waits for a load before the tile's matrix products have been issued
-  uint4 kst[K_PER_THREAD], vst[V_PER_THREAD];
-  auto fetch = [&](int k0) {                             // global -> registers
-    const int pbase = (k0 >> ps_shift) - first_page;
-    const int in_page = (k0 & (ps - 1));                 // not 0 only for pages larger than a tile
-#pragma unroll
-    for (int i = 0; i < K_PER_THREAD; ++i) {
-      const int key = k0 + kkey[i];
-      const bool ok = key >= kv_min && key <= kv_max;
-      const int64_t page = ok ? pages_s[pbase + (kkey[i] >> ps_shift)] : 0;
-      const int64_t at = ok ? page * page_stride + kin[i] + in_page * HD : 0;
-      kst[i] = *reinterpret_cast<const uint4*>(k_pages + at);
-    }
-#pragma unroll
-    for (int i = 0; i < V_PER_THREAD; ++i) {
-      const int key = k0 + vkey[i];
-      const bool ok = key + 7 >= kv_min && key <= kv_max;
-      const int64_t page = ok ? pages_s[pbase + (vkey[i] >> ps_shift)] : 0;
-      const int64_t at = ok ? page * page_stride + vin[i] + in_page : 0;
-      vst[i] = *reinterpret_cast<const uint4*>(v_pages + at);
-    }
-  };
-  auto stash = [&](int stage, int k0) {                  // registers -> LDS, clearing what lies outside the keys
-    bf16_t* ks = lds_kv + (int64_t)stage * LDS_TILE;
-    bf16_t* vs = ks + LBN * KROW;
-    // an empty statement that "changes" the fetched registers: no arithmetic on them (and so no wait for
-    // their loads) can be moved up in front of the tile's computation
-#pragma unroll
-    for (int i = 0; i < K_PER_THREAD; ++i)
-      asm volatile("" : "+v"(kst[i].x), "+v"(kst[i].y), "+v"(kst[i].z), "+v"(kst[i].w));
-#pragma unroll
-    for (int i = 0; i < V_PER_THREAD; ++i)
-      asm volatile("" : "+v"(vst[i].x), "+v"(vst[i].y), "+v"(vst[i].z), "+v"(vst[i].w));
-#pragma unroll
-    for (int i = 0; i < K_PER_THREAD; ++i) {
-      if (kout[i] >= 0) {
-        const int key = k0 + kkey[i];
-        const bool ok = key >= kv_min && key <= kv_max;
-        *reinterpret_cast<uint4*>(ks + kout[i]) = ok ? kst[i] : uint4{0u, 0u, 0u, 0u};
-      }
-    }
-#pragma unroll
-    for (int i = 0; i < V_PER_THREAD; ++i) {
-      if (vout[i] >= 0) {
-        const int key = k0 + vkey[i];
-        uint4 v = vst[i];
-        if (key < kv_min || key + 7 > kv_max) {          // slots outside the request's keys hold anything
-          uint32_t w[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            const bool lo_ok = key + 2 * j >= kv_min && key + 2 * j <= kv_max;
-            const bool hi_ok = key + 2 * j + 1 >= kv_min && key + 2 * j + 1 <= kv_max;
-            w[j] &= (lo_ok ? 0x0000ffffu : 0u) | (hi_ok ? 0xffff0000u : 0u);
-          }
-          v = uint4{w[0], w[1], w[2], w[3]};
-        }
-        *reinterpret_cast<uint4*>(vs + vout[i]) = v;
-      }
-    }
-  };
-
-  fetch(t_begin);
-  stash(0, t_begin);
-  __syncthreads();
-  int stage = 0;
-  for (int k0 = t_begin; k0 < t_end; k0 += LBN, stage ^= 1) {
-    const bool more = k0 + LBN < t_end;
-    if (more) fetch(k0 + LBN);
-    __builtin_amdgcn_sched_barrier(0);     // what uses the fetched registers stays below the computation
-    if (wave_live && k0 <= wave_max) {
-      const bf16_t* ks = lds_kv + (int64_t)stage * LDS_TILE;
-      const bf16_t* vs = ks + LBN * KROW;
-#pragma unroll
-      for (int sub = 0; sub < LBN / 32; ++sub) {
-        const int kt = k0 + sub * 32;
-        if (kt > wave_max) break;
-        f32x4 s[NB][2];
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb) {
-          s[nb][0] = f32x4{0.f, 0.f, 0.f, 0.f};
-          s[nb][1] = f32x4{0.f, 0.f, 0.f, 0.f};
-        }
-#pragma unroll
-        for (int t = 0; t < 2; ++t)
-#pragma unroll
-          for (int kb = 0; kb < KB; ++kb) {
-            bf16x8 a = zero8();
-            if (kb * 32 + g * 8 < HD) a = load8(ks + (sub * 32 + t * 16 + c) * KROW + kb * 32 + g * 8);
-#pragma unroll
-            for (int nb = 0; nb < NB; ++nb)
-              s[nb][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qr[nb][kb], s[nb][t], 0, 0, 0);
-          }
-        const bool interior = kt >= full_lo && kt + 31 <= full_hi;
-        bf16x8 pb[NB];
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb) {
-          float sv[8];
-          float mx = -INFINITY;
-          if (interior && cpos[nb] >= 0) {
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-              sv[j] = s[nb][j >> 2][j & 3] * scale;
-              mx = fmaxf(mx, sv[j]);
-            }
-          } else {
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-              const int key = kt + 8 * g + j;
-              const bool valid = key >= clo[nb] && key <= cpos[nb];
-              sv[j] = valid ? s[nb][j >> 2][j & 3] * scale : -INFINITY;
-              mx = fmaxf(mx, sv[j]);
-            }
-          }
-          mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
-          mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
-          const float m_new = fmaxf(m[nb], mx);
-          float alpha = 1.f, sum = 0.f;
-          float p[8];
-          if (m_new == -INFINITY) {
-#pragma unroll
-            for (int j = 0; j < 8; ++j) p[j] = 0.f;
-          } else {
-            alpha = fast_exp2(m[nb] - m_new);
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-              p[j] = fast_exp2(sv[j] - m_new);
-              sum += p[j];
-            }
-          }
-          sum += __shfl_xor(sum, 16, WAVE);
-          sum += __shfl_xor(sum, 32, WAVE);
-          l[nb] = l[nb] * alpha + sum;
-          m[nb] = m_new;
-          if (__any(alpha != 1.f)) {
-#pragma unroll
-            for (int db = 0; db < DB; ++db) o[nb][db] *= alpha;
-          }
-#pragma unroll
-          for (int j = 0; j < 8; ++j) pb[nb][j] = (__bf16)p[j];
-        }
-#pragma unroll
-        for (int db = 0; db < DB; ++db) {
-          const bf16x8 a = load8(vs + (db * 16 + c) * VROW + sub * 32 + g * 8);
-#pragma unroll
-          for (int nb = 0; nb < NB; ++nb)
-            o[nb][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb[nb], o[nb][db], 0, 0, 0);
-        }
-      }
-    }
-    __builtin_amdgcn_sched_barrier(0);
-    if (more) stash(stage ^ 1, k0 + LBN);
-    __syncthreads();
-  }
-  if (!wave_live) return;
-#pragma unroll
-  for (int nb = 0; nb < NB; ++nb) {
-    const int j = wrow + nb * 16 + c;
-    if (j >= rows) continue;
-    const float inv = 1.f / l[nb];
-    bf16_t* op = out + (int64_t)(row0 + j) * out_stride + (int64_t)head * HD + g * 4;
-#pragma unroll
-    for (int db = 0; db < DB; ++db) {
-      union { uint2 u; bf16_t e[4]; } pk;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) pk.e[i] = f32_to_bf16(o[nb][db][i] * inv);
-      *reinterpret_cast<uint2*>(op + db * 16) = pk.u;
-    }
-  }
-}
-
-// how the wavefronts of an LDS-prefill workgroup are shared out: hpw heads (a divisor of the group, at
-// most 4) times rbw row blocks, 4 to 8 wavefronts in all
-static void lds_prefill_shape(int group, int* hpw, int* rbw) {
-  int h = 1;
-  for (int d = 2; d <= 4; ++d)
-    if (group % d == 0) h = d;
-  *hpw = h;
-  *rbw = h == 3 ? 2 : 8 / h > 4 ? 4 : 8 / h;
-}
-
-// the staging registers of the LDS kernel grow with the head size; beyond 128 the register kernel stands
-extern "C" int ga_attn_prefill_lds_supported() { return HD <= 128 ? 1 : 0; }
-
-extern "C" int ga_attn_prefill_lds_tile_rows(int nh, int nkv, int wide) {
-  int hpw, rbw;
-  lds_prefill_shape(nh / nkv, &hpw, &rbw);
-  return rbw * 16 * (wide ? PREFILL_NB : 1);
-}
-
-extern "C" int ga_attn_prefill_lds(void* out, int64_t out_stride, const void* q, int64_t q_stride,
-                                   const void* k_pages, const void* v_pages, const void* block_table,
-                                   int table_width, const void* tiles, int n_tiles, int wide, int nh, int nkv,
-                                   int page_size, int window, float scale, hipStream_t stream) {
-  if (n_tiles <= 0) return 0;
-  if (nkv <= 0 || nh % nkv) return -1;
-  if (HD > 128) return -9;
-  int ps_shift = 0;
-  while ((1 << ps_shift) < page_size) ++ps_shift;
-  if ((1 << ps_shift) != page_size || page_size < 8) return -2;
-  const int group = nh / nkv;
-  int hpw, rbw;
-  lds_prefill_shape(group, &hpw, &rbw);
-  const int head_blocks = group / hpw;
-  if ((int64_t)nkv * head_blocks > 65535) return -4;
-  const int nb = wide ? PREFILL_NB : 1;
-  if (table_width > 8192) return -10;        // the page ids of one request must fit beside the tiles in LDS
-  const size_t lds = (size_t)2 * LDS_TILE * sizeof(bf16_t) + (size_t)table_width * sizeof(int32_t);
-  dim3 grid(n_tiles, nkv * head_blocks), block(64 * hpw * rbw);
-  if (block.x < LDS_MIN_THREADS) return -8;
-  const void* fn = nb == 1 ? (const void*)attn_prefill_lds_kernel<1> : (const void*)attn_prefill_lds_kernel<PREFILL_NB>;
-  if (lds > 48 * 1024 && hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
-    return -7;
-#define LAUNCH(NB)                                                                                        \
-  hipLaunchKernelGGL(attn_prefill_lds_kernel<NB>, grid, block, lds, stream, (bf16_t*)out, out_stride,     \
-                     (const bf16_t*)q, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages,           \
-                     (const int32_t*)block_table, table_width, (const int32_t*)tiles, nh, nkv, head_blocks, \
-                     hpw, rbw, ps_shift, window, scale * LOG2E)
-  if (nb == 1) LAUNCH(1); else LAUNCH(PREFILL_NB);
-#undef LAUNCH
-  return GA_CHECK_LAUNCH();
-}
-
 extern "C" int ga_attn_head_dim() { return HD; }
 // rows of a prefill tile: 16 or (head sizes up to 128) 32
 extern "C" int ga_attn_prefill_max_tile_rows() { return 16 * PREFILL_NB; }

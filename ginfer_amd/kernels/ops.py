@@ -425,9 +425,6 @@ _DECODE_TARGET_WORKGROUPS = 256       # four wavefronts each, one workgroup per 
 _MIN_SPLIT_KEYS = 128                 # one tile of 32 keys for each wavefront of a workgroup
 _MAX_SPLITS = 256
 PREFILL_WIDE_TILES_FROM = 1024        # tokens in a step from which prompt rows go 32 to a wavefront
-# tokens in a step from which key tiles are shared through LDS: never, as measured on MI355X the
-# register kernel is as fast up to 8k-token prompts; the LDS kernel stays tested for longer ones
-PREFILL_LDS_FROM = 1 << 30
 
 
 def attention_mfma_supported(dtype, head_dim, page_size):
@@ -496,14 +493,9 @@ def paged_attention_mfma(q, k_pages, v_pages, block_table, step, num_heads, num_
     _need(q.stride(0) % 8 == 0 and q.data_ptr() % 16 == 0, "q rows must be 16-byte aligned")
     lib = build.load("attention_mfma", {"HEAD_DIM": head_dim})
     _need(lib.ga_attn_head_dim() == head_dim, "attention library was built for another head size")
-    # rows of a prompt portion per wavefront: 32 where the kernel has it and the step is long, else 16; long
-    # steps share each key tile among the wavefronts of a workgroup through LDS
+    # rows of a prompt portion per wavefront: 32 where the kernel has it and the step is long, else 16
     wide = T >= PREFILL_WIDE_TILES_FROM and lib.ga_attn_prefill_max_tile_rows() == 32
-    through_lds = T >= PREFILL_LDS_FROM and bool(lib.ga_attn_prefill_lds_supported()) and block_table.shape[1] <= 8192
-    if through_lds:
-        tile_rows = lib.ga_attn_prefill_lds_tile_rows(_i(num_heads), _i(num_kv_heads), _i(1 if wide else 0))
-    else:
-        tile_rows = 32 if wide else 16
+    tile_rows = 32 if wide else 16
     plan = _attention_plan(step, tile_rows, q.device)
     _need(sum(step.host_q_len) == T, "the step's entries do not add up to its tokens")
     if out is None:
@@ -520,12 +512,7 @@ def paged_attention_mfma(q, k_pages, v_pages, block_table, step, num_heads, num_
             _ptr(out), _i64(out.stride(0)), _ptr(q), _i64(q.stride(0)), _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
             _i(block_table.shape[1]), _ptr(plan["decode_info"]), _i(plan["n_decode"]), _i(num_heads), _i(num_kv_heads), _i(page_size), _i(w), _f(scale), _i(split_keys),
             _i(num_splits), _ptr(ws_o), _ptr(ws_ml), _stream()), "attn_decode")
-    if plan["n_tiles"] and through_lds:
-        _check(lib.ga_attn_prefill_lds(
-            _ptr(out), _i64(out.stride(0)), _ptr(q), _i64(q.stride(0)), _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
-            _i(block_table.shape[1]), _ptr(plan["tiles"]), _i(plan["n_tiles"]), _i(1 if wide else 0), _i(num_heads),
-            _i(num_kv_heads), _i(page_size), _i(w), _f(scale), _stream()), "attn_prefill_lds")
-    elif plan["n_tiles"]:
+    if plan["n_tiles"]:
         _check(lib.ga_attn_prefill(
             _ptr(out), _i64(out.stride(0)), _ptr(q), _i64(q.stride(0)), _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
             _i(block_table.shape[1]), _ptr(plan["tiles"]), _i(plan["n_tiles"]), _i(tile_rows), _i(num_heads), _i(num_kv_heads),

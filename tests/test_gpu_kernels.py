@@ -345,14 +345,13 @@ MFMA_SEQS = ATTN_SEQS + [[(1, 31), (1, 32), (1, 33), (1, 64), (1, 65)], [(31, 31
                          [(1, 5000)], [(300, 700)]]
 
 
-@pytest.mark.parametrize("wide,lds", [(False, False), (True, False), (False, True), (True, True)])
+@pytest.mark.parametrize("wide", [False, True])
 @pytest.mark.parametrize("nh,nkv,hd", ATTN_HEADS + [(40, 2, 64), (3, 1, 256), (18, 1, 16), (7, 1, 64), (8, 4, 256)])
 @pytest.mark.parametrize("seqs", MFMA_SEQS)
-def test_paged_attention_mfma(nh, nkv, hd, seqs, wide, lds, monkeypatch):
+def test_paged_attention_mfma(nh, nkv, hd, seqs, wide, monkeypatch):
     from ginfer_amd.kernels import ops
     monkeypatch.setattr(ops, "PREFILL_WIDE_TILES_FROM", 0 if wide else 1 << 30)    # 32 or 16 rows to a wavefront
-    monkeypatch.setattr(ops, "PREFILL_LDS_FROM", 0 if lds else 1 << 30)            # key tiles through LDS or not
-    if (wide or lds) and max(q for q, _ in seqs) == 1:
+    if wide and max(q for q, _ in seqs) == 1:
         pytest.skip("no prompt rows in this case")
     if sum(kv for _, kv in seqs) * nkv * hd > 3e6 and (nh, nkv, hd) not in ((12, 2, 128), (6, 1, 32)):
         pytest.skip("large case kept for two head shapes")
@@ -376,11 +375,11 @@ def test_paged_attention_mfma_every_head_size(hd, wide, monkeypatch):
     close(out, ref, 2e-2)
 
 
-@pytest.mark.parametrize("lds", [False, True])
+@pytest.mark.parametrize("wide", [False, True])
 @pytest.mark.parametrize("window", [1, 5, 16, 40, 64, 100])
-def test_paged_attention_mfma_window(window, lds, monkeypatch):
+def test_paged_attention_mfma_window(window, wide, monkeypatch):
     from ginfer_amd.kernels import ops
-    monkeypatch.setattr(ops, "PREFILL_LDS_FROM", 0 if lds else 1 << 30)
+    monkeypatch.setattr(ops, "PREFILL_WIDE_TILES_FROM", 0 if wide else 1 << 30)
     nh, nkv, hd, ps = 6, 3, 48, 16
     seqs = [(1, 200), (30, 90), (7, 7), (1, window), (1, window + 1), (50, 130), (1, 2000)]
     a, ref, _ = _paged_case(seqs, nh, nkv, hd, ps, torch.bfloat16, seed=window, window=window)
@@ -389,12 +388,12 @@ def test_paged_attention_mfma_window(window, lds, monkeypatch):
     close(out, ref, 2e-2)
 
 
-@pytest.mark.parametrize("lds", [False, True])
+@pytest.mark.parametrize("wide", [False, True])
 @pytest.mark.parametrize("where", ["first", "page_edge", "before_page_edge", "tile_edge", "before_tile_edge", "split_edge",
                                    "last", "window_edge", "behind_window"])
-def test_paged_attention_mfma_finds_one_far_key(where, lds, monkeypatch):
+def test_paged_attention_mfma_finds_one_far_key(where, wide, monkeypatch):
     from ginfer_amd.kernels import ops
-    monkeypatch.setattr(ops, "PREFILL_LDS_FROM", 0 if lds else 1 << 30)
+    monkeypatch.setattr(ops, "PREFILL_WIDE_TILES_FROM", 0 if wide else 1 << 30)
     nh, nkv, hd, ps = 4, 2, 32, 16
     kv = 300
     window = 100 if "window" in where else None
