@@ -41,6 +41,8 @@ constexpr int PREFILL_NB = HD <= 128 ? 2 : 1;
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(2))) float f32x2;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
 
 // The kernels keep scores, running maxima and the maxima of partial results in units of log2(e): the
 // launchers multiply the score scale by LOG2E once, and every exponential is a bare exp2.
@@ -191,21 +193,22 @@ __device__ __forceinline__ void attend_tiles(f32x4 (&o)[NB][DB], float (&m)[NB],
         }
         m[nb] = m_new;
       }
+      // A column that has seen no key yet has m == -inf and only dead keys (-inf) in this tile: with 0 in
+      // place of m every exponent is -inf and every p is 0, without a branch.
+      const float m_use = m[nb] == -INFINITY ? 0.f : m[nb];
       float sum = 0.f;
       float p[8];
-      if (m[nb] == -INFINITY) {            // the column has seen no key yet
 #pragma unroll
-        for (int j = 0; j < 8; ++j) p[j] = 0.f;
-      } else {
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          p[j] = fast_exp2(__builtin_fmaf(sv[j], scale, -m[nb]));
-          sum += p[j];
-        }
+      for (int j = 0; j < 8; ++j) {
+        p[j] = fast_exp2(__builtin_fmaf(sv[j], scale, -m_use));
+        sum += p[j];
       }
       l[nb] += sum;
+      // two values to a conversion (v_cvt_pk_bf16_f32), round to nearest even
+      union { bf16x8 v; bf16x2 h[4]; } packed;
 #pragma unroll
-      for (int j = 0; j < 8; ++j) pb[nb][j] = (__bf16)p[j];
+      for (int j = 0; j < 4; ++j) packed.h[j] = __builtin_convertvector(f32x2{p[2 * j], p[2 * j + 1]}, bf16x2);
+      pb[nb] = packed.v;
     }
     // ---- output: O^T += V^T P.  In a tile that reaches past the ends of the key range the values read
     // for dead keys (anything: the slot may never have been written) are cleared: 0 * NaN is not 0.
