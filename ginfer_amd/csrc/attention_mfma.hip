@@ -38,6 +38,17 @@ constexpr int HD = HEAD_DIM;
 constexpr int KB = (HD + 31) / 32;   // 32-dim blocks of the q.k product (the last may be half empty)
 constexpr int DB = HD / 16;          // 16-dim blocks of the output
 constexpr int PREFILL_NB = HD <= 128 ? 2 : 1;
+// Measured on MI355X (12 heads in 2 groups, head size 128, prompts of 2k to 16k tokens): workgroups of 8
+// wavefronts with one set of key and value registers in flight are fastest (66 us at 2k, 530 us at 8k).  4
+// wavefronts (one per SIMD, 512 registers each) take 78 and 638 us, with one set or two: the loads' latency is
+// not what the kernel waits for; its vector instructions (softmax) take 1.7 times the issue time of its matrix
+// products, and two wavefronts per SIMD overlap the two.
+#ifndef PREFILL_DEPTH
+#define PREFILL_DEPTH 1              // sets of key and value registers in flight in the prefill kernel
+#endif
+#ifndef PREFILL_WAVES
+#define PREFILL_WAVES 8              // wavefronts of a prefill workgroup
+#endif
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
@@ -106,13 +117,120 @@ __device__ __forceinline__ void load_v_tile(bf16x8 (&vr)[DB], const bf16_t* __re
   for (int db = 0; db < DB; ++db) vr[db] = load8(vp + (int64_t)db * 16 * ps);
 }
 
+// One tile of 32 keys starting at k0, with its operands in kr and vr: scores, online softmax, output.  As soon
+// as the products that read kr (then vr) have been issued the registers are refilled with the tile k_refill
+// (< 0: none), whose pages pg holds; after that pg takes the pages of the tile k_lookup (< 0: none).
+template <int NB>
+__device__ __forceinline__ void attend_one_tile(f32x4 (&o)[NB][DB], float (&m)[NB], float (&l)[NB],
+                                                const bf16x8 (&q)[NB][KB], const int (&cpos)[NB],
+                                                const int (&clo)[NB], bf16x8 (&kr)[2][KB], bf16x8 (&vr)[DB],
+                                                TilePages& pg, const bf16_t* __restrict__ k_pages,
+                                                const bf16_t* __restrict__ v_pages,
+                                                const int32_t* __restrict__ bt, int kvh, int nkv, int ps_shift,
+                                                int kv_min, int kv_max, int full_lo, int full_hi, int k0,
+                                                int k_refill, int k_lookup, float scale, int c, int g) {
+  // ---- scores: S^T = K Q^T
+  f32x4 s[NB][2];
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) {
+    s[nb][0] = f32x4{0.f, 0.f, 0.f, 0.f};
+    s[nb][1] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+#pragma unroll
+  for (int t = 0; t < 2; ++t)
+#pragma unroll
+    for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+        s[nb][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kr[t][kb], q[nb][kb], s[nb][t], 0, 0, 0);
+  if (k_refill >= 0) load_k_tile(kr, k_pages, pg, kvh, nkv, ps_shift, k_refill, c, g);
+  // ---- mask and online softmax; the lane holds keys k0 + 8g + j, j = 0..7, of column c.  The running
+  // max is kept in scaled units; the scale rides on the exponent's multiply-add.
+  const bool interior = k0 >= full_lo && k0 + 31 <= full_hi;      // the same for the whole wavefront
+  bf16x8 pb[NB];
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) {
+    float sv[8];
+    float mx = -INFINITY;
+    if (interior && cpos[nb] >= 0) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        sv[j] = s[nb][j >> 2][j & 3];
+        mx = fmaxf(mx, sv[j]);
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int key = k0 + 8 * g + j;
+        const bool valid = key >= clo[nb] && key <= cpos[nb];
+        sv[j] = valid ? s[nb][j >> 2][j & 3] : -INFINITY;      // a select: what was read for a dead key is dropped
+        mx = fmaxf(mx, sv[j]);
+      }
+    }
+    // The running max is raised lazily: only when some score of the tile exceeds it by more than
+    // LAZY_MAX (in log2 units), which after the first tiles is rare.  Until then exponentials may reach
+    // 2^LAZY_MAX, harmless in 32-bit sums, and the tile costs no exchange between lanes: the four lanes
+    // of a column keep partial sums of their own keys (added up once, by finish_sums, after the loop).
+    if (__any(mx * scale > m[nb] + LAZY_MAX)) {
+      mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+      const float m_new = fmaxf(m[nb], mx * scale);
+      if (m_new != -INFINITY) {
+        const float alpha = fast_exp2(m[nb] - m_new);      // exp2(-inf) = 0 the first time
+        l[nb] *= alpha;
+#pragma unroll
+        for (int db = 0; db < DB; ++db) o[nb][db] *= alpha;
+      }
+      m[nb] = m_new;
+    }
+    // A column that has seen no key yet has m == -inf and only dead keys (-inf) in this tile: with 0 in
+    // place of m every exponent is -inf and every p is 0, without a branch.
+    const float m_use = m[nb] == -INFINITY ? 0.f : m[nb];
+    float sum = 0.f;
+    float p[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      p[j] = fast_exp2(__builtin_fmaf(sv[j], scale, -m_use));
+      sum += p[j];
+    }
+    l[nb] += sum;
+    // two values to a conversion (v_cvt_pk_bf16_f32), round to nearest even
+    union { bf16x8 v; bf16x2 h[4]; } packed;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) packed.h[j] = __builtin_convertvector(f32x2{p[2 * j], p[2 * j + 1]}, bf16x2);
+    pb[nb] = packed.v;
+  }
+  // ---- output: O^T += V^T P.  In a tile that reaches past the ends of the key range the values read
+  // for dead keys (anything: the slot may never have been written) are cleared: 0 * NaN is not 0.
+  if (k0 < kv_min || k0 + 31 > kv_max) {
+    const int kbase = k0 + 8 * g;
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+      union { bf16x8 v; bf16_t e[8]; } u;
+      u.v = vr[db];
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        if (kbase + j < kv_min || kbase + j > kv_max) u.e[j] = 0;
+      vr[db] = u.v;
+    }
+  }
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb)
+      o[nb][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vr[db], pb[nb], o[nb][db], 0, 0, 0);
+  if (k_refill >= 0) load_v_tile(vr, v_pages, pg, kvh, nkv, ps_shift, k_refill, c, g);
+  if (k_lookup >= 0) lookup_pages(pg, bt, ps_shift, kv_min, kv_max, k_lookup, c, g);
+}
+
 // Attends columns to the key tiles tile_begin, tile_begin + tile_stride, ... < tile_end (multiples of 32).
 // kv_min..kv_max is the inclusive range of keys that any column of the wavefront may see; full_lo..full_hi
-// the range that EVERY live column sees (tiles inside it need no mask).  The loop is software-pipelined:
-// page ids are looked up a tile before they are needed, and the keys and values of tile i+1 are requested
-// right after the products of tile i that free their registers, so that no load waits for a look-up and
-// each has most of a tile's matrix products and softmax to arrive in.
-template <int NB>
+// the range that EVERY live column sees (tiles inside it need no mask).  The loop is software-pipelined
+// DEPTH tiles deep: DEPTH sets of operand registers are filled ahead, each refilled with the tile DEPTH
+// further on as soon as the products that read it have been issued, and the pages of a tile are looked up
+// DEPTH tiles before its loads; so no load waits for a look-up and each has (nearly) DEPTH tiles' products and
+// softmax to arrive in.  DEPTH 2 costs a second set of registers.
+template <int NB, int DEPTH>
 __device__ __forceinline__ void attend_tiles(f32x4 (&o)[NB][DB], float (&m)[NB], float (&l)[NB],
                                              const bf16x8 (&q)[NB][KB], const int (&cpos)[NB],
                                              const int (&clo)[NB], const bf16_t* __restrict__ k_pages,
@@ -120,119 +238,35 @@ __device__ __forceinline__ void attend_tiles(f32x4 (&o)[NB][DB], float (&m)[NB],
                                              const int32_t* __restrict__ bt, int kvh, int nkv, int ps_shift,
                                              int kv_min, int kv_max, int full_lo, int full_hi, int tile_begin,
                                              int tile_end, int tile_stride, float scale) {
+  static_assert(DEPTH == 1 || DEPTH == 2, "one or two sets of operand registers");
   const int lane = threadIdx.x & 63, c = lane & 15, g = lane >> 4;
   if (tile_begin >= tile_end) return;
-  // pg_nxt: pages of the tile after the current one; they are looked up a whole tile before the loads
-  // that need them are issued.  kr and vr hold the operands of the CURRENT tile at the top of the loop;
-  // each is refilled with the next tile's as soon as its matrix products have been issued, so every load
-  // has most of a tile's work to arrive in, and no operand is held twice.
-  TilePages pg_nxt;
-  bf16x8 kr[2][KB], vr[DB];
-  {
-    TilePages pg;
-    lookup_pages(pg, bt, ps_shift, kv_min, kv_max, tile_begin, c, g);
-    load_k_tile(kr, k_pages, pg, kvh, nkv, ps_shift, tile_begin, c, g);
-    load_v_tile(vr, v_pages, pg, kvh, nkv, ps_shift, tile_begin, c, g);
-    pg_nxt = pg;
-    if (tile_begin + tile_stride < tile_end)
-      lookup_pages(pg_nxt, bt, ps_shift, kv_min, kv_max, tile_begin + tile_stride, c, g);
+  TilePages pg[DEPTH];
+  bf16x8 kr[DEPTH][2][KB], vr[DEPTH][DB];
+#pragma unroll
+  for (int d = 0; d < DEPTH; ++d) {
+    const int k0 = tile_begin + d * tile_stride;
+    if (k0 < tile_end) {
+      lookup_pages(pg[d], bt, ps_shift, kv_min, kv_max, k0, c, g);
+      load_k_tile(kr[d], k_pages, pg[d], kvh, nkv, ps_shift, k0, c, g);
+      load_v_tile(vr[d], v_pages, pg[d], kvh, nkv, ps_shift, k0, c, g);
+    }
   }
-  for (int k0 = tile_begin; k0 < tile_end; k0 += tile_stride) {
-    const bool more = k0 + tile_stride < tile_end;
-    // ---- scores: S^T = K Q^T
-    f32x4 s[NB][2];
 #pragma unroll
-    for (int nb = 0; nb < NB; ++nb) {
-      s[nb][0] = f32x4{0.f, 0.f, 0.f, 0.f};
-      s[nb][1] = f32x4{0.f, 0.f, 0.f, 0.f};
-    }
+  for (int d = 0; d < DEPTH; ++d) {
+    const int k0 = tile_begin + (DEPTH + d) * tile_stride;
+    if (k0 < tile_end) lookup_pages(pg[d], bt, ps_shift, kv_min, kv_max, k0, c, g);
+  }
+  for (int kbase = tile_begin; kbase < tile_end; kbase += DEPTH * tile_stride) {
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
-#pragma unroll
-      for (int kb = 0; kb < KB; ++kb)
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb)
-          s[nb][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kr[t][kb], q[nb][kb], s[nb][t], 0, 0, 0);
-    if (more) load_k_tile(kr, k_pages, pg_nxt, kvh, nkv, ps_shift, k0 + tile_stride, c, g);
-    // ---- mask and online softmax; the lane holds keys k0 + 8g + j, j = 0..7, of column c.  The running
-    // max is kept in scaled units; the scale rides on the exponent's multiply-add.
-    const bool interior = k0 >= full_lo && k0 + 31 <= full_hi;      // the same for the whole wavefront
-    bf16x8 pb[NB];
-#pragma unroll
-    for (int nb = 0; nb < NB; ++nb) {
-      float sv[8];
-      float mx = -INFINITY;
-      if (interior && cpos[nb] >= 0) {
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          sv[j] = s[nb][j >> 2][j & 3];
-          mx = fmaxf(mx, sv[j]);
-        }
-      } else {
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          const int key = k0 + 8 * g + j;
-          const bool valid = key >= clo[nb] && key <= cpos[nb];
-          sv[j] = valid ? s[nb][j >> 2][j & 3] : -INFINITY;      // a select: what was read for a dead key is dropped
-          mx = fmaxf(mx, sv[j]);
-        }
+    for (int d = 0; d < DEPTH; ++d) {
+      const int k0 = kbase + d * tile_stride;
+      if (k0 < tile_end) {                    // the same for the whole wavefront
+        const int k_refill = k0 + DEPTH * tile_stride, k_lookup = k0 + 2 * DEPTH * tile_stride;
+        attend_one_tile<NB>(o, m, l, q, cpos, clo, kr[d], vr[d], pg[d], k_pages, v_pages, bt, kvh, nkv, ps_shift, kv_min,
+                            kv_max, full_lo, full_hi, k0, k_refill < tile_end ? k_refill : -1,
+                            k_lookup < tile_end ? k_lookup : -1, scale, c, g);
       }
-      // The running max is raised lazily: only when some score of the tile exceeds it by more than
-      // LAZY_MAX (in log2 units), which after the first tiles is rare.  Until then exponentials may reach
-      // 2^LAZY_MAX, harmless in 32-bit sums, and the tile costs no exchange between lanes: the four lanes
-      // of a column keep partial sums of their own keys (added up once, by finish_sums, after the loop).
-      if (__any(mx * scale > m[nb] + LAZY_MAX)) {
-        mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
-        mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
-        const float m_new = fmaxf(m[nb], mx * scale);
-        if (m_new != -INFINITY) {
-          const float alpha = fast_exp2(m[nb] - m_new);      // exp2(-inf) = 0 the first time
-          l[nb] *= alpha;
-#pragma unroll
-          for (int db = 0; db < DB; ++db) o[nb][db] *= alpha;
-        }
-        m[nb] = m_new;
-      }
-      // A column that has seen no key yet has m == -inf and only dead keys (-inf) in this tile: with 0 in
-      // place of m every exponent is -inf and every p is 0, without a branch.
-      const float m_use = m[nb] == -INFINITY ? 0.f : m[nb];
-      float sum = 0.f;
-      float p[8];
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        p[j] = fast_exp2(__builtin_fmaf(sv[j], scale, -m_use));
-        sum += p[j];
-      }
-      l[nb] += sum;
-      // two values to a conversion (v_cvt_pk_bf16_f32), round to nearest even
-      union { bf16x8 v; bf16x2 h[4]; } packed;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) packed.h[j] = __builtin_convertvector(f32x2{p[2 * j], p[2 * j + 1]}, bf16x2);
-      pb[nb] = packed.v;
-    }
-    // ---- output: O^T += V^T P.  In a tile that reaches past the ends of the key range the values read
-    // for dead keys (anything: the slot may never have been written) are cleared: 0 * NaN is not 0.
-    if (k0 < kv_min || k0 + 31 > kv_max) {
-      const int kbase = k0 + 8 * g;
-#pragma unroll
-      for (int db = 0; db < DB; ++db) {
-        union { bf16x8 v; bf16_t e[8]; } u;
-        u.v = vr[db];
-#pragma unroll
-        for (int j = 0; j < 8; ++j)
-          if (kbase + j < kv_min || kbase + j > kv_max) u.e[j] = 0;
-        vr[db] = u.v;
-      }
-    }
-#pragma unroll
-    for (int db = 0; db < DB; ++db)
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb)
-        o[nb][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vr[db], pb[nb], o[nb][db], 0, 0, 0);
-    if (more) {
-      load_v_tile(vr, v_pages, pg_nxt, kvh, nkv, ps_shift, k0 + tile_stride, c, g);
-      if (k0 + 2 * tile_stride < tile_end)
-        lookup_pages(pg_nxt, bt, ps_shift, kv_min, kv_max, k0 + 2 * tile_stride, c, g);
     }
   }
 }
@@ -304,7 +338,7 @@ __global__ __launch_bounds__(64 * DEC_WAVES) void attn_decode_split_kernel(
     const int cpos[1] = {col_ok ? pos : -1}, clo[1] = {lo};
     const int32_t* bt = block_table + (int64_t)info.z * table_width;
     // every live column of a decode wavefront sees the same keys: lo..pos
-    attend_tiles<1>(o, m, l, qr, cpos, clo, k_pages, v_pages, bt, kvh, nkv, ps_shift, lo, pos, lo, pos,
+    attend_tiles<1, 1>(o, m, l, qr, cpos, clo, k_pages, v_pages, bt, kvh, nkv, ps_shift, lo, pos, lo, pos,
                     begin + 32 * wave, end, 32 * DEC_WAVES, scale);
     finish_sums<1>(l);
   }
@@ -396,7 +430,7 @@ __global__ __launch_bounds__(64) void attn_decode_combine_kernel(
 // states of a head's wavefronts meet in LDS: wavefront 0 of the head merges and writes the rows.
 // tiles: int32 [n][4] = (entry, first token row of the step, rows (<= 16*NB), first position).
 template <int NB>
-__global__ __launch_bounds__(512) void attn_prefill_kernel(
+__global__ __launch_bounds__(64 * PREFILL_WAVES) void attn_prefill_kernel(
     bf16_t* __restrict__ out, int64_t out_stride, const bf16_t* __restrict__ q, int64_t q_stride,
     const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
     const int32_t* __restrict__ block_table, int table_width, const int32_t* __restrict__ tiles, int nh,
@@ -430,7 +464,7 @@ __global__ __launch_bounds__(512) void attn_prefill_kernel(
     const int kv_max = pos0 + rows - 1;
     // every row of the tile sees the keys from the last row's window start up to the first row's position
     const int full_lo = (window > 0 && kv_max - window + 1 > 0) ? kv_max - window + 1 : 0;
-    attend_tiles<NB>(o, m, l, qr, cpos, clo, k_pages, v_pages, block_table + (int64_t)entry * table_width, kvh,
+    attend_tiles<NB, PREFILL_DEPTH>(o, m, l, qr, cpos, clo, k_pages, v_pages, block_table + (int64_t)entry * table_width, kvh,
                      nkv, ps_shift, kv_min, kv_max, full_lo, pos0, (kv_min / 32) * 32 + 32 * split,
                      (kv_max / 32 + 1) * 32, 32 * splits, scale);
     finish_sums<NB>(l);
@@ -544,7 +578,7 @@ extern "C" int ga_attn_prefill(void* out, int64_t out_stride, const void* q, int
   int hpw = 1;
   for (int d = 2; d <= 4; ++d)
     if (group % d == 0 && (int64_t)n_tiles * nkv * (group / d) >= 256) hpw = d;
-  int splits = 8 / hpw;
+  int splits = PREFILL_WAVES / hpw;
   if (hpw > 1 && splits > 4) splits = 4;
   const int head_blocks = group / hpw;
   if ((int64_t)nkv * head_blocks > 65535) return -4;
