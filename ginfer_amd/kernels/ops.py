@@ -494,8 +494,8 @@ def paged_attention_mfma(q, k_pages, v_pages, block_table, step, num_heads, num_
     lib = build.load("attention_mfma", {"HEAD_DIM": head_dim})
     _need(lib.ga_attn_head_dim() == head_dim, "attention library was built for another head size")
     # rows of a prompt portion per wavefront: 32 where the kernel has it and the step is long, else 16
-    wide = T >= PREFILL_WIDE_TILES_FROM and lib.ga_attn_prefill_max_tile_rows() == 32
-    tile_rows = 32 if wide else 16
+    wide = T >= PREFILL_WIDE_TILES_FROM
+    tile_rows = lib.ga_attn_prefill_max_tile_rows() if wide else 16
     plan = _attention_plan(step, tile_rows, q.device)
     _need(sum(step.host_q_len) == T, "the step's entries do not add up to its tokens")
     if out is None:
