@@ -23,6 +23,10 @@ SHAPE = dict(architectures=["Qwen2ForCausalLM"], model_type="qwen2", num_hidden_
              rope_theta=10000.0, rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=131072,
              use_sliding_window=False, sliding_window=4096, max_window_layers=21)
 FULL_LAYERS = 28
+# a larger shape of the same architecture, for looking at the kernels at other sizes (--shape 7b): Qwen2-7B's sizes
+SHAPE_7B = dict(SHAPE, hidden_size=3584, num_attention_heads=28, num_key_value_heads=4, intermediate_size=18944,
+                vocab_size=152064, rope_theta=1e6, max_position_embeddings=32768, max_window_layers=28)
+SHAPES = {"1.5b": ("qwen2-1.5b-shape", SHAPE), "7b": ("qwen2-7b-shape", SHAPE_7B)}
 HBM_PEAK = 8.0e12            # bytes/s, MI355X HBM3E
 PEAK_FLOPS = {"bf16": 2.5e15, "fp16": 2.5e15, "fp8": 5.0e15, "fp32": 157.3e12}   # dense matrix peaks
 
@@ -53,6 +57,7 @@ def main():
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--points", default="1,64", help="other decode batch sizes to report")
     ap.add_argument("--model-dir", default=None, help="reuse a model folder written earlier")
+    ap.add_argument("--shape", default="1.5b", choices=sorted(SHAPES), help="layer sizes (the headline is 1.5b)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this engine runs on ONE GPU; --gpus %d is not supported" % args.gpus)
@@ -62,7 +67,8 @@ def main():
     from ginfer_amd import ModelRunner, StepEntry, config_from_dict, write_random_model
     from ginfer_amd.sampling import Sampler, SamplingParams
 
-    cfg = dict(SHAPE, num_hidden_layers=args.layers)
+    shape_name, shape = SHAPES[args.shape]
+    cfg = dict(shape, num_hidden_layers=args.layers)
     weight_bytes, kv_per_token, prefill_flops = model_numbers(cfg, args.layers)
     tmp = None
     folder = args.model_dir
@@ -140,11 +146,11 @@ def main():
     step_bytes = weight_bytes + args.batch * mean_ctx * kv_per_token
     achieved = step_bytes / dt / 1e9
     out = {
-        "metric": "decode tok/s at batch %d (Qwen2 1.5B shape, context %d)" % (args.batch, args.context),
+        "metric": "decode tok/s at batch %d (Qwen2 %s shape, context %d)" % (args.batch, args.shape.upper(), args.context),
         "value": round(args.batch / dt, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(dt * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic tokens, random weights N(0, 0.02)",
-        "config": {"model": "qwen2-1.5b-shape", "global_batch": args.batch, "seq_len": args.context,
+        "config": {"model": shape_name, "global_batch": args.batch, "seq_len": args.context,
                    "parallelism": "single-gpu", "layers": args.layers, "layers_full": FULL_LAYERS,
                    "hidden_size": cfg["hidden_size"], "num_attention_heads": cfg["num_attention_heads"],
                    "num_key_value_heads": cfg["num_key_value_heads"], "head_dim": cfg["head_dim"],

@@ -11,7 +11,7 @@ import torch
 from ..kernels import ops
 
 
-# a product with at least this many input features whose consumer adds partial sums is split over K
+# from this many input features on, a product is "long": a folded norm gives way to a split over workgroups
 SPLIT_K_FROM = 4096
 MAX_SPLIT_K_PARTS = 16
 # a folded norm keeps K within a workgroup; measured on MI355X, a product with a long K still gains from
@@ -32,15 +32,10 @@ def linear(x, weight, bias=None, out_dtype=None, parts_ok=False):
         # 16-row tile of W per wavefront streams best; beyond, four tiles halve the re-reading of x; a
         # long K is split over workgroups where the consumer can add the parts
         many = x.shape[0] > 16
-        if parts_ok and out_dtype is None and x.shape[1] >= SPLIT_K_FROM:
-            # enough parts that a wavefront's share of K is one trip of loads (4 steps of 64 with one tile,
-            # 2 with four), and a tenth more, which was measured faster than an exact fit
-            per_trip = 2 if many else 4
-            steps = -(-x.shape[1] // 64)
-            splits = min(MAX_SPLIT_K_PARTS, max(2, -(-steps * 11 // (10 * 8 * per_trip))))
-            return ops.gemm_skinny(x, weight, bias, out_dtype=torch.float32, nt=4 if many else 1, grid_splits=splits)
         if parts_ok and out_dtype is None and x.shape[1] >= 1024:
-            return ops.gemm_skinny(x, weight, bias, out_dtype=torch.float32, nt=1, grid_splits=2)
+            nt, splits = _split_plan(x.shape[0], weight.shape[0], x.shape[1])
+            if splits > 1:
+                return ops.gemm_skinny(x, weight, bias, out_dtype=torch.float32, nt=nt, grid_splits=splits)
         return ops.gemm_skinny(x, weight, bias, out_dtype=out_dtype, nt=4 if (many and weight.shape[0] >= 4096) else 1)
     if parts_ok and out_dtype is None and bias is None:
         parts = _library_split(x.shape[0], weight.shape[0], x.shape[1])
@@ -60,6 +55,32 @@ def linear(x, weight, bias=None, out_dtype=None, parts_ok=False):
     if bias is not None:
         return torch.addmm(bias, x, weight.t())
     return torch.mm(x, weight.t())
+
+
+def _split_plan(rows, out_features, in_features):
+    """(tiles of W per wavefront, parts of K) for a product whose consumer adds partial sums.  Measured on
+    MI355X at the sizes of a 1.5B and a 7B model: the kernel wants some 250 workgroups with four tiles per
+    wavefront (more than 16 rows, and enough columns) or some 500 with one, and parts of equal length: the count
+    of parts divides K's steps of 64 (down projection of the 1.5B shape at 64 rows: 10 parts 14 us, 11 parts
+    23 us).  That gives 10 parts at 64 rows and 5 at 8 for the 1.5B shape's down projection, 4 for the 7B
+    shape's; a product with a short K and few columns keeps 2 parts."""
+    steps = -(-in_features // 64)
+    cap = max(1, min(MAX_SPLIT_K_PARTS, steps // 8))       # parts that leave every wavefront a step
+    tiles4 = -(-out_features // 64)
+    if rows > 16 and tiles4 * cap >= 192:
+        return 4, _nearest_divisor(steps, 256.0 / tiles4, cap)
+    if in_features < SPLIT_K_FROM:
+        return 1, min(2, cap)
+    return 1, _nearest_divisor(steps, 512.0 / -(-out_features // 16), cap)
+
+
+def _nearest_divisor(n, target, cap):
+    """The divisor of n in 1..cap nearest to target (the smaller of two equally near)."""
+    best = 1
+    for d in range(1, cap + 1):
+        if n % d == 0 and abs(d - target) < abs(best - target):
+            best = d
+    return best
 
 
 def _library_is_faster(rows, out_features):
