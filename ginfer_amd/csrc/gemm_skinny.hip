@@ -301,14 +301,17 @@ struct GaSkinnyNorm {
   float* out_sumsq;        // [M][ga_skinny_norm_parts(M, N)]
 };
 
-// Tiles of a product of M rows when the caller leaves the choice to the library: packed whenever they can be
-// (measured on MI355X: up to a third faster where a product has few columns; ga_gemm_skinny leaves products
-// with many workgroups as they are: the head, and the gated product, which was measured slower packed).
-static int auto_pack(int M) { return M <= 8 ? 2 : 1; }
+// Tiles of a product of M rows when the caller leaves the choice to the library: packed where they can be and
+// full tiles would make fewer than 192 workgroups.  Measured on MI355X: a third faster where a product has few
+// columns (1536: 96 workgroups of full tiles); no gain or a loss from 224 workgroups on (down projection of a 7B
+// shape at 8 rows: 35 us with full tiles, 44 packed); the gated product was measured slower packed.
+static int auto_pack(int M, int workgroups_of_full_tiles) {
+  return (M <= 8 && workgroups_of_full_tiles < 192) ? 2 : 1;
+}
 
 // Partial sums a row gets from a product of M rows and N columns that feeds a norm.
 extern "C" int ga_skinny_norm_parts(int M, int N) {
-  const int cp = 16 / auto_pack(M);
+  const int cp = 16 / auto_pack(M, (N + 15) / 16);
   return (N + cp - 1) / cp;
 }
 
@@ -333,7 +336,7 @@ extern "C" int ga_gemm_skinny(void* C, int64_t ldc, const void* A, int64_t lda, 
     if (mb != 1 || gated || grid_splits != 1 || !norm->gain || !norm->scaled || !norm->out_sumsq) return -6;
     nt = 1;
     ks = SK_WAVES;
-    pack = auto_pack(M);          // what ga_skinny_norm_parts promised
+    pack = auto_pack(M, (N + 15) / 16);          // what ga_skinny_norm_parts promised
     norm_out = NormOut{norm->residual, norm->ldr, norm->gain, norm->gain_f32, (bf16_t*)norm->scaled, norm->lds,
                        norm->out_sumsq};
   }
@@ -345,7 +348,7 @@ extern "C" int ga_gemm_skinny(void* C, int64_t ldc, const void* A, int64_t lda, 
   if (grid_splits > 1 && !out_f32) return -3;
   if (gated && (grid_splits > 1 || bias)) return -4;
   const int groups = SK_WAVES / ks;
-  if (pack == 0) pack = (grid_splits == 1 && !gated && N / (groups * nt * 16) <= 1024) ? auto_pack(M) : 1;
+  if (pack == 0) pack = (grid_splits == 1 && !gated) ? auto_pack(M, (N + groups * nt * 16 - 1) / (groups * nt * 16)) : 1;
   if (pack != 1 && (pack != 2 || M > 8)) return -2;
   const int cp = 16 / pack;
   const int ncol = gated ? cp : nt * cp;
@@ -563,7 +566,7 @@ extern "C" int ga_qkv_rope_skinny(void* q_out, const void* A, int64_t lda, const
     if (mb != 1 || norm->in_parts < 1 || norm->in_parts > NORM_IN_MAX_PARTS) return -5;
     norm_in = NormIn{norm->in_sumsq, norm->in_parts, norm->inv_width, norm->eps};
   }
-  if (pack == 0) pack = auto_pack(M);
+  if (pack == 0) pack = auto_pack(M, (nh + 2 * nkv) * hd / 32);
   if (pack != 1 && (pack != 2 || M > 8)) return -2;
   const int ks = 8, groups = SK_WAVES / ks;
   // with more than 8 rows and so few columns that full tiles leave most of the chip idle: half tiles (measured on

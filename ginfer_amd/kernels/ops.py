@@ -298,7 +298,7 @@ def folded_norm_supported(a, w, residual, gain):
     x = a.scaled if isinstance(a, ScaledRows) else a
     N = w.shape[0]
     return (gemm_skinny_supported(x, w) and x.shape[0] <= FOLDED_NORM_MAX_ROWS and N % 8 == 0
-            and N <= (8 if x.shape[0] <= 8 else 16) * 512
+            and build.load("gemm_skinny").ga_skinny_norm_parts(_i(x.shape[0]), _i(N)) <= 512
             and residual.dtype == torch.float32 and residual.shape == (x.shape[0], N) and residual.stride(1) == 1
             and gain.dtype in (torch.bfloat16, torch.float32) and gain.shape == (N,) and gain.is_contiguous())
 
@@ -329,7 +329,7 @@ def gemm_skinny(a, w, bias=None, out=None, out_dtype=None, nt=0, ks=0, grid_spli
         residual, gain, eps = into_norm
         _need(folded_norm_supported(a, w, residual, gain) and not gated and grid_splits == 1 and out is None,
               "a product folds the norm after it for at most %d bfloat16 rows, a float32 residual [M, N] and a "
-              "gain [N], N a multiple of 8 up to 4096 (8192 from 9 rows on)" % FOLDED_NORM_MAX_ROWS)
+              "gain [N], N a multiple of 8 with at most 512 partial sums a row" % FOLDED_NORM_MAX_ROWS)
         _dev(residual, gain)
         norm = norm or _SkinnyNorm()
         M, N = residual.shape

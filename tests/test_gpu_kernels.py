@@ -489,7 +489,7 @@ def test_gemm_skinny_gated(M, I, K):
 @pytest.mark.parametrize("M", [1, 3, 8, 16])
 @pytest.mark.parametrize("N,K,bias,gain_dtype", [(1536, 1536, False, torch.bfloat16), (1536, 8960, False, torch.float32),
                                                  (88, 136, True, torch.bfloat16), (200, 64, True, torch.float32),
-                                                 (4096, 72, False, torch.bfloat16)])
+                                                 (4096, 72, False, torch.bfloat16), (8192, 136, False, torch.bfloat16)])
 def test_gemm_skinny_folds_the_norm_after_it(M, N, K, bias, gain_dtype):
     """The product that adds itself to the residual and hands on the norm's rows in two factors, and the
     products that take such rows: together they equal add, norm, product."""
@@ -509,7 +509,8 @@ def test_gemm_skinny_folds_the_norm_after_it(M, N, K, bias, gain_dtype):
     normed = pm.rms_norm(h, gain.double(), eps)
     close(rows.rows(), normed, 1e-2)
     # the partial sums come from the 32-bit residual that was written, column block by column block
-    cols = 8 if M <= 8 else 16
+    cols = 8 if rows.sumsq.shape[1] == -(-N // 8) else 16
+    assert rows.sumsq.shape[1] == -(-N // cols)
     parts = torch.stack([(res[:, c:c + cols].double() ** 2).sum(dim=1) for c in range(0, N, cols)], dim=1)
     close(rows.sumsq, parts, 1e-6)
     # products that take the rows: plain, gated, and the fused q|k|v projection
@@ -537,7 +538,7 @@ def test_gemm_skinny_folds_the_norm_after_it(M, N, K, bias, gain_dtype):
     if M > 1:
         res1 = res0[M - 1:M].clone()
         alone = ops.gemm_skinny(a[M - 1:M], w, b, into_norm=(res1, gain, eps))
-        if M <= 8:       # the same tiling: bit for bit
+        if M <= 8 or alone.sumsq.shape[1] == rows.sumsq.shape[1]:       # the same tiling: bit for bit
             assert torch.equal(alone.scaled[0], rows.scaled[M - 1]) and torch.equal(alone.sumsq[0], rows.sumsq[M - 1])
             assert torch.equal(res1[0], res[M - 1])
         else:            # from 9 rows on the tiles are not packed: the same sums in another order
