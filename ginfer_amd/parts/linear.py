@@ -14,8 +14,8 @@ from ..kernels import ops
 # from this many input features on, a product is "long": a folded norm gives way to a split over workgroups
 SPLIT_K_FROM = 4096
 MAX_SPLIT_K_PARTS = 16
-# a folded norm keeps K within a workgroup; measured on MI355X, a product with a long K still gains from
-# folding while its tiles are packed (up to 8 rows)
+# a folded norm keeps K within a workgroup; measured on MI355X, a product with a long K and fewer than 192
+# workgroups of full tiles still gains from folding while its tiles are packed (up to 8 rows)
 FOLD_LONG_K_UP_TO_ROWS = 8
 
 
@@ -111,8 +111,8 @@ def linear_into_norm(x, weight, bias, residual, norm):
     root-mean-square norm with a gain): the caller then takes the ordinary way."""
     if not getattr(norm, "foldable", False) or x.dtype != torch.bfloat16 or residual is None:
         return None
-    if x.shape[1] >= SPLIT_K_FROM and x.shape[0] > FOLD_LONG_K_UP_TO_ROWS:
-        return None      # a long K wants its split over workgroups more than it wants the norm folded
+    if x.shape[1] >= SPLIT_K_FROM and x.shape[0] > FOLD_LONG_K_UP_TO_ROWS and weight.shape[0] < 16 * 192:
+        return None      # a long K and few columns: the split over workgroups is worth more than the folded norm
     if not ops.folded_norm_supported(x, weight, residual, norm.weight):
         return None
     return ops.gemm_skinny(x, weight, bias, into_norm=(residual, norm.weight, norm.eps))

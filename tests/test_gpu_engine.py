@@ -427,3 +427,31 @@ def test_configurations_drawn_at_random(tmp_path, seed, dtype):
         got = H.run_steps(runner, steps)
         runner.cache.check()
         H.compare_with_plain(got, reqs, folder, H.TOL[dtype], "drawn %d %s %s %s" % (seed, dtype, what, cfg))
+
+
+@pytest.mark.parametrize("live", [6, 12, 40])
+def test_layer_sizes_of_a_7b_model_decoding_together(tmp_path, live):
+    """Two layers of a 7B shape (width 3584, 28 heads in 4 groups, feed-forward 18944) with 6, 12 and 40 requests
+    decoding side by side: the products' plans for wider matrices (no packed tiles, norms folded up to 16 rows,
+    K split in few parts), against the plain implementation."""
+    from ginfer_amd import ModelRunner
+    V = 1500
+    cfg = dict(architectures=["Qwen2ForCausalLM"], num_hidden_layers=2, hidden_size=3584, num_attention_heads=28,
+               num_key_value_heads=4, intermediate_size=18944, vocab_size=V, rope_theta=1e6, rms_norm_eps=1e-6,
+               tie_word_embeddings=False, max_position_embeddings=512)
+    folder = H.make_model_folder(tmp_path / "wide", cfg, 4, "float32")
+    prompt, decoded = 18, 6
+    reqs = {"r%d" % i: H.random_tokens(prompt + decoded, V, 100 + i) for i in range(live)}
+    steps = [dict(entries=[dict(id=rid, tokens=ids[:prompt], want=[prompt - 1])], end=[]) for rid, ids in reqs.items()]
+    for k in range(decoded):
+        steps.append(dict(entries=[dict(id=rid, tokens=[ids[prompt + k]], want=[0]) for rid, ids in reqs.items()],
+                          end=list(reqs) if k == decoded - 1 else []))
+    runner = ModelRunner(folder, dtype="bfloat16", page_size=16, num_pages=2 * live, max_requests=live)
+    got = H.run_steps(runner, steps)
+    runner.cache.check()
+    pcfg, w = pm.read_config(folder), pm.read_weights(folder, torch.float32)
+    for rid in list(reqs)[:3] + list(reqs)[-2:]:
+        ref = pm.forward(pcfg, w, reqs[rid]).numpy()
+        for p in range(prompt - 1, prompt + decoded):
+            err = np.abs(got[(rid, p)] - ref[p]).max() / np.abs(ref).max()
+            assert err <= H.TOL["bfloat16"], "request %s position %d: %.3g" % (rid, p, err)
