@@ -3,6 +3,8 @@
 tokenizer: prompts are lists of token ids and so are the results."""
 import time
 from dataclasses import dataclass
+
+import torch
 from typing import List, Optional
 
 from ..sampling import SamplingParams, Sampler
@@ -21,6 +23,7 @@ class EngineConfig:
     gpu_memory_utilization: float = 0.9   # share of the free device memory that becomes cache pages
     kvcache_block_size: int = 16          # tokens per cache page
     num_kvcache_blocks: Optional[int] = None   # pages per cache group; None: from free memory
+    pipeline_decode: bool = True          # launch a decode step before the tokens of the step before it are read
 
 
 @dataclass
@@ -45,7 +48,14 @@ class Engine:
                                    self.runner.spec.eos_token_ids, self.runner.max_model_len)
         self.sampler = Sampler(self.runner.device)
         self._next_id = 0
-        self.stats = dict(prefill_tokens=0, prefill_time=0.0, decode_tokens=0, decode_time=0.0, steps=0)
+        self._launched = None            # a step that is on the device and whose tokens have not been read yet
+        # sampled tokens come to the host through pinned buffers, each with an event: a step's tokens can then be
+        # waited for while the step launched after it is still running
+        self._token_ring = [(torch.empty(max(config.max_num_seqs, 1), dtype=torch.int32, pin_memory=True),
+                             torch.cuda.Event()) for _ in range(4)]
+        self._ring_at = 0
+        self.stats = dict(prefill_tokens=0, prefill_time=0.0, decode_tokens=0, decode_time=0.0, steps=0,
+                          steps_launched_ahead=0)
 
     def add_request(self, prompt_token_ids, params: Optional[SamplingParams] = None):
         params = params or SamplingParams()
@@ -60,26 +70,62 @@ class Engine:
         return rid
 
     def has_unfinished(self):
-        return not self.scheduler.is_finished()
+        return self._launched is not None or not self.scheduler.is_finished()
 
-    def step(self) -> List[RequestOutput]:
-        """One scheduled batch through the model; returns the requests that finished in it."""
-        t0 = time.perf_counter()
-        scheduled = self.scheduler.schedule()
+    def _launch(self, scheduled, device_tokens=None):
+        """Hands a scheduled step to the device: model step and sampling are queued, nothing is waited for.
+        device_tokens: the ids of single-token items that are still on the device (a step launched ahead)."""
         entries = []
         for sc in scheduled:
             s = sc.seq
-            toks = s.token_ids[s.num_computed:s.num_computed + sc.num_tokens]
+            toks = [0] if device_tokens is not None else s.token_ids[s.num_computed:s.num_computed + sc.num_tokens]
             entries.append(StepEntry(s.request_id, toks, [sc.num_tokens - 1] if sc.samples else []))
-        logits = self.runner.step(entries, borrow=True)
+        logits = self.runner.step(entries, borrow=True, device_tokens=device_tokens)
         sampling = [sc.seq for sc in scheduled if sc.samples]
-        tokens = self.sampler.sample(logits, [s.params for s in sampling],
-                                     [s.num_output_tokens for s in sampling])
+        ahead = 1 if device_tokens is not None else 0      # the token before is not in the request's list yet
+        tokens = self.sampler.sample_on_device(logits, [s.params for s in sampling],
+                                               [s.num_output_tokens + ahead for s in sampling])
+        arrival = None
+        if tokens is not None:               # the copy to the host is queued now, behind this step only
+            host, event = self._token_ring[self._ring_at]
+            self._ring_at = (self._ring_at + 1) % len(self._token_ring)
+            host[:tokens.shape[0]].copy_(tokens, non_blocking=True)
+            event.record()
+            arrival = (host, event, tokens.shape[0])
+        n_prefill = sum(sc.num_tokens for sc in scheduled if sc.num_tokens > 1 or sc.seq.num_computed == 0)
+        self.scheduler.advance(scheduled)
+        return dict(scheduled=scheduled, tokens=tokens, arrival=arrival, n_prefill=n_prefill,
+                    n_decode=sum(sc.num_tokens for sc in scheduled) - n_prefill)
+
+    def step(self) -> List[RequestOutput]:
+        """One scheduled batch through the model; returns the requests that finished in it.  While every
+        running request just decodes, the next step is launched before this step's tokens are read
+        (`pipeline_decode`): the host's work on a step then overlaps the device's work on the next."""
+        t0 = time.perf_counter()
+        cur = self._launched
+        self._launched = None
+        if cur is None:
+            cur = self._launch(self.scheduler.schedule())
+        nxt = None
+        if self.config.pipeline_decode and cur["tokens"] is not None:
+            ahead = self.scheduler.schedule_ahead(cur["scheduled"])
+            if ahead is not None:
+                items, index = ahead
+                toks = cur["tokens"]
+                if len(index) != toks.shape[0]:
+                    toks = toks[torch.as_tensor(index, device=toks.device)]
+                nxt = self._launch(items, device_tokens=toks)
+                self.stats["steps_launched_ahead"] += 1
+        tokens = []
+        if cur["arrival"] is not None:
+            host, event, n = cur["arrival"]
+            event.synchronize()
+            tokens = host[:n].tolist()
         now = time.perf_counter()
-        finished = self.scheduler.postprocess(scheduled, tokens, now)
+        finished = self.scheduler.absorb(cur["scheduled"], tokens, now)
+        self._launched = nxt
         dt = now - t0
-        n_prefill = sum(sc.num_tokens for sc in scheduled if sc.num_tokens > 1 or sc.seq.num_computed == sc.num_tokens)
-        n_decode = sum(sc.num_tokens for sc in scheduled) - n_prefill
+        n_prefill, n_decode = cur["n_prefill"], cur["n_decode"]
         st = self.stats
         st["steps"] += 1
         # a mixed step's time is shared out by tokens

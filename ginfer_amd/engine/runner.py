@@ -81,10 +81,14 @@ class ModelRunner:
         return self.spec.vocab_size
 
     # ---- the step
-    def step(self, entries: List[StepEntry], borrow=False):
+    def step(self, entries: List[StepEntry], borrow=False, device_tokens=None):
         """Returns float32 logits [R, V] on the device: the wanted places in the order of the entries
         and of each entry's `want`.  With borrow=True the result may be a buffer that the next step
-        overwrites (the engine samples from it at once)."""
+        overwrites (the engine samples from it at once).
+        device_tokens (int32 [len(entries)] on the device): every entry brings ONE token whose id the host does
+        not know yet (the entry's own token is a placeholder): the ids are taken from this tensor on the device,
+        in the order of the entries.  This lets a caller launch a decode step before it has read the tokens of
+        the step before."""
         if not entries:
             return torch.empty((0, self.vocab_size), dtype=torch.float32, device=self.device)
         cache = self.cache
@@ -99,6 +103,11 @@ class ModelRunner:
             for w in e.want:
                 if not 0 <= w < n:
                     raise ValueError("request %r wants place %r of %d tokens" % (e.request_id, w, n))
+        if device_tokens is not None:
+            if any(len(e.tokens) != 1 for e in entries):
+                raise ValueError("tokens that are still on the device stand for single-token entries only")
+            if device_tokens.dtype != torch.int32 or tuple(device_tokens.shape) != (len(entries),) or not device_tokens.is_cuda:
+                raise ValueError("device_tokens must be int32 [%d] on the device" % len(entries))
         reserved_here = []
         try:
             for e in entries:
@@ -115,7 +124,7 @@ class ModelRunner:
                     raise ValueError("request %r has %d tokens reserved but brings %d"
                                      % (e.request_id, cache.pending(e.request_id), len(e.tokens)))
             host = self._host_arrays(entries)
-            logits = self._run(host, borrow)
+            logits = self._run(host, borrow, device_tokens)
         except Exception:
             for rid in reserved_here:       # nothing is committed: the requests stay as long as they were
                 cache.requests[rid].pending = 0
@@ -203,7 +212,7 @@ class ModelRunner:
             host_q_start=host["q_start"].tolist(), host_q_len=host["q_len"].tolist(), caches=caches,
             extra={"decode_info": buf.dev["decode_info"], "decode_span": _context_bucket(host["max_kv"])})
 
-    def _run(self, host, borrow):
+    def _run(self, host, borrow, device_tokens=None):
         E, T = host["E"], host["T"]
         graphable = self.use_graphs and T == E and E <= GRAPH_MAX_ROWS and len(host["rows"]) == E and \
             bool((host["rows"] == np.arange(E)).all())
@@ -221,10 +230,14 @@ class ModelRunner:
                     g = self._capture(key, host)
             if g is not None:
                 g["buf"].fill(host)
+                if device_tokens is not None:
+                    g["buf"].buf.dev["ids"].copy_(device_tokens)
                 g["graph"].replay()
                 return g["logits"] if borrow else g["logits"].clone()
         buf = self._buffers.get(T, E, len(host["rows"]), host["width"], len(host["decode_info"]))
         ctx = self._context(host, buf)
+        if device_tokens is not None:
+            buf.dev["ids"].copy_(device_tokens)
         return self.model.forward(ctx)
 
     def _capture(self, key, host):

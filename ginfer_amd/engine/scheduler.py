@@ -155,15 +155,31 @@ class Scheduler:
         """tokens: one sampled token for every scheduled item that samples, in order.  Appends them,
         finishes what is done (end-of-sequence id unless ignore_eos, max_tokens, max_model_len), frees
         their pages.  Returns the sequences that finished."""
+        self.advance(scheduled)
+        return self.absorb(scheduled, tokens, now)
+
+    def advance(self, scheduled: List[Scheduled]):
+        """The step has been handed to the device: its tokens count as computed."""
+        cache = self.cache
+        for sc in scheduled:
+            rid = sc.seq.request_id
+            if cache.pending(rid):
+                cache.commit(rid)
+            sc.seq.num_computed += sc.num_tokens
+
+    def absorb(self, scheduled: List[Scheduled], tokens: List[int], now=None) -> List[Sequence]:
+        """The step's sampled tokens have arrived (one for every item that samples, in order): appends them and
+        finishes what is done.  An item whose request finished meanwhile (a step launched ahead of the token that
+        ended it) is passed over."""
         finished = []
         it = iter(tokens)
         for sc in scheduled:
             seq = sc.seq
-            self.cache.commit(seq.request_id) if self.cache.pending(seq.request_id) else None
-            seq.num_computed += sc.num_tokens
             if not sc.samples:
                 continue
             tok = int(next(it))
+            if seq.state is not State.RUNNING:
+                continue
             seq.token_ids.append(tok)
             if seq.first_token_ts is None:
                 seq.first_token_ts = now
@@ -181,3 +197,35 @@ class Scheduler:
                 self.running.remove(seq)
                 finished.append(seq)
         return finished
+
+    # ---- a step launched before the tokens of the step before it are known
+    def schedule_ahead(self, scheduled: List[Scheduled]):
+        """`scheduled` has been launched (and advanced) but its tokens have not been read yet.  If the step
+        after it is certain to be one more token for every request that is still running, and nothing else,
+        reserves that step and returns (its items, for each the index of its request in `scheduled`); else None,
+        with nothing changed.  Certain means: every running request is in `scheduled` and samples there, none of
+        them reaches max_tokens or max_model_len with the token it is about to get, no waiting request could be
+        admitted, and the pages are there.  A request that ends on an end-of-sequence token nobody has seen yet
+        runs one step too many; its result is dropped by absorb()."""
+        alive = [(i, sc) for i, sc in enumerate(scheduled) if sc.seq.state is State.RUNNING]
+        if not alive or len(alive) != len(self.running) or len(alive) > self.max_num_batched_tokens:
+            return None
+        if self.waiting and len(self.running) < self.max_num_seqs and self.cache.can_admit():
+            return None
+        for _, sc in alive:
+            seq = sc.seq
+            # every known token is computed and the next one is on its way: the request will hold `known` tokens
+            known = len(seq.token_ids) + 1
+            if not sc.samples or seq.num_computed != len(seq.token_ids) \
+                    or known - seq.num_prompt_tokens >= seq.params.max_tokens or known >= self.max_model_len:
+                return None
+        reserved = []
+        for _, sc in alive:
+            try:
+                self.cache.append(sc.seq.request_id, 1)
+                reserved.append(sc.seq.request_id)
+            except OutOfPages:
+                for rid in reserved:
+                    self.cache.requests[rid].pending = 0
+                return None
+        return [Scheduled(sc.seq, 1, True) for _, sc in alive], [i for i, _ in alive]

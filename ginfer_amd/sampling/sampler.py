@@ -13,14 +13,17 @@ class Sampler:
     def sample(self, logits, params, output_positions):
         """logits float32 [R, V]; params: R SamplingParams; output_positions: which output token of its
         request each row decides (indexes the request's random stream).  Returns a list of R ints."""
+        out = self.sample_on_device(logits, params, output_positions)
+        return [] if out is None else out.cpu().tolist()
+
+    def sample_on_device(self, logits, params, output_positions):
+        """As sample(), but the tokens stay on the device: int32 [R] (None for no rows).  Nothing waits."""
         R = logits.shape[0]
         if R == 0:
-            return []
+            return None
         if all(p.temperature <= 0 for p in params):
-            out = ops.sample_rows(logits)
-        else:
-            temp = torch.tensor([float(p.temperature) for p in params], dtype=torch.float32, device=self.device)
-            uni = torch.tensor(np.asarray([uniform(p.seed, n) for p, n in zip(params, output_positions)],
-                                          dtype=np.float32), device=self.device)
-            out = ops.sample_rows(logits, temp, uni)
-        return out.cpu().tolist()
+            return ops.sample_rows(logits)
+        temp = torch.tensor([float(p.temperature) for p in params], dtype=torch.float32, device=self.device)
+        uni = torch.tensor(np.asarray([uniform(p.seed, n) for p, n in zip(params, output_positions)],
+                                      dtype=np.float32), device=self.device)
+        return ops.sample_rows(logits, temp, uni)

@@ -455,3 +455,41 @@ def test_layer_sizes_of_a_7b_model_decoding_together(tmp_path, live):
         for p in range(prompt - 1, prompt + decoded):
             err = np.abs(got[(rid, p)] - ref[p]).max() / np.abs(ref).max()
             assert err <= H.TOL["bfloat16"], "request %s position %d: %.3g" % (rid, p, err)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_steps_launched_ahead_change_nothing(folders, dtype):
+    """While every running request decodes, the engine launches the next step before it has read the tokens
+    of this one.  The tokens are the same as without that, bit for bit: greedy and sampled requests, requests that
+    stop on a token nobody had seen when the step after it was launched, requests that reach max_tokens, and
+    others arriving while the pipeline runs."""
+    from ginfer_amd import Engine, EngineConfig, SamplingParams
+    name = "B"
+    vocab = H.TINY[name][0]["vocab_size"]
+    prompts = [H.random_tokens(n, vocab, 900 + n) for n in (5, 17, 33, 9, 12, 21, 3, 40)]
+
+    def run(pipeline):
+        eng = Engine(EngineConfig(model_path=folders[name], dtype=dtype, max_num_batched_tokens=64, max_num_seqs=5,
+                                  max_seq_len=128, kvcache_block_size=8, num_kvcache_blocks=80, pipeline_decode=pipeline))
+        free = eng.generate(prompts[:2], SamplingParams(max_tokens=12, ignore_eos=True))      # to find tokens to stop on
+        stops = sorted({o.token_ids[5] for o in free} | {o.token_ids[8] for o in free})
+        params = [SamplingParams(max_tokens=m, temperature=t, seed=7, ignore_eos=False, stop_token_ids=stops if st else None)
+                  for m, t, st in ((12, 0.0, True), (12, 0.0, True), (25, 0.8, False), (7, 0.0, False), (30, 0.0, True),
+                                   (1, 0.0, False), (16, 1.1, True), (20, 0.0, False))]
+        ids = [eng.add_request(p, sp) for p, sp in zip(prompts[:5], params[:5])]
+        done, steps = {}, 0
+        while eng.has_unfinished():
+            for o in eng.step():
+                done[o.request_id] = o
+            steps += 1
+            if steps == 6:             # three more arrive while the others decode
+                ids += [eng.add_request(p, sp) for p, sp in zip(prompts[5:], params[5:])]
+        eng.runner.cache.check()
+        assert not eng.runner.cache.requests
+        return [(done[i].token_ids, done[i].finish_reason) for i in ids], eng.stats["steps_launched_ahead"]
+
+    with_ahead, n_ahead = run(True)
+    without, none_ahead = run(False)
+    assert n_ahead > 5 and none_ahead == 0
+    assert with_ahead == without
+    assert {r for _, r in with_ahead} >= {"eos", "max_tokens"}

@@ -174,3 +174,117 @@ def test_uniform_numbers_are_a_function_of_seed_and_place():
     assert abs(sum(us) / 1000 - 0.5) < 0.05
     import numpy as np
     assert all(float(np.float32(u)) == u for u in us)          # exact in 32-bit
+
+
+def run_ahead(sched, cache, seqs, arrivals=None, max_steps=10000):
+    """As the engine drives the scheduler when it launches decode steps ahead: a step is advanced at once, the
+    step after it is reserved (if schedule_ahead allows) before the first one's tokens are absorbed.  The
+    stand-in model can name a token only once the tokens before it are known, so tokens of a step launched ahead
+    are worked out when they are absorbed."""
+    for s in seqs:
+        sched.add(s)
+    done, launched, ahead_steps, steps = [], None, 0, 0
+    while launched is not None or not sched.is_finished():
+        cur = launched
+        if cur is None:
+            cur = sched.schedule()
+            assert cur
+            sched.advance(cur)
+        nxt = sched.schedule_ahead(cur)
+        if nxt is not None:
+            items, index = nxt
+            assert [cur[i].seq for i in index] == [sc.seq for sc in items]
+            assert all(cache.pending(sc.seq.request_id) == 1 for sc in items)
+            sched.advance(items)
+            ahead_steps += 1
+        toks = [fake_token(b.seq.token_ids) for b in cur if b.samples]
+        done += sched.absorb(cur, toks, now=float(steps))
+        cache.check()
+        launched = None if nxt is None else nxt[0]
+        steps += 1
+        if arrivals and steps in arrivals:
+            sched.add(arrivals[steps])
+        assert steps < max_steps
+    return done, ahead_steps
+
+
+def test_steps_launched_ahead_give_the_same_tokens():
+    sched, cache = make(num_pages=64, max_num_seqs=3, budget=16)
+    seqs = [seq(0, 5, 9), seq(1, 11, 4), seq(2, 3, 12), seq(3, 7, 6)]
+    want = {s.request_id: expected(s) for s in seqs}
+    done, ahead = run_ahead(sched, cache, seqs)
+    assert ahead > 5
+    assert {s.request_id: s.token_ids for s in done} == want
+    assert not cache.requests
+
+
+def test_a_request_that_stops_on_an_unseen_token_runs_one_step_too_many_and_is_dropped():
+    sched, cache = make(num_pages=64, max_num_seqs=2, budget=16)
+    a, b = seq(0, 4, 20), seq(1, 6, 20)
+    stop = expected(a)[4 + 3]                                    # a's fourth output token ends it
+    a.params.stop_token_ids = [stop]
+    a.params.ignore_eos = False
+    done, ahead = run_ahead(sched, cache, [a, b])
+    by_id = {s.request_id: s for s in done}
+    assert by_id[0].finish_reason == "eos" and by_id[0].token_ids[-1] == stop and by_id[0].num_output_tokens <= 4
+    assert by_id[1].token_ids == expected(b) and by_id[1].finish_reason == "max_tokens"
+    assert ahead > 5 and not cache.requests
+
+
+def test_no_step_ahead_when_the_next_step_is_not_certain():
+    sched, cache = make(num_pages=64, max_num_seqs=2, budget=16)
+    a = seq(0, 4, 2)
+    sched.add(a)
+    first = sched.schedule()
+    sched.advance(first)
+    assert sched.schedule_ahead(first) is not None               # token 1 of 2 is on its way: one more step is certain
+    cache.requests[0].pending = 0                                # (undo the reservation of the probe)
+    sched.absorb(first, [fake_token(a.token_ids)], 0.0)
+    second = sched.schedule()
+    sched.advance(second)
+    assert sched.schedule_ahead(second) is None                  # the token on its way is the last: max_tokens
+    sched.absorb(second, [fake_token(a.token_ids)], 1.0)
+    assert sched.is_finished()
+    # a waiting request that could be admitted goes first
+    sched, cache = make(num_pages=64, max_num_seqs=2, budget=16)
+    sched.add(seq(0, 4, 9))
+    first = sched.schedule()
+    sched.advance(first)
+    sched.add(seq(1, 4, 9))
+    assert sched.schedule_ahead(first) is None
+    # a prompt that is not through yet
+    sched, cache = make(num_pages=64, max_num_seqs=2, budget=4)
+    sched.add(seq(0, 9, 9))
+    first = sched.schedule()
+    sched.advance(first)
+    assert not first[0].samples and sched.schedule_ahead(first) is None
+
+
+def test_no_step_ahead_without_pages_and_nothing_stays_reserved():
+    """Two requests that outgrow the pool together: where the step ahead lacks a page it is not taken, what it had
+    reserved is undone, and the ordinary schedule (which may evict) decides instead; the tokens stay the same."""
+    sched, cache = make(num_pages=5, page_size=4, max_num_seqs=2, budget=16)
+    seqs = [seq(0, 4, 9), seq(1, 4, 9)]
+    want = {s.request_id: expected(s) for s in seqs}
+    for s in seqs:
+        sched.add(s)
+    refused_for_pages, done, steps = 0, [], 0
+    while not sched.is_finished():
+        batch = sched.schedule()
+        sched.advance(batch)
+        free_before = cache.groups[0].pool.num_free
+        ahead = sched.schedule_ahead(batch)
+        if ahead is None:
+            assert all(r.pending == 0 for r in cache.requests.values())
+            if len(batch) == 2 and all(b.samples for b in batch) and free_before < 2 \
+                    and all(cache.length(b.seq.request_id) % 4 == 0 for b in batch):
+                refused_for_pages += 1
+        else:                                       # this test drives the steps one by one: give the probe back
+            for sc in ahead[0]:
+                cache.requests[sc.seq.request_id].pending = 0
+        cache.check()
+        done += sched.absorb(batch, [fake_token(b.seq.token_ids) for b in batch if b.samples], float(steps))
+        steps += 1
+        assert steps < 200
+    assert refused_for_pages >= 1 and sched.num_evictions >= 1
+    assert {s.request_id: s.token_ids for s in done} == want
