@@ -5,7 +5,8 @@ on one MI355X, with the achieved fraction of the HBM and matrix-core rooflines.
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B] [--context C]
 
 A step is one decode step of the engine's own step function plus sampling: every request of the batch
-gets one token, from the paged cache, and its next token comes back to the host.  Prints ONE JSON line.
+gets one token, from the paged cache, and its next token comes back to the host; as in the engine, the next
+step is launched before this step's tokens have been waited for.  Prints ONE JSON line.
 """
 import argparse
 import json
@@ -123,15 +124,38 @@ def main():
         tokens = torch.randint(0, vocab, (B,), generator=g).tolist()
         params = [SamplingParams() for _ in range(B)]
 
-        def one(tokens):
-            logits = runner.step([StepEntry(("d", b), [tokens[b]], [0]) for b in range(B)])
-            return sampler.sample(logits, params, [0] * B)
-        for _ in range(warmup):
-            tokens = one(tokens)
+        ring = [(torch.empty(B, dtype=torch.int32, pin_memory=True), torch.cuda.Event()) for _ in range(3)]
+        at = [0]
+
+        def launch(tokens=None, device_tokens=None):
+            """One step handed to the device: model, sampling, and the tokens' copy to the host behind it."""
+            ids = tokens if tokens is not None else [0] * B
+            logits = runner.step([StepEntry(("d", b), [ids[b]], [0]) for b in range(B)], borrow=True,
+                                 device_tokens=device_tokens)
+            dev = sampler.sample_on_device(logits, params, [0] * B)
+            host, event = ring[at[0] % len(ring)]
+            at[0] += 1
+            host.copy_(dev, non_blocking=True)
+            event.record()
+            return dev, host, event
+
+        def run(n, tokens):
+            """n steps, as the engine drives them: the next step is launched (its ids taken on the device) before
+            this step's tokens, which come to the host every step, have been waited for."""
+            if n <= 0:
+                return tokens
+            cur = launch(tokens=tokens)
+            for _ in range(n - 1):
+                nxt = launch(device_tokens=cur[0])
+                cur[2].synchronize()
+                tokens = cur[1].tolist()
+                cur = nxt
+            cur[2].synchronize()
+            return cur[1].tolist()
+        tokens = run(warmup, tokens)
         sync()
         t0 = time.perf_counter()
-        for _ in range(steps):
-            tokens = one(tokens)
+        tokens = run(steps, tokens)
         sync()
         dt = (time.perf_counter() - t0) / steps
         mean_ctx = args.context - steps / 2.0
