@@ -32,6 +32,8 @@ def _engine_args(p):
     p.add_argument("--ignore-eos", action="store_true", help="do not stop at an end-of-sequence token")
     p.add_argument("--temperature", type=float, default=0.0, help="0: greedy")
     p.add_argument("--seed", type=int, default=0, help="seed of the sampler's random stream")
+    p.add_argument("--no-pipeline-decode", action="store_true",
+                   help="read every step's tokens before the next step is launched")
 
 
 def _engine(args):
@@ -42,7 +44,7 @@ def _engine(args):
         model_path=args.model_path, dtype=args.dtype, max_num_batched_tokens=args.max_num_batched_tokens,
         max_num_seqs=args.max_num_seqs, max_seq_len=args.max_seq_len,
         gpu_memory_utilization=args.gpu_memory_utilization, kvcache_block_size=args.kvcache_block_size,
-        num_kvcache_blocks=args.num_kvcache_blocks))
+        num_kvcache_blocks=args.num_kvcache_blocks, pipeline_decode=not args.no_pipeline_decode))
 
 
 def _params(args, n):
@@ -59,9 +61,10 @@ def _report(engine, outs, wall):
             "%.3f ms" % (o.tpot * 1e3) if o.tpot else "-", o.evictions))
     pf = st["prefill_tokens"] / st["prefill_time"] if st["prefill_time"] else 0.0
     dc = st["decode_tokens"] / st["decode_time"] if st["decode_time"] else 0.0
-    sys.stderr.write("steps=%d prefill=%.1f tok/s decode=%.1f tok/s wall=%.3f s evictions=%d\n"
-                     % (st["steps"], pf, dc, wall, engine.scheduler.num_evictions))
-    return dict(steps=st["steps"], prefill_tok_s=pf, decode_tok_s=dc, wall_s=wall)
+    sys.stderr.write("steps=%d (launched ahead: %d) prefill=%.1f tok/s decode=%.1f tok/s wall=%.3f s evictions=%d\n"
+                     % (st["steps"], st["steps_launched_ahead"], pf, dc, wall, engine.scheduler.num_evictions))
+    return dict(steps=st["steps"], steps_launched_ahead=st["steps_launched_ahead"], prefill_tok_s=pf, decode_tok_s=dc,
+                wall_s=wall)
 
 
 def cmd_generate(args):
