@@ -438,12 +438,23 @@ __global__ __launch_bounds__(64 * PREFILL_WAVES) void attn_prefill_kernel(
   extern __shared__ float lds[];          // [hpw][splits-1][NB] x { o[HD][17], m[16], l[16] }
   constexpr int STATE = HD * 17 + 32;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c = lane & 15, g = lane >> 4;
-  const int kvh = blockIdx.y / head_blocks, hb = blockIdx.y % head_blocks;
+  // Workgroups go to the 8 XCDs in turn, each with an L2 of its own.  Where the grid's y (kv head x head block)
+  // divides 8 and its x is a multiple of 8 / y, the workgroups are renumbered so that an XCD sees one y only: its
+  // L2 then holds the keys and values of one kv head instead of all of them.  The tiles of a y keep their order
+  // (heaviest first).  With linear = 8a + b the new place is (y = b / per, x = a * per + b % per): one to one
+  // exactly when x's extent is a multiple of per (else the last x would fall outside, and the grid stays as it is).
+  int by = blockIdx.y, bx = blockIdx.x;
+  if (gridDim.y > 1 && 8 % gridDim.y == 0 && gridDim.x % (8 / gridDim.y) == 0) {
+    const int linear = blockIdx.x + blockIdx.y * gridDim.x, per = 8 / gridDim.y;
+    by = (linear % 8) / per;
+    bx = (linear / 8) * per + (linear % 8) % per;
+  }
+  const int kvh = by / head_blocks, hb = by % head_blocks;
   const int group = nh / nkv;
   const int hl = wave / splits, split = wave % splits;
   const bool head_ok = hb * hpw + hl < group;
   const int head = kvh * group + hb * hpw + hl;
-  const int32_t* tile = tiles + (int64_t)blockIdx.x * 4;
+  const int32_t* tile = tiles + (int64_t)bx * 4;
   const int entry = tile[0], row0 = tile[1], rows = tile[2], pos0 = tile[3];
 
   f32x4 o[NB][DB];
