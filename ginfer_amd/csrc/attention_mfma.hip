@@ -46,6 +46,9 @@ constexpr int PREFILL_NB = HD <= 128 ? 2 : 1;
 #ifndef PREFILL_DEPTH
 #define PREFILL_DEPTH 1              // sets of key and value registers in flight in the prefill kernel
 #endif
+#ifndef DECODE_DEPTH
+#define DECODE_DEPTH 1               // ... and in the decode kernel (2 was measured no faster from 1k to 128k tokens)
+#endif
 #ifndef PREFILL_WAVES
 #define PREFILL_WAVES 8              // wavefronts of a prefill workgroup
 #endif
@@ -338,7 +341,7 @@ __global__ __launch_bounds__(64 * DEC_WAVES) void attn_decode_split_kernel(
     const int cpos[1] = {col_ok ? pos : -1}, clo[1] = {lo};
     const int32_t* bt = block_table + (int64_t)info.z * table_width;
     // every live column of a decode wavefront sees the same keys: lo..pos
-    attend_tiles<1, 1>(o, m, l, qr, cpos, clo, k_pages, v_pages, bt, kvh, nkv, ps_shift, lo, pos, lo, pos,
+    attend_tiles<1, DECODE_DEPTH>(o, m, l, qr, cpos, clo, k_pages, v_pages, bt, kvh, nkv, ps_shift, lo, pos, lo, pos,
                     begin + 32 * wave, end, 32 * DEC_WAVES, scale);
     finish_sums<1>(l);
   }
