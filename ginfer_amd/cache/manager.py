@@ -10,6 +10,16 @@ next token to be computed; its table keeps a -1 there.  Pages return to the pool
 released and are used again by later requests.  The reference has one pool, one table per sequence,
 no window and no state (ginfer/engine/block_manager.cc:63-148, ginfer/engine/model_runner.cc:52-87).
 
+Shared prefixes (optional; the reference always does it, block_manager.cc:63-110): a page that is full and
+whose tokens are known is remembered under (what came before it, its tokens).  A request that is admitted
+with its tokens takes over the remembered pages of its longest known prefix, as one more holder of each, and
+starts behind them; at least its last token is left to run.  A remembered page that nobody holds lies in the
+free queue like any other and is forgotten when it is taken for something else.  What came before a page is
+named by a number that is never used twice, so a hit is exact: it compares tokens, not hashes of them (the
+reference compares a 64-bit chain hash and the page's own tokens).  Only for models whose every cache group
+keeps all keys and that have no per-request state: a window gives pages of a prefix back, and state has to
+see every token.
+
 Device layout of one group: one allocation [entries_in_group, 2 (k, v), pages, nkv * page_size * hd]; an
 entry's keys are viewed [pages, nkv, page_size, hd] and its values [pages, nkv, hd, page_size]
 (transposed inside a page, which is what the matrix-core attention kernels read fastest).
@@ -29,6 +39,7 @@ class _Request:
     length: int = 0                      # tokens whose keys/values (or state) are in the cache
     pending: int = 0                     # tokens reserved by append() and not yet committed
     tables: List[List[int]] = field(default_factory=list)   # per group: logical block -> page or -1
+    contents: List[List[int]] = field(default_factory=list) # per group: content number of each remembered block
 
 
 class CacheGroup:
@@ -36,6 +47,35 @@ class CacheGroup:
         self.spec, self.entries, self.page_size = spec, list(entries), page_size
         self.pool = PagePool(num_pages)
         self.tensor = None               # device tensor, set by allocate_device
+        # full pages whose tokens are known, for requests that share a prefix
+        self._page_of = {}               # (content number of the block before or 0, the block's tokens) -> page
+        self._key_of = {}                # page -> its key in _page_of
+        self._content_of = {}            # page -> content number, never used twice
+        self._contents = 0
+
+    def lookup(self, before, tokens):
+        """(page, content number) of the remembered block with these tokens after the content `before`, or None."""
+        page = self._page_of.get((before, tokens))
+        return None if page is None else (page, self._content_of[page])
+
+    def remember(self, before, tokens, page):
+        """The page holds the block with these tokens after `before`.  Returns the block's content number: a new
+        one, or that of a page remembered earlier for the same content (this page then stays unknown)."""
+        known = self._page_of.get((before, tokens))
+        if known is not None:
+            return self._content_of[known]
+        self.forget(page)
+        self._contents += 1
+        self._page_of[(before, tokens)] = page
+        self._key_of[page] = (before, tokens)
+        self._content_of[page] = self._contents
+        return self._contents
+
+    def forget(self, page):
+        key = self._key_of.pop(page, None)
+        if key is not None:
+            del self._page_of[key]
+            del self._content_of[page]
 
     @property
     def window(self):
@@ -50,9 +90,14 @@ class CacheGroup:
 
 
 class CacheManager:
-    def __init__(self, cache_specs, page_size, num_pages, max_requests):
+    def __init__(self, cache_specs, page_size, num_pages, max_requests, prefix_caching=False):
         """cache_specs: per schedule entry KVCacheSpec | StateSpec | None (None: keeps nothing, or reads
-        another entry's cache).  num_pages: pages of every group's pool."""
+        another entry's cache).  num_pages: pages of every group's pool.  prefix_caching: requests admitted with
+        their tokens share the pages of a known prefix."""
+        if prefix_caching and not self.supports_prefix_caching(cache_specs):
+            raise ValueError("prefixes cannot be shared in a model with a window or with per-request state")
+        self.prefix_caching = bool(prefix_caching)
+        self.prefix_hit_tokens = 0
         if page_size < 1:
             raise ValueError("page_size must be positive")
         self.page_size, self.max_requests = int(page_size), int(max_requests)
@@ -75,6 +120,12 @@ class CacheManager:
         self._table_np = [np.full((self.max_requests, 16), -1, dtype=np.int32) for _ in self.groups]
         self._length_np = np.zeros(self.max_requests, dtype=np.int64)
         self._any_window = any(g.window is not None for g in self.groups)
+
+    @staticmethod
+    def supports_prefix_caching(cache_specs):
+        return (any(isinstance(s, KVCacheSpec) for s in cache_specs)
+                and not any(isinstance(s, StateSpec) or (isinstance(s, KVCacheSpec) and s.window is not None)
+                            for s in cache_specs))
 
     # ---- device memory
     def bytes_per_page(self, element_size):
@@ -104,15 +155,63 @@ class CacheManager:
     def can_admit(self):
         return self.slots.num_free > 0
 
-    def admit(self, rid):
+    def admit(self, rid, token_ids=None):
+        """A state slot and empty block tables for the request.  With token_ids (and prefix caching): the pages of
+        the longest remembered prefix are taken over, and length(rid) tells how many tokens they hold."""
         if rid in self.requests:
             raise ValueError("request %r is already in the cache" % (rid,))
-        self.requests[rid] = _Request(slot=self.slots.take(), tables=[[] for _ in self.groups])
-        slot = self.requests[rid].slot
+        req = self.requests[rid] = _Request(slot=self.slots.take(), tables=[[] for _ in self.groups],
+                                            contents=[[] for _ in self.groups])
+        slot = req.slot
         for t in self._table_np:
             t[slot, :] = -1
         self._length_np[slot] = 0
+        if self.prefix_caching and token_ids is not None:
+            self._share_prefix(req, token_ids)
         return slot
+
+    def _share_prefix(self, req, token_ids):
+        ps = self.page_size
+        blocks = (len(token_ids) - 1) // ps          # the last token at least is left to run
+        chains = []
+        for g in self.groups:
+            chain, before = [], 0
+            for i in range(blocks):
+                hit = g.lookup(before, tuple(token_ids[i * ps:(i + 1) * ps]))
+                if hit is None:
+                    break
+                chain.append(hit)
+                before = hit[1]
+            chains.append(chain)
+            blocks = len(chain)
+        if blocks == 0:
+            return
+        for gi, g in enumerate(self.groups):
+            for page, content in chains[gi][:blocks]:
+                g.pool.share(page)
+                req.tables[gi].append(page)
+                req.contents[gi].append(content)
+            self._mirror_table(gi, req)
+        req.length = blocks * ps
+        self._length_np[req.slot] = req.length
+        self.prefix_hit_tokens += req.length
+
+    def _remember(self, req, token_ids):
+        """Remembers the request's full pages whose tokens are known and whose keys and values are committed."""
+        ps = self.page_size
+        full = min(req.length, len(token_ids)) // ps
+        for gi, g in enumerate(self.groups):
+            chain, table = req.contents[gi], req.tables[gi]
+            for i in range(len(chain), full):
+                chain.append(g.remember(chain[i - 1] if i else 0, tuple(token_ids[i * ps:(i + 1) * ps]), table[i]))
+
+    def _mirror_table(self, gi, req):
+        table, mirror = req.tables[gi], self._table_np[gi]
+        if len(table) > mirror.shape[1]:
+            wider = np.full((self.max_requests, max(len(table), 2 * mirror.shape[1])), -1, dtype=np.int32)
+            wider[:, :mirror.shape[1]] = mirror
+            self._table_np[gi] = mirror = wider
+        mirror[req.slot, :len(table)] = table
 
     def length(self, rid):
         return self.requests[rid].length
@@ -193,16 +292,14 @@ class CacheManager:
                 table[i] = -1
             while len(table) < need_blocks:
                 table.append(-1)
-            new_pages = iter(g.pool.take(take))
+            taken = g.pool.take(take)
+            for p in taken:
+                g.forget(p)              # what the page held for requests to come is gone
+            new_pages = iter(taken)
             for i in range(max(first, 0), need_blocks):
                 if table[i] < 0:
                     table[i] = next(new_pages)
-            mirror = self._table_np[gi]
-            if len(table) > mirror.shape[1]:
-                wider = np.full((self.max_requests, max(len(table), 2 * mirror.shape[1])), -1, dtype=np.int32)
-                wider[:, :mirror.shape[1]] = mirror
-                self._table_np[gi] = mirror = wider
-            mirror[req.slot, :len(table)] = table
+            self._mirror_table(gi, req)
         req.pending = n_new
         return req.length
 
@@ -218,17 +315,24 @@ class CacheManager:
     def lengths_array(self, slots):
         return self._length_np[slots]
 
-    def commit(self, rid):
+    def commit(self, rid, token_ids=None):
+        """The reserved tokens are in the cache (or on their way there, in stream order).  token_ids: the
+        request's tokens as far as they are known, for remembering pages that are full now."""
         req = self.requests[rid]
         req.length += req.pending
         req.pending = 0
         self._length_np[req.slot] = req.length
+        if self.prefix_caching and token_ids is not None:
+            self._remember(req, token_ids)
 
-    def release(self, rid):
-        """The request ends (or is evicted): every page and its slot go back."""
+    def release(self, rid, token_ids=None):
+        """The request ends (or is evicted): every page and its slot go back, the pages of its end first, so
+        that the start of what it held is the last to be taken for something else."""
         req = self.requests.pop(rid)
+        if self.prefix_caching and token_ids is not None:
+            self._remember(req, token_ids)
         for gi, g in enumerate(self.groups):
-            g.pool.give_back([p for p in req.tables[gi] if p >= 0])
+            g.pool.give_back([p for p in reversed(req.tables[gi]) if p >= 0])
         self.slots.give_back(req.slot)
 
     # ---- checks (tests call this after every operation)
@@ -239,9 +343,22 @@ class CacheManager:
                 for p in req.tables[gi]:
                     if p < 0:
                         continue
-                    if p in seen:
-                        raise AssertionError("page %d of group %d is held by %r and %r" % (p, gi, seen[p], rid))
-                    seen[p] = rid
+                    if p in seen and not self.prefix_caching:
+                        raise AssertionError("page %d of group %d is held by %r and %r" % (p, gi, seen[p][0], rid))
+                    seen.setdefault(p, []).append(rid)
+                if len(set(p for p in req.tables[gi] if p >= 0)) != sum(1 for p in req.tables[gi] if p >= 0):
+                    raise AssertionError("group %d: %r holds a page twice" % (gi, rid))
+            for p, rids in seen.items():
+                if g.pool.holders(p) != len(rids):
+                    raise AssertionError("page %d of group %d has %d holders, tables say %r"
+                                         % (p, gi, g.pool.holders(p), rids))
+                if len(rids) > 1 and p not in g._key_of:
+                    raise AssertionError("page %d of group %d is shared by %r but not remembered" % (p, gi, rids))
+            for key, p in g._page_of.items():
+                if g._key_of.get(p) != key or p not in g._content_of:
+                    raise AssertionError("group %d: the records of remembered page %d disagree" % (gi, p))
+            if len(g._key_of) != len(g._page_of) or len(g._content_of) != len(g._page_of):
+                raise AssertionError("group %d: records of remembered pages left over" % gi)
             held = set(g.pool.held())
             if held != set(seen):
                 raise AssertionError("group %d: pool holds %s, tables hold %s" % (gi, sorted(held), sorted(seen)))

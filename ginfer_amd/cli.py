@@ -34,6 +34,8 @@ def _engine_args(p):
     p.add_argument("--seed", type=int, default=0, help="seed of the sampler's random stream")
     p.add_argument("--no-pipeline-decode", action="store_true",
                    help="read every step's tokens before the next step is launched")
+    p.add_argument("--no-prefix-caching", action="store_true",
+                   help="requests do not share the cache pages of a common prefix")
 
 
 def _engine(args):
@@ -44,7 +46,8 @@ def _engine(args):
         model_path=args.model_path, dtype=args.dtype, max_num_batched_tokens=args.max_num_batched_tokens,
         max_num_seqs=args.max_num_seqs, max_seq_len=args.max_seq_len,
         gpu_memory_utilization=args.gpu_memory_utilization, kvcache_block_size=args.kvcache_block_size,
-        num_kvcache_blocks=args.num_kvcache_blocks, pipeline_decode=not args.no_pipeline_decode))
+        num_kvcache_blocks=args.num_kvcache_blocks, pipeline_decode=not args.no_pipeline_decode,
+        enable_prefix_caching=False if args.no_prefix_caching else None))
 
 
 def _params(args, n):
@@ -61,10 +64,12 @@ def _report(engine, outs, wall):
             "%.3f ms" % (o.tpot * 1e3) if o.tpot else "-", o.evictions))
     pf = st["prefill_tokens"] / st["prefill_time"] if st["prefill_time"] else 0.0
     dc = st["decode_tokens"] / st["decode_time"] if st["decode_time"] else 0.0
-    sys.stderr.write("steps=%d (launched ahead: %d) prefill=%.1f tok/s decode=%.1f tok/s wall=%.3f s evictions=%d\n"
-                     % (st["steps"], st["steps_launched_ahead"], pf, dc, wall, engine.scheduler.num_evictions))
+    shared = engine.runner.cache.prefix_hit_tokens
+    sys.stderr.write("steps=%d (launched ahead: %d) prefill=%.1f tok/s decode=%.1f tok/s wall=%.3f s evictions=%d "
+                     "prompt tokens found in the cache=%d\n"
+                     % (st["steps"], st["steps_launched_ahead"], pf, dc, wall, engine.scheduler.num_evictions, shared))
     return dict(steps=st["steps"], steps_launched_ahead=st["steps_launched_ahead"], prefill_tok_s=pf, decode_tok_s=dc,
-                wall_s=wall)
+                wall_s=wall, prefix_hit_tokens=shared)
 
 
 def cmd_generate(args):
@@ -93,7 +98,8 @@ def cmd_benchmark(args):
     vocab = min(engine.runner.vocab_size, 10001)
     prompts = [[rng.randrange(vocab) for _ in range(args.prompt_len)] for _ in range(args.num_prompts)]
     args.ignore_eos = True
-    engine.generate(prompts[:2], _params(args, 2))
+    # the warm-up has prompts of its own: the timed run finds nothing of its prompts in the cache
+    engine.generate([[rng.randrange(vocab) for _ in range(args.prompt_len)] for _ in range(2)], _params(args, 2))
     for k in engine.stats:
         engine.stats[k] = 0 if isinstance(engine.stats[k], int) else 0.0
     t0 = time.perf_counter()

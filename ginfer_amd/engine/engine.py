@@ -24,6 +24,9 @@ class EngineConfig:
     kvcache_block_size: int = 16          # tokens per cache page
     num_kvcache_blocks: Optional[int] = None   # pages per cache group; None: from free memory
     pipeline_decode: bool = True          # launch a decode step before the tokens of the step before it are read
+    # requests share the cache pages of a common prefix (ginfer/engine/block_manager.cc:63-110, where it cannot be
+    # switched off).  None: wherever the model allows it (no window, no per-request state); True: or refuse
+    enable_prefix_caching: Optional[bool] = None
 
 
 @dataclass
@@ -43,7 +46,8 @@ class Engine:
         self.runner = ModelRunner(config.model_path, dtype=config.dtype, page_size=config.kvcache_block_size,
                                   num_pages=config.num_kvcache_blocks, max_requests=config.max_num_seqs,
                                   max_model_len=config.max_seq_len,
-                                  gpu_memory_utilization=config.gpu_memory_utilization)
+                                  gpu_memory_utilization=config.gpu_memory_utilization,
+                                  prefix_caching=config.enable_prefix_caching)
         self.scheduler = Scheduler(self.runner.cache, config.max_num_seqs, config.max_num_batched_tokens,
                                    self.runner.spec.eos_token_ids, self.runner.max_model_len)
         self.sampler = Sampler(self.runner.device)
@@ -92,7 +96,7 @@ class Engine:
             host[:tokens.shape[0]].copy_(tokens, non_blocking=True)
             event.record()
             arrival = (host, event, tokens.shape[0])
-        n_prefill = sum(sc.num_tokens for sc in scheduled if sc.num_tokens > 1 or sc.seq.num_computed == 0)
+        n_prefill = sum(sc.num_tokens for sc in scheduled if not sc.seq.decoding)   # prompts, and evicted requests fed again
         self.scheduler.advance(scheduled)
         return dict(scheduled=scheduled, tokens=tokens, arrival=arrival, n_prefill=n_prefill,
                     n_decode=sum(sc.num_tokens for sc in scheduled) - n_prefill)

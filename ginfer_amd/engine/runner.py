@@ -38,7 +38,8 @@ def require_gpu():
 
 class ModelRunner:
     def __init__(self, model_path, dtype="bfloat16", page_size=16, num_pages=None, max_requests=64,
-                 max_model_len=None, gpu_memory_utilization=0.9, device=None, config=None, use_graphs=True):
+                 max_model_len=None, gpu_memory_utilization=0.9, device=None, config=None, use_graphs=True,
+                 prefix_caching=False):
         self.device = device or require_gpu()
         if dtype not in DTYPES:
             raise ValueError("dtype must be one of %s, got %r" % (sorted(DTYPES), dtype))
@@ -56,7 +57,9 @@ class ModelRunner:
         specs = self.model.cache_specs()
         if num_pages is None:
             num_pages = self._pages_from_free_memory(specs, gpu_memory_utilization)
-        self.cache = CacheManager(specs, self.page_size, int(num_pages), int(max_requests))
+        if prefix_caching is None:       # where the model allows it
+            prefix_caching = CacheManager.supports_prefix_caching(specs)
+        self.cache = CacheManager(specs, self.page_size, int(num_pages), int(max_requests), prefix_caching=prefix_caching)
         self.cache.allocate_device(self.dtype, self.device)
         self._owner_of = [i if e.cache_of is None else e.cache_of for i, e in enumerate(self.model.schedule)]
         self._buffers = _BufferCache(len(self.cache.groups), self.device)

@@ -6,7 +6,9 @@ then what is left of the budget goes to prompt portions, first of running reques
 not through yet, then of waiting requests in arrival order, while fewer than max_num_seqs requests
 run and a state slot is free.  A portion is cut to what the budget and the free pages allow.  The
 reference runs prompts whole and never beside decoding (ginfer/engine/scheduler.cc:20-71); its queues,
-its finishing rule (:83-99) and its answer to a full cache are kept:
+its finishing rule (:83-99) and its answer to a full cache are kept.  A request is admitted with its tokens:
+where the cache shares prefixes it starts behind the part that the cache already holds
+(ginfer/engine/block_manager.cc:83-96), an evicted request behind what is left of its own pages.
 
 When pages run out for a decoding request, the newest running request is evicted: its pages are given
 back, it keeps its tokens, returns to the FRONT of the waiting queue and is later fed again from its
@@ -110,10 +112,12 @@ class Scheduler:
         # 3. admissions in arrival order; no skipping ahead of the head of the queue
         while self.waiting and budget > 0 and len(self.running) < self.max_num_seqs and cache.can_admit():
             seq = self.waiting[0]
-            cache.admit(seq.request_id)
+            cache.admit(seq.request_id, seq.token_ids)
+            seq.num_computed = cache.length(seq.request_id)     # a known prefix is in the cache already
             n = self._portion(seq, budget)
             if n == 0:
                 cache.release(seq.request_id)
+                seq.num_computed = 0
                 break
             self.waiting.popleft()
             seq.state = State.RUNNING
@@ -142,10 +146,11 @@ class Scheduler:
         return 0
 
     def _evict(self, seq):
-        self.cache.release(seq.request_id)
+        self.cache.release(seq.request_id, seq.token_ids)
         self.running.remove(seq)
         seq.state = State.WAITING
         seq.num_computed = 0
+        seq.decoding = False
         seq.evictions += 1
         self.num_evictions += 1
         self.waiting.appendleft(seq)
@@ -164,8 +169,10 @@ class Scheduler:
         for sc in scheduled:
             rid = sc.seq.request_id
             if cache.pending(rid):
-                cache.commit(rid)
+                cache.commit(rid, sc.seq.token_ids)
             sc.seq.num_computed += sc.num_tokens
+            if sc.samples:
+                sc.seq.decoding = True
 
     def absorb(self, scheduled: List[Scheduled], tokens: List[int], now=None) -> List[Sequence]:
         """The step's sampled tokens have arrived (one for every item that samples, in order): appends them and
@@ -193,7 +200,7 @@ class Scheduler:
                 reason = "max_model_len"
             if reason:
                 seq.state, seq.finish_reason, seq.finish_ts = State.FINISHED, reason, now
-                self.cache.release(seq.request_id)
+                self.cache.release(seq.request_id, seq.token_ids)
                 self.running.remove(seq)
                 finished.append(seq)
         return finished

@@ -22,6 +22,7 @@ class Sequence:
     params: SamplingParams
     state: State = State.WAITING
     num_computed: int = 0                # tokens whose keys and values are in the cache
+    decoding: bool = False               # every known token has been handed to the device; it gets one a step now
     finish_reason: Optional[str] = None
     evictions: int = 0
     request_ts: float = field(default_factory=time.perf_counter)

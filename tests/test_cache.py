@@ -28,6 +28,21 @@ def test_page_pool():
     assert sorted(p.held()) == [0, 1, 2, 3]
 
 
+def test_page_pool_with_several_holders():
+    p = PagePool(3)
+    assert p.take(2) == [0, 1]
+    p.share(0)
+    assert p.holders(0) == 2
+    p.give_back([0])
+    assert p.holders(0) == 1 and p.num_free == 1          # still held by the other
+    p.give_back([0, 1])
+    assert p.num_free == 3
+    p.share(0)                                            # out of the free queue again, with what it held
+    assert p.holders(0) == 1 and p.num_free == 2 and p.take(2) == [2, 1]
+    with pytest.raises(ValueError, match="not held"):
+        p.give_back([2, 2])
+
+
 def test_slot_pool():
     s = SlotPool(2)
     assert (s.take(), s.take()) == (0, 1)
@@ -67,7 +82,8 @@ def test_append_commit_release_and_reuse():
     m.release("a")
     m.check()
     m.append("b", 40)
-    assert m.table("b", 0) == [4, 5, 0, 1, 2]    # the pages of "a" are used again, after those that were free
+    # the pages of "a" are used again, after those that were free; the pages of its end first
+    assert m.table("b", 0) == [4, 5, 3, 2, 1]
     with pytest.raises(ValueError, match="already"):
         m.admit("b")
     m.admit("c")
@@ -148,3 +164,139 @@ def test_random_orders_keep_every_page_accounted(seed):
         m.release(rid)
     m.check()
     assert all(g.pool.num_free == g.pool.num_pages for g in m.groups) and m.slots.num_free == 4
+
+
+# ---- shared prefixes
+
+def _run(m, rid, tokens, upto=None):
+    """Appends and commits the request's tokens from its length up to `upto`."""
+    upto = len(tokens) if upto is None else upto
+    n = upto - m.length(rid)
+    if n > 0:
+        m.append(rid, n)
+        m.commit(rid, tokens)
+
+
+def test_prefix_is_shared_exactly():
+    m = CacheManager([FULL], page_size=8, num_pages=8, max_requests=3, prefix_caching=True)
+    a = list(range(100, 120))                      # 20 tokens: two full pages and a half
+    m.admit("a", a)
+    assert m.length("a") == 0
+    _run(m, "a", a)
+    assert m.table("a", 0) == [0, 1, 2]
+    b = a[:16] + [7, 7, 7]
+    m.admit("b", b)
+    assert m.length("b") == 16 and m.table("b", 0) == [0, 1] and m.prefix_hit_tokens == 16
+    assert m.groups[0].pool.holders(0) == 2 and m.groups[0].pool.holders(2) == 1
+    m.check()
+    _run(m, "b", b)
+    assert m.table("b", 0) == [0, 1, 3]            # its own page from the first token that differs
+    m.release("a", a)
+    assert m.groups[0].pool.holders(0) == 1 and m.groups[0].pool.num_free == 5
+    # a prompt that ends at a page's edge: its last token is left to run, so the last page is not taken over
+    m.admit("c", a[:16])
+    assert m.length("c") == 8 and m.table("c", 0) == [0]
+    m.release("c", a[:16])
+    # tokens that differ inside the first page: nothing is shared, although later pages would match
+    d = [1] + a[1:]
+    m.admit("d", d)
+    assert m.length("d") == 0
+    m.release("d")
+    m.release("b", b)
+    m.check()
+    assert m.groups[0].pool.num_free == 8
+    # everything is free, and still remembered: the same prompt finds its pages again
+    m.admit("e", a)
+    assert m.length("e") == 16 and m.table("e", 0) == [0, 1]
+    m.check()
+
+
+def test_a_page_taken_for_something_else_is_forgotten_with_what_follows_it():
+    m = CacheManager([FULL], page_size=4, num_pages=4, max_requests=2, prefix_caching=True)
+    a = [1, 2, 3, 4, 5, 6, 7, 8, 9]
+    m.admit("a", a)
+    _run(m, "a", a)                                # pages 0, 1 full, 2 begun
+    m.release("a", a)                              # free queue: 3, then a's pages from its end: 2, 1, 0
+    x = [9] * 13
+    m.admit("x", x)
+    _run(m, "x", x)                                # takes all four pages: a's are forgotten
+    m.release("x")                                 # without tokens: nothing of x is remembered
+    m.admit("b", a)
+    assert m.length("b") == 0
+    _run(m, "b", a, upto=4)                        # the first block again, under a new number
+    m.admit("c", a)
+    assert m.length("c") == 4                      # the second block of "a" is not found behind the new first one
+    m.check()
+
+
+def test_without_tokens_nothing_is_shared():
+    m = CacheManager([FULL], page_size=4, num_pages=6, max_requests=2, prefix_caching=True)
+    a = list(range(9))
+    m.admit("a")
+    m.append("a", 9)
+    m.commit("a")
+    m.release("a")
+    m.admit("b", a)
+    assert m.length("b") == 0
+    with pytest.raises(ValueError, match="window or with per-request state"):
+        CacheManager([FULL, WIN], page_size=4, num_pages=6, max_requests=2, prefix_caching=True)
+    with pytest.raises(ValueError, match="window or with per-request state"):
+        CacheManager([FULL, StateSpec((4,), torch.float32)], page_size=4, num_pages=6, max_requests=2, prefix_caching=True)
+    assert not CacheManager.supports_prefix_caching([None]) and CacheManager.supports_prefix_caching([FULL, None])
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_random_orders_with_shared_prefixes(seed):
+    """Requests whose token lists share beginnings come and go in random order.  A shadow of what every page holds
+    (the whole sequence up to the page's end, as the request that wrote it knew it) shows that a page taken over
+    holds exactly the newcomer's own beginning."""
+    rng = random.Random(100 + seed)
+    ps = rng.choice([2, 4, 8])
+    specs = [FULL, None, KVCacheSpec(1, 32, None)]
+    m = CacheManager(specs, page_size=ps, num_pages=rng.choice([10, 24]), max_requests=4, prefix_caching=True)
+    stems = [[rng.randrange(3) for _ in range(40)] for _ in range(3)]
+    shadow = [dict() for _ in m.groups]
+    live, tokens, next_id, hits = [], {}, 0, 0
+    for _ in range(800):
+        op = rng.random()
+        if op < 0.25 and m.can_admit():
+            stem = rng.choice(stems)
+            cut = rng.randrange(1, 40)
+            toks = stem[:cut] + [rng.randrange(3) for _ in range(rng.randrange(0, 12))]
+            m.admit(next_id, toks)
+            got = m.length(next_id)
+            assert got % ps == 0 and got <= len(toks) - 1
+            for gi in range(len(m.groups)):
+                for i, page in enumerate(m.table(next_id, gi)):
+                    assert shadow[gi][page] == toks[:(i + 1) * ps]
+            hits += got
+            live.append(next_id)
+            tokens[next_id] = toks
+            next_id += 1
+        elif op < 0.8 and live:
+            rid = rng.choice(live)
+            toks = tokens[rid]
+            start = m.length(rid)
+            n = min(rng.choice([1, 1, 2, 3, 7, 20]), len(toks) - start)
+            if n == 0:                                   # decoding: a new token becomes known
+                toks.append(rng.randrange(3))
+                n = 1
+            try:
+                m.append(rid, n)
+            except OutOfPages:
+                m.check()
+                continue
+            for gi in range(len(m.groups)):
+                t = m.table(rid, gi)
+                for blk in range(start // ps, (start + n - 1) // ps + 1):
+                    shadow[gi][t[blk]] = toks[:min(start + n, (blk + 1) * ps)]
+            m.commit(rid, toks if rng.random() < 0.8 else None)
+        elif live:
+            rid = live.pop(rng.randrange(len(live)))
+            m.release(rid, tokens[rid] if rng.random() < 0.8 else None)
+        m.check()
+    for rid in live:
+        m.release(rid, tokens[rid])
+    m.check()
+    assert all(g.pool.num_free == g.pool.num_pages for g in m.groups) and m.slots.num_free == 4
+    assert hits > 0 and hits == m.prefix_hit_tokens

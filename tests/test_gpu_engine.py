@@ -116,11 +116,16 @@ def test_greedy_generation_through_the_entry_point(folders, dtype):
     outs = eng.generate(prompts, SamplingParams(max_tokens=12, ignore_eos=True))
     eng.runner.cache.check()
     assert not eng.runner.cache.requests
-    cfg, w = pm.read_config(folder), pm.read_weights(folder)
     for p, o in zip(prompts, outs):
         assert o.prompt_token_ids == p and len(o.token_ids) == 12 and o.finish_reason == "max_tokens"
-        # every generated token is the plain implementation's greedy choice given the engine's own
-        # prefix, unless the plain top two are within rounding of each other
+    _greedy_as_plain(folder, prompts, outs, dtype)
+
+
+def _greedy_as_plain(folder, prompts, outs, dtype):
+    """Every generated token is the plain implementation's greedy choice given the engine's own prefix, unless the
+    plain top two are within rounding of each other."""
+    cfg, w = pm.read_config(folder), pm.read_weights(folder)
+    for p, o in zip(prompts, outs):
         ids = p + o.token_ids
         logits = pm.forward(cfg, w, ids[:-1])
         for k, tok in enumerate(o.token_ids):
@@ -129,6 +134,57 @@ def test_greedy_generation_through_the_entry_point(folders, dtype):
             if tok != best:
                 gap = float(row[best] - row[tok]) / float(row.abs().max())
                 assert gap <= H.TOL[dtype], "token %d of prompt %d: engine %d, plain %d, gap %.3g" % (k, len(p), tok, best, gap)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_requests_that_share_a_prefix_share_its_pages(folders, dtype):
+    """A request whose first tokens the cache already holds (from a request before it, finished or still running)
+    starts behind them.  Its tokens are the plain implementation's, and in 32-bit the same, bit for bit, as
+    without sharing; fewer prompt tokens are run."""
+    from ginfer_amd import Engine, EngineConfig, SamplingParams
+    name = "B"
+    folder = folders[name]
+    vocab = H.TINY[name][0]["vocab_size"]
+    stem = H.random_tokens(70, vocab, 1200)
+    first = [stem[:50], H.random_tokens(23, vocab, 1201)]
+    # the whole first prompt again; its beginning with another end; one that leaves the stem inside the first page;
+    # the first request's prompt and output as a prompt (a conversation that goes on)
+    later = [stem[:50], stem[:41] + H.random_tokens(9, vocab, 1202), stem[:5] + H.random_tokens(30, vocab, 1203), None,
+             stem[:64]]
+    results = {}
+    for share in (True, False):
+        eng = Engine(EngineConfig(model_path=folder, dtype=dtype, max_num_batched_tokens=32, max_num_seqs=4,
+                                  max_seq_len=256, kvcache_block_size=8, num_kvcache_blocks=60,
+                                  enable_prefix_caching=share))
+        sp = SamplingParams(max_tokens=10, ignore_eos=True)
+        outs = eng.generate(first, sp)
+        prompts = [p if p is not None else first[0] + outs[0].token_ids for p in later]
+        # the last one arrives while the others run: it finds pages of a request that is still running
+        ids = [eng.add_request(p, SamplingParams(max_tokens=10, ignore_eos=True)) for p in prompts[:4]]
+        done, steps = {}, 0
+        while eng.has_unfinished():
+            for o in eng.step():
+                done[o.request_id] = o
+            steps += 1
+            if steps == 3:
+                ids.append(eng.add_request(prompts[4], SamplingParams(max_tokens=10, ignore_eos=True)))
+        eng.runner.cache.check()
+        assert not eng.runner.cache.requests
+        outs2 = [done[i] for i in ids]
+        _greedy_as_plain(folder, first + prompts, outs + outs2, dtype)
+        results[share] = ([o.token_ids for o in outs + outs2], eng.runner.cache.prefix_hit_tokens, eng.stats["prefill_tokens"])
+    (shared, hits, ran), (alone, no_hits, ran_alone) = results[True], results[False]
+    # pages of 8: 48 of 50, 40 of 41, none of 5, 56 of the 60 of prompt and output, 48 of 64 (what the first holds)
+    assert hits == 48 + 40 + 0 + 56 + 48 and no_hits == 0
+    assert ran == ran_alone - hits
+    if dtype == "float32":
+        assert shared == alone
+    # a model with a window cannot share: asked for, it is refused; left open, it goes without
+    with pytest.raises(ValueError, match="window"):
+        Engine(EngineConfig(model_path=folders["C"], dtype=dtype, max_seq_len=128, num_kvcache_blocks=20,
+                            enable_prefix_caching=True))
+    assert not Engine(EngineConfig(model_path=folders["C"], dtype=dtype, max_seq_len=128,
+                                   num_kvcache_blocks=20)).runner.cache.prefix_caching
 
 
 def test_temperature_sampling_matches_plain_with_same_uniforms(folders):

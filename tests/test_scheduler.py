@@ -11,8 +11,9 @@ from ginfer_amd.parts import KVCacheSpec
 from ginfer_amd.sampling import SamplingParams, uniform
 
 
-def make(num_pages, page_size=4, max_num_seqs=4, budget=16, eos=(999,), max_model_len=256, window=None):
-    cache = CacheManager([KVCacheSpec(1, 16, window)], page_size, num_pages, max_num_seqs)
+def make(num_pages, page_size=4, max_num_seqs=4, budget=16, eos=(999,), max_model_len=256, window=None,
+         prefix_caching=False):
+    cache = CacheManager([KVCacheSpec(1, 16, window)], page_size, num_pages, max_num_seqs, prefix_caching=prefix_caching)
     return Scheduler(cache, max_num_seqs, budget, eos, max_model_len), cache
 
 
@@ -288,3 +289,58 @@ def test_no_step_ahead_without_pages_and_nothing_stays_reserved():
         assert steps < 200
     assert refused_for_pages >= 1 and sched.num_evictions >= 1
     assert {s.request_id: s.token_ids for s in done} == want
+
+
+# ---- requests that share a prefix
+
+def test_a_request_starts_behind_the_prefix_that_the_cache_holds():
+    sched, cache = make(num_pages=16, budget=32, prefix_caching=True)
+    a = seq(0, 10, max_tokens=3)
+    done, steps = run(sched, cache, [a])
+    assert steps[0] == [(0, 10)] and done[0].token_ids == expected(a)
+    # the same prompt with another end: two pages of four are known, the rest runs
+    b = Sequence(1, a.token_ids[:9] + [5, 6, 7], 12, SamplingParams(max_tokens=3))
+    # the whole of a's prompt and output again: everything up to the last full page is known
+    c = Sequence(2, list(a.token_ids), len(a.token_ids), SamplingParams(max_tokens=2))
+    done, steps = run(sched, cache, [b, c])
+    assert steps[0] == [(1, 4), (2, 1)]
+    assert cache.prefix_hit_tokens == 8 + 12
+    assert {s.request_id: s.token_ids for s in done} == {1: expected(b), 2: expected(c)}
+    assert all(g.pool.num_free == g.pool.num_pages for g in cache.groups)
+
+
+def test_an_evicted_request_finds_its_own_pages_again():
+    sched, cache = make(num_pages=8, page_size=4, max_num_seqs=2, budget=32, prefix_caching=True)
+    a, b = seq(0, 9, max_tokens=12), seq(1, 9, max_tokens=12)
+    fed_again = []
+
+    def check(batch):
+        for sc in batch:
+            if sc.seq is b and sc.seq.evictions and sc.num_tokens > 1:
+                fed_again.append((sc.seq.num_computed, sc.num_tokens))
+
+    done, steps = run(sched, cache, [a, b], check=check)
+    assert b.evictions == 1 and a.evictions == 0
+    # b is fed again from behind the pages of its own that nobody had taken meanwhile, not from its first token
+    assert fed_again and fed_again[0][0] > 0 and fed_again[0][0] % 4 == 0
+    assert {s.request_id: s.token_ids for s in done} == {0: expected(a), 1: expected(b)}
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_workloads_with_shared_prefixes_finish_with_the_same_tokens(seed):
+    rng = random.Random(50 + seed)
+    sched, cache = make(num_pages=rng.choice([16, 24, 40]), page_size=rng.choice([2, 4, 8]),
+                        max_num_seqs=rng.choice([2, 4]), budget=rng.choice([8, 24, 64]), prefix_caching=True)
+    stems = [[rng.randrange(900) for _ in range(40)] for _ in range(2)]
+    seqs = []
+    for i in range(14):
+        ids = rng.choice(stems)[:rng.randint(1, 14)] + [rng.randrange(900) for _ in range(rng.randint(0, 6))]
+        seqs.append(Sequence(i, ids, len(ids), SamplingParams(max_tokens=rng.randint(1, 12))))
+    want = {s.request_id: expected(s) for s in seqs}
+    if seed % 2:
+        done, _ = run_ahead(sched, cache, seqs)
+    else:
+        done, _ = run(sched, cache, seqs)
+    assert {s.request_id: s.token_ids for s in done} == want
+    assert cache.prefix_hit_tokens > 0
+    assert not cache.requests and all(g.pool.num_free == g.pool.num_pages for g in cache.groups)
