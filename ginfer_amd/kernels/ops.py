@@ -491,6 +491,9 @@ def paged_attention_mfma(q, k_pages, v_pages, block_table, step, num_heads, num_
           "the matrix-core attention kernels take bfloat16, head sizes in steps of 16 up to 256 and page sizes that "
           "are powers of two from 8; got %s, head %d, page %d" % (q.dtype, head_dim, page_size))
     _need(q.stride(0) % 8 == 0 and q.data_ptr() % 16 == 0, "q rows must be 16-byte aligned")
+    _need(k_pages.shape[0] * num_kv_heads * max(page_size, head_dim) < 2 ** 31,
+          "the matrix-core attention kernels count the rows of a layer's cache in 32 bits: %d pages x %d kv heads x "
+          "%d is too many" % (k_pages.shape[0], num_kv_heads, max(page_size, head_dim)))
     lib = build.load("attention_mfma", {"HEAD_DIM": head_dim})
     _need(lib.ga_attn_head_dim() == head_dim, "attention library was built for another head size")
     # rows of a prompt portion per wavefront: 32 where the kernel has it and the step is long, else 16
