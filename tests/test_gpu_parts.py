@@ -309,6 +309,150 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped(tmp_path):
             assert err < 1e-4, "request %s position %d: %.3g" % (rid, p, err)
 
 
+def _register_routed_toy():
+    """A second toy architecture defined here, in the test: a feed-forward that routes every token to one of
+    three experts (router logits in 32-bit), in one layer only, beside the package's dense one in the other; and
+    a position encoding of its own (rotation by a fraction of the position), used by one layer's attention while
+    the other keeps the package's.  None of it touches the package's files."""
+    from ginfer_amd.config import register_architecture, PartSpec, LayerSpec, ScheduleEntry, ModelSpec
+    from ginfer_amd.parts import register_feed_forward, register_position, Part
+    from ginfer_amd.weights import WeightSpec
+
+    @register_position("toy_slow_rotation")
+    class SlowRotation(Part):
+        """Rotary tables of the angle (p / slow) * inv_freq: what the attention kernels need is the tables."""
+        capturable = True
+
+        def __init__(self, theta, rotary_dim, max_positions, slow, dtype=None, device=None):
+            self.theta, self.rotary_dim, self.max_positions, self.slow = float(theta), int(rotary_dim), int(max_positions), float(slow)
+            self.device, self._limit, self._tables = device, None, None
+
+        def limit_positions(self, n):
+            self._limit, self._tables = min(self.max_positions, int(n)), None
+
+        def tables(self):
+            if self._tables is None:
+                half = self.rotary_dim // 2
+                inv = 1.0 / torch.pow(torch.tensor(self.theta, dtype=torch.float32), torch.arange(half, dtype=torch.float32) / half)
+                ang = (torch.arange(self._limit or self.max_positions, dtype=torch.float32) / self.slow)[:, None] * inv[None, :]
+                self._tables = (torch.cos(ang).to(self.device).contiguous(), torch.sin(ang).to(self.device).contiguous())
+            return self._tables
+
+    @register_feed_forward("toy_one_of_n")
+    class OneOfN(Part):
+        """y = p_e * W2_e . relu(W1_e . x) for the expert e with the largest router logit, p_e its softmax weight
+        (32-bit).  Routing is a function of the token alone."""
+
+        def __init__(self, hidden_size, intermediate_size, num_experts, dtype, device):
+            self.H, self.I, self.E, self.dtype, self.device = hidden_size, intermediate_size, num_experts, dtype, device
+
+        def weight_specs(self):
+            specs = {"router.weight": WeightSpec((self.E, self.H), keep_32bit=True)}
+            for e in range(self.E):
+                specs["experts.%d.w1.weight" % e] = WeightSpec((self.I, self.H))
+                specs["experts.%d.w2.weight" % e] = WeightSpec((self.H, self.I))
+            return specs
+
+        def bind_weights(self, t):
+            self.router = t["router.weight"]
+            self.w1 = torch.stack([t["experts.%d.w1.weight" % e] for e in range(self.E)])
+            self.w2 = torch.stack([t["experts.%d.w2.weight" % e] for e in range(self.E)])
+
+        def forward(self, x):
+            logits = x.float() @ self.router.float().t()
+            prob, choice = torch.softmax(logits, dim=-1).max(dim=-1)
+            hidden = torch.relu(torch.einsum("th,tih->ti", x, self.w1[choice]))
+            return (torch.einsum("ti,thi->th", hidden, self.w2[choice]).float() * prob[:, None]).to(x.dtype)
+
+    @register_architecture("ToyRoutedLM")
+    @dataclass
+    class ToyRoutedConfig:
+        hidden_size: int = 40
+        vocab_size: int = 173
+        architecture = "ToyRoutedLM"
+
+        @classmethod
+        def from_dict(cls, d):
+            return cls(d["hidden_size"], d["vocab_size"])
+
+        def to_dict(self):
+            return dict(architectures=["ToyRoutedLM"], hidden_size=self.hidden_size, vocab_size=self.vocab_size)
+
+        def model_spec(self):
+            Hd = self.hidden_size
+            norm = PartSpec("rmsnorm", dict(size=Hd, eps=1e-6))
+            slow = PartSpec("toy_slow_rotation", dict(theta=500.0, rotary_dim=16, max_positions=128, slow=4.0))
+            rope = PartSpec("rope_neox", dict(theta=500.0, rotary_dim=16, max_positions=128))
+
+            def attn(pos):
+                return PartSpec("attention", dict(hidden_size=Hd, num_heads=2, num_kv_heads=2, head_dim=16, qkv_bias=True,
+                                                  out_bias=False, window=None, position=pos, scale=None))
+            dense = PartSpec("swiglu", dict(hidden_size=Hd, intermediate_size=56))
+            routed = PartSpec("toy_one_of_n", dict(hidden_size=Hd, intermediate_size=24, num_experts=3))
+            layers = [LayerSpec("model.layers.0", attn(slow), routed, norm, norm),
+                      LayerSpec("model.layers.1", attn(rope), dense, norm, norm)]
+            return ModelSpec(hidden_size=Hd, vocab_size=self.vocab_size, layers=layers,
+                             schedule=[ScheduleEntry(0), ScheduleEntry(1)],
+                             embedding=PartSpec("embedding", dict(vocab_size=self.vocab_size, hidden_size=Hd)),
+                             final_norm=norm, head=PartSpec("lm_head", dict(vocab_size=self.vocab_size, hidden_size=Hd,
+                                                                            tied=False)),
+                             max_positions=128, eos_token_ids=[0])
+    return ToyRoutedConfig
+
+
+def _routed_toy_plain(folder, ids):
+    w = pm.read_weights(folder)
+    T = len(ids)
+    cfg = dict(num_attention_heads=2, num_key_value_heads=2, head_dim=16)
+    half = 8
+    inv = 1.0 / torch.pow(torch.tensor(500.0, dtype=torch.float32), torch.arange(half, dtype=torch.float32) / half)
+    slow_ang = (torch.arange(T, dtype=torch.float32) / 4.0)[:, None] * inv[None, :]
+    tables = {0: (torch.sin(slow_ang).double(), torch.cos(slow_ang).double()), 1: pm.rope_tables(500.0, 16, T)}
+    x = pm.embedding(w["model.embed_tokens.weight"], ids)
+    choices = None
+    for layer in (0, 1):
+        p = "model.layers.%d" % layer
+        n = pm.rms_norm(x, w[p + ".input_layernorm.weight"], 1e-6)
+        sin, cos = tables[layer]
+        a, _ = pm.attention_block(n, w, p + ".self_attn", cfg, list(range(T)), sin, cos, None)
+        h = x + a
+        n = pm.rms_norm(h, w[p + ".post_attention_layernorm.weight"], 1e-6)
+        if layer == 0:
+            prob = torch.softmax(n @ w[p + ".mlp.router.weight"].t(), dim=-1)
+            choices = prob.argmax(dim=-1)
+            out = torch.zeros_like(n)
+            for t in range(T):
+                e = int(choices[t])
+                hid = torch.relu(w[p + ".mlp.experts.%d.w1.weight" % e] @ n[t])
+                out[t] = prob[t, e] * (w[p + ".mlp.experts.%d.w2.weight" % e] @ hid)
+            x = h + out
+        else:
+            x = h + pm.feed_forward(n, w, p + ".mlp")
+    return pm.linear(pm.rms_norm(x, w["model.norm.weight"], 1e-6), w["lm_head.weight"]).float().numpy(), choices
+
+
+def test_toy_routed_feed_forward_and_toy_position_encoding(tmp_path):
+    """Layers of one model with different feed-forwards and different position encodings, both toys registered
+    here: built from the configuration, stepped whole, in portions and mixed, against a plain statement of them."""
+    from ginfer_amd import ModelRunner, write_random_model, config_from_folder
+    Toy = _register_routed_toy()
+    folder = write_random_model(str(tmp_path / "routed"), Toy(), seed=9, dtype="float32")
+    assert type(config_from_folder(folder)).__name__ == "ToyRoutedConfig"
+    reqs = {"a": H.random_tokens(45, 173, 11), "b": H.random_tokens(18, 173, 12), "c": H.random_tokens(31, 173, 13)}
+    runner = ModelRunner(folder, dtype="float32", page_size=8, num_pages=24, max_requests=3)
+    assert len(runner.model.position_parts()) == 2                  # one table set per encoding
+    assert not runner.use_graphs                                     # the toy says nothing of being recordable
+    refs = {rid: _routed_toy_plain(folder, ids) for rid, ids in reqs.items()}
+    assert len({int(c) for _, ch in refs.values() for c in ch}) == 3  # every expert is used
+    for steps in (H.steps_whole(reqs), H.steps_portions(reqs, sizes=(7, 2, 13)), H.steps_mixed(reqs, max_live=3, seed=2)):
+        got = H.run_steps(runner, steps)
+        runner.cache.check()
+        for (rid, p), row in got.items():
+            ref = refs[rid][0]
+            err = np.abs(row - ref[p]).max() / np.abs(ref).max()
+            assert err < 1e-4, "request %s position %d: %.3g" % (rid, p, err)
+
+
 def test_schedule_names_a_layer_twice_and_shares_a_cache(tmp_path):
     """The order of layers is data: a Qwen2 folder run with another schedule."""
     from ginfer_amd import ModelRunner, config_from_folder
