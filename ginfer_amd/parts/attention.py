@@ -10,6 +10,14 @@ from .linear import linear, linear_into_norm
 from .registry import register_mixer
 
 
+def _library_then_rotation_is_faster(rows, in_features):
+    """The fused projection kernel cannot split K over workgroups (its epilogue needs whole sums).  Measured on
+    MI355X at a 7B model's sizes (K 3584, 4608 outputs): from 17 rows on the BLAS library's product followed by
+    the rotation kernel is faster (32 rows: 17.6 us against 20.6; 64 rows: 23.4 against 28.1); at a 1.5B model's
+    (K 1536) the fused kernel stays ahead or level up to 64 rows."""
+    return rows > 16 and in_features >= 3072
+
+
 @register_mixer("attention")
 class Attention(Part):
     """q/k/v projections (one fused product over the stacked weights; results equal the three separate
@@ -67,7 +75,8 @@ class Attention(Part):
         """into_norm = (residual, norm): where the output projection's kernel can, the result is added to the
         residual here and the rows of `norm` come back as ops.ScaledRows; else the result comes back as ever."""
         cos, sin = self.position.tables()
-        if ops.qkv_rope_skinny_supported(x, self.w_qkv, self.hd, self.position.rotary_dim):
+        if (ops.qkv_rope_skinny_supported(x, self.w_qkv, self.hd, self.position.rotary_dim)
+                and not _library_then_rotation_is_faster(x.shape[0], x.shape[1])):
             # few rows (decode): projection, rotation and cache write in one kernel
             qkv = ops.qkv_rope_skinny(x, self.w_qkv, self.b_qkv, step.positions, cos, sin, cache.slot_mapping,
                                       cache.k_pages, cache.v_pages, self.nh, self.nkv, self.hd, write_kv=cache.owner)
