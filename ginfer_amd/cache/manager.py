@@ -24,6 +24,7 @@ Device layout of one group: one allocation [entries_in_group, 2 (k, v), pages, n
 entry's keys are viewed [pages, nkv, page_size, hd] and its values [pages, nkv, hd, page_size]
 (transposed inside a page, which is what the matrix-core attention kernels read fastest).
 """
+from array import array
 from dataclasses import dataclass, field
 from typing import Dict, List, Optional
 
@@ -40,6 +41,11 @@ class _Request:
     pending: int = 0                     # tokens reserved by append() and not yet committed
     tables: List[List[int]] = field(default_factory=list)   # per group: logical block -> page or -1
     contents: List[List[int]] = field(default_factory=list) # per group: content number of each remembered block
+
+
+def _block_tokens(token_ids, block, page_size):
+    """The tokens of one full block as a key: their 32-bit values as bytes (compact, and compared exactly)."""
+    return array("i", token_ids[block * page_size:(block + 1) * page_size]).tobytes()
 
 
 class CacheGroup:
@@ -177,7 +183,7 @@ class CacheManager:
         for g in self.groups:
             chain, before = [], 0
             for i in range(blocks):
-                hit = g.lookup(before, tuple(token_ids[i * ps:(i + 1) * ps]))
+                hit = g.lookup(before, _block_tokens(token_ids, i, ps))
                 if hit is None:
                     break
                 chain.append(hit)
@@ -203,7 +209,7 @@ class CacheManager:
         for gi, g in enumerate(self.groups):
             chain, table = req.contents[gi], req.tables[gi]
             for i in range(len(chain), full):
-                chain.append(g.remember(chain[i - 1] if i else 0, tuple(token_ids[i * ps:(i + 1) * ps]), table[i]))
+                chain.append(g.remember(chain[i - 1] if i else 0, _block_tokens(token_ids, i, ps), table[i]))
 
     def _mirror_table(self, gi, req):
         table, mirror = req.tables[gi], self._table_np[gi]
