@@ -21,7 +21,7 @@ def _tensor_seed(seed, name):
     return int.from_bytes(h[:8], "little") & ((1 << 63) - 1)
 
 
-def draw(spec, seed, name, dtype):
+def draw(spec, seed, name, dtype, std_scale=1.0):
     g = torch.Generator(device="cpu")
     g.manual_seed(_tensor_seed(seed, name))
     if spec.kind == "int":
@@ -31,7 +31,7 @@ def draw(spec, seed, name, dtype):
     elif spec.init == "ones":
         t = torch.ones(spec.shape, dtype=torch.float32)
     else:
-        t = torch.empty(spec.shape, dtype=torch.float32).normal_(0.0, spec.std, generator=g)
+        t = torch.empty(spec.shape, dtype=torch.float32).normal_(0.0, spec.std * std_scale, generator=g)
         if spec.init == "one_plus_normal":
             t += 1.0
         elif spec.init != "normal":
@@ -39,8 +39,10 @@ def draw(spec, seed, name, dtype):
     return t.to(dtype)
 
 
-def write_random_model(folder, config, seed, dtype="bfloat16"):
-    """Writes `folder/config.json` and `folder/model.safetensors`; returns the folder."""
+def write_random_model(folder, config, seed, dtype="bfloat16", std_scale=1.0):
+    """Writes `folder/config.json` and `folder/model.safetensors`; returns the folder.  std_scale widens every
+    normal draw: with the usual 0.02 a tiny model's blocks add so little to the embedding that greedy generation
+    repeats one token."""
     from ..parts.model import build_model
     if dtype not in _STORAGE:
         raise ValueError("dtype must be one of %s" % sorted(_STORAGE))
@@ -52,7 +54,7 @@ def write_random_model(folder, config, seed, dtype="bfloat16"):
     model = build_model(config.model_spec(), _STORAGE[dtype], device=None)
     tensors = {}
     for name, spec in model.weight_specs().items():
-        tensors[name] = draw(spec, seed, name, _STORAGE[dtype])
+        tensors[name] = draw(spec, seed, name, _STORAGE[dtype], std_scale)
     write_safetensors(os.path.join(folder, "model.safetensors"), tensors,
                       metadata={"format": "pt", "seed": seed})
     return folder

@@ -31,9 +31,9 @@ TINY_C = dict(  # explicit head_dim 48 with nh*hd != hidden, widths no power of 
 TINY = {"A": (TINY_A, 0, 16), "B": (TINY_B, 1, 8), "C": (TINY_C, 2, 16)}   # config, seed, page size
 
 
-def make_model_folder(folder, config_dict, seed, dtype="float32"):
+def make_model_folder(folder, config_dict, seed, dtype="float32", std_scale=1.0):
     from ginfer_amd import config_from_dict, write_random_model
-    return write_random_model(str(folder), config_from_dict(config_dict), seed, dtype)
+    return write_random_model(str(folder), config_from_dict(config_dict), seed, dtype, std_scale=std_scale)
 
 
 def random_tokens(n, vocab, seed):

@@ -18,6 +18,17 @@ def folders(tmp_path_factory):
     return out
 
 
+@pytest.fixture(scope="module")
+def sharp_folders(tmp_path_factory):
+    """The same configurations with every weight drawn three times as wide.  With the usual N(0, 0.02) a tiny model's
+    scores are all but equal, its attention is a plain mean of the values, and one wrong or missing key moves a logit
+    by less than bfloat16's rounding; with wide draws the softmax has peaks and such a fault shows."""
+    out = {}
+    for name, (cfg, seed, _) in H.TINY.items():
+        out[name] = H.make_model_folder(tmp_path_factory.mktemp("sharp" + name), cfg, seed, "float32", std_scale=3.0)
+    return out
+
+
 def _requests(name, lengths, seed=10):
     vocab = H.TINY[name][0]["vocab_size"]
     return {"r%d" % i: H.random_tokens(n, vocab, seed + i) for i, n in enumerate(lengths)}
@@ -33,7 +44,9 @@ LENGTHS = {"A": [5, 17, 33, 70, 131], "B": [1, 9, 40, 64, 100, 150], "C": [3, 50
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", ["A", "B", "C"])
-def test_whole_last_decoded_and_portions(folders, name, dtype):
+@pytest.mark.parametrize("weights", ["usual", "wide"])
+def test_whole_last_decoded_and_portions(folders, sharp_folders, name, dtype, weights):
+    folders = folders if weights == "usual" else sharp_folders
     reqs = _requests(name, LENGTHS[name])
     ps = H.TINY[name][2]
     runner = _runner(folders[name], name, dtype, pages=-(-256 // ps))
@@ -54,7 +67,9 @@ def test_whole_last_decoded_and_portions(folders, name, dtype):
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", ["A", "B", "C"])
-def test_mixed_with_pages_used_again(folders, name, dtype):
+@pytest.mark.parametrize("weights", ["usual", "wide"])
+def test_mixed_with_pages_used_again(folders, sharp_folders, name, dtype, weights):
+    folders = folders if weights == "usual" else sharp_folders
     lengths = {"A": [40, 75, 110, 33, 90, 61, 130], "B": [9, 100, 64, 31, 150, 77, 18], "C": [60, 97, 140, 45, 120, 80]}
     reqs = _requests(name, lengths[name], seed=40)
     steps = H.steps_mixed(reqs, max_live=4, seed=3)
