@@ -170,21 +170,11 @@ __device__ __forceinline__ void load_v_tile(bf16x8 (&vr)[DB], const bf16_t* __re
   for (int db = 0; db < DB; ++db) vr[db] = load8(vp + (int64_t)db * 16 * ps);
 }
 
-// One tile of 32 keys starting at k0, with its operands in kr and vr: scores, online softmax, output.  As soon
-// as the products that read kr (then vr) have been issued the registers are refilled with the tile k_refill
-// (< 0: none), whose pages pg holds; after that pg takes the pages of the tile k_lookup (< 0: none).
+// The steps of one tile of 32 keys starting at k0, shared by the loops that keep the tile's operands in registers
+// and the one that reads them from LDS.
+// ---- scores: S^T = K Q^T
 template <int NB>
-__device__ __forceinline__ void attend_one_tile(f32x4 (&o)[NB][DB], float (&m)[NB], float (&l)[NB],
-                                                const bf16x8 (&q)[NB][KB], const int (&cpos)[NB],
-                                                const int (&clo)[NB], bf16x8 (&kr)[2][KB], bf16x8 (&vr)[DB],
-                                                TilePages& pg, const LaneKeys& lk,
-                                                const bf16_t* __restrict__ k_pages,
-                                                const bf16_t* __restrict__ v_pages,
-                                                const int32_t* __restrict__ bt, int table_width, int kvh, int nkv,
-                                                int ps_shift, int kv_min, int kv_max, int full_lo, int full_hi,
-                                                int k0, int k_refill, int k_lookup, float scale, int c, int g) {
-  // ---- scores: S^T = K Q^T
-  f32x4 s[NB][2];
+__device__ __forceinline__ void tile_scores(f32x4 (&s)[NB][2], const bf16x8 (&kr)[2][KB], const bf16x8 (&q)[NB][KB]) {
 #pragma unroll
   for (int nb = 0; nb < NB; ++nb) {
     s[nb][0] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -197,13 +187,17 @@ __device__ __forceinline__ void attend_one_tile(f32x4 (&o)[NB][DB], float (&m)[N
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb)
         s[nb][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kr[t][kb], q[nb][kb], s[nb][t], 0, 0, 0);
-  const bool refill_edge = k_refill < kv_min || k_refill + 31 > kv_max;
-  if (k_refill >= 0) load_k_tile(kr, k_pages, pg, lk, kvh, nkv, ps_shift, k_refill, refill_edge, kv_min, kv_max, g);
-  // ---- mask and online softmax; the lane holds keys k0 + 8g + j, j = 0..7, of column c.  The running
-  // max is kept in scaled units; the scale rides on the exponent's multiply-add.  An empty column (no
-  // query: its q is zero) goes along unmasked in interior tiles; nothing of it is ever written.
+}
+
+// ---- mask and online softmax; the lane holds keys k0 + 8g + j, j = 0..7, of column c.  The running max is
+// kept in scaled units; the scale rides on the exponent's multiply-add.  An empty column (no query: its q is
+// zero) goes along unmasked in interior tiles; nothing of it is ever written.
+template <int NB>
+__device__ __forceinline__ void tile_softmax(bf16x8 (&pb)[NB], const f32x4 (&s)[NB][2], f32x4 (&o)[NB][DB],
+                                             float (&m)[NB], float (&l)[NB], const int (&cpos)[NB],
+                                             const int (&clo)[NB], int full_lo, int full_hi, int k0, float scale,
+                                             int g) {
   const bool interior = k0 >= full_lo && k0 + 31 <= full_hi;      // the same for the whole wavefront
-  bf16x8 pb[NB];
 #pragma unroll
   for (int nb = 0; nb < NB; ++nb) {
     float sv[8];
@@ -256,8 +250,13 @@ __device__ __forceinline__ void attend_one_tile(f32x4 (&o)[NB][DB], float (&m)[N
     for (int j = 0; j < 4; ++j) packed.h[j] = __builtin_convertvector(f32x2{p[2 * j], p[2 * j + 1]}, bf16x2);
     pb[nb] = packed.v;
   }
-  // ---- output: O^T += V^T P.  In a tile that reaches past the ends of the key range the values read
-  // for dead keys (anything: the slot may never have been written) are cleared: 0 * NaN is not 0.
+}
+
+// ---- output: O^T += V^T P.  In a tile that reaches past the ends of the key range the values read for dead
+// keys (anything: the slot may never have been written) are cleared first: 0 * NaN is not 0.
+template <int NB>
+__device__ __forceinline__ void tile_output(f32x4 (&o)[NB][DB], bf16x8 (&vr)[DB], const bf16x8 (&pb)[NB], int kv_min,
+                                            int kv_max, int k0, int g) {
   if (k0 < kv_min || k0 + 31 > kv_max) {
     const int kbase = k0 + 8 * g;
 #pragma unroll
@@ -275,6 +274,28 @@ __device__ __forceinline__ void attend_one_tile(f32x4 (&o)[NB][DB], float (&m)[N
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb)
       o[nb][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vr[db], pb[nb], o[nb][db], 0, 0, 0);
+}
+
+// One tile with its operands in the registers kr and vr.  As soon as the products that read kr (then vr) have
+// been issued the registers are refilled with the tile k_refill (< 0: none), whose pages pg holds; after that pg
+// takes the pages of the tile k_lookup (< 0: none).
+template <int NB>
+__device__ __forceinline__ void attend_one_tile(f32x4 (&o)[NB][DB], float (&m)[NB], float (&l)[NB],
+                                                const bf16x8 (&q)[NB][KB], const int (&cpos)[NB],
+                                                const int (&clo)[NB], bf16x8 (&kr)[2][KB], bf16x8 (&vr)[DB],
+                                                TilePages& pg, const LaneKeys& lk,
+                                                const bf16_t* __restrict__ k_pages,
+                                                const bf16_t* __restrict__ v_pages,
+                                                const int32_t* __restrict__ bt, int table_width, int kvh, int nkv,
+                                                int ps_shift, int kv_min, int kv_max, int full_lo, int full_hi,
+                                                int k0, int k_refill, int k_lookup, float scale, int c, int g) {
+  f32x4 s[NB][2];
+  tile_scores<NB>(s, kr, q);
+  const bool refill_edge = k_refill < kv_min || k_refill + 31 > kv_max;
+  if (k_refill >= 0) load_k_tile(kr, k_pages, pg, lk, kvh, nkv, ps_shift, k_refill, refill_edge, kv_min, kv_max, g);
+  bf16x8 pb[NB];
+  tile_softmax<NB>(pb, s, o, m, l, cpos, clo, full_lo, full_hi, k0, scale, g);
+  tile_output<NB>(o, vr, pb, kv_min, kv_max, k0, g);
   if (k_refill >= 0) load_v_tile(vr, v_pages, pg, lk, kvh, nkv, ps_shift, k_refill, refill_edge, kv_min, kv_max, c);
   if (k_lookup >= 0) lookup_pages(pg, bt, table_width, ps_shift, k_lookup);
 }
@@ -605,6 +626,247 @@ __global__ __launch_bounds__(64 * PREFILL_WAVES) void attn_prefill_kernel(
   }
 }
 
+// ----------------------------------------------------------------------------- prefill, operands through LDS
+// For head sizes of 64, 128 and 256.  The wavefronts of a workgroup that attend the same rows to the same key
+// tiles (the heads of a kv group, side by side) take their K and V operands from LDS, where ONE further
+// wavefront per stream of tiles, the producer, has put them with loads that go from global memory straight
+// into LDS.  What this saves is the vector memory unit's time, which is what the register kernel above waits
+// for (its time follows the number of tile visits of its wavefronts, whatever each visit computes): a load
+// instruction there brings 16 rows of 64 bytes, half a cache line each, once per head; here every instruction
+// brings whole lines, once per workgroup, and the heads read LDS.
+//   ring: per stream STAGES stages of a tile's keys (32 * HD * 2 bytes) followed by its values (as many).
+//   keys of a stage: 16-byte piece `ch` of key row r lies at piece r * CPR + (ch ^ (swz(r) mod CPR)), CPR = HD / 8
+//     pieces to a row and swz(r) = 4 * (r / 8) + r % 4: the 16 rows that one matrix-core operand takes, 8 lanes to a
+//     clock, then fall into different banks.  Values: piece g (8 keys) of dim d at piece d * 4 + g: an operand is
+//     1 KB in a row.
+//   every iteration: the producer waits for the loads of the tile the consumers are about to read, all meet at a
+//   barrier, the producer issues the loads of the tile STAGES - 1 further on into the stage that was read last.
+#if HEAD_DIM == 64 || HEAD_DIM == 128 || HEAD_DIM == 256
+#define HAVE_PREFILL_SHARED 1
+constexpr int CPR = HD / 8;
+constexpr int TILE_K_BYTES = 32 * HD * 2;
+constexpr int STAGE_BYTES = 2 * TILE_K_BYTES;
+typedef __attribute__((address_space(3))) void lds_void_t;
+typedef const __attribute__((address_space(1))) void global_void_t;
+
+__device__ __forceinline__ int swz(int r) { return ((r >> 3) << 2) | (r & 3); }
+
+template <int N>
+__device__ __forceinline__ void wait_vector_loads_but() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+// The producer's loads of one tile.  p0..p3: the pages of the tile (scalars; 0 for a page with no live key).
+__device__ __forceinline__ void produce_tile(unsigned char* stage, const bf16_t* __restrict__ k_pages,
+                                             const bf16_t* __restrict__ v_pages, int p0, int p1, int p2, int p3,
+                                             int kvh, int nkv, int ps_shift, int k0, int lane) {
+  const int ps = 1 << ps_shift;
+  const int in_page = k0 & (ps - 1);                 // not 0 only where a page holds several tiles
+  // keys: instruction i brings the pieces i * 64 .. + 63 of the stage: 64 / CPR whole rows, all of one page
+#pragma unroll
+  for (int i = 0; i < DB; ++i) {
+    const int piece = i * 64 + lane, r = piece / CPR, ch = (piece % CPR) ^ (swz(r) & (CPR - 1));
+    const int which = (i * (64 / CPR)) >> ps_shift;
+    const int page = which == 0 ? p0 : which == 1 ? p1 : which == 2 ? p2 : p3;
+    const int64_t row = (((int64_t)page * nkv + kvh) << ps_shift) + in_page + (r & (ps - 1));
+    __builtin_amdgcn_global_load_lds((global_void_t*)(k_pages + row * HD + ch * 8), (lds_void_t*)(stage + i * 1024), 16,
+                                     0, 0);
+  }
+  // values: instruction i brings dims 16 i .. + 15, four pieces of 8 keys each
+  const int d = lane >> 2, piece_keys = (lane & 3) * 8, which = piece_keys >> ps_shift;
+  int q0 = p0, q1 = p1, q2 = p2, q3 = p3;           // pinned as values: see pick_page
+  asm("" : "+s"(q0));
+  asm("" : "+s"(q1));
+  asm("" : "+s"(q2));
+  asm("" : "+s"(q3));
+  int page = q0;
+  page = which == 1 ? q1 : page;
+  page = which == 2 ? q2 : page;
+  page = which == 3 ? q3 : page;
+  const int64_t head = ((int64_t)page * nkv + kvh) * HD;
+  const int slot = in_page + (piece_keys & (ps - 1));
+#pragma unroll
+  for (int i = 0; i < DB; ++i)
+    __builtin_amdgcn_global_load_lds((global_void_t*)(v_pages + ((head + 16 * i + d) << ps_shift) + slot),
+                                     (lds_void_t*)(stage + TILE_K_BYTES + i * 1024), 16, 0, 0);
+}
+
+// grid (tiles, nkv * head_blocks); a workgroup holds hpw * splits consumers (hpw heads, each head's keys dealt
+// to `splits` wavefronts as in the kernel above) and after them `splits` producers, one per stream of tiles.
+template <int NB, int STAGES>
+__global__ __launch_bounds__(64 * PREFILL_WAVES) void attn_prefill_shared_kernel(
+    bf16_t* __restrict__ out, int64_t out_stride, const bf16_t* __restrict__ q, int64_t q_stride,
+    const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
+    const int32_t* __restrict__ block_table, int table_width, const int32_t* __restrict__ tiles, int nh,
+    int nkv, int head_blocks, int hpw, int splits, int ps_shift, int window, float scale) {
+  static_assert(STAGES == 2 || STAGES == 3, "two or three stages");
+  extern __shared__ __attribute__((aligned(16))) unsigned char ring[];
+  float* lds = reinterpret_cast<float*>(ring);      // after the loop: [hpw][splits-1][NB] x { o[HD][17], m[16], l[16] }
+  constexpr int STATE = HD * 17 + 32;
+  const int lane = threadIdx.x & 63, c = lane & 15, g = lane >> 4;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  int by = blockIdx.y, bx = blockIdx.x;             // renumbered as in the kernel above
+  if (gridDim.y > 1 && 8 % gridDim.y == 0 && gridDim.x % (8 / gridDim.y) == 0) {
+    const int linear = blockIdx.x + blockIdx.y * gridDim.x, per = 8 / gridDim.y;
+    by = (linear % 8) / per;
+    bx = (linear / 8) * per + (linear % 8) % per;
+  }
+  const int kvh = by / head_blocks, hb = by % head_blocks;
+  const int group = nh / nkv;
+  const int consumers = hpw * splits;
+  const bool producer = wave >= consumers;
+  const int stream = producer ? wave - consumers : wave % splits;
+  const int hl = producer ? 0 : wave / splits;
+  const bool head_ok = !producer && hb * hpw + hl < group;
+  const int head = kvh * group + hb * hpw + hl;
+  const int32_t* tile = tiles + (int64_t)bx * 4;
+  const int entry = __builtin_amdgcn_readfirstlane(tile[0]), row0 = __builtin_amdgcn_readfirstlane(tile[1]),
+            rows = __builtin_amdgcn_readfirstlane(tile[2]), pos0 = __builtin_amdgcn_readfirstlane(tile[3]);
+  const int kv_min = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;
+  const int kv_max = pos0 + rows - 1;
+  // every row of the tile sees the keys from the last row's window start up to the first row's position
+  const int full_lo = (window > 0 && kv_max - window + 1 > 0) ? kv_max - window + 1 : 0;
+  const int first = (kv_min / 32) * 32, tile_end = (kv_max / 32 + 1) * 32, stride = 32 * splits;
+  const int iterations = (tile_end - first + stride - 1) / stride;       // of stream 0, the longest
+  const int begin = first + 32 * stream;
+  unsigned char* my_ring = ring + (size_t)stream * STAGES * STAGE_BYTES;
+
+  f32x4 o[NB][DB];
+  float m[NB], l[NB];
+  init_state<NB>(o, m, l);
+  if (producer) {
+    const int32_t* bt = block_table + (int64_t)entry * table_width;
+    const int ps = 1 << ps_shift;
+    // the loads of tile number j of the stream, into its stage
+    auto produce = [&](int j) {
+      const int k0 = begin + j * stride;
+      if (k0 >= tile_end) return;
+      const int first_page = k0 >> ps_shift;
+      int pages[4];
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        const int lo = k0 + (w << ps_shift);                              // the page's first key
+        const bool live = (w << ps_shift) < 32 && lo <= kv_max && lo + ps - 1 >= kv_min;
+        const int id = table_entry(bt, table_width, first_page + w);
+        pages[w] = live ? id : 0;
+      }
+      produce_tile(my_ring + (j % STAGES) * STAGE_BYTES, k_pages, v_pages, pages[0], pages[1], pages[2], pages[3], kvh,
+                   nkv, ps_shift, k0, lane);
+    };
+#pragma unroll
+    for (int j = 0; j < STAGES - 1; ++j) produce(j);
+    for (int i = 0; i < iterations; ++i) {
+      // tile i is in LDS (a load into LDS counts as done when LDS holds it): what may still be on its way is the
+      // tile after it, if the stream has one and the ring a third stage.  No fence here: it would wait for that
+      // tile as well.
+      if (STAGES == 3 && begin + (i + 1) * stride < tile_end) wait_vector_loads_but<2 * DB>();
+      else wait_vector_loads_but<0>();
+      __builtin_amdgcn_s_barrier();
+      produce(i + STAGES - 1);                             // into the stage that was read in iteration i - 1
+    }
+  } else {
+    bf16x8 qr[NB][KB];
+    int cpos[NB], clo[NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+      const int j = nb * 16 + c;
+      const bool ok = head_ok && j < rows;
+      cpos[nb] = ok ? pos0 + j : -1;
+      clo[nb] = (window > 0 && pos0 + j - window + 1 > 0) ? pos0 + j - window + 1 : 0;
+      load_q(qr[nb], ok ? q + (int64_t)(row0 + j) * q_stride + (int64_t)head * HD : nullptr, g);
+    }
+    // where this lane's operands lie in a stage: the two key rows of its products, piece by piece, and its values
+    int k_at[2][KB];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      const int r = 8 * (c >> 2) + 4 * t + (c & 3);
+#pragma unroll
+      for (int kb = 0; kb < KB; ++kb) k_at[t][kb] = (r * CPR + ((kb * 4 + g) ^ (swz(r) & (CPR - 1)))) * 16;
+    }
+    const int v_at = TILE_K_BYTES + (c * 4 + g) * 16;
+    for (int i = 0; i < iterations; ++i) {
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+      const int k0 = begin + i * stride;
+      if (head_ok && k0 < tile_end) {                      // the same for the whole wavefront
+        const unsigned char* stage = my_ring + (i % STAGES) * STAGE_BYTES;
+        bf16x8 kr[2][KB], vr[DB];
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int kb = 0; kb < KB; ++kb) kr[t][kb] = *reinterpret_cast<const bf16x8*>(stage + k_at[t][kb]);
+#pragma unroll
+        for (int db = 0; db < DB; ++db) vr[db] = *reinterpret_cast<const bf16x8*>(stage + v_at + db * 1024);
+        f32x4 s[NB][2];
+        tile_scores<NB>(s, kr, qr);
+        bf16x8 pb[NB];
+        tile_softmax<NB>(pb, s, o, m, l, cpos, clo, full_lo, pos0, k0, scale, g);
+        tile_output<NB>(o, vr, pb, kv_min, kv_max, k0, g);
+      }
+    }
+    if (head_ok) finish_sums<NB>(l);
+  }
+  // the wavefronts of a head meet as in the kernel above; first everybody is through with the ring
+  __syncthreads();
+  const int split = stream;
+  if (splits > 1) {
+    if (head_ok && split > 0) {
+      float* st = lds + (int64_t)((hl * (splits - 1) + split - 1) * NB) * STATE;
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) {
+        float* sn = st + nb * STATE;
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) sn[(db * 16 + g * 4 + i) * 17 + c] = o[nb][db][i];
+        if (g == 0) {
+          sn[HD * 17 + c] = m[nb];
+          sn[HD * 17 + 16 + c] = l[nb];
+        }
+      }
+    }
+    __syncthreads();
+    if (!head_ok || split > 0) return;
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+      float mx = m[nb];
+      for (int sp = 1; sp < splits; ++sp)
+        mx = fmaxf(mx, lds[(int64_t)((hl * (splits - 1) + sp - 1) * NB + nb) * STATE + HD * 17 + c]);
+      const float f0 = m[nb] == -INFINITY ? 0.f : fast_exp2(m[nb] - mx);
+      l[nb] *= f0;
+#pragma unroll
+      for (int db = 0; db < DB; ++db) o[nb][db] *= f0;
+      for (int sp = 1; sp < splits; ++sp) {      // in split order
+        const float* sn = lds + (int64_t)((hl * (splits - 1) + sp - 1) * NB + nb) * STATE;
+        const float ms = sn[HD * 17 + c];
+        const float f = ms == -INFINITY ? 0.f : fast_exp2(ms - mx);
+        l[nb] += sn[HD * 17 + 16 + c] * f;
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) o[nb][db][i] += sn[(db * 16 + g * 4 + i) * 17 + c] * f;
+      }
+    }
+  } else if (!head_ok) {
+    return;
+  }
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) {
+    const int j = nb * 16 + c;
+    if (j >= rows) continue;
+    const float inv = 1.f / l[nb];
+    bf16_t* op = out + (int64_t)(row0 + j) * out_stride + (int64_t)head * HD + g * 4;
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+      union { uint2 u; bf16_t e[4]; } pk;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) pk.e[i] = f32_to_bf16(o[nb][db][i] * inv);
+      *reinterpret_cast<uint2*>(op + db * 16) = pk.u;
+    }
+  }
+}
+#endif
+
 extern "C" int ga_attn_head_dim() { return HD; }
 // rows of a prefill tile: 16 or (head sizes up to 128) 32
 extern "C" int ga_attn_prefill_max_tile_rows() { return 16 * PREFILL_NB; }
@@ -643,7 +905,7 @@ extern "C" int ga_attn_decode(void* out, int64_t out_stride, const void* q, int6
 extern "C" int ga_attn_prefill(void* out, int64_t out_stride, const void* q, int64_t q_stride,
                                const void* k_pages, const void* v_pages, const void* block_table,
                                int table_width, const void* tiles, int n_tiles, int tile_rows, int nh, int nkv,
-                               int page_size, int window, float scale, hipStream_t stream) {
+                               int page_size, int window, float scale, int fill_workgroups, hipStream_t stream) {
   if (n_tiles <= 0) return 0;
   if (nkv <= 0 || nh % nkv) return -1;
   if (tile_rows != 16 && tile_rows != 16 * PREFILL_NB) return -6;
@@ -651,6 +913,47 @@ extern "C" int ga_attn_prefill(void* out, int64_t out_stride, const void* q, int
   while ((1 << ps_shift) < page_size) ++ps_shift;
   if ((1 << ps_shift) != page_size || page_size < 8) return -2;
   const int group = nh / nkv;
+  const int nb = tile_rows / 16;
+#if defined(HAVE_PREFILL_SHARED) && !defined(PREFILL_SHARED_OFF)
+  {
+    // at least two heads of a group side by side, and tiles enough to fill the chip with such workgroups: the
+    // kernel that shares the operands through LDS.  A workgroup's wavefronts: heads x streams of tiles, and a
+    // producer for every stream.
+    int heads = 1;
+    for (int d = 2; d < PREFILL_WAVES; ++d)
+      if (group % d == 0 && (int64_t)n_tiles * nkv * (group / d) >= fill_workgroups) heads = d;
+    if (heads >= 2) {
+      int streams = PREFILL_WAVES / (heads + 1), stages = 3;
+      const size_t room = 150 * 1024;
+      if ((size_t)streams * stages * STAGE_BYTES > room) stages = 2;
+      while (streams > 1 && (size_t)streams * stages * STAGE_BYTES > room) --streams;
+      const int head_blocks = group / heads;
+      if ((int64_t)nkv * head_blocks > 65535) return -4;
+      size_t lds = (size_t)streams * stages * STAGE_BYTES;
+      const size_t merge = (size_t)heads * (streams - 1) * nb * (HD * 17 + 32) * sizeof(float);
+      if (merge > lds) lds = merge;
+      dim3 grid(n_tiles, nkv * head_blocks), block(64 * (heads + 1) * streams);
+#define LAUNCH_SHARED(NB, ST)                                                                                  \
+  do {                                                                                                         \
+    const void* fn = (const void*)attn_prefill_shared_kernel<NB, ST>;                                          \
+    if (lds > 48 * 1024 &&                                                                                     \
+        hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)           \
+      return -7;                                                                                               \
+    hipLaunchKernelGGL((attn_prefill_shared_kernel<NB, ST>), grid, block, lds, stream, (bf16_t*)out,           \
+                       out_stride, (const bf16_t*)q, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages, \
+                       (const int32_t*)block_table, table_width, (const int32_t*)tiles, nh, nkv, head_blocks,  \
+                       heads, streams, ps_shift, window, scale * LOG2E);                                       \
+  } while (0)
+      if (nb == 1) {
+        if (stages == 3) LAUNCH_SHARED(1, 3); else LAUNCH_SHARED(1, 2);
+      } else {
+        if (stages == 3) LAUNCH_SHARED(PREFILL_NB, 3); else LAUNCH_SHARED(PREFILL_NB, 2);
+      }
+#undef LAUNCH_SHARED
+      return GA_CHECK_LAUNCH();
+    }
+  }
+#endif
   // heads of a group that share a workgroup, and so the keys they stream: the largest divisor of the group that a
   // workgroup has wavefronts for, smaller where the step has too few tiles to fill the chip, which leaves more
   // wavefronts of a workgroup to split the keys of each head.  Measured on MI355X: 7 heads of a group side by side
@@ -658,12 +961,11 @@ extern "C" int ga_attn_prefill(void* out, int64_t out_stride, const void* q, int
   // 178; 6 heads side by side 491 us for 8k tokens of 12 heads in 2 groups where 3 heads split two ways take 500
   int hpw = 1;
   for (int d = 2; d <= PREFILL_WAVES; ++d)
-    if (group % d == 0 && (int64_t)n_tiles * nkv * (group / d) >= 256) hpw = d;
+    if (group % d == 0 && (int64_t)n_tiles * nkv * (group / d) >= fill_workgroups) hpw = d;
   int splits = PREFILL_WAVES / hpw;
   if (hpw > 1 && splits > 4) splits = 4;
   const int head_blocks = group / hpw;
   if ((int64_t)nkv * head_blocks > 65535) return -4;
-  const int nb = tile_rows / 16;
   const size_t lds = (size_t)hpw * (splits - 1) * nb * (HD * 17 + 32) * sizeof(float);
   dim3 grid(n_tiles, nkv * head_blocks), block(64 * hpw * splits);
 #define LAUNCH(NB)                                                                                        \

@@ -425,6 +425,9 @@ _DECODE_TARGET_WORKGROUPS = 256       # four wavefronts each, one workgroup per 
 _MIN_SPLIT_KEYS = 128                 # one tile of 32 keys for each wavefront of a workgroup
 _MAX_SPLITS = 256
 PREFILL_WIDE_TILES_FROM = 1024        # tokens in a step from which prompt rows go 32 to a wavefront
+# workgroups that fill the chip: heads of a kv group go side by side into a prefill workgroup only while the step
+# still makes this many workgroups
+PREFILL_FILL_WORKGROUPS = 256
 
 
 def attention_mfma_supported(dtype, head_dim, page_size):
@@ -519,7 +522,7 @@ def paged_attention_mfma(q, k_pages, v_pages, block_table, step, num_heads, num_
         _check(lib.ga_attn_prefill(
             _ptr(out), _i64(out.stride(0)), _ptr(q), _i64(q.stride(0)), _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
             _i(block_table.shape[1]), _ptr(plan["tiles"]), _i(plan["n_tiles"]), _i(tile_rows), _i(num_heads), _i(num_kv_heads),
-            _i(page_size), _i(w), _f(scale), _stream()), "attn_prefill")
+            _i(page_size), _i(w), _f(scale), _i(PREFILL_FILL_WORKGROUPS), _stream()), "attn_prefill")
     return out
 
 

@@ -363,6 +363,65 @@ def test_paged_attention_mfma(nh, nkv, hd, seqs, wide, monkeypatch):
 
 
 @pytest.mark.parametrize("wide", [False, True])
+@pytest.mark.parametrize("nh,nkv,hd", [(12, 2, 128), (28, 4, 128), (6, 3, 64), (14, 2, 64), (4, 2, 256), (6, 1, 256), (9, 3, 128),
+                                       (8, 2, 128), (5, 1, 64), (12, 2, 48)])
+@pytest.mark.parametrize("seqs", [[(300, 700)], [(31, 31), (33, 95), (2, 2), (17, 100)], [(125, 260), (63, 63), (1, 40)],
+                                  [(64, 64), (128, 128)], [(257, 1300)]])
+def test_paged_attention_mfma_heads_side_by_side(nh, nkv, hd, seqs, wide, monkeypatch):
+    """The prefill kernel that shares keys and values among the heads of a kv group through LDS runs where a step
+    has tiles enough to fill the chip; here it is made to run on small cases too (every head size it is built for,
+    groups of 2 to 7 heads with one or two streams of tiles, page sizes of 8 to 64, portions that start inside a
+    sequence), beside a head size that it is not built for."""
+    from ginfer_amd.kernels import ops
+    monkeypatch.setattr(ops, "PREFILL_WIDE_TILES_FROM", 0 if wide else 1 << 30)
+    monkeypatch.setattr(ops, "PREFILL_FILL_WORKGROUPS", 1)
+    for ps in (16, 8, 32, 64):
+        a, ref, _ = _paged_case(seqs, nh, nkv, hd, ps, torch.bfloat16, seed=hd + ps)
+        out = ops.paged_attention_mfma(a["q"], a["k_pages"], a["v_pages"], a["block_table"], _Step(seqs, a), nh, nkv, hd,
+                                       1.0 / math.sqrt(hd))
+        close(out, ref, 2e-2)
+
+
+@pytest.mark.parametrize("wide", [False, True])
+@pytest.mark.parametrize("window", [1, 5, 16, 40, 64, 100])
+def test_paged_attention_mfma_heads_side_by_side_window(window, wide, monkeypatch):
+    from ginfer_amd.kernels import ops
+    monkeypatch.setattr(ops, "PREFILL_WIDE_TILES_FROM", 0 if wide else 1 << 30)
+    monkeypatch.setattr(ops, "PREFILL_FILL_WORKGROUPS", 1)
+    nh, nkv, hd = 6, 2, 64
+    seqs = [(30, 90), (7, 7), (50, 130), (200, 330), (1, 2000)]
+    for ps in (16, 8):
+        a, ref, _ = _paged_case(seqs, nh, nkv, hd, ps, torch.bfloat16, seed=window, window=window)
+        out = ops.paged_attention_mfma(a["q"], a["k_pages"], a["v_pages"], a["block_table"], _Step(seqs, a), nh, nkv, hd,
+                                       1.0 / math.sqrt(hd), window=window)
+        close(out, ref, 2e-2)
+
+
+@pytest.mark.parametrize("wide", [False, True])
+@pytest.mark.parametrize("where", ["first", "page_edge", "before_page_edge", "tile_edge", "before_tile_edge", "split_edge",
+                                   "last", "window_edge", "behind_window"])
+def test_paged_attention_mfma_heads_side_by_side_finds_one_far_key(where, wide, monkeypatch):
+    from ginfer_amd.kernels import ops
+    monkeypatch.setattr(ops, "PREFILL_WIDE_TILES_FROM", 0 if wide else 1 << 30)
+    monkeypatch.setattr(ops, "PREFILL_FILL_WORKGROUPS", 1)
+    nh, nkv, hd, ps = 6, 2, 64, 16
+    kv = 300
+    window = 100 if "window" in where else None
+    place = {"first": 0, "page_edge": 16 * 9, "before_page_edge": 16 * 9 - 1, "tile_edge": 32 * 3, "before_tile_edge": 95,
+             "split_edge": 64, "last": kv - 1, "window_edge": kv - 100, "behind_window": kv - 101}[where]
+    seqs = [(20, kv), (40, kv)]
+    a, ref, _ = _paged_case(seqs, nh, nkv, hd, ps, torch.bfloat16, seed=5, window=window, spike=lambda e, ql, n: place)
+    out = ops.paged_attention_mfma(a["q"], a["k_pages"], a["v_pages"], a["block_table"], _Step(seqs, a), nh, nkv, hd,
+                                   1.0 / math.sqrt(hd), window=window)
+    close(out, ref, 2e-2)
+    last_rows = out.float().cpu()[[19, 59]]
+    if where == "behind_window":
+        assert (last_rows.abs() < 3).all()
+    else:
+        assert (last_rows - 7.0).abs().max() < 0.1
+
+
+@pytest.mark.parametrize("wide", [False, True])
 @pytest.mark.parametrize("hd", list(range(16, 257, 16)))
 def test_paged_attention_mfma_every_head_size(hd, wide, monkeypatch):
     """Head sizes in steps of 16 up to 256, each with a group of 3 heads: portions of prompts beside single tokens."""
