@@ -80,7 +80,7 @@ def _writable_dir():
     for d in _build_dirs():
         try:
             os.makedirs(d, exist_ok=True)
-            probe = os.path.join(d, ".probe_%d" % os.getpid())
+            probe = os.path.join(d, ".probe_%d_%d" % (os.getpid(), threading.get_ident()))
             with open(probe, "w"):
                 pass
             os.remove(probe)
@@ -122,7 +122,8 @@ def compile_module(module, out_dir=None, quiet=False):
            + ["-I", CSRC, "-o", tmp, os.path.join(CSRC, src + ".hip")])
     module = stem
     env = dict(os.environ)
-    env.setdefault("HOME", tempfile.gettempdir())   # hipcc wants a home for its caches
+    if not env.get("HOME"):
+        env["HOME"] = tempfile.gettempdir()          # hipcc wants a home for its caches
     t0 = time.time()
     proc = subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, env=env, text=True)
     # a line now and then while a long compile runs
