@@ -5,6 +5,8 @@ Every part
     has one, arrives already built under the parameter `position`);
   * says which tensors it needs: `weight_specs() -> {local name: WeightSpec}`; local names are joined
     to the part's prefix by the model, e.g. "model.layers.3.self_attn" + "." + "q_proj.weight";
+  * may name tensors that a checkpoint is allowed to carry although the part never reads them:
+    `unread_weights() -> [local name, ...]` (a tied head's own copy of the table);
   * receives them, already on the device and in the right dtype: `bind_weights({local name: tensor})`;
   * names the kernel libraries it launches: `kernel_modules() -> [module, ...]`;
   * says whether its forward may be recorded into a HIP graph: `capturable` (False unless the part sets
@@ -55,6 +57,9 @@ class Part:
 
     def weight_specs(self):
         return {}
+
+    def unread_weights(self):
+        return []
 
     def bind_weights(self, tensors):
         if tensors:

@@ -48,6 +48,11 @@ class LMHead(Part):
     def weight_specs(self):
         return {} if self.tied else {"weight": WeightSpec((self.vocab_size, self.hidden_size))}
 
+    def unread_weights(self):
+        # a checkpoint of a tied model may still hold the head's copy of the table; like the reference
+        # (ginfer/model/qwen2.cc:42-46) the model does not read it
+        return ["weight"] if self.tied else []
+
     def bind_weights(self, t):
         if not self.tied:
             self.weight = t["weight"]

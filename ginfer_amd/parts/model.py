@@ -112,6 +112,11 @@ class DecoderModel:
                 specs[prefix + "." + local] = ws
         return specs
 
+    def unread_weights(self):
+        """Full names of tensors that a checkpoint may carry although no part reads them."""
+        return [prefix + "." + local for prefix, part in self._named_parts()
+                for local in getattr(part, "unread_weights", list)()]
+
     def bind_weights(self, tensors):
         for prefix, part in self._named_parts():
             local = {n: tensors[prefix + "." + n] for n in part.weight_specs()}

@@ -28,11 +28,12 @@ class WeightError(ValueError):
     pass
 
 
-def check_against(specs, available, where):
-    """specs: name -> WeightSpec; available: name -> (dtype, shape).  Raises one WeightError that
-    lists everything that is wrong, or returns."""
+def check_against(specs, available, where, unread=()):
+    """specs: name -> WeightSpec; available: name -> (dtype, shape); unread: names the file may hold
+    although the model reads none of them.  Raises one WeightError that lists everything that is wrong,
+    or returns."""
     missing = [n for n in specs if n not in available]
-    unexpected = [n for n in available if n not in specs]
+    unexpected = [n for n in available if n not in specs and n not in unread]
     wrong = []
     for n, s in specs.items():
         if n not in available:
@@ -73,7 +74,7 @@ def load_weights(model, folder, device):
     specs = model.weight_specs()
     files = open_model_files(folder)
     available = {n: f.info(n) for n, f in files.items()}
-    check_against(specs, available, folder)
+    check_against(specs, available, folder, unread=set(getattr(model, "unread_weights", list)()))
     tensors = {}
     for name, spec in specs.items():
         cpu = files[name].tensor(name)

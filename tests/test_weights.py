@@ -76,17 +76,22 @@ def test_one_error_lists_missing_unexpected_and_wrong(tmp_path):
     tensors = {n: f.tensor(n).clone() for n in f.names()}
     del tensors["model.norm.weight"]
     del tensors["model.layers.1.mlp.up_proj.weight"]
-    tensors["lm_head.weight"] = torch.zeros(512, 64)                                  # tied: not expected
+    tensors["lm_head.weight"] = torch.zeros(512, 64)                                  # tied: carried, never read
+    tensors["model.layers.0.self_attn.o_proj.bias"] = torch.zeros(64)                 # not expected
     tensors["model.layers.0.self_attn.q_proj.weight"] = torch.zeros(64, 65)           # wrong shape
     tensors["model.layers.0.self_attn.k_proj.bias"] = torch.zeros(32, dtype=torch.int32)   # wrong kind
     write_safetensors(os.path.join(folder, "model.safetensors"), tensors)
     model = build_model(cfg.model_spec(), torch.float32, None)
     files = open_model_files(folder)
     with pytest.raises(WeightError) as e:
-        check_against(model.weight_specs(), {n: fl.info(n) for n, fl in files.items()}, folder)
+        check_against(model.weight_specs(), {n: fl.info(n) for n, fl in files.items()}, folder,
+                      unread=model.unread_weights())
     msg = str(e.value)
     assert "model.norm.weight" in msg and "model.layers.1.mlp.up_proj.weight" in msg and "missing tensors (2)" in msg
-    assert "unexpected tensors (1): lm_head.weight" in msg
+    assert model.unread_weights() == ["lm_head.weight"]
+    assert "unexpected tensors (1): model.layers.0.self_attn.o_proj.bias" in msg
+    untied = build_model(config_from_dict(H.TINY_B).model_spec(), torch.float32, None)
+    assert untied.unread_weights() == []
     assert "q_proj.weight: expected shape [64, 64], found [64, 65]" in msg
     assert "k_proj.bias: expected a floating tensor" in msg
     assert e.value.missing == ["model.layers.1.mlp.up_proj.weight", "model.norm.weight"]
