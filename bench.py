@@ -23,11 +23,14 @@ SHAPE = dict(architectures=["Qwen2ForCausalLM"], model_type="qwen2", num_hidden_
              num_attention_heads=12, num_key_value_heads=2, head_dim=128, intermediate_size=8960, vocab_size=151936,
              rope_theta=10000.0, rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=131072,
              use_sliding_window=False, sliding_window=4096, max_window_layers=21)
-FULL_LAYERS = 28
 # a larger shape of the same architecture, for looking at the kernels at other sizes (--shape 7b): Qwen2-7B's sizes
 SHAPE_7B = dict(SHAPE, hidden_size=3584, num_attention_heads=28, num_key_value_heads=4, intermediate_size=18944,
                 vocab_size=152064, rope_theta=1e6, max_position_embeddings=32768, max_window_layers=28)
-SHAPES = {"1.5b": ("qwen2-1.5b-shape", SHAPE), "7b": ("qwen2-7b-shape", SHAPE_7B)}
+# Qwen2.5-72B's sizes: 145 GB of bfloat16 weights on the one GPU, drawn on the device (no model folder)
+SHAPE_72B = dict(SHAPE, num_hidden_layers=80, hidden_size=8192, num_attention_heads=64, num_key_value_heads=8,
+                 intermediate_size=29568, vocab_size=152064, rope_theta=1e6, max_position_embeddings=32768,
+                 max_window_layers=70)
+SHAPES = {"1.5b": ("qwen2-1.5b-shape", SHAPE), "7b": ("qwen2-7b-shape", SHAPE_7B), "72b": ("qwen2.5-72b-shape", SHAPE_72B)}
 HBM_PEAK = 8.0e12            # bytes/s, MI355X HBM3E
 PEAK_FLOPS = {"bf16": 2.5e15, "fp16": 2.5e15, "fp8": 5.0e15, "fp32": 157.3e12}   # dense matrix peaks
 
@@ -51,7 +54,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--layers", type=int, default=FULL_LAYERS)
+    ap.add_argument("--layers", type=int, default=None, help="fewer layers than the shape has (default: all)")
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--context", type=int, default=4096, help="context length the timed decode steps end at")
     ap.add_argument("--prefill-tokens", type=int, default=2048)
@@ -59,6 +62,8 @@ def main():
     ap.add_argument("--points", default="1,64", help="other decode batch sizes to report")
     ap.add_argument("--model-dir", default=None, help="reuse a model folder written earlier")
     ap.add_argument("--shape", default="1.5b", choices=sorted(SHAPES), help="layer sizes (the headline is 1.5b)")
+    ap.add_argument("--device-weights", action="store_true",
+                    help="draw the weights on the device instead of writing and reading a model folder (always for 72b)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this engine runs on ONE GPU; --gpus %d is not supported" % args.gpus)
@@ -69,11 +74,17 @@ def main():
     from ginfer_amd.sampling import Sampler, SamplingParams
 
     shape_name, shape = SHAPES[args.shape]
+    full_layers = shape["num_hidden_layers"]
+    if args.layers is None:
+        args.layers = full_layers
+    device_weights = args.device_weights or args.shape == "72b"
     cfg = dict(shape, num_hidden_layers=args.layers)
     weight_bytes, kv_per_token, prefill_flops = model_numbers(cfg, args.layers)
     tmp = None
     folder = args.model_dir
-    if folder is None or not os.path.isfile(os.path.join(folder, "config.json")):
+    if device_weights:
+        folder = None
+    elif folder is None or not os.path.isfile(os.path.join(folder, "config.json")):
         if folder is None:
             tmp = tempfile.TemporaryDirectory(prefix="ginfer_bench_")
             folder = tmp.name
@@ -87,7 +98,9 @@ def main():
     ctx_pages = -(-(args.context + 1) // page)
     pages = max_b * ctx_pages + -(-args.prefill_tokens // page) + 8
     runner = ModelRunner(folder, dtype=args.dtype, page_size=page, num_pages=pages, max_requests=max_b + 1,
-                         max_model_len=max(args.context, args.prefill_tokens) + 8)
+                         max_model_len=max(args.context, args.prefill_tokens) + 8,
+                         config=config_from_dict(cfg) if device_weights else None,
+                         random_seed=0 if device_weights else None)
     sampler = Sampler(runner.device)
     g = torch.Generator().manual_seed(0)
     vocab = cfg["vocab_size"]
@@ -175,7 +188,7 @@ def main():
         "ms_per_step": round(dt * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic tokens, random weights N(0, 0.02)",
         "config": {"model": shape_name, "global_batch": args.batch, "seq_len": args.context,
-                   "parallelism": "single-gpu", "layers": args.layers, "layers_full": FULL_LAYERS,
+                   "parallelism": "single-gpu", "layers": args.layers, "layers_full": full_layers,
                    "hidden_size": cfg["hidden_size"], "num_attention_heads": cfg["num_attention_heads"],
                    "num_key_value_heads": cfg["num_key_value_heads"], "head_dim": cfg["head_dim"],
                    "intermediate_size": cfg["intermediate_size"], "vocab_size": cfg["vocab_size"],

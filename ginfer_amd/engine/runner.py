@@ -18,7 +18,7 @@ from ..config import config_from_folder
 from ..kernels import build
 from ..parts.base import KVCacheSpec, StateSpec
 from ..parts.model import build_model, StepContext, KVView, StateView
-from ..weights import load_weights
+from ..weights import load_weights, bind_random_weights
 
 DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32}
 
@@ -39,11 +39,16 @@ def require_gpu():
 class ModelRunner:
     def __init__(self, model_path, dtype="bfloat16", page_size=16, num_pages=None, max_requests=64,
                  max_model_len=None, gpu_memory_utilization=0.9, device=None, config=None, use_graphs=True,
-                 prefix_caching=False):
+                 prefix_caching=False, random_seed=None):
+        """model_path: a folder with config.json and the weights.  With model_path None, `config` (a typed
+        configuration) and `random_seed` make a model whose weights are drawn on the device, for shapes too
+        large to pass through a file."""
         self.device = device or require_gpu()
         if dtype not in DTYPES:
             raise ValueError("dtype must be one of %s, got %r" % (sorted(DTYPES), dtype))
         self.dtype = DTYPES[dtype]
+        if model_path is None and (config is None or random_seed is None):
+            raise ValueError("without a model folder, a configuration and a random_seed are needed")
         self.config = config or config_from_folder(model_path)
         self.spec = self.config.model_spec()
         self.model = build_model(self.spec, self.dtype, self.device)
@@ -52,7 +57,10 @@ class ModelRunner:
             p.limit_positions(self.max_model_len)
         # compile what this model needs, all at once, before anything runs
         build.build_all(modules=self.model.kernel_modules())
-        load_weights(self.model, model_path, self.device)
+        if model_path is None:
+            bind_random_weights(self.model, int(random_seed), self.device)
+        else:
+            load_weights(self.model, model_path, self.device)
         self.page_size = int(page_size)
         specs = self.model.cache_specs()
         if num_pages is None:

@@ -68,6 +68,26 @@ def target_dtype(spec, stored_dtype, compute_dtype):
     return compute_dtype
 
 
+class TensorsOnDemand:
+    """A mapping name -> tensor that makes a tensor when it is asked for and keeps nothing: a model that binds
+    part by part then never holds a second copy of more than one part's tensors (a part may stack or
+    re-lay-out what it is given)."""
+
+    def __init__(self, names, make):
+        self._names, self._make = set(names), make
+
+    def __getitem__(self, name):
+        if name not in self._names:
+            raise KeyError(name)
+        return self._make(name)
+
+    def __contains__(self, name):
+        return name in self._names
+
+    def keys(self):
+        return sorted(self._names)
+
+
 def load_weights(model, folder, device):
     """Reads every tensor the model expects from `folder`, converts, uploads, and hands the
     dictionary to `model.bind_weights`."""
@@ -75,11 +95,10 @@ def load_weights(model, folder, device):
     files = open_model_files(folder)
     available = {n: f.info(n) for n, f in files.items()}
     check_against(specs, available, folder, unread=set(getattr(model, "unread_weights", list)()))
-    tensors = {}
-    for name, spec in specs.items():
+    def fetch(name):
         cpu = files[name].tensor(name)
-        dt = target_dtype(spec, cpu.dtype, model.dtype)
+        dt = target_dtype(specs[name], cpu.dtype, model.dtype)
         # upload in the stored dtype, convert on the device: no host copy of a large checkpoint
-        tensors[name] = cpu.to(device=device).to(dt).contiguous()
-    model.bind_weights(tensors)
+        return cpu.to(device=device).to(dt).contiguous()
+    model.bind_weights(TensorsOnDemand(specs, fetch))
     return model

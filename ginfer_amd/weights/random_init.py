@@ -39,6 +39,32 @@ def draw(spec, seed, name, dtype, std_scale=1.0):
     return t.to(dtype)
 
 
+def bind_random_weights(model, seed, device, std_scale=1.0):
+    """Draws every tensor the model expects on the device and binds it: for shapes too large to pass
+    through a file in reasonable time (a 72B shape is 145 GB).  Same distributions and the same seeding by
+    (seed, tensor name) as `draw`, but the device's generator gives other numbers than the host's: a model
+    made here is not the one `write_random_model` writes for the same seed."""
+    from .loader import TensorsOnDemand
+    specs = model.weight_specs()
+
+    def make(name):
+        spec = specs[name]
+        if spec.kind == "int":
+            return torch.zeros(spec.shape, dtype=torch.int32, device=device)
+        dt = model.dtype                 # as a checkpoint stored in the compute dtype would load
+        if spec.init in ("zeros", "ones"):
+            return torch.full(spec.shape, 0.0 if spec.init == "zeros" else 1.0, dtype=dt, device=device)
+        if spec.init not in ("normal", "one_plus_normal"):
+            raise ValueError("unknown init %r for %s" % (spec.init, name))
+        g = torch.Generator(device=device)
+        g.manual_seed(_tensor_seed(seed, name))
+        return torch.empty(spec.shape, dtype=dt, device=device).normal_(
+            1.0 if spec.init == "one_plus_normal" else 0.0, spec.std * std_scale, generator=g)
+    tensors = TensorsOnDemand(specs, make)
+    model.bind_weights(tensors)
+    return model
+
+
 def write_random_model(folder, config, seed, dtype="bfloat16", std_scale=1.0):
     """Writes `folder/config.json` and `folder/model.safetensors`; returns the folder.  std_scale widens every
     normal draw: with the usual 0.02 a tiny model's blocks add so little to the embedding that greedy generation

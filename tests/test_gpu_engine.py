@@ -564,3 +564,24 @@ def test_steps_launched_ahead_change_nothing(folders, dtype):
     assert n_ahead > 5 and none_ahead == 0
     assert with_ahead == without
     assert {r for _, r in with_ahead} >= {"eos", "max_tokens"}
+
+
+def test_weights_drawn_on_the_device():
+    """A model without a folder: a configuration and a seed, every tensor drawn on the device.  The same seed
+    gives the same logits, another seed others; cutting a request changes nothing."""
+    from ginfer_amd import ModelRunner, StepEntry, config_from_dict
+    cfg = config_from_dict(H.TINY_B)
+    ids = H.random_tokens(40, 1000, 5)
+    outs = []
+    for seed in (3, 3, 4):
+        r = ModelRunner(None, dtype="float32", page_size=8, num_pages=16, max_requests=2, config=cfg, random_seed=seed)
+        whole = r.step([StepEntry("a", ids, [39])]).cpu()
+        r.release("a")
+        r.step([StepEntry("a", ids[:17], [])])
+        cut = r.step([StepEntry("a", ids[17:], [22])]).cpu()
+        assert torch.isfinite(whole).all() and torch.equal(whole, cut)
+        outs.append(whole)
+        del r
+    assert torch.equal(outs[0], outs[1]) and not torch.equal(outs[0], outs[2])
+    with pytest.raises(ValueError):
+        ModelRunner(None, dtype="float32", config=cfg)
