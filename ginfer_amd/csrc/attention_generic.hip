@@ -1,5 +1,5 @@
 // Paged attention, the general kernel: any mix of prompt portions and single decoded tokens, any
-// head size that is a multiple of 8 up to 256, full or windowed, 32-bit or bfloat16 storage with
+// head size up to 256, full or windowed, 32-bit or bfloat16 storage with
 // 32-bit scores, softmax and accumulators.  It is the whole of the 32-bit path and the fallback of
 // the bfloat16 path.
 //

@@ -186,8 +186,7 @@ def paged_attention_generic(q, k_pages, v_pages, block_table, token_entry, posit
     [max(0, p - window + 1), p], p = positions[t].  Returns [T, nh*hd]."""
     T = _check_attention_operands(q, k_pages, v_pages, block_table, token_entry, positions, num_heads,
                                   num_kv_heads, head_dim)
-    _need(head_dim % 8 == 0 and 0 < head_dim <= 256, "head_dim %d is not supported by the general attention kernel "
-          "(multiples of 8 up to 256)" % head_dim)
+    _need(0 < head_dim <= 256, "head_dim %d is not supported by the general attention kernel (up to 256)" % head_dim)
     if out is None:
         out = torch.empty((T, num_heads * head_dim), dtype=q.dtype, device=q.device)
     _need(out.dtype == q.dtype and out.shape == (T, num_heads * head_dim) and out.stride(1) == 1, "out must be [T, nh*hd]")

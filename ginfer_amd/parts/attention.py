@@ -33,9 +33,9 @@ class Attention(Part):
                  scale, dtype, device):
         if num_heads % num_kv_heads:
             raise ValueError("num_heads %d is not a multiple of num_kv_heads %d" % (num_heads, num_kv_heads))
-        if head_dim % 16 or not 0 < head_dim <= 256:
-            raise ValueError("head_dim %d is not supported: the attention kernels take multiples of 16 up to 256"
-                             % head_dim)
+        if not 0 < head_dim <= 256:
+            raise ValueError("head_dim %d is not supported: the attention kernels take head sizes up to 256 "
+                             "(the matrix-core kernels multiples of 16, the general kernel the others)" % head_dim)
         self.hidden_size, self.nh, self.nkv, self.hd = hidden_size, num_heads, num_kv_heads, head_dim
         self.qkv_bias, self.out_bias = bool(qkv_bias), bool(out_bias)
         self.window = int(window) if window else None
@@ -68,7 +68,9 @@ class Attention(Part):
     def kernel_modules(self):
         mods = ["rope_kv", "attention_generic", "gemm"]
         if self.dtype == torch.bfloat16:
-            mods += [("attention_mfma", {"HEAD_DIM": self.hd}), "gemm_skinny"]
+            mods += ["gemm_skinny"]
+            if self.hd in ops.MFMA_HEAD_DIMS:
+                mods += [("attention_mfma", {"HEAD_DIM": self.hd})]
         return mods
 
     def forward(self, x, step, cache, into_norm=None):

@@ -480,6 +480,24 @@ def _drawn_configuration(seed):
     return cfg, rng.choice([8, 16, 32])
 
 
+@pytest.mark.parametrize("head_dim", [2, 8, 12, 24, 36, 40, 100, 200])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_head_sizes_between_the_steps_of_16(tmp_path, dtype, head_dim):
+    """Even head sizes that are no multiple of 16 go to the general attention kernel in both dtypes."""
+    from ginfer_amd import ModelRunner
+    cfg = dict(architectures=["Qwen2ForCausalLM"], num_hidden_layers=2, hidden_size=72, num_attention_heads=4,
+               num_key_value_heads=2, head_dim=head_dim, intermediate_size=120, vocab_size=300, rope_theta=1e4,
+               rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=128)
+    folder = H.make_model_folder(tmp_path / "hd", cfg, 7, "float32")
+    reqs = {"a": H.random_tokens(75, 300, 1), "b": H.random_tokens(34, 300, 2)}
+    runner = ModelRunner(folder, dtype=dtype, page_size=16, num_pages=10, max_requests=2)
+    for what, steps in (("whole", H.steps_whole(reqs)), ("mixed", H.steps_mixed(reqs, max_live=2, seed=1)),
+                        ("last 32 decoded", H.steps_last_decoded(reqs))):
+        got = H.run_steps(runner, steps)
+        runner.cache.check()
+        H.compare_with_plain(got, reqs, folder, H.TOL[dtype], "head size %d %s %s" % (head_dim, dtype, what))
+
+
 @pytest.mark.parametrize("seed", list(range(8)))
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_configurations_drawn_at_random(tmp_path, seed, dtype):
