@@ -85,9 +85,10 @@ def test_mixed_with_pages_used_again(folders, sharp_folders, name, dtype, weight
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_trace_run_program(folders, tmp_path, dtype):
-    """bin/trace_run as a user runs it: whole, then mixed with few pages, in one process."""
-    name = "B"
+@pytest.mark.parametrize("name", ["B", "C"])
+def test_trace_run_program(folders, tmp_path, dtype, name):
+    """bin/trace_run as a user runs it: whole, then mixed with few pages, in one process (C: layers with a
+    window beside layers without, so two groups of pages)."""
     reqs = _requests(name, [70, 33, 120, 64, 90], seed=70)
     whole = H.steps_whole(reqs)
     mixed = H.steps_mixed({k + "m": v for k, v in reqs.items()}, max_live=4, seed=5)
