@@ -7,6 +7,7 @@ environment variable, the engine settings carry the names of its `engine::Config
     python -m ginfer_amd generate  --model-path DIR --prompt-ids 1,2,3 --prompt-ids 4,5 --max-tokens 16
     python -m ginfer_amd benchmark --model-path DIR --num-prompts 256 --prompt-len 512 --max-tokens 128
     python -m ginfer_amd random-weights --config config.json --seed 0 --out DIR
+    python -m ginfer_amd generate  --random-config config.json --prompt-ids 1,2,3      (weights drawn on the device)
 """
 import argparse
 import json
@@ -19,6 +20,9 @@ import time
 def _engine_args(p):
     p.add_argument("--model-path", default=os.environ.get("MODEL_PATH"),
                    help="folder with config.json and model.safetensors (default: $MODEL_PATH)")
+    p.add_argument("--random-config", default=None, metavar="CONFIG.json",
+                   help="instead of a model folder: a config.json whose weights are drawn on the device")
+    p.add_argument("--weights-seed", type=int, default=0, help="seed of the weights drawn for --random-config")
     p.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"],
                    help="bfloat16: the serving kernels; float32: everything in true 32-bit")
     p.add_argument("--max-num-batched-tokens", type=int, default=2048, help="token budget of one step")
@@ -39,11 +43,17 @@ def _engine_args(p):
 
 
 def _engine(args):
-    from . import Engine, EngineConfig
-    if not args.model_path:
-        sys.exit("no model: give --model-path or set MODEL_PATH")
+    from . import Engine, EngineConfig, config_from_dict
+    model_config = None
+    if args.random_config:
+        with open(args.random_config) as f:
+            model_config = config_from_dict(json.load(f))
+        args.model_path = None
+    elif not args.model_path:
+        sys.exit("no model: give --model-path, set MODEL_PATH, or give --random-config")
     return Engine(EngineConfig(
-        model_path=args.model_path, dtype=args.dtype, max_num_batched_tokens=args.max_num_batched_tokens,
+        model_path=args.model_path, model_config=model_config,
+        random_seed=args.weights_seed if model_config is not None else None, dtype=args.dtype, max_num_batched_tokens=args.max_num_batched_tokens,
         max_num_seqs=args.max_num_seqs, max_seq_len=args.max_seq_len,
         gpu_memory_utilization=args.gpu_memory_utilization, kvcache_block_size=args.kvcache_block_size,
         num_kvcache_blocks=args.num_kvcache_blocks, pipeline_decode=not args.no_pipeline_decode,

@@ -15,7 +15,7 @@ from .sequence import Sequence
 
 @dataclass
 class EngineConfig:
-    model_path: str
+    model_path: Optional[str]             # folder with config.json and the weights; None: model_config and random_seed
     dtype: str = "bfloat16"               # "bfloat16" or "float32" (everything in true 32-bit)
     max_num_batched_tokens: int = 2048    # token budget of one step
     max_num_seqs: int = 64                # requests running at a time
@@ -27,6 +27,10 @@ class EngineConfig:
     # requests share the cache pages of a common prefix (ginfer/engine/block_manager.cc:63-110, where it cannot be
     # switched off).  None: wherever the model allows it (no window, no per-request state); True: or refuse
     enable_prefix_caching: Optional[bool] = None
+    # without a model folder: a typed configuration (the reference's `model_config` field, ginfer/engine/config.h:8-21)
+    # and the seed that its weights are drawn from on the device
+    model_config: Optional[object] = None
+    random_seed: Optional[int] = None
 
 
 @dataclass
@@ -47,7 +51,9 @@ class Engine:
                                   num_pages=config.num_kvcache_blocks, max_requests=config.max_num_seqs,
                                   max_model_len=config.max_seq_len,
                                   gpu_memory_utilization=config.gpu_memory_utilization,
-                                  prefix_caching=config.enable_prefix_caching)
+                                  prefix_caching=config.enable_prefix_caching,
+                                  config=config.model_config if config.model_path is None else None,
+                                  random_seed=config.random_seed if config.model_path is None else None)
         self.scheduler = Scheduler(self.runner.cache, config.max_num_seqs, config.max_num_batched_tokens,
                                    self.runner.spec.eos_token_ids, self.runner.max_model_len)
         self.sampler = Sampler(self.runner.device)

@@ -338,6 +338,16 @@ def test_command_line(folders, tmp_path):
     cfg, w = pm.read_config(folders[name]), pm.read_weights(folders[name])
     assert [l["token_ids"] for l in lines] == [pm.generate(cfg, w, p, 6, ignore_eos=True) for p in ([5, 17, 3], [9, 8, 7, 6])]
     assert "decode=" in out.stderr and "ttft=" in out.stderr
+    # without a folder: the configuration alone, weights drawn on the device; the same seed gives the same tokens
+    runs = []
+    for _ in range(2):
+        cmd = [sys.executable, os.path.join(H.ROOT, "bin", "ginfer"), "generate", "--random-config",
+               os.path.join(str(folders[name]), "config.json"), "--weights-seed", "3", "--dtype", "float32", "--prompt-ids", "5,17,3",
+               "--max-tokens", "4", "--ignore-eos", "--max-num-seqs", "2", "--max-seq-len", "64", "--num-kvcache-blocks", "16"]
+        out = subprocess.run(cmd, env=dict(os.environ, MODEL_PATH=""), capture_output=True, text=True, timeout=300)
+        assert out.returncode == 0, out.stderr
+        runs.append(json.loads(out.stdout.strip().splitlines()[0])["token_ids"])
+    assert runs[0] == runs[1] and len(runs[0]) == 4
 
 
 def test_real_layer_sizes(tmp_path):
