@@ -62,6 +62,8 @@ def main():
     ap.add_argument("--points", default="1,64", help="other decode batch sizes to report")
     ap.add_argument("--model-dir", default=None, help="reuse a model folder written earlier")
     ap.add_argument("--shape", default="1.5b", choices=sorted(SHAPES), help="layer sizes (the headline is 1.5b)")
+    ap.add_argument("--no-measured-peaks", action="store_true",
+                    help="leave out the box's own copy bandwidth and product rate (the fractions use the published peaks)")
     ap.add_argument("--device-weights", action="store_true",
                     help="draw the weights on the device instead of writing and reading a model folder (always for 72b)")
     args = ap.parse_args()
@@ -176,6 +178,26 @@ def main():
             runner.release(("d", b))
         return dt, mean_ctx
 
+    def measured_peaks():
+        """What this box reaches with library routines, beside the published peaks that the fractions are quoted on:
+        a device copy of 2 GB (bytes read + bytes written per second) and a bfloat16 product of 8192^3."""
+        src = torch.empty(1 << 30, dtype=torch.int16, device=runner.device)
+        dst = torch.empty_like(src)
+        a = torch.randn(8192, 8192, device=runner.device).bfloat16()
+        b = torch.randn(8192, 8192, device=runner.device).bfloat16()
+        out = {}
+        for name, fn, work in (("copy_GBps", lambda: dst.copy_(src), 2 * src.numel() * 2 / 1e9),
+                               ("bf16_product_TFLOPs", lambda: torch.mm(a, b.t()), 2 * 8192 ** 3 / 1e12)):
+            for _ in range(3):
+                fn()
+            sync()
+            t0 = time.perf_counter()
+            for _ in range(10):
+                fn()
+            sync()
+            out[name] = round(work / ((time.perf_counter() - t0) / 10), 1)
+        return out
+
     results = {}
     for B in points:
         results[B] = decode(B, args.steps, args.warmup)
@@ -198,6 +220,8 @@ def main():
                      "frac": round(achieved * 1e9 / HBM_PEAK, 4)},
         "points": {"decode_b%d" % B: round(B / results[B][0], 1) for B in points if B != args.batch},
     }
+    if not args.no_measured_peaks:
+        out["measured"] = measured_peaks()
     print(json.dumps(out))
     if tmp is not None:
         tmp.cleanup()
