@@ -31,6 +31,10 @@ class EngineConfig:
     # and the seed that its weights are drawn from on the device
     model_config: Optional[object] = None
     random_seed: Optional[int] = None
+    # one portion of a prompt and one decoded token run through the model when the engine starts, so that the first
+    # request does not pay for what is set up at a kernel's or a library's first call
+    # (ginfer/engine/model_runner.cc:34-50 warms up with one token)
+    warmup: bool = True
 
 
 @dataclass
@@ -66,6 +70,35 @@ class Engine:
         self._ring_at = 0
         self.stats = dict(prefill_tokens=0, prefill_time=0.0, decode_tokens=0, decode_time=0.0, steps=0,
                           steps_launched_ahead=0)
+        if config.warmup:
+            self._warm_up()
+
+    def _warm_up(self):
+        """Prompt portions of several lengths (the library picks other kernels for other numbers of rows, and loads each
+        at its first use), then decoded tokens, with sampling, through the model's own step; the request is given
+        back afterwards and leaves nothing behind (it is admitted without its tokens, so no page of it is remembered)."""
+        runner, cfg = self.runner, self.config
+        room = min(runner.max_model_len - 3, cfg.max_num_batched_tokens,
+                   min(g.pool.num_free for g in runner.cache.groups) * runner.page_size - 3 if runner.cache.groups else 1 << 30)
+        rid = ("warm-up",)
+        greedy = [SamplingParams()]
+        try:
+            done = set()
+            for n in (2048, 1024, 512, 256, 160, 96, 48, 24, 8):
+                n = min(n, room)
+                if n < 1 or n in done:
+                    continue
+                done.add(n)
+                logits = runner.step([StepEntry(rid, [0] * n, [n - 1])], borrow=True)
+                self.sampler.sample_on_device(logits, greedy, [0])
+                if len(done) == 1:
+                    for _ in range(2):
+                        logits = runner.step([StepEntry(rid, [0], [0])], borrow=True)
+                        self.sampler.sample_on_device(logits, greedy, [0])
+                runner.release(rid)
+            torch.cuda.synchronize()
+        finally:
+            runner.release(rid)
 
     def add_request(self, prompt_token_ids, params: Optional[SamplingParams] = None):
         params = params or SamplingParams()
