@@ -105,3 +105,27 @@ def test_partial_sums_are_added_up_for_norms_that_do_not_take_them():
     assert whole(parts, Taking()) is parts
     x = torch.randn(3, 8)
     assert whole(x, Plain()) is x and whole(None, Plain()) is None
+
+
+def test_header_declares_every_entry_point_as_it_is_defined():
+    """ginfer_amd/csrc/ginfer_amd.h repeats the parameter lists of the `extern "C"` definitions in the sources."""
+    import glob
+    import os
+    import re
+    csrc = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "ginfer_amd", "csrc")
+
+    def squeeze(text):
+        return re.sub(r"\s+", " ", text.replace("struct ", "")).strip()
+    defined = {}
+    for path in glob.glob(os.path.join(csrc, "*.hip")):
+        src = open(path).read()
+        for m in re.finditer(r'extern "C"\s+([\w ]+?)\s*\b(ga_\w+)\s*\(([^)]*)\)\s*\{', src):
+            defined[m.group(2)] = (squeeze(m.group(1)), squeeze(m.group(3)))
+    header = open(os.path.join(csrc, "ginfer_amd.h")).read()
+    header = re.sub(r"//[^\n]*", "", header)
+    declared = {}
+    for m in re.finditer(r'([\w ]+?)\s*\b(ga_\w+)\s*\(([^)]*)\)\s*;', header):
+        declared[m.group(2)] = (squeeze(m.group(1)), squeeze(m.group(3)))
+    assert defined and set(defined) == set(declared), (sorted(set(defined) ^ set(declared)))
+    for name in defined:
+        assert defined[name] == declared[name], "%s: defined %s, declared %s" % (name, defined[name], declared[name])
