@@ -40,9 +40,10 @@ def _check(rc, name):
         raise KernelError("kernel %s failed to launch (code %d)" % (name, rc))
 
 
-def _need(cond, msg):
+def _need(cond, msg, *args):
+    """Raises KernelError(msg % args) unless cond holds; the message is put together only then."""
     if not cond:
-        raise KernelError(msg)
+        raise KernelError(msg % args if args else msg)
 
 
 def _dev(*tensors):
@@ -59,8 +60,10 @@ def _dev(*tensors):
 
 
 def _is_bf16(dtype):
-    _need(dtype in (torch.float32, torch.bfloat16), "compute dtype must be float32 or bfloat16, got %s" % dtype)
-    return 1 if dtype == torch.bfloat16 else 0
+    if dtype is torch.bfloat16:
+        return 1
+    _need(dtype is torch.float32, "compute dtype must be float32 or bfloat16, got %s", dtype)
+    return 0
 
 
 def embedding_gather(table, ids, out=None):
@@ -89,13 +92,16 @@ def add_rmsnorm(residual, delta, gain, eps, dtype, rows=None, out=None):
     parts = 0
     if delta is not None and delta.dim() == 3:
         _need(delta.dtype == torch.float32 and delta.shape[1:] == (T, H) and delta.is_contiguous() and delta.shape[0] >= 1,
-              "partial sums must be contiguous float32 [parts, %d, %d], got %s %s" % (T, H, delta.dtype, tuple(delta.shape)))
+              "partial sums must be contiguous float32 [parts, %d, %d], got %s %s",
+              T, H, delta.dtype, tuple(delta.shape))
         parts = delta.shape[0]
     elif delta is not None:
         _need(delta.dtype == dtype and delta.shape == (T, H) and delta.is_contiguous(),
-              "delta must be contiguous %s [%d, %d], got %s %s" % (dtype, T, H, delta.dtype, tuple(delta.shape)))
+              "delta must be contiguous %s [%d, %d], got %s %s",
+              dtype, T, H, delta.dtype, tuple(delta.shape))
     _need(gain.shape == (H,) and gain.is_contiguous() and gain.dtype in (dtype, torch.float32),
-          "gain must be contiguous [%d] in %s or float32" % (H, dtype))
+          "gain must be contiguous [%d] in %s or float32",
+          H, dtype)
     R = T
     if rows is not None:
         _need(rows.dtype == torch.int32 and rows.dim() == 1 and rows.is_contiguous(), "rows must be contiguous int32 [R]")
@@ -134,13 +140,17 @@ def rope_kv_write(qkv, positions, cos, sin, slot_mapping, k_pages, v_pages, num_
     _dev(qkv, positions, cos, sin, slot_mapping, k_pages, v_pages)
     T = qkv.shape[0]
     width = (num_heads + 2 * num_kv_heads) * head_dim
-    _need(qkv.dim() == 2 and qkv.shape[1] == width and qkv.is_contiguous(), "qkv must be contiguous [T, %d]" % width)
+    _need(qkv.dim() == 2 and qkv.shape[1] == width and qkv.is_contiguous(),
+          "qkv must be contiguous [T, %d]",
+          width)
     _need(positions.dtype == torch.int32 and positions.shape == (T,) and positions.is_contiguous(),
           "positions must be contiguous int32 [T]")
     _need(cos.dtype == torch.float32 and sin.dtype == torch.float32 and cos.shape == sin.shape and cos.dim() == 2
           and cos.is_contiguous() and sin.is_contiguous(), "cos and sin must be contiguous float32 [P, rotary_dim/2]")
     rotary_dim = 2 * cos.shape[1]
-    _need(0 < rotary_dim <= head_dim, "rotary_dim %d must lie in (0, head_dim %d]" % (rotary_dim, head_dim))
+    _need(0 < rotary_dim <= head_dim,
+          "rotary_dim %d must lie in (0, head_dim %d]",
+          rotary_dim, head_dim)
     page_size = 1
     if write_kv:
         _need(slot_mapping is not None and slot_mapping.dtype == torch.int64 and slot_mapping.shape == (T,)
@@ -158,11 +168,12 @@ def _check_pages(k_pages, v_pages, dtype, nkv, hd):
     _need(k_pages is not None and v_pages is not None, "cache pages are missing")
     for p in (k_pages, v_pages):
         _need(p.dtype == dtype and p.dim() == 4 and p.is_contiguous() and p.shape[1] == nkv,
-              "cache pages must be contiguous %s with %d kv heads" % (dtype, nkv))
+              "cache pages must be contiguous %s with %d kv heads",
+              dtype, nkv)
     ps = k_pages.shape[2]
     _need(k_pages.shape[3] == hd and tuple(v_pages.shape) == (k_pages.shape[0], nkv, hd, ps),
-          "cache pages must be k [pages, %d, page_size, %d] and v [pages, %d, %d, page_size], got %s and %s"
-          % (nkv, hd, nkv, hd, tuple(k_pages.shape), tuple(v_pages.shape)))
+          "cache pages must be k [pages, %d, page_size, %d] and v [pages, %d, %d, page_size], got %s and %s",
+          nkv, hd, nkv, hd, tuple(k_pages.shape), tuple(v_pages.shape))
     return ps
 
 
@@ -170,12 +181,16 @@ def _check_attention_operands(q, k_pages, v_pages, block_table, token_entry, pos
     _dev(q, k_pages, v_pages, block_table, token_entry, positions)
     T = q.shape[0]
     _need(q.dim() == 2 and q.stride(1) == 1 and q.shape[1] >= nh * hd, "q must be [T, >= nh*hd] with unit inner stride")
-    _need(nkv > 0 and nh % nkv == 0, "num_heads %d is not a multiple of num_kv_heads %d" % (nh, nkv))
+    _need(nkv > 0 and nh % nkv == 0,
+          "num_heads %d is not a multiple of num_kv_heads %d",
+          nh, nkv)
     _check_pages(k_pages, v_pages, q.dtype, nkv, hd)
     _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous(),
           "block_table must be contiguous int32 [entries, width]")
     for name, x in (("token_entry", token_entry), ("positions", positions)):
-        _need(x.dtype == torch.int32 and x.shape == (T,) and x.is_contiguous(), "%s must be contiguous int32 [T]" % name)
+        _need(x.dtype == torch.int32 and x.shape == (T,) and x.is_contiguous(),
+              "%s must be contiguous int32 [T]",
+              name)
     return T
 
 
@@ -186,7 +201,9 @@ def paged_attention_generic(q, k_pages, v_pages, block_table, token_entry, posit
     [max(0, p - window + 1), p], p = positions[t].  Returns [T, nh*hd]."""
     T = _check_attention_operands(q, k_pages, v_pages, block_table, token_entry, positions, num_heads,
                                   num_kv_heads, head_dim)
-    _need(0 < head_dim <= 256, "head_dim %d is not supported by the general attention kernel (up to 256)" % head_dim)
+    _need(0 < head_dim <= 256,
+          "head_dim %d is not supported by the general attention kernel (up to 256)",
+          head_dim)
     if out is None:
         out = torch.empty((T, num_heads * head_dim), dtype=q.dtype, device=q.device)
     _need(out.dtype == q.dtype and out.shape == (T, num_heads * head_dim) and out.stride(1) == 1, "out must be [T, nh*hd]")
@@ -203,8 +220,9 @@ def gemm_nt(a, w, bias=None, out=None, out_dtype=None):
     """a [M, K] . w [N, K]^T (+ bias [N]) -> [M, N]; 32-bit accumulation, plain FMA.  a and w share a
     dtype (float32 or bfloat16); out is that dtype or float32."""
     _dev(a, w, bias, out)
-    _need(a.dim() == 2 and w.dim() == 2 and a.shape[1] == w.shape[1], "gemm_nt: a [M, K] and w [N, K] do not agree: %s, %s"
-          % (tuple(a.shape), tuple(w.shape)))
+    _need(a.dim() == 2 and w.dim() == 2 and a.shape[1] == w.shape[1],
+          "gemm_nt: a [M, K] and w [N, K] do not agree: %s, %s",
+          tuple(a.shape), tuple(w.shape))
     _need(a.dtype == w.dtype and a.stride(1) == 1 and w.is_contiguous(), "gemm_nt: a and w must share a dtype; w contiguous")
     M, K = a.shape
     N = w.shape[0]
@@ -232,7 +250,9 @@ def sample_rows(logits, temperature=None, uniform=None, out=None):
     if temperature is not None:
         _need(uniform is not None, "temperature sampling needs uniform numbers")
         for name, x in (("temperature", temperature), ("uniform", uniform)):
-            _need(x.dtype == torch.float32 and x.shape == (R,) and x.is_contiguous(), "%s must be contiguous float32 [R]" % name)
+            _need(x.dtype == torch.float32 and x.shape == (R,) and x.is_contiguous(),
+                  "%s must be contiguous float32 [R]",
+                  name)
     if out is None:
         out = torch.empty((R,), dtype=torch.int32, device=logits.device)
     _need(out.dtype == torch.int32 and out.shape == (R,) and out.is_contiguous(), "out must be contiguous int32 [R]")
@@ -282,7 +302,8 @@ class _SkinnyNorm(ctypes.Structure):
 def _norm_in(norm, a):
     """Fills the in_ fields from ScaledRows; returns the rows the product runs on."""
     _need(a.scaled.dtype == torch.bfloat16 and a.scaled.dim() == 2 and a.scaled.shape[0] <= FOLDED_NORM_MAX_ROWS,
-          "rows of a folded norm are bfloat16 [M <= %d, H]" % FOLDED_NORM_MAX_ROWS)
+          "rows of a folded norm are bfloat16 [M <= %d, H]",
+          FOLDED_NORM_MAX_ROWS)
     M, H = a.scaled.shape
     _need(a.sumsq.dtype == torch.float32 and a.sumsq.dim() == 2 and a.sumsq.shape[0] == M and a.sumsq.is_contiguous()
           and 1 <= a.sumsq.shape[1] <= 512, "partial sums of a folded norm are contiguous float32 [M, parts <= 512]")
@@ -328,7 +349,8 @@ def gemm_skinny(a, w, bias=None, out=None, out_dtype=None, nt=0, ks=0, grid_spli
         residual, gain, eps = into_norm
         _need(folded_norm_supported(a, w, residual, gain) and not gated and grid_splits == 1 and out is None,
               "a product folds the norm after it for at most %d bfloat16 rows, a float32 residual [M, N] and a "
-              "gain [N], N a multiple of 8 with at most 512 partial sums a row" % FOLDED_NORM_MAX_ROWS)
+              "gain [N], N a multiple of 8 with at most 512 partial sums a row",
+              FOLDED_NORM_MAX_ROWS)
         _dev(residual, gain)
         norm = norm or _SkinnyNorm()
         M, N = residual.shape
@@ -339,10 +361,13 @@ def gemm_skinny(a, w, bias=None, out=None, out_dtype=None, nt=0, ks=0, grid_spli
         norm.gain, norm.gain_f32 = gain.data_ptr(), 1 if gain.dtype == torch.float32 else 0
         norm.scaled, norm.lds, norm.out_sumsq = scaled.data_ptr(), scaled.stride(0), sumsq.data_ptr()
     _dev(a, w, bias, out)
-    _need(a.dim() == 2 and w.dim() == 2 and a.shape[1] == w.shape[1], "gemm_skinny: a [M, K] and w [N, K] do not agree: %s, %s"
-          % (tuple(a.shape), tuple(w.shape)))
-    _need(gemm_skinny_supported(a, w), "gemm_skinny takes bfloat16, at most %d rows, K a multiple of 8 and 16-byte "
-          "aligned rows; got a %s %s, w %s %s" % (SKINNY_MAX_ROWS, a.dtype, tuple(a.shape), w.dtype, tuple(w.shape)))
+    _need(a.dim() == 2 and w.dim() == 2 and a.shape[1] == w.shape[1],
+          "gemm_skinny: a [M, K] and w [N, K] do not agree: %s, %s",
+          tuple(a.shape), tuple(w.shape))
+    _need(gemm_skinny_supported(a, w),
+          "gemm_skinny takes bfloat16, at most %d rows, K a multiple of 8 and 16-byte "
+          "aligned rows; got a %s %s, w %s %s",
+          SKINNY_MAX_ROWS, a.dtype, tuple(a.shape), w.dtype, tuple(w.shape))
     M, K = a.shape
     N = w.shape[0]
     if gated:       # w stacks gate over up: the result has half as many columns
@@ -395,11 +420,17 @@ def qkv_rope_skinny(x, w, bias, positions, cos, sin, slot_mapping, k_pages, v_pa
     _dev(x, w, bias, positions, cos, sin, slot_mapping, k_pages, v_pages)
     M, K = x.shape
     width = (num_heads + 2 * num_kv_heads) * head_dim
-    _need(w.shape == (width, K), "qkv weight must be [%d, %d], got %s" % (width, K, tuple(w.shape)))
-    _need(qkv_rope_skinny_supported(x, w, head_dim, 2 * cos.shape[1]), "the fused q|k|v kernel takes bfloat16, at most %d "
-          "rows, head sizes that are multiples of 32 and a rotation of the whole head" % SKINNY_MAX_ROWS)
+    _need(w.shape == (width, K),
+          "qkv weight must be [%d, %d], got %s",
+          width, K, tuple(w.shape))
+    _need(qkv_rope_skinny_supported(x, w, head_dim, 2 * cos.shape[1]),
+          "the fused q|k|v kernel takes bfloat16, at most %d "
+          "rows, head sizes that are multiples of 32 and a rotation of the whole head",
+          SKINNY_MAX_ROWS)
     if bias is not None:
-        _need(bias.dtype == torch.bfloat16 and bias.shape == (width,) and bias.is_contiguous(), "qkv bias must be bfloat16 [%d]" % width)
+        _need(bias.dtype == torch.bfloat16 and bias.shape == (width,) and bias.is_contiguous(),
+              "qkv bias must be bfloat16 [%d]",
+              width)
     _need(positions.dtype == torch.int32 and positions.shape == (M,) and positions.is_contiguous(), "positions must be int32 [M]")
     _need(cos.dtype == torch.float32 and sin.dtype == torch.float32 and cos.shape == sin.shape and cos.is_contiguous()
           and sin.is_contiguous(), "cos and sin must be contiguous float32 [P, head_dim/2]")
@@ -491,11 +522,13 @@ def paged_attention_mfma(q, k_pages, v_pages, block_table, step, num_heads, num_
     page_size = k_pages.shape[2]
     _need(attention_mfma_supported(q.dtype, head_dim, page_size),
           "the matrix-core attention kernels take bfloat16, head sizes in steps of 16 up to 256 and page sizes that "
-          "are powers of two from 8; got %s, head %d, page %d" % (q.dtype, head_dim, page_size))
+          "are powers of two from 8; got %s, head %d, page %d",
+          q.dtype, head_dim, page_size)
     _need(q.stride(0) % 8 == 0 and q.data_ptr() % 16 == 0, "q rows must be 16-byte aligned")
     _need(k_pages.shape[0] * num_kv_heads * max(page_size, head_dim) < 2 ** 31,
           "the matrix-core attention kernels count the rows of a layer's cache in 32 bits: %d pages x %d kv heads x "
-          "%d is too many" % (k_pages.shape[0], num_kv_heads, max(page_size, head_dim)))
+          "%d is too many",
+          k_pages.shape[0], num_kv_heads, max(page_size, head_dim))
     lib = build.load("attention_mfma", {"HEAD_DIM": head_dim})
     _need(lib.ga_attn_head_dim() == head_dim, "attention library was built for another head size")
     # rows of a prompt portion per wavefront: 32 where the kernel has it and the step is long, else 16
