@@ -112,6 +112,11 @@ class Engine:
         self.scheduler.add(Sequence(rid, ids, len(ids), params))
         return rid
 
+    def abort(self, request_id) -> Optional[RequestOutput]:
+        """Ends a request now, wherever it stands; returns what it has produced, or None if it is not alive."""
+        seq = self.scheduler.abort(request_id, time.perf_counter())
+        return None if seq is None else self._output(seq)
+
     def has_unfinished(self):
         return self._launched is not None or not self.scheduler.is_finished()
 

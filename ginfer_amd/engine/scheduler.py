@@ -67,6 +67,25 @@ class Scheduler:
     def is_finished(self):
         return not self.waiting and not self.running
 
+    def abort(self, request_id, now=None):
+        """Takes a request out, waiting or running: its pages and its state slot are given back at once and it
+        finishes with the reason "aborted", keeping the tokens it has.  Returns the sequence, or None when no
+        such request is alive.  A step that is already on the device may still hold the request: its token is
+        passed over by absorb(), and what it writes lies in pages that nobody reads before they are written anew."""
+        for seq in list(self.waiting) + self.running:
+            if seq.request_id == request_id:
+                break
+        else:
+            return None
+        if seq.state is State.RUNNING:
+            self.running.remove(seq)
+        else:
+            self.waiting.remove(seq)
+        if self.cache.has(request_id):
+            self.cache.release(request_id, seq.token_ids)
+        seq.state, seq.finish_reason, seq.finish_ts = State.FINISHED, "aborted", now
+        return seq
+
     # ---- one step
     def schedule(self) -> List[Scheduled]:
         cache = self.cache

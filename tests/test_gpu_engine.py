@@ -614,3 +614,30 @@ def test_weights_drawn_on_the_device():
     assert torch.equal(outs[0], outs[1]) and not torch.equal(outs[0], outs[2])
     with pytest.raises(ValueError):
         ModelRunner(None, dtype="float32", config=cfg)
+
+
+def test_abort_in_the_middle_leaves_the_others_untouched(folders):
+    """A request is ended from outside while steps launched ahead are on the device: it keeps what it has, its pages
+    go back, and the other requests generate what they generate alone."""
+    from ginfer_amd import Engine, EngineConfig, SamplingParams
+    name = "A"
+    eng = Engine(EngineConfig(model_path=str(folders[name]), dtype="float32", max_num_batched_tokens=32, max_num_seqs=4,
+                              max_seq_len=128, kvcache_block_size=16, num_kvcache_blocks=24))
+    prompts = [H.random_tokens(n, 512, 60 + n) for n in (9, 21, 14)]
+    ids = [eng.add_request(p, SamplingParams(max_tokens=24, ignore_eos=True)) for p in prompts]
+    done = {}
+    for _ in range(8):
+        for o in eng.step():
+            done[o.request_id] = o
+    out = eng.abort(ids[1])
+    assert out is not None and out.finish_reason == "aborted" and 0 < len(out.token_ids) < 24
+    assert eng.abort(ids[1]) is None
+    while eng.has_unfinished():
+        for o in eng.step():
+            done[o.request_id] = o
+    cfg, w = pm.read_config(folders[name]), pm.read_weights(folders[name])
+    for k in (0, 2):
+        assert done[ids[k]].token_ids == pm.generate(cfg, w, prompts[k], 24, ignore_eos=True)
+    assert out.token_ids == pm.generate(cfg, w, prompts[1], 24, ignore_eos=True)[:len(out.token_ids)]
+    eng.runner.cache.check()
+    assert not eng.runner.cache.requests

@@ -344,3 +344,43 @@ def test_random_workloads_with_shared_prefixes_finish_with_the_same_tokens(seed)
     assert {s.request_id: s.token_ids for s in done} == want
     assert cache.prefix_hit_tokens > 0
     assert not cache.requests and all(g.pool.num_free == g.pool.num_pages for g in cache.groups)
+
+
+def test_abort_gives_everything_back_wherever_the_request_stands():
+    sched, cache = make(num_pages=16, budget=8, max_num_seqs=2)
+    seqs = [seq(i, 10, max_tokens=20) for i in range(3)]
+    for s in seqs:
+        sched.add(s)
+    free0 = cache.groups[0].pool.num_free
+    batch = sched.schedule()                       # request 0 gets a portion; 1 and 2 wait or start
+    sched.postprocess(batch, [fake_token(b.seq.token_ids) for b in batch if b.samples], now=1.0)
+    running = {s.request_id for s in sched.running}
+    assert 0 in running and 2 not in running
+    # a running request in the middle of its prompt, and one that still waits
+    a = sched.abort(0, now=2.0)
+    w = sched.abort(2, now=2.0)
+    assert a is seqs[0] and a.state is State.FINISHED and a.finish_reason == "aborted" and a.finish_ts == 2.0
+    assert w is seqs[2] and w.finish_reason == "aborted" and w.num_output_tokens == 0
+    assert sched.abort(0) is None and sched.abort(77) is None
+    assert not cache.has(0) and not cache.has(2)
+    cache.check()
+    # the rest runs to its end as if the others had never been there
+    done = []
+    steps = 0
+    while not sched.is_finished():
+        batch = sched.schedule()
+        assert all(b.seq.request_id == 1 for b in batch)
+        done += sched.postprocess(batch, [fake_token(b.seq.token_ids) for b in batch if b.samples], now=3.0)
+        steps += 1
+        assert steps < 100
+    assert [s.request_id for s in done] == [1] and done[0].token_ids == expected(seqs[1])
+    assert not cache.requests and cache.groups[0].pool.num_free == free0
+    # a step that is on the device when its request is aborted: the token that arrives is passed over
+    sched2, cache2 = make(num_pages=16, budget=8)
+    b = seq(5, 4, max_tokens=20)
+    sched2.add(b)
+    batch = sched2.schedule()
+    sched2.advance(batch)
+    sched2.abort(5)
+    assert sched2.absorb(batch, [123]) == [] and b.num_output_tokens == 0 and sched2.is_finished()
+    cache2.check()
