@@ -38,6 +38,8 @@ def _engine_args(p):
     p.add_argument("--seed", type=int, default=0, help="seed of the sampler's random stream")
     p.add_argument("--no-pipeline-decode", action="store_true",
                    help="read every step's tokens before the next step is launched")
+    p.add_argument("--no-graph-mixed-steps", action="store_true",
+                   help="steps with prompt portions are launched kernel by kernel, never replayed from a recording")
     p.add_argument("--no-prefix-caching", action="store_true",
                    help="requests do not share the cache pages of a common prefix")
 
@@ -57,6 +59,7 @@ def _engine(args):
         max_num_seqs=args.max_num_seqs, max_seq_len=args.max_seq_len,
         gpu_memory_utilization=args.gpu_memory_utilization, kvcache_block_size=args.kvcache_block_size,
         num_kvcache_blocks=args.num_kvcache_blocks, pipeline_decode=not args.no_pipeline_decode,
+        graph_mixed_steps=not args.no_graph_mixed_steps,
         enable_prefix_caching=False if args.no_prefix_caching else None))
 
 
@@ -78,8 +81,9 @@ def _report(engine, outs, wall):
     sys.stderr.write("steps=%d (launched ahead: %d) prefill=%.1f tok/s decode=%.1f tok/s wall=%.3f s evictions=%d "
                      "prompt tokens found in the cache=%d\n"
                      % (st["steps"], st["steps_launched_ahead"], pf, dc, wall, engine.scheduler.num_evictions, shared))
+    sys.stderr.write("how the steps ran: %s\n" % engine.runner.counts)
     return dict(steps=st["steps"], steps_launched_ahead=st["steps_launched_ahead"], prefill_tok_s=pf, decode_tok_s=dc,
-                wall_s=wall, prefix_hit_tokens=shared)
+                wall_s=wall, prefix_hit_tokens=shared, ran=dict(engine.runner.counts))
 
 
 def cmd_generate(args):
@@ -113,12 +117,44 @@ def cmd_benchmark(args):
     for k in engine.stats:
         engine.stats[k] = 0 if isinstance(engine.stats[k], int) else 0.0
     t0 = time.perf_counter()
-    outs = engine.generate(prompts, _params(args, len(prompts)))
+    if args.request_rate > 0:
+        outs = _generate_as_they_arrive(engine, prompts, _params(args, len(prompts)), args.request_rate, rng)
+    else:
+        outs = engine.generate(prompts, _params(args, len(prompts)))
     wall = time.perf_counter() - t0
     rep = _report(engine, [], wall)
     total = sum(len(o.prompt_token_ids) + len(o.token_ids) for o in outs)
     rep.update(total_tokens=total, total_tok_s=total / wall, output_tok_s=sum(len(o.token_ids) for o in outs) / wall)
+    for name, values in (("ttft_ms", [o.ttft * 1e3 for o in outs if o.ttft is not None]),
+                         ("tpot_ms", [o.tpot * 1e3 for o in outs if o.tpot is not None])):
+        values.sort()
+        if values:
+            rep[name] = dict(mean=round(sum(values) / len(values), 3), p50=round(values[len(values) // 2], 3),
+                             p99=round(values[min(len(values) - 1, int(len(values) * 0.99))], 3))
     print(json.dumps(rep))
+
+
+def _generate_as_they_arrive(engine, prompts, params, rate, rng):
+    """Requests arrive one by one, `rate` a second on average (exponential gaps from the seeded generator), while
+    the engine steps: what a request waits for its first token and for every further one then depends on what
+    else is running, as in serving."""
+    arrivals, t = [], 0.0
+    for _ in prompts:
+        t += rng.expovariate(rate)
+        arrivals.append(t)
+    start = time.perf_counter()
+    ids, done, nxt = [], {}, 0
+    while nxt < len(prompts) or engine.has_unfinished():
+        now = time.perf_counter() - start
+        while nxt < len(prompts) and arrivals[nxt] <= now:
+            ids.append(engine.add_request(prompts[nxt], params[nxt]))
+            nxt += 1
+        if engine.has_unfinished():
+            for out in engine.step():
+                done[out.request_id] = out
+        else:
+            time.sleep(max(0.0, min(arrivals[nxt] - now, 0.001)))
+    return [done[i] for i in ids]
 
 
 def cmd_random_weights(args):
@@ -141,6 +177,8 @@ def main(argv=None):
     _engine_args(b)
     b.add_argument("--num-prompts", type=int, default=256)
     b.add_argument("--prompt-len", type=int, default=512)
+    b.add_argument("--request-rate", type=float, default=0.0,
+                   help="requests a second arriving while the engine runs (0: all at once, the reference's benchmark)")
     b.set_defaults(fn=cmd_benchmark, max_num_batched_tokens=16384, max_num_seqs=256, max_tokens=128)
     r = sub.add_parser("random-weights", help="write a model folder with random weights")
     r.add_argument("--config", required=True, help="a config.json of a registered architecture")

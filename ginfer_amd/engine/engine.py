@@ -35,6 +35,9 @@ class EngineConfig:
     # request does not pay for what is set up at a kernel's or a library's first call
     # (ginfer/engine/model_runner.cc:34-50 warms up with one token)
     warmup: bool = True
+    # steps with prompt portions of up to 512 token rows are laid into recorded steps of padded sizes: their launches
+    # would cost the host more than the device works on them
+    graph_mixed_steps: bool = True
 
 
 @dataclass
@@ -56,6 +59,7 @@ class Engine:
                                   max_model_len=config.max_seq_len,
                                   gpu_memory_utilization=config.gpu_memory_utilization,
                                   prefix_caching=config.enable_prefix_caching,
+                                  graph_mixed_steps=config.graph_mixed_steps,
                                   config=config.model_config if config.model_path is None else None,
                                   random_seed=config.random_seed if config.model_path is None else None)
         self.scheduler = Scheduler(self.runner.cache, config.max_num_seqs, config.max_num_batched_tokens,

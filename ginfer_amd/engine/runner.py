@@ -39,7 +39,7 @@ def require_gpu():
 class ModelRunner:
     def __init__(self, model_path, dtype="bfloat16", page_size=16, num_pages=None, max_requests=64,
                  max_model_len=None, gpu_memory_utilization=0.9, device=None, config=None, use_graphs=True,
-                 prefix_caching=False, random_seed=None):
+                 prefix_caching=False, random_seed=None, graph_mixed_steps=True):
         """model_path: a folder with config.json and the weights.  With model_path None, `config` (a typed
         configuration) and `random_seed` make a model whose weights are drawn on the device, for shapes too
         large to pass through a file."""
@@ -73,6 +73,11 @@ class ModelRunner:
         self._buffers = _BufferCache(len(self.cache.groups), self.device)
         self.use_graphs = bool(use_graphs) and self.model.capturable()
         self._graphs, self._graph_seen = {}, {}
+        self.graph_mixed_steps = bool(graph_mixed_steps)
+        self._padded_buffers = {}
+        # how steps ran: launched kernel by kernel, replayed as a recorded decode step, replayed as a recorded step
+        # with prompt portions; and how many steps were recorded
+        self.counts = dict(launched=0, replayed_decode=0, replayed_padded=0, recorded=0)
 
     def _pages_from_free_memory(self, specs, utilization):
         """Pages = free device memory (after the weights are resident) * utilization / bytes per page, the
@@ -244,12 +249,136 @@ class ModelRunner:
                 if device_tokens is not None:
                     g["buf"].buf.dev["ids"].copy_(device_tokens)
                 g["graph"].replay()
+                self.counts["replayed_decode"] += 1
                 return g["logits"] if borrow else g["logits"].clone()
+        if not graphable and device_tokens is None and self.use_graphs and self.graph_mixed_steps:
+            logits = self._run_padded(host, borrow)
+            if logits is not None:
+                return logits
         buf = self._buffers.get(T, E, len(host["rows"]), host["width"], len(host["decode_info"]))
         ctx = self._context(host, buf)
         if device_tokens is not None:
             buf.dev["ids"].copy_(device_tokens)
+        self.counts["launched"] += 1
         return self.model.forward(ctx)
+
+    # ---- recorded steps that hold prompt portions
+    def _run_padded(self, host, borrow):
+        """A step with prompt portions, short enough that the host's launches would take longer than the device's
+        work: it is laid into a recorded step of fixed sizes (token rows and entries powers of two, the context
+        bucket), recorded the second time such sizes are seen.  Rows and entries beyond the step's own
+        are padding: tokens of an extra entry whose one page is page 0, which write nothing to the cache; the tiles
+        and single-token records that fill the plan point at the first padding row.  Rows do not mix in any kernel,
+        so what the padding computes stays in the padding.  None: the step runs launch by launch."""
+        T, E, R = host["T"], host["E"], len(host["rows"])
+        if T + 1 > MIXED_GRAPH_MAX_TOKENS or E > GRAPH_MAX_ROWS:
+            return None
+        t_pad = 64                       # coarse sizes, so that few recorded steps serve many: rows 64, 128, 256, 512
+        while t_pad < T + 1:
+            t_pad *= 2
+        e_pad = 8                        # entries 8, 16, ... 256
+        while e_pad < E:
+            e_pad *= 2
+        if R > e_pad:
+            return None
+        bucket = _context_bucket(host["max_kv"])
+        key = ("padded", t_pad, e_pad, bucket)
+        g = self._graphs.pop(key, None)
+        if g is not None:
+            self._graphs[key] = g
+        else:
+            self._graph_seen[key] = self._graph_seen.get(key, 0) + 1
+            if self._graph_seen[key] >= GRAPH_AFTER:
+                while len(self._graphs) >= GRAPH_KEEP:
+                    self._graphs.pop(next(iter(self._graphs)))
+                g = self._capture_padded(key, host)
+        if g is None:
+            # not recorded yet: launched kernel by kernel, but with the same padded sizes, so that a step's bits do not
+            # depend on whether its sizes have been seen before
+            width = max(1, -(-bucket // self.page_size))
+            buf = self._padded_buffers.pop(key, None)
+            if buf is None:
+                buf = _StepBuffers(t_pad, e_pad + 1, e_pad, width, e_pad, len(self.cache.groups), self.device,
+                                   n_tiles=self._padded_tiles(t_pad, e_pad))
+                while len(self._padded_buffers) >= 8:
+                    self._padded_buffers.pop(next(iter(self._padded_buffers)))
+            self._padded_buffers[key] = buf
+            ctx = self._padded_context(host, buf, t_pad, e_pad, width, bucket)
+            self.counts["launched"] += 1
+            return self.model.forward(ctx)[:R]
+        g["buf"].fill(self._pad(host, t_pad, e_pad, g["width"]))
+        g["graph"].replay()
+        self.counts["replayed_padded"] += 1
+        out = g["logits"][:R]
+        return out if borrow else out.clone()
+
+    @staticmethod
+    def _padded_tiles(t_pad, e_pad):
+        from ..kernels import ops
+        return t_pad // ops.PLAN_TILE_ROWS + e_pad
+
+    def _padded_context(self, host, buf, t_pad, e_pad, width, bucket):
+        from ..kernels import ops
+        ctx = self._context(self._pad(host, t_pad, e_pad, width), buf)
+        ctx.extra = {"decode_info": buf.dev["decode_info"], "decode_span": bucket,
+                     "static_plan": dict(tiles=buf.dev["tiles"], n_tiles=self._padded_tiles(t_pad, e_pad), n_decode=e_pad,
+                                         tile_rows=ops.PLAN_TILE_ROWS)}
+        return ctx
+
+    def _pad(self, host, t_pad, e_pad, width):
+        from ..kernels import ops
+        T, E, R = host["T"], host["E"], len(host["rows"])
+        dummy, entries = e_pad, e_pad + 1
+        def grown(a, n, fill):
+            out = np.full((n,) + a.shape[1:], fill, dtype=a.dtype)
+            out[:a.shape[0]] = a
+            return out
+        cu = np.full(entries + 1, T, dtype=np.int32)
+        cu[:E + 1] = host["cu"]
+        cu[entries] = t_pad
+        q_len = grown(host["q_len"], entries, 0)
+        q_len[dummy] = t_pad - T
+        tables = []
+        for t in host["tables"]:
+            bt = np.full((entries, width), -1, dtype=np.int32)
+            bt[:E, :t.shape[1]] = t
+            bt[dummy, 0] = 0
+            tables.append(bt)
+        _, _, _, tiles = ops.plan_rows(host["q_len"].tolist(), host["q_start"].tolist(), ops.PLAN_TILE_ROWS)
+        tile_arr = np.empty((self._padded_tiles(t_pad, e_pad), 4), dtype=np.int32)
+        tile_arr[:] = (dummy, T, 1, 0)
+        if tiles:
+            tile_arr[:len(tiles)] = np.asarray(tiles, dtype=np.int32)
+        info = np.empty((e_pad, 4), dtype=np.int32)
+        info[:] = (T, 0, dummy, 0)
+        info[:len(host["decode_info"])] = host["decode_info"]
+        return dict(host, T=t_pad, E=entries, ids=grown(host["ids"], t_pad, 0), pos=grown(host["pos"], t_pad, 0),
+                    ent=grown(host["ent"], t_pad, dummy), cu=cu, q_start=grown(host["q_start"], entries, 0), q_len=q_len,
+                    rows=grown(host["rows"], e_pad, 0), width=width, tables=tables,
+                    slot_maps=[grown(sm, t_pad, -1) for sm in host["slot_maps"]],
+                    state_slots=grown(host["state_slots"], entries, 0), decode_info=info, tiles=tile_arr)
+
+    def _capture_padded(self, key, host):
+        _, t_pad, e_pad, bucket = key
+        width = max(1, -(-bucket // self.page_size))
+        buf = _StepBuffers(t_pad, e_pad + 1, e_pad, width, e_pad, len(self.cache.groups), self.device,
+                           n_tiles=self._padded_tiles(t_pad, e_pad))
+        ctx = self._padded_context(host, buf, t_pad, e_pad, width, bucket)
+        extra = dict(ctx.extra)
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            self.model.forward(ctx)          # outside the graph first: libraries load, the allocator settles
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        self.counts["recorded"] += 1
+        graph = torch.cuda.CUDAGraph()
+        ctx.extra = extra
+        with torch.cuda.graph(graph):
+            logits = self.model.forward(ctx)
+        g = dict(graph=graph, buf=buf, logits=logits, ctx=ctx, width=width)
+        self._graphs[key] = g
+        return g
 
     def _capture(self, key, host):
         """Records the decode step of E single tokens (contexts up to `bucket`) into a HIP graph.  All
@@ -266,6 +395,7 @@ class ModelRunner:
             self.model.forward(ctx)          # warm-up outside the graph: libraries load, allocator settles
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
+        self.counts["recorded"] += 1
         graph = torch.cuda.CUDAGraph()
         ctx.extra = {"decode_info": buf.dev["decode_info"], "decode_span": bucket}
         with torch.cuda.graph(graph):
@@ -294,19 +424,21 @@ def _context_bucket(max_kv):
 
 GRAPH_MAX_ROWS = 256     # decode batches up to this many requests are recorded
 GRAPH_AFTER = 2          # a batch shape is recorded the second time it is seen
-GRAPH_KEEP = 32          # recorded shapes kept at a time (least recently used goes first)
+GRAPH_KEEP = 128         # recorded shapes kept at a time (least recently used goes first)
+MIXED_GRAPH_MAX_TOKENS = 512    # steps with prompt portions are recorded up to this many token rows (padding included)
 
 
 class _StepBuffers:
     """One pinned host buffer and one device buffer that hold all side inputs of a step; `fill` copies the
     host arrays in and uploads them in one transfer."""
 
-    def __init__(self, T, E, R, width, n_decode, ngroups, device):
+    def __init__(self, T, E, R, width, n_decode, ngroups, device, n_tiles=0):
         self.shape = (T, E, R, width, n_decode)
         fields = [("slots%d" % g, np.int64, (T,)) for g in range(ngroups)]
         fields += [("state_slots", np.int64, (E,))]
         fields += [("ids", np.int32, (T,)), ("pos", np.int32, (T,)), ("ent", np.int32, (T,)), ("cu", np.int32, (E + 1,)),
-                   ("q_start", np.int32, (E,)), ("rows", np.int32, (R,)), ("decode_info", np.int32, (n_decode, 4))]
+                   ("q_start", np.int32, (E,)), ("rows", np.int32, (R,)), ("decode_info", np.int32, (n_decode, 4)),
+                   ("tiles", np.int32, (n_tiles, 4))]
         fields += [("table%d" % g, np.int32, (E, max(width, 1))) for g in range(ngroups)]
         offset, self.layout = 0, {}
         for name, dt, shape in fields:
@@ -339,6 +471,8 @@ class _StepBuffers:
         h["rows"][:] = host["rows"]
         h["decode_info"][:] = host["decode_info"]
         h["state_slots"][:] = host["state_slots"]
+        if "tiles" in host:
+            h["tiles"][:] = host["tiles"]
         for g, (bt, sm) in enumerate(zip(host["tables"], host["slot_maps"])):
             h["table%d" % g][:, :bt.shape[1]] = bt
             h["slots%d" % g][:] = sm

@@ -465,30 +465,49 @@ def attention_mfma_supported(dtype, head_dim, page_size):
             and page_size & (page_size - 1) == 0)
 
 
-def _attention_plan(step, tile_rows, device):
-    """Which rows of the step are single new tokens and how the rows of prompt portions fall into tiles;
-    made once per step and shared by all layers."""
-    key = ("attention_plan", tile_rows)
-    plan = step.extra.get(key)
-    if plan is not None:
-        return plan
-    import numpy as np
-    decode_rows, decode_pos, tiles = [], [], []
+def plan_rows(q_len, q_start, tile_rows):
+    """How a step's rows go to the attention kernels: (rows, positions, entries of the single new tokens,
+    tiles of the prompt portions as (entry, first row of the step, rows, first position), heaviest first)."""
+    decode_rows, decode_pos, decode_entries, tiles = [], [], [], []
     o = 0
-    for e in range(step.num_entries):
-        n, start = step.host_q_len[e], step.host_q_start[e]
+    for e, (n, start) in enumerate(zip(q_len, q_start)):
         if n == 1:
             decode_rows.append(o)
             decode_pos.append(start)
+            decode_entries.append(e)
         else:
             for r in range(0, n, tile_rows):
                 tiles.append((e, o + r, min(tile_rows, n - r), start + r))
         o += n
     tiles.sort(key=lambda t: -(t[3] + t[2]))      # the tiles with the most keys first
+    return decode_rows, decode_pos, decode_entries, tiles
+
+
+PLAN_TILE_ROWS = 16       # rows of a prompt portion per wavefront in steps of fewer than PREFILL_WIDE_TILES_FROM tokens
+
+
+def _attention_plan(step, tile_rows, device):
+    """Which rows of the step are single new tokens and how the rows of prompt portions fall into tiles;
+    made once per step and shared by all layers.  A recorded step brings its plan along (`static_plan` in the
+    step's extra: device arrays of fixed size that the runner refills, counts that include padding)."""
+    key = ("attention_plan", tile_rows)
+    plan = step.extra.get(key)
+    if plan is not None:
+        return plan
+    static = step.extra.get("static_plan")
+    if static is not None:
+        _need(tile_rows == static["tile_rows"], "a recorded step was planned for tiles of %d rows, not %d",
+              static["tile_rows"], tile_rows)
+        plan = dict(n_decode=static["n_decode"], decode_pos=None, n_tiles=static["n_tiles"],
+                    decode_span=step.extra.get("decode_span"), decode_info=step.extra.get("decode_info"),
+                    tiles=static["tiles"])
+        step.extra[key] = plan
+        return plan
+    import numpy as np
+    decode_rows, decode_pos, entries, tiles = plan_rows(step.host_q_len, step.host_q_start, tile_rows)
     # (row, position, entry, -) of every single new token; the runner uploads it with the step's other inputs
     decode_info = step.extra.get("decode_info")
     if decode_info is None and decode_rows:
-        entries = [e for e in range(step.num_entries) if step.host_q_len[e] == 1]
         decode_info = torch.tensor([[r, p, e, 0] for r, p, e in zip(decode_rows, decode_pos, entries)], dtype=torch.int32,
                                    device=device)
     plan = dict(
