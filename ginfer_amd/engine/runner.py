@@ -75,6 +75,7 @@ class ModelRunner:
         self._graphs, self._graph_seen = {}, {}
         self.graph_mixed_steps = bool(graph_mixed_steps)
         self._padded_buffers = {}
+        self._graph_budget, self._graph_bytes, self._graph_bytes_seen = None, 0, {}
         # how steps ran: launched kernel by kernel, replayed as a recorded decode step, replayed as a recorded step
         # with prompt portions; and how many steps were recorded
         self.counts = dict(launched=0, replayed_decode=0, replayed_padded=0, recorded=0)
@@ -241,9 +242,7 @@ class ModelRunner:
             else:
                 self._graph_seen[key] = self._graph_seen.get(key, 0) + 1
                 if self._graph_seen[key] >= GRAPH_AFTER:
-                    while len(self._graphs) >= GRAPH_KEEP:      # each graph holds its buffers: forget the oldest
-                        self._graphs.pop(next(iter(self._graphs)))
-                    g = self._capture(key, host)
+                    g = self._record(self._capture, key, host)
             if g is not None:
                 g["buf"].fill(host)
                 if device_tokens is not None:
@@ -261,6 +260,30 @@ class ModelRunner:
             buf.dev["ids"].copy_(device_tokens)
         self.counts["launched"] += 1
         return self.model.forward(ctx)
+
+    def _record(self, capture, key, host):
+        """Records a step unless the device memory that recorded steps may hold is used up (each holds its buffers and
+        its activations): the least recently used ones are forgotten first, by count and by bytes.  None: not
+        recorded, the step runs launch by launch."""
+        if self._graph_budget is None:
+            # half of what the cache pool left free, at most 1/8 of the card
+            free, total = torch.cuda.mem_get_info(self.device)
+            self._graph_budget = min((free + torch.cuda.memory_reserved(self.device)
+                                      - torch.cuda.memory_allocated(self.device)) // 2, total // 8)
+        need = self._graph_bytes_seen.get(key[0] == "padded", 0)
+        while self._graphs and (len(self._graphs) >= GRAPH_KEEP or self._graph_bytes + need > self._graph_budget):
+            old = self._graphs.pop(next(iter(self._graphs)))
+            self._graph_bytes -= old["bytes"]
+            del old
+        if need > self._graph_budget:
+            return None
+        before = torch.cuda.memory_reserved(self.device)     # a recorded step keeps a pool of its own reserved
+        g = capture(key, host)
+        g["bytes"] = max(0, torch.cuda.memory_reserved(self.device) - before)
+        self._graph_bytes += g["bytes"]
+        kind = key[0] == "padded"
+        self._graph_bytes_seen[kind] = max(self._graph_bytes_seen.get(kind, 0), g["bytes"])
+        return g
 
     # ---- recorded steps that hold prompt portions
     def _run_padded(self, host, borrow):
@@ -289,9 +312,7 @@ class ModelRunner:
         else:
             self._graph_seen[key] = self._graph_seen.get(key, 0) + 1
             if self._graph_seen[key] >= GRAPH_AFTER:
-                while len(self._graphs) >= GRAPH_KEEP:
-                    self._graphs.pop(next(iter(self._graphs)))
-                g = self._capture_padded(key, host)
+                g = self._record(self._capture_padded, key, host)
         if g is None:
             # not recorded yet: launched kernel by kernel, but with the same padded sizes, so that a step's bits do not
             # depend on whether its sizes have been seen before
