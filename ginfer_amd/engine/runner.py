@@ -7,6 +7,7 @@ prompts or all single tokens and returns token ids (ginfer/engine/model_runner.c
 ginfer/model/model.cc:180-228); the side inputs built here are the same in kind (ids, positions,
 block tables, slot mapping: model_runner.cc:145-298), flattened per token.
 """
+import time
 from dataclasses import dataclass, field
 from typing import List, Sequence
 
@@ -78,7 +79,7 @@ class ModelRunner:
         self._graph_budget, self._graph_bytes, self._graph_bytes_seen = None, 0, {}
         # how steps ran: launched kernel by kernel, replayed as a recorded decode step, replayed as a recorded step
         # with prompt portions; and how many steps were recorded
-        self.counts = dict(launched=0, replayed_decode=0, replayed_padded=0, recorded=0)
+        self.counts = dict(launched=0, replayed_decode=0, replayed_padded=0, recorded=0, recording_seconds=0.0)
 
     def _pages_from_free_memory(self, specs, utilization):
         """Pages = free device memory (after the weights are resident) * utilization / bytes per page, the
@@ -278,7 +279,9 @@ class ModelRunner:
         if need > self._graph_budget:
             return None
         before = torch.cuda.memory_reserved(self.device)     # a recorded step keeps a pool of its own reserved
+        t0 = time.perf_counter()
         g = capture(key, host)
+        self.counts["recording_seconds"] = round(self.counts["recording_seconds"] + time.perf_counter() - t0, 4)
         g["bytes"] = max(0, torch.cuda.memory_reserved(self.device) - before)
         self._graph_bytes += g["bytes"]
         kind = key[0] == "padded"
