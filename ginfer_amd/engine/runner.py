@@ -6,6 +6,10 @@ side by side; a request may be cut anywhere.  The reference's runner takes a bat
 prompts or all single tokens and returns token ids (ginfer/engine/model_runner.cc:177-317,
 ginfer/model/model.cc:180-228); the side inputs built here are the same in kind (ids, positions,
 block tables, slot mapping: model_runner.cc:145-298), flattened per token.
+
+Steps whose shapes come again are recorded into HIP graphs and replayed: steps of single tokens by their exact
+number of requests, short steps with prompt portions laid into padded sizes (`_run_padded`); all side inputs of
+a recorded step live in one static buffer that every replay refills.
 """
 import time
 from dataclasses import dataclass, field
