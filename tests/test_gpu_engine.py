@@ -511,6 +511,21 @@ def test_head_sizes_between_the_steps_of_16(tmp_path, dtype, head_dim):
         got = H.run_steps(runner, steps)
         runner.cache.check()
         H.compare_with_plain(got, reqs, folder, H.TOL[dtype], "head size %d %s %s" % (head_dim, dtype, what))
+    if head_dim == 24:
+        # as in serving (only an entry's last place wanted), twice over, so that the steps are laid into recorded steps
+        # of padded sizes: the general attention kernel meets the padding rows too
+        steps = H.steps_mixed(reqs, max_live=2, seed=1) + H.steps_mixed({k + "x": v for k, v in reqs.items()}, max_live=2, seed=1)
+        for st in steps:
+            for e in st["entries"]:
+                e["want"] = [len(e["tokens"]) - 1]
+        got = H.run_steps(runner, steps)
+        assert any(k[0] == "padded" for k in runner._graphs)
+        both = dict(reqs)
+        both.update({k + "x": v for k, v in reqs.items()})
+        refs = {rid: H.plain_logits(folder, ids) for rid, ids in both.items()}
+        for (rid, p), row in got.items():
+            err = float(np.abs(row.astype(np.float64) - refs[rid][p]).max() / np.abs(refs[rid]).max())
+            assert np.isfinite(row).all() and err <= H.TOL[dtype], "head size 24 %s padded: %s %d: %.3g" % (dtype, rid, p, err)
 
 
 @pytest.mark.parametrize("seed", list(range(8)))
