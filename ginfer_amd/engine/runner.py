@@ -284,7 +284,16 @@ class ModelRunner:
             return None
         before = torch.cuda.memory_reserved(self.device)     # a recorded step keeps a pool of its own reserved
         t0 = time.perf_counter()
-        g = capture(key, host)
+        try:
+            g = capture(key, host)
+        except Exception as e:           # recording is a matter of speed only: the steps go on launch by launch
+            import sys
+            sys.stderr.write("[ginfer_amd] recording a step failed (%s: %s); steps are launched kernel by kernel from "
+                             "now on\n" % (type(e).__name__, e))
+            self._graphs.pop(key, None)
+            self.use_graphs = False
+            torch.cuda.synchronize()
+            return None
         self.counts["recording_seconds"] = round(self.counts["recording_seconds"] + time.perf_counter() - t0, 4)
         g["bytes"] = max(0, torch.cuda.memory_reserved(self.device) - before)
         self._graph_bytes += g["bytes"]
