@@ -41,6 +41,7 @@ class _Request:
     pending: int = 0                     # tokens reserved by append() and not yet committed
     tables: List[List[int]] = field(default_factory=list)   # per group: logical block -> page or -1
     contents: List[List[int]] = field(default_factory=list) # per group: content number of each remembered block
+    gone: List[int] = field(default_factory=list)           # per group: every block before this one was given back
 
 
 def _block_tokens(token_ids, block, page_size):
@@ -167,7 +168,7 @@ class CacheManager:
         if rid in self.requests:
             raise ValueError("request %r is already in the cache" % (rid,))
         req = self.requests[rid] = _Request(slot=self.slots.take(), tables=[[] for _ in self.groups],
-                                            contents=[[] for _ in self.groups])
+                                            contents=[[] for _ in self.groups], gone=[0] * len(self.groups))
         slot = req.slot
         for t in self._table_np:
             t[slot, :] = -1
@@ -239,7 +240,7 @@ class CacheManager:
         for gi, g in enumerate(self.groups):
             table = req.tables[gi]
             first = g.first_needed_block(start)
-            give = [i for i in range(min(first, len(table))) if table[i] >= 0]
+            give = [i for i in range(req.gone[gi], min(first, len(table))) if table[i] >= 0]
             take = 0
             for i in range(max(first, 0), need_blocks):
                 if i >= len(table) or table[i] < 0:
@@ -267,7 +268,7 @@ class CacheManager:
         for gi, g in enumerate(self.groups):
             table = req.tables[gi]
             first = g.first_needed_block(req.length)
-            give = sum(1 for i in range(min(first, len(table))) if table[i] >= 0)
+            give = sum(1 for i in range(req.gone[gi], min(first, len(table))) if table[i] >= 0)
             have_blocks = len(table)
             room = have_blocks * self.page_size - req.length if have_blocks * self.page_size > req.length else 0
             cap = room + (g.pool.num_free + give) * self.page_size
@@ -296,6 +297,7 @@ class CacheManager:
             g.pool.give_back([table[i] for i in give])
             for i in give:
                 table[i] = -1
+            req.gone[gi] = max(req.gone[gi], min(first, len(table)))
             while len(table) < need_blocks:
                 table.append(-1)
             taken = g.pool.take(take)
