@@ -212,13 +212,18 @@ class CacheManager:
             for i in range(len(chain), full):
                 chain.append(g.remember(chain[i - 1] if i else 0, _block_tokens(token_ids, i, ps), table[i]))
 
-    def _mirror_table(self, gi, req):
+    def _mirror_table(self, gi, req, changed=None):
+        """Copies the request's table of a group into the host mirror: all of it, or the blocks named."""
         table, mirror = req.tables[gi], self._table_np[gi]
         if len(table) > mirror.shape[1]:
             wider = np.full((self.max_requests, max(len(table), 2 * mirror.shape[1])), -1, dtype=np.int32)
             wider[:, :mirror.shape[1]] = mirror
             self._table_np[gi] = mirror = wider
-        mirror[req.slot, :len(table)] = table
+        if changed is None:
+            mirror[req.slot, :len(table)] = table
+        else:
+            for i in changed:
+                mirror[req.slot, i] = table[i]
 
     def length(self, rid):
         return self.requests[rid].length
@@ -239,6 +244,9 @@ class CacheManager:
         need_blocks = -(-end // self.page_size)
         for gi, g in enumerate(self.groups):
             table = req.tables[gi]
+            if g.window is None:         # a table without a window has no gaps: what is missing lies at its end
+                plan.append(([], max(0, need_blocks - len(table)), 0, need_blocks))
+                continue
             first = g.first_needed_block(start)
             give = [i for i in range(req.gone[gi], min(first, len(table))) if table[i] >= 0]
             take = 0
@@ -298,16 +306,19 @@ class CacheManager:
             for i in give:
                 table[i] = -1
             req.gone[gi] = max(req.gone[gi], min(first, len(table)))
+            scan_from = max(first, 0) if g.window is not None else len(table)
             while len(table) < need_blocks:
                 table.append(-1)
             taken = g.pool.take(take)
             for p in taken:
                 g.forget(p)              # what the page held for requests to come is gone
             new_pages = iter(taken)
-            for i in range(max(first, 0), need_blocks):
+            changed = list(give)
+            for i in range(scan_from, need_blocks):
                 if table[i] < 0:
                     table[i] = next(new_pages)
-            self._mirror_table(gi, req)
+                    changed.append(i)
+            self._mirror_table(gi, req, changed)
         req.pending = n_new
         return req.length
 
