@@ -81,6 +81,11 @@ class ModelRunner:
         self.graph_mixed_steps = bool(graph_mixed_steps)
         self._padded_buffers = {}
         self._graph_budget, self._graph_bytes, self._graph_bytes_seen = None, 0, {}
+        # Padding pays while the host's launches (~5 ms a step) outlast the device's work on the padded rows, which may
+        # be twice the step's own: with some 1e15 operations a second that is rows * weights < ~1.5e12 (512 rows for a
+        # 1.5B model, 128 for a 7B one, none for a 72B one)
+        weights = sum(int(np.prod(ws.shape)) for ws in self.model.weight_specs().values())
+        self._padded_max_rows = min(MIXED_GRAPH_MAX_TOKENS, int(1.5e12 // max(weights, 1)))
         # how steps ran: launched kernel by kernel, replayed as a recorded decode step, replayed as a recorded step
         # with prompt portions; and how many steps were recorded
         self.counts = dict(launched=0, replayed_decode=0, replayed_padded=0, recorded=0, recording_seconds=0.0)
@@ -310,11 +315,13 @@ class ModelRunner:
         and single-token records that fill the plan point at the first padding row.  Rows do not mix in any kernel,
         so what the padding computes stays in the padding.  None: the step runs launch by launch."""
         T, E, R = host["T"], host["E"], len(host["rows"])
-        if T + 1 > MIXED_GRAPH_MAX_TOKENS or E > GRAPH_MAX_ROWS:
+        if T + 1 > self._padded_max_rows or E > GRAPH_MAX_ROWS:
             return None
         t_pad = 64                       # coarse sizes, so that few recorded steps serve many: rows 64, 128, 256, 512
         while t_pad < T + 1:
             t_pad *= 2
+        if t_pad > self._padded_max_rows:
+            return None
         e_pad = 8                        # entries 8, 16, ... 256
         while e_pad < E:
             e_pad *= 2
