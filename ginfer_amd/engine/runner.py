@@ -370,37 +370,7 @@ class ModelRunner:
         return ctx
 
     def _pad(self, host, t_pad, e_pad, width):
-        from ..kernels import ops
-        T, E, R = host["T"], host["E"], len(host["rows"])
-        dummy, entries = e_pad, e_pad + 1
-        def grown(a, n, fill):
-            out = np.full((n,) + a.shape[1:], fill, dtype=a.dtype)
-            out[:a.shape[0]] = a
-            return out
-        cu = np.full(entries + 1, T, dtype=np.int32)
-        cu[:E + 1] = host["cu"]
-        cu[entries] = t_pad
-        q_len = grown(host["q_len"], entries, 0)
-        q_len[dummy] = t_pad - T
-        tables = []
-        for t in host["tables"]:
-            bt = np.full((entries, width), -1, dtype=np.int32)
-            bt[:E, :t.shape[1]] = t
-            bt[dummy, 0] = 0
-            tables.append(bt)
-        _, _, _, tiles = ops.plan_rows(host["q_len"].tolist(), host["q_start"].tolist(), ops.PLAN_TILE_ROWS)
-        tile_arr = np.empty((self._padded_tiles(t_pad, e_pad), 4), dtype=np.int32)
-        tile_arr[:] = (dummy, T, 1, 0)
-        if tiles:
-            tile_arr[:len(tiles)] = np.asarray(tiles, dtype=np.int32)
-        info = np.empty((e_pad, 4), dtype=np.int32)
-        info[:] = (T, 0, dummy, 0)
-        info[:len(host["decode_info"])] = host["decode_info"]
-        return dict(host, T=t_pad, E=entries, ids=grown(host["ids"], t_pad, 0), pos=grown(host["pos"], t_pad, 0),
-                    ent=grown(host["ent"], t_pad, dummy), cu=cu, q_start=grown(host["q_start"], entries, 0), q_len=q_len,
-                    rows=grown(host["rows"], e_pad, 0), width=width, tables=tables,
-                    slot_maps=[grown(sm, t_pad, -1) for sm in host["slot_maps"]],
-                    state_slots=grown(host["state_slots"], entries, 0), decode_info=info, tiles=tile_arr)
+        return pad_step(host, t_pad, e_pad, width)
 
     def _capture_padded(self, key, host):
         _, t_pad, e_pad, bucket = key
@@ -455,6 +425,43 @@ class ModelRunner:
         out = np.full((table.shape[0], width), -1, dtype=np.int32)
         out[:, :table.shape[1]] = table
         return out
+
+
+def pad_step(host, t_pad, e_pad, width):
+    """The host arrays of a step laid into t_pad token rows and e_pad + 1 entries: the step's own come first, the
+    rest is padding (see ModelRunner._run_padded).  Tables are `width` wide."""
+    from ..kernels import ops
+    T, E = host["T"], host["E"]
+    dummy, entries = e_pad, e_pad + 1
+
+    def grown(a, n, fill):
+        out = np.full((n,) + a.shape[1:], fill, dtype=a.dtype)
+        out[:a.shape[0]] = a
+        return out
+    cu = np.full(entries + 1, T, dtype=np.int32)
+    cu[:E + 1] = host["cu"]
+    cu[entries] = t_pad
+    q_len = grown(host["q_len"], entries, 0)
+    q_len[dummy] = t_pad - T
+    tables = []
+    for t in host["tables"]:
+        bt = np.full((entries, width), -1, dtype=np.int32)
+        bt[:E, :t.shape[1]] = t
+        bt[dummy, 0] = 0
+        tables.append(bt)
+    _, _, _, tiles = ops.plan_rows(host["q_len"].tolist(), host["q_start"].tolist(), ops.PLAN_TILE_ROWS)
+    tile_arr = np.empty(((t_pad // ops.PLAN_TILE_ROWS + e_pad), 4), dtype=np.int32)
+    tile_arr[:] = (dummy, T, 1, 0)
+    if tiles:
+        tile_arr[:len(tiles)] = np.asarray(tiles, dtype=np.int32)
+    info = np.empty((e_pad, 4), dtype=np.int32)
+    info[:] = (T, 0, dummy, 0)
+    info[:len(host["decode_info"])] = host["decode_info"]
+    return dict(host, T=t_pad, E=entries, ids=grown(host["ids"], t_pad, 0), pos=grown(host["pos"], t_pad, 0),
+                ent=grown(host["ent"], t_pad, dummy), cu=cu, q_start=grown(host["q_start"], entries, 0), q_len=q_len,
+                rows=grown(host["rows"], e_pad, 0), width=width, tables=tables,
+                slot_maps=[grown(sm, t_pad, -1) for sm in host["slot_maps"]],
+                state_slots=grown(host["state_slots"], entries, 0), decode_info=info, tiles=tile_arr)
 
 
 def _context_bucket(max_kv):
