@@ -149,10 +149,11 @@ class Engine:
         return dict(scheduled=scheduled, tokens=tokens, arrival=arrival, n_prefill=n_prefill,
                     n_decode=sum(sc.num_tokens for sc in scheduled) - n_prefill)
 
-    def step(self) -> List[RequestOutput]:
+    def step(self, on_token=None) -> List[RequestOutput]:
         """One scheduled batch through the model; returns the requests that finished in it.  While every
         running request just decodes, the next step is launched before this step's tokens are read
-        (`pipeline_decode`): the host's work on a step then overlaps the device's work on the next."""
+        (`pipeline_decode`): the host's work on a step then overlaps the device's work on the next.
+        on_token(request_id, token): called for every token that a request gets in this step, as soon as it is read."""
         t0 = time.perf_counter()
         cur = self._launched
         self._launched = None
@@ -174,7 +175,11 @@ class Engine:
             event.synchronize()
             tokens = host[:n].tolist()
         now = time.perf_counter()
+        before = [(sc.seq, sc.seq.num_tokens) for sc in cur["scheduled"] if sc.samples] if on_token else ()
         finished = self.scheduler.absorb(cur["scheduled"], tokens, now)
+        for seq, n in before:
+            if seq.num_tokens > n:
+                on_token(seq.request_id, seq.token_ids[-1])
         self._launched = nxt
         dt = now - t0
         n_prefill, n_decode = cur["n_prefill"], cur["n_decode"]
@@ -197,9 +202,10 @@ class Engine:
         return RequestOutput(s.request_id, s.token_ids[:s.num_prompt_tokens], s.output_ids, s.finish_reason,
                              ttft, tpot, s.evictions)
 
-    def generate(self, prompts, params=None) -> List[RequestOutput]:
+    def generate(self, prompts, params=None, on_token=None) -> List[RequestOutput]:
         """prompts: lists of token ids; params: one SamplingParams for all, or one per prompt.  Returns the
-        outputs in the order of the prompts."""
+        outputs in the order of the prompts.  on_token(request_id, token): called as the tokens arrive; the
+        request ids are those of add_request, counted up from the engine's first request."""
         if params is None or isinstance(params, SamplingParams):
             params = [params] * len(prompts)
         if len(params) != len(prompts):
@@ -208,6 +214,6 @@ class Engine:
         ids = [self.add_request(p, copy.copy(sp)) for p, sp in zip(prompts, params)]
         done = {}
         while self.has_unfinished():
-            for out in self.step():
+            for out in self.step(on_token):
                 done[out.request_id] = out
         return [done[i] for i in ids]

@@ -129,11 +129,14 @@ def test_greedy_generation_through_the_entry_point(folders, dtype):
     prompts = [H.random_tokens(n, vocab, 200 + n) for n in (1, 9, 40, 64, 100)]
     eng = Engine(EngineConfig(model_path=folder, dtype=dtype, max_num_batched_tokens=24, max_num_seqs=4,
                               max_seq_len=256, kvcache_block_size=8, num_kvcache_blocks=40))
-    outs = eng.generate(prompts, SamplingParams(max_tokens=12, ignore_eos=True))
+    streamed = {}
+    outs = eng.generate(prompts, SamplingParams(max_tokens=12, ignore_eos=True),
+                        on_token=lambda rid, tok: streamed.setdefault(rid, []).append(tok))
     eng.runner.cache.check()
     assert not eng.runner.cache.requests
     for p, o in zip(prompts, outs):
         assert o.prompt_token_ids == p and len(o.token_ids) == 12 and o.finish_reason == "max_tokens"
+        assert streamed[o.request_id] == o.token_ids          # every token was handed out as it came, in order
     _greedy_as_plain(folder, prompts, outs, dtype)
 
 
