@@ -60,12 +60,13 @@ def main():
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--points", default="1,64", help="other decode batch sizes to report")
-    ap.add_argument("--model-dir", default=None, help="reuse a model folder written earlier")
+    ap.add_argument("--model-dir", default=None, help="a model folder: reused if it holds a model, else written (implies --file-weights)")
     ap.add_argument("--shape", default="1.5b", choices=sorted(SHAPES), help="layer sizes (the headline is 1.5b)")
     ap.add_argument("--no-measured-peaks", action="store_true",
                     help="leave out the box's own copy bandwidth and product rate (the fractions use the published peaks)")
-    ap.add_argument("--device-weights", action="store_true",
-                    help="draw the weights on the device instead of writing and reading a model folder (always for 72b)")
+    ap.add_argument("--file-weights", action="store_true",
+                    help="write the random weights into a model folder and load them from there, instead of drawing them "
+                         "on the device (not for 72b: 145 GB)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this engine runs on ONE GPU; --gpus %d is not supported" % args.gpus)
@@ -79,7 +80,7 @@ def main():
     full_layers = shape["num_hidden_layers"]
     if args.layers is None:
         args.layers = full_layers
-    device_weights = args.device_weights or args.shape == "72b"
+    device_weights = args.shape == "72b" or not (args.file_weights or args.model_dir)
     cfg = dict(shape, num_hidden_layers=args.layers)
     weight_bytes, kv_per_token, prefill_flops = model_numbers(cfg, args.layers)
     tmp = None
