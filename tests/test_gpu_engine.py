@@ -352,6 +352,16 @@ def test_command_line(folders, tmp_path):
         assert out.returncode == 0, out.stderr
         runs.append(json.loads(out.stdout.strip().splitlines()[0])["token_ids"])
     assert runs[0] == runs[1] and len(runs[0]) == 4
+    # the benchmark with requests that arrive while the engine runs
+    cmd = [sys.executable, os.path.join(H.ROOT, "bin", "ginfer"), "benchmark", "--random-config",
+           os.path.join(str(folders[name]), "config.json"), "--dtype", "bfloat16", "--num-prompts", "12", "--prompt-len", "9",
+           "--max-tokens", "5", "--request-rate", "2000", "--max-num-seqs", "4", "--max-num-batched-tokens", "32",
+           "--max-seq-len", "64", "--num-kvcache-blocks", "32"]
+    out = subprocess.run(cmd, env=dict(os.environ, MODEL_PATH=""), capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stderr
+    rep = json.loads(out.stdout.strip().splitlines()[-1])
+    assert rep["total_tokens"] == 12 * (9 + 5) and rep["ttft_ms"]["p50"] > 0 and rep["tpot_ms"]["mean"] > 0
+    assert sum(rep["ran"][k] for k in ("launched", "replayed_decode", "replayed_padded")) >= rep["steps"]
 
 
 def test_real_layer_sizes(tmp_path):
