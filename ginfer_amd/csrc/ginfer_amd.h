@@ -63,6 +63,8 @@ int ga_qkv_rope_skinny(void* q_out, const void* A, int64_t lda, const void* W, c
 
 // ---- activation.hip: out [tokens, inter] = silu(gu[:, :inter]) * gu[:, inter:]
 int ga_silu_mul(void* out, const void* gu, int tokens, int inter, int is_bf16, hipStream_t stream);
+// the same on a product that lies transposed, gu_t [2 inter, tokens] bfloat16; tokens and inter multiples of 8
+int ga_silu_mul_transposed(void* out, const void* gu_t, int tokens, int inter, hipStream_t stream);
 
 // ---- attention_generic.hip: every token attends to its request's pages; any head size up to 256, window or 0
 int ga_paged_attention_generic(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* k_pages,

@@ -132,6 +132,21 @@ def silu_mul(gate_up, out=None):
     return out
 
 
+def silu_mul_transposed(gate_up_t, out=None):
+    """gate_up_t [2I, T] (the gate-up product lying transposed) -> [T, I]: silu(gate) * up."""
+    _dev(gate_up_t, out)
+    _need(gate_up_t.dim() == 2 and gate_up_t.is_contiguous() and gate_up_t.dtype == torch.bfloat16
+          and gate_up_t.shape[0] % 16 == 0 and gate_up_t.shape[1] % 8 == 0,
+          "gate_up_t must be contiguous bfloat16 [2I, T] with I and T multiples of 8")
+    I, T = gate_up_t.shape[0] // 2, gate_up_t.shape[1]
+    if out is None:
+        out = torch.empty((T, I), dtype=torch.bfloat16, device=gate_up_t.device)
+    _need(out.dtype == torch.bfloat16 and out.shape == (T, I) and out.is_contiguous(), "out must be contiguous bfloat16 [T, I]")
+    lib = build.load("activation")
+    _check(lib.ga_silu_mul_transposed(_ptr(out), _ptr(gate_up_t), _i(T), _i(I), _stream()), "silu_mul_transposed")
+    return out
+
+
 def rope_kv_write(qkv, positions, cos, sin, slot_mapping, k_pages, v_pages, num_heads, num_kv_heads,
                   head_dim, write_kv=True):
     """Rotates q and k inside qkv [T, (nh + 2 nkv) hd] in place and writes k, v to the paged cache

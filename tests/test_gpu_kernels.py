@@ -85,6 +85,22 @@ def test_silu_mul(dtype, tol, T, I):
     assert out[0, 0] == 0 and abs(out[0, 1] - 100.0) < 1 and abs(out[0, 2]) < 1e-6
 
 
+@pytest.mark.parametrize("T,I", [(8, 8), (64, 64), (72, 136), (512, 1000), (2048, 8960), (264, 24)])
+def test_silu_mul_on_a_transposed_product(T, I):
+    """The same activation on a product that lies transposed, [2I, T]: equal to the usual kernel on the same numbers,
+    bit for bit, at sizes with whole and with broken tiles."""
+    from ginfer_amd.kernels import ops
+    gu = rnd((T, 2 * I), torch.bfloat16, 6, scale=3.0)
+    got = ops.silu_mul_transposed(gu.t().contiguous())
+    assert got.shape == (T, I) and torch.equal(got, ops.silu_mul(gu))
+    ref = torch.nn.functional.silu(gu[:, :I].double()) * gu[:, I:].double()
+    close(got, ref, 1e-2)
+    with pytest.raises(ops.KernelError):
+        ops.silu_mul_transposed(rnd((2 * 12, 16), torch.bfloat16, 1))        # I = 12 is no multiple of 8
+    with pytest.raises(ops.KernelError):
+        ops.silu_mul_transposed(rnd((16, 12), torch.bfloat16, 1))            # nor are 12 tokens
+
+
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 5e-5), (torch.bfloat16, 1e-2)])
 @pytest.mark.parametrize("M,N,K,bias", [(2, 8, 9, True), (1031, 2000, 408, False), (512, 1024, 256, True),
                                         (130, 1001, 1000, True), (1, 1000, 128, True), (1, 197, 4216, False),

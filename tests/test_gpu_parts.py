@@ -33,7 +33,7 @@ PART_DTYPES = [(torch.float32, 1e-5), (torch.bfloat16, 2e-2)]
 
 
 @pytest.mark.parametrize("dtype,tol", PART_DTYPES)
-@pytest.mark.parametrize("T", [1, 7, 200])
+@pytest.mark.parametrize("T", [1, 7, 200, 512, 768])     # 512, 768: the product with the weights first, transposed
 def test_swiglu_part(dtype, tol, T):
     from ginfer_amd.parts import lookup
     Hd, I = 88, 136
