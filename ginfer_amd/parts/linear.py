@@ -135,7 +135,7 @@ def gated_linear(x, weight_gate_up):
 def _transposed_product_is_faster(x, weight):
     """Measured on MI355X at the 1.5B, 7B and 72B shapes' gate-up product: with a number of rows that is a multiple of
     256 (the portions that a token budget of 2,048 cuts) the library's tiles fit the rows when the weights are its
-    first operand: level to 15 % faster (2,048 rows of the 1.5B shape: 115 -> 98 us); with other row counts it is up
-    to 20 % slower, so they keep the usual product."""
-    return (x.dtype == torch.bfloat16 and x.shape[0] >= 512 and x.shape[0] % 256 == 0 and x.is_contiguous()
+    first operand: level to 15 % faster (2,048 rows of the 1.5B shape: 115 -> 98 us; 256 rows, a decode step of 256
+    requests: 3 to 8 %); with other row counts it is up to 20 % slower, so they keep the usual product."""
+    return (x.dtype == torch.bfloat16 and x.shape[0] >= 256 and x.shape[0] % 256 == 0 and x.is_contiguous()
             and weight.shape[0] % 16 == 0 and x.shape[1] % 8 == 0)
