@@ -193,29 +193,27 @@ __device__ __forceinline__ void tile_scores(f32x4 (&s)[NB][2], const bf16x8 (&kr
 // kept in scaled units; the scale rides on the exponent's multiply-add.  An empty column (no query: its q is
 // zero) goes along unmasked in interior tiles; nothing of it is ever written.
 template <int NB>
-__device__ __forceinline__ void tile_softmax(bf16x8 (&pb)[NB], const f32x4 (&s)[NB][2], f32x4 (&o)[NB][DB],
+__device__ __forceinline__ void tile_softmax(bf16x8 (&pb)[NB], f32x4 (&s)[NB][2], f32x4 (&o)[NB][DB],
                                              float (&m)[NB], float (&l)[NB], const int (&cpos)[NB],
                                              const int (&clo)[NB], int full_lo, int full_hi, int k0, float scale,
                                              int g) {
   const bool interior = k0 >= full_lo && k0 + 31 <= full_hi;      // the same for the whole wavefront
 #pragma unroll
   for (int nb = 0; nb < NB; ++nb) {
+    if (!interior) {
+      // The lane's key j is live where lo <= j <= hi: two subtractions here, none on the path without a mask.  The
+      // scores are masked where they lie (a select: what was read for a dead key is dropped), so that the path
+      // without a mask copies nothing.
+      const int lo = clo[nb] - (k0 + 8 * g), hi = cpos[nb] - (k0 + 8 * g);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) s[nb][j >> 2][j & 3] = (j >= lo && j <= hi) ? s[nb][j >> 2][j & 3] : -INFINITY;
+    }
     float sv[8];
     float mx = -INFINITY;
-    if (interior) {
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        sv[j] = s[nb][j >> 2][j & 3];
-        mx = fmaxf(mx, sv[j]);
-      }
-    } else {
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const int key = k0 + 8 * g + j;
-        const bool valid = key >= clo[nb] && key <= cpos[nb];
-        sv[j] = valid ? s[nb][j >> 2][j & 3] : -INFINITY;      // a select: what was read for a dead key is dropped
-        mx = fmaxf(mx, sv[j]);
-      }
+    for (int j = 0; j < 8; ++j) {
+      sv[j] = s[nb][j >> 2][j & 3];
+      mx = fmaxf(mx, sv[j]);
     }
     // The running max is raised lazily: only when some score of the tile exceeds it by more than
     // LAZY_MAX (in log2 units), which after the first tiles is rare.  Until then exponentials may reach
