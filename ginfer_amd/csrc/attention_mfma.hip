@@ -25,8 +25,9 @@
 //   O^T += V^T P: which is exactly the k-slot layout of operand B for P, with no shuffle; operand A is
 //                 16 dims x 8 consecutive keys of V^T: one 16-byte load per lane because the cache keeps
 //                 values transposed inside a page ([page][kv_head][dim][slot]).
-// Nothing is staged through LDS: each operand element is loaded once per wavefront, and the heads of a
-// group that run side by side hit the same lines in the vector cache.
+// The decode kernel and the first prefill kernel stage nothing through LDS: each operand element is loaded
+// once per wavefront, and the heads of a group that run side by side hit the same lines in the vector cache.
+// The second prefill kernel (head sizes 64, 128, 256) has one wavefront load each tile into LDS for all heads.
 #include "common.cuh"
 
 #ifndef HEAD_DIM
