@@ -58,3 +58,11 @@ __device__ __forceinline__ float block_sum(float v, float* scratch) {
 }
 
 #define GA_CHECK_LAUNCH() ((int)hipGetLastError())
+
+// Page and place in the page of a cache slot (slot >= 0).  Page sizes are powers of two nearly always: then a shift,
+// for a 64-bit division is some hundred instructions, in every thread, before the first store can go out.
+__device__ __forceinline__ void slot_page(int64_t slot, int page_size, int64_t& page, int64_t& off) {
+  if ((page_size & (page_size - 1)) == 0) page = slot >> (__ffs(page_size) - 1);
+  else page = slot / page_size;
+  off = slot - page * page_size;
+}

@@ -524,7 +524,8 @@ __global__ __launch_bounds__(SK_THREADS) void qkv_rope_skinny_kernel(
     lo += e_blo[it];
     hi += e_bhi[it];
     const int64_t slot = e_slot[it];
-    const int64_t page = slot >= 0 ? slot / page_size : 0, off = slot >= 0 ? slot - page * page_size : 0;
+    int64_t page = 0, off = 0;
+    if (slot >= 0) slot_page(slot, page_size, page, off);
     if (u < qk_units) {
       const int head = u / upq, j = (u % upq) * CP + nl;
       const float c = e_cos[it], sn = e_sin[it];

@@ -30,7 +30,8 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, const int32_t* __restr
     const int64_t slot = slot_mapping[t];
     if (slot >= 0) {
       const int g = is_k ? head - nh : head - nh - nkv;
-      const int64_t page = slot / page_size, off = slot - page * page_size;
+      int64_t page, off;
+      slot_page(slot, page_size, page, off);
       dst = is_k ? k_pages + ((page * nkv + g) * page_size + off) * hd
                  : v_pages + (page * nkv + g) * (int64_t)hd * page_size + off;
     }
@@ -79,8 +80,7 @@ __global__ __launch_bounds__(256) void rope_kv_write_vec_kernel(
   if (write_kv) {
     const int64_t slot = slot_mapping[t];
     if (slot >= 0) {
-      page = slot / page_size;
-      off = slot - page * page_size;
+      slot_page(slot, page_size, page, off);
     }
   }
   for (int item = threadIdx.x; item < total; item += blockDim.x) {

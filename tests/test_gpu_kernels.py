@@ -170,6 +170,43 @@ def test_rope_and_cache_write(dtype, tol, T, nh, nkv, hd, rd, theta):
     assert torch.equal(kp1, kp0) and torch.equal(vp1, vp0)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("ps", [4, 8, 12, 16, 32])
+def test_cache_write_of_slots_in_a_row(dtype, ps):
+    """Prompt portions: tokens whose slots follow each other, starting anywhere in a page, across page ends, with
+    tokens that write nothing and single tokens of other requests between them.  Every value lands in its slot of
+    the transposed page and nothing else changes."""
+    from ginfer_amd.kernels import ops
+    nh, nkv, hd, pages = 4, 2, 64, 100
+    runs = [(5, 35), (-1, 1), (100, 20), (311, 1), (-1, 2), (160, 9), (330 + ps - 1, 1), (200, 17), (250, 3)]
+    slots = []
+    for first, n in runs:
+        slots += [-1] * n if first < 0 else list(range(first, first + n))
+    assert len(set(x for x in slots if x >= 0)) == sum(1 for x in slots if x >= 0) and max(slots) < pages * ps
+    T = len(slots)
+    slots = torch.tensor(slots, dtype=torch.int64)
+    qkv = rnd((T, (nh + 2 * nkv) * hd), dtype, 21)
+    positions = torch.arange(T, dtype=torch.int32, device=dev())
+    sin, cos = pm.rope_tables(1e4, hd, T)
+    kp, vp = rnd((pages, nkv, ps, hd), dtype, 22), rnd((pages, nkv, hd, ps), dtype, 23)
+    kexp, vexp = kp.clone().cpu(), vp.clone().cpu()
+    x = qkv.clone()
+    ops.rope_kv_write(x, positions, cos.to(dev()), sin.to(dev()), slots.to(dev()), kp, vp, nh, nkv, hd)
+    xk = x[:, nh * hd:(nh + nkv) * hd].cpu().view(T, nkv, hd)
+    v = qkv[:, (nh + nkv) * hd:].cpu().view(T, nkv, hd)
+    for t in range(T):
+        sl = int(slots[t])
+        if sl >= 0:
+            kexp[sl // ps, :, sl % ps, :] = xk[t]
+            vexp[sl // ps, :, :, sl % ps] = v[t]
+    assert torch.equal(kp.cpu(), kexp) and torch.equal(vp.cpu(), vexp)
+    # the rotation is the one of single tokens
+    one = qkv[40:41].clone()
+    ops.rope_kv_write(one, positions[40:41].contiguous(), cos.to(dev()), sin.to(dev()), slots[40:41].to(dev()),
+                      kp.clone(), vp.clone(), nh, nkv, hd)
+    assert torch.equal(one[0], x[40])
+
+
 # ----------------------------------------------------------------------------- attention
 
 def _paged_case(seqs, nh, nkv, hd, ps, dtype, seed, window=None, spike=None):
