@@ -57,6 +57,76 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, const int32_t* __restr
   }
 }
 
+// The values of ROPE_ROWS consecutive tokens of the step, written by one workgroup.  In the transposed pages an
+// element of v lies page_size elements from the next of its token, so a token alone writes 2 or 4 bytes at a time,
+// each into a 32-byte sector of its own.  Here the tokens' v rows wait in LDS, and the thread that owns one
+// (kv head, dim) writes the tokens whose slots follow each other inside a page in one store of up to 16 bytes: the
+// tokens of a prompt portion do.  Which tokens form a run depends on the slots alone, so the threads branch together.
+// Dynamic LDS: ROPE_ROWS * nkv * hd elements.
+#define ROPE_ROWS 8
+#define ROPE_VALUE_BLOCKS_FROM 512
+template <typename T>
+__device__ __forceinline__ void write_values_in_runs(const T* __restrict__ qkv, const int64_t* __restrict__ slot_mapping,
+                                                     T* __restrict__ v_pages, int tokens, int64_t t0, int nh, int nkv,
+                                                     int hd, int page_size) {
+  constexpr int V = 16 / sizeof(T);
+  extern __shared__ __attribute__((aligned(16))) unsigned char rows_lds[];
+  T* v_rows = reinterpret_cast<T*>(rows_lds);                       // [ROPE_ROWS][nkv * hd]
+  __shared__ int64_t s_slot[ROPE_ROWS];
+  const int rows = tokens - t0 < ROPE_ROWS ? (int)(tokens - t0) : ROPE_ROWS;
+  const int width = nkv * hd, chunks = width / V;
+  if ((int)threadIdx.x < rows) s_slot[threadIdx.x] = slot_mapping[t0 + threadIdx.x];
+  for (int idx = threadIdx.x; idx < rows * chunks; idx += blockDim.x) {
+    const int r = idx / chunks, ch = idx % chunks;
+    *reinterpret_cast<uint4*>(v_rows + r * width + ch * V) =
+        *reinterpret_cast<const uint4*>(qkv + (t0 + r) * (int64_t)(nh + 2 * nkv) * hd + (int64_t)(nh + nkv) * hd + ch * V);
+  }
+  __syncthreads();
+  for (int pair = threadIdx.x; pair < width; pair += blockDim.x) {
+    const int g = pair / hd, j = pair % hd;
+    const T* mine = v_rows + pair;                                  // this (kv head, dim) of row r: mine[r * width]
+    int r = 0;
+    while (r < rows) {                                              // the same walk in every thread
+      const int64_t slot = s_slot[r];
+      if (slot < 0) {
+        ++r;
+        continue;
+      }
+      int64_t page, off;
+      slot_page(slot, page_size, page, off);
+      int len = 1;                                                  // tokens of the run: a power of two, at most V
+      for (int c = V; c > 1; c >>= 1) {
+        if (r + c > rows || page_size % c || off % c) continue;
+        bool follow = true;
+        for (int i = 1; i < c; ++i) follow = follow && s_slot[r + i] == slot + i;
+        if (follow) {
+          len = c;
+          break;
+        }
+      }
+      T* dst = v_pages + ((page * nkv + g) * (int64_t)hd + j) * page_size + off;
+      union { uint4 u; uint2 d; uint32_t w; T e[V]; } out;
+      if (len == V) {
+#pragma unroll
+        for (int i = 0; i < V; ++i) out.e[i] = mine[(r + i) * width];
+        *reinterpret_cast<uint4*>(dst) = out.u;
+      } else if (len * sizeof(T) == 8) {
+#pragma unroll
+        for (int i = 0; i < (int)(8 / sizeof(T)); ++i) out.e[i] = mine[(r + i) * width];
+        *reinterpret_cast<uint2*>(dst) = out.d;
+      } else if (len == 2 && sizeof(T) == 2) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) out.e[i] = mine[(r + i) * width];
+        *reinterpret_cast<uint32_t*>(dst) = out.w;
+      } else {
+        len = 1;
+        dst[0] = mine[r * width];
+      }
+      r += len;
+    }
+  }
+}
+
 // The same with 16-byte accesses: one workgroup per token walks all heads; an item is a chunk of V
 // consecutive pairs (j, j + half) of a q or k head, a chunk of the unrotated tail, or a chunk of a v head.
 // For rotary_dim / 2, head_dim - rotary_dim and head_dim multiples of V = 16 / sizeof(T).
@@ -64,8 +134,14 @@ template <typename T>
 __global__ __launch_bounds__(256) void rope_kv_write_vec_kernel(
     T* __restrict__ qkv, const int32_t* __restrict__ positions, const float* __restrict__ cos_t,
     const float* __restrict__ sin_t, const int64_t* __restrict__ slot_mapping, T* __restrict__ k_pages,
-    T* __restrict__ v_pages, int nh, int nkv, int hd, int rotary_dim, int page_size, int write_kv) {
+    T* __restrict__ v_pages, int nh, int nkv, int hd, int rotary_dim, int page_size, int write_kv, int tokens,
+    int value_blocks) {
   constexpr int V = 16 / sizeof(T);
+  if (value_blocks && (int)blockIdx.x >= tokens) {
+    write_values_in_runs<T>(qkv, slot_mapping, v_pages, tokens, ((int64_t)blockIdx.x - tokens) * ROPE_ROWS, nh, nkv, hd,
+                            page_size);
+    return;
+  }
   const int64_t t = blockIdx.x;
   const int half = rotary_dim >> 1;
   const int rot_chunks = half / V, tail_chunks = (hd - rotary_dim) / V, v_chunks = hd / V;
@@ -93,10 +169,17 @@ __global__ __launch_bounds__(256) void rope_kv_write_vec_kernel(
         union { uint4 u; T e[V]; } lo, hi, olo, ohi;
         lo.u = *reinterpret_cast<const uint4*>(x + j);
         hi.u = *reinterpret_cast<const uint4*>(x + j + half);
+        // the tables' rows in 16-byte loads too (a row starts at a multiple of V floats, and so does j)
+        union { float4 q[V / 4]; float e[V]; } cv, sv;
+#pragma unroll
+        for (int i = 0; i < V / 4; ++i) {
+          cv.q[i] = *reinterpret_cast<const float4*>(c + j + 4 * i);
+          sv.q[i] = *reinterpret_cast<const float4*>(s + j + 4 * i);
+        }
 #pragma unroll
         for (int i = 0; i < V; ++i) {
           const float l = Num<T>::ld(&lo.e[i]), h = Num<T>::ld(&hi.e[i]);
-          const float cj = c[j + i], sj = s[j + i];
+          const float cj = cv.e[i], sj = sv.e[i];
           Num<T>::st(&olo.e[i], l * cj - h * sj);
           Num<T>::st(&ohi.e[i], l * sj + h * cj);
         }
@@ -110,7 +193,7 @@ __global__ __launch_bounds__(256) void rope_kv_write_vec_kernel(
         const int j = rotary_dim + (ch - rot_chunks) * V;
         *reinterpret_cast<uint4*>(dst + j) = *reinterpret_cast<const uint4*>(x + j);
       }
-    } else if (page >= 0) {
+    } else if (page >= 0 && !value_blocks) {
       const int vi = item - qk_items;
       const int g = vi / v_chunks, j = (vi % v_chunks) * V;
       union { uint4 u; T e[V]; } val;
@@ -129,16 +212,23 @@ extern "C" int ga_rope_kv_write(void* qkv, const void* positions, const void* co
   if (tokens <= 0) return 0;
   const int v = is_bf16 ? 8 : 4;
   if ((rotary_dim / 2) % v == 0 && (hd - rotary_dim) % v == 0 && hd % v == 0) {
+    // Further workgroups that write the values of ROPE_ROWS tokens each, where their rows fit in LDS and the step is
+    // long (measured on MI355X, 12 + 2 x 2 heads of 128, slots 5 past a page's start: 8.2 -> 7.7 us at 2,048 tokens,
+    // 37 -> 31 at 16,384; at 256 tokens, where the launch is what counts, 3.6 -> 4.2)
+    const size_t rows_lds = (size_t)ROPE_ROWS * nkv * hd * (is_bf16 ? 2 : 4);
+    const int value_blocks =
+        (write_kv && tokens >= ROPE_VALUE_BLOCKS_FROM && rows_lds <= 32 * 1024) ? (tokens + ROPE_ROWS - 1) / ROPE_ROWS : 0;
+    dim3 grid(tokens + value_blocks), block(256);
     if (is_bf16)
-      hipLaunchKernelGGL(rope_kv_write_vec_kernel<bf16_t>, dim3(tokens), dim3(256), 0, stream, (bf16_t*)qkv,
-                         (const int32_t*)positions, (const float*)cos_t, (const float*)sin_t,
+      hipLaunchKernelGGL(rope_kv_write_vec_kernel<bf16_t>, grid, block, value_blocks ? rows_lds : 0, stream,
+                         (bf16_t*)qkv, (const int32_t*)positions, (const float*)cos_t, (const float*)sin_t,
                          (const int64_t*)slot_mapping, (bf16_t*)k_pages, (bf16_t*)v_pages, nh, nkv, hd, rotary_dim,
-                         page_size, write_kv);
+                         page_size, write_kv, tokens, value_blocks);
     else
-      hipLaunchKernelGGL(rope_kv_write_vec_kernel<float>, dim3(tokens), dim3(256), 0, stream, (float*)qkv,
-                         (const int32_t*)positions, (const float*)cos_t, (const float*)sin_t,
+      hipLaunchKernelGGL(rope_kv_write_vec_kernel<float>, grid, block, value_blocks ? rows_lds : 0, stream,
+                         (float*)qkv, (const int32_t*)positions, (const float*)cos_t, (const float*)sin_t,
                          (const int64_t*)slot_mapping, (float*)k_pages, (float*)v_pages, nh, nkv, hd, rotary_dim,
-                         page_size, write_kv);
+                         page_size, write_kv, tokens, value_blocks);
     return GA_CHECK_LAUNCH();
   }
   dim3 grid(tokens, nh + 2 * nkv), block(64);

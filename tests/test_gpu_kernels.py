@@ -172,13 +172,17 @@ def test_rope_and_cache_write(dtype, tol, T, nh, nkv, hd, rd, theta):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("ps", [4, 8, 12, 16, 32])
-def test_cache_write_of_slots_in_a_row(dtype, ps):
+@pytest.mark.parametrize("long_run", [0, 530])
+def test_cache_write_of_slots_in_a_row(dtype, ps, long_run):
     """Prompt portions: tokens whose slots follow each other, starting anywhere in a page, across page ends, with
     tokens that write nothing and single tokens of other requests between them.  Every value lands in its slot of
-    the transposed page and nothing else changes."""
+    the transposed page and nothing else changes.  With the long run the step has tokens enough for the kernel to
+    write the values of 8 tokens at a time."""
     from ginfer_amd.kernels import ops
-    nh, nkv, hd, pages = 4, 2, 64, 100
+    nh, nkv, hd, pages = 4, 2, 64, 400
     runs = [(5, 35), (-1, 1), (100, 20), (311, 1), (-1, 2), (160, 9), (330 + ps - 1, 1), (200, 17), (250, 3)]
+    if long_run:
+        runs.insert(3, (701, long_run))
     slots = []
     for first, n in runs:
         slots += [-1] * n if first < 0 else list(range(first, first + n))
