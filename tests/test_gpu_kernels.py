@@ -676,10 +676,11 @@ def test_folded_norm_refuses_what_it_cannot_take():
 @pytest.mark.parametrize("M,pack", [(1, 1), (1, 2), (5, 2), (8, 1), (8, 2), (12, 1), (33, 1), (64, 1)])
 @pytest.mark.parametrize("nh,nkv,hd,K,theta", [(12, 2, 128, 1536, 1e4), (6, 1, 32, 192, 1e6), (4, 4, 64, 88, 1e4), (5, 1, 96, 72, 5e5),
                                                (28, 4, 128, 72, 1e4)])     # the last: so many columns that tiles stay full
-def test_qkv_rope_skinny(M, pack, nh, nkv, hd, K, theta):
+@pytest.mark.parametrize("ps", [8, 12])         # 12: the page of a slot by division, not by a shift
+def test_qkv_rope_skinny(M, pack, nh, nkv, hd, K, theta, ps):
     """The fused decode kernel equals projection, then rotation and cache write."""
     from ginfer_amd.kernels import ops
-    ps, pages = 8, 40
+    pages = 40
     width = (nh + 2 * nkv) * hd
     x, w, b = rnd((M, K), torch.bfloat16, 60), rnd((width, K), torch.bfloat16, 61, scale=0.2), rnd((width,), torch.bfloat16, 62)
     positions = torch.randint(0, 300, (M,), dtype=torch.int32, device=dev())
