@@ -4,7 +4,8 @@
 // attention once per head size, libattention_mfma_HEAD_DIM<n>.so).  All entry points are `extern "C"`, take raw
 // device pointers and the stream to launch on, check what can be checked on the host, and return 0 or a
 // negative number without launching anything.  Sizes are in elements unless bytes are named.  bfloat16 values
-// are raw 16-bit patterns.  Nothing here allocates device memory: scratch memory is the caller's.
+// are raw 16-bit patterns.  Nothing here allocates device memory: scratch memory is the caller's (or, for
+// ga_sample_rows_static, a static array of the library).
 //
 // The declarations repeat the definitions' parameter lists; tests/test_config.py compares the two.
 #pragma once
@@ -92,6 +93,20 @@ int ga_attn_prefill(void* out, int64_t out_stride, const void* q, int64_t q_stri
 int64_t ga_sample_scratch_floats(int rows, int vocab);
 int ga_sample_rows(void* out, const void* logits, int64_t row_stride, int rows, int vocab, const void* temperature,
                    const void* uniform, void* scratch, hipStream_t stream);
+
+// ---- sampling.hip, for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+// loops, harnesses that forbid allocation).  This entry point has no counterpart in the reference, whose argmax takes
+// its buffers from the caller's allocator.  ga_sample_rows_static is ga_sample_rows with its scratch in a static
+// device array of 196,608 bytes that each GPU holds until the process ends: at most
+// ga_sample_rows_static_max_rows() (256) rows a call, more are refused with -2 and nothing is launched
+// (ga_sample_rows_static_error(code) says what a negative code means).  It allocates nothing and calls nothing that
+// does.  Calls on one GPU share the array: calls that overlap there (other streams, other threads) race.
+// ga_sample_rows_static_init() looks the array up on the current device ahead of the first call (optional).
+int ga_sample_rows_static_max_rows();
+int ga_sample_rows_static_init();
+const char* ga_sample_rows_static_error(int code);
+int ga_sample_rows_static(void* out, const void* logits, int64_t row_stride, int rows, int vocab,
+                          const void* temperature, const void* uniform, hipStream_t stream);
 
 #ifdef __cplusplus
 }

@@ -9,6 +9,8 @@
 //     the cut into segments depends on the vocabulary alone, never on the rows beside it.
 // The reference samples greedily only (ginfer/engine/sampling_params.h:5-8).
 #include "common.cuh"
+#include <atomic>
+#include <mutex>
 
 #define SCAN_THREADS 256
 #define SCAN_WAVES (SCAN_THREADS / WAVE)
@@ -184,4 +186,77 @@ extern "C" int ga_sample_rows(void* out, const void* logits, int64_t row_stride,
                      seg_arg, seg_sum, (const float*)logits, row_stride, vocab, seg, segments,
                      (const float*)temperature, (const float*)uniform);
   return GA_CHECK_LAUNCH();
+}
+
+// ---- the same choice for callers that cannot allocate
+//
+// ga_sample_rows takes its scratch memory from the caller, who has to allocate it.  Code that runs under HIP
+// graph capture, a tight serving loop or a harness that forbids allocation cannot: for them the scratch lies in
+// a file-scope device array of a fixed, modest size, which every GPU that this library runs on holds until the
+// process ends (STATIC_SCRATCH_FLOATS * 4 = 196,608 bytes).  In host code the array's name stands for the symbol,
+// not for device memory: its address on a device is looked up once per device (hipGetSymbolAddress, with that
+// device current) and only that address is ever handed to a kernel.
+#define STATIC_MAX_ROWS 256
+#define STATIC_SCRATCH_FLOATS (3 * STATIC_MAX_ROWS * MAX_SEGMENTS)
+#define STATIC_MAX_DEVICES 64
+static __device__ __align__(256) float scratch[STATIC_SCRATCH_FLOATS];
+
+static std::mutex scratch_lock;
+static std::atomic<float*> scratch_on_device[STATIC_MAX_DEVICES];   // the array's address on each device, once known
+
+// The address of `scratch` on the current device, looked up at the first call on that device; null (and *rc set)
+// if the runtime refuses.
+static float* static_scratch(int* rc) {
+  int device = -1;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess) { *rc = (int)e; return nullptr; }
+  if (device < 0 || device >= STATIC_MAX_DEVICES) { *rc = -3; return nullptr; }
+  float* p = scratch_on_device[device].load(std::memory_order_acquire);
+  if (p) return p;
+  std::lock_guard<std::mutex> hold(scratch_lock);
+  p = scratch_on_device[device].load(std::memory_order_acquire);
+  if (p) return p;
+  void* address = nullptr;
+  e = hipGetSymbolAddress(&address, HIP_SYMBOL(scratch));
+  if (e != hipSuccess || !address) { *rc = e != hipSuccess ? (int)e : -4; return nullptr; }
+  p = (float*)address;
+  scratch_on_device[device].store(p, std::memory_order_release);
+  return p;
+}
+
+// Rows that ga_sample_rows_static takes in one call.
+extern "C" int ga_sample_rows_static_max_rows() { return STATIC_MAX_ROWS; }
+
+// Looks up the scratch array on the current device, so that the first ga_sample_rows_static there does nothing
+// but launch (a caller that is about to record a graph calls this before).  0, or the runtime's error code.
+extern "C" int ga_sample_rows_static_init() {
+  int rc = 0;
+  return static_scratch(&rc) ? 0 : rc;
+}
+
+// What a negative return value of ga_sample_rows_static means.
+extern "C" const char* ga_sample_rows_static_error(int code) {
+  switch (code) {
+    case 0: return "ok";
+    case -1: return "vocab must be positive";
+    case -2: return "more rows than ga_sample_rows_static_max_rows(): the static scratch array holds 256 rows";
+    case -3: return "the current device's number is beyond the devices this library keeps an address for (64)";
+    case -4: return "the scratch array has no address on the current device";
+    default: return code > 0 ? "an error code of the HIP runtime" : "unknown";
+  }
+}
+
+// ga_sample_rows without a scratch argument and without any allocation: the segments' results go through the
+// static array.  At most ga_sample_rows_static_max_rows() rows a call (more: -2, nothing launched).  Every call
+// on a GPU shares that GPU's array: calls that overlap there (two streams, two threads) race; calls in one stream
+// do not.  Nothing in the array has to start at zero: the first kernel writes every word the second one reads.
+extern "C" int ga_sample_rows_static(void* out, const void* logits, int64_t row_stride, int rows, int vocab,
+                                     const void* temperature, const void* uniform, hipStream_t stream) {
+  if (rows <= 0) return 0;
+  if (vocab <= 0) return -1;
+  if (rows > STATIC_MAX_ROWS) return -2;
+  int rc = 0;
+  float* ptr = static_scratch(&rc);
+  if (!ptr) return rc;
+  return ga_sample_rows(out, logits, row_stride, rows, vocab, temperature, uniform, ptr, stream);
 }

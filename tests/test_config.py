@@ -119,12 +119,12 @@ def test_header_declares_every_entry_point_as_it_is_defined():
     defined = {}
     for path in glob.glob(os.path.join(csrc, "*.hip")):
         src = open(path).read()
-        for m in re.finditer(r'extern "C"\s+([\w ]+?)\s*\b(ga_\w+)\s*\(([^)]*)\)\s*\{', src):
+        for m in re.finditer(r'extern "C"\s+([\w \*]+?)\s*\b(ga_\w+)\s*\(([^)]*)\)\s*\{', src):
             defined[m.group(2)] = (squeeze(m.group(1)), squeeze(m.group(3)))
     header = open(os.path.join(csrc, "ginfer_amd.h")).read()
     header = re.sub(r"//[^\n]*", "", header)
     declared = {}
-    for m in re.finditer(r'([\w ]+?)\s*\b(ga_\w+)\s*\(([^)]*)\)\s*;', header):
+    for m in re.finditer(r'([\w \*]+?)\s*\b(ga_\w+)\s*\(([^)]*)\)\s*;', header):
         declared[m.group(2)] = (squeeze(m.group(1)), squeeze(m.group(3)))
     assert defined and set(defined) == set(declared), (sorted(set(defined) ^ set(declared)))
     for name in defined:
