@@ -163,8 +163,9 @@ def feed_forward(n, w, prefix):
     return linear(swiglu(g, u), w[prefix + ".down_proj.weight"])
 
 
-def forward(cfg, w, ids, schedule=None):
-    """Logits [T, V] for one whole sequence at positions 0..T-1.
+def forward(cfg, w, ids, schedule=None, rows=None):
+    """Logits [T, V] for one whole sequence at positions 0..T-1 (with `rows`, a list of positions: the
+    logits [len(rows), V] at those alone; the final norm and the head act on every row by itself).
     Block order ginfer/core/layer/transformer/encoder.cc:33-39: n = norm1(x); h = x + attn(n);
     n = norm2(h); x = h + mlp(n).  Then the final norm and the output head (tied to the embedding
     or `lm_head.weight`), ginfer/model/model.cc:158-165, ginfer/model/qwen2.cc:41-46.
@@ -189,6 +190,8 @@ def forward(cfg, w, ids, schedule=None):
         h = x + a
         n = rms_norm(h, w[p + ".post_attention_layernorm.weight"], eps)
         x = h + feed_forward(n, w, p + ".mlp")
+    if rows is not None:
+        x = x[torch.as_tensor(rows, dtype=torch.long)]
     n = rms_norm(x, w["model.norm.weight"], eps)
     head = w["model.embed_tokens.weight"] if cfg["tie_word_embeddings"] else w["lm_head.weight"]
     return linear(n, head)
