@@ -115,7 +115,10 @@ class ModelRunner:
         device_tokens (int32 [len(entries)] on the device): every entry brings ONE token whose id the host does
         not know yet (the entry's own token is a placeholder): the ids are taken from this tensor on the device,
         in the order of the entries.  This lets a caller launch a decode step before it has read the tokens of
-        the step before."""
+        the step before.
+        Cache pages: a request that the step meets for the first time is admitted; tokens that the caller has not
+        reserved (`cache.append`) are reserved and committed here; tokens that the caller reserved stay for the caller to
+        commit once the step is launched."""
         if not entries:
             return torch.empty((0, self.vocab_size), dtype=torch.float32, device=self.device)
         cache = self.cache
@@ -137,27 +140,18 @@ class ModelRunner:
                 raise ValueError("device_tokens must be int32 [%d] on the device" % len(entries))
         reserved_here = []
         try:
-            for e in entries:
-                if not cache.has(e.request_id):
-                    cache.admit(e.request_id)
-                if cache.pending(e.request_id) == 0:
-                    if cache.length(e.request_id) + len(e.tokens) > self.max_model_len:
-                        raise ValueError("request %r would grow to %d tokens, beyond max_model_len %d"
-                                         % (e.request_id, cache.length(e.request_id) + len(e.tokens),
-                                            self.max_model_len))
-                    cache.append(e.request_id, len(e.tokens))
-                    reserved_here.append(e.request_id)
-                elif cache.pending(e.request_id) != len(e.tokens):
-                    raise ValueError("request %r has %d tokens reserved but brings %d"
-                                     % (e.request_id, cache.pending(e.request_id), len(e.tokens)))
+            reserve_for_step(cache, entries, self.max_model_len, reserved_here)
             host = self._host_arrays(entries)
             logits = self._run(host, borrow, device_tokens)
         except Exception:
             for rid in reserved_here:       # nothing is committed: the requests stay as long as they were
                 cache.requests[rid].pending = 0
             raise
-        for e in entries:
-            cache.commit(e.request_id)
+        # What this step reserved it also commits.  A caller that reserved the tokens itself (the scheduler) commits them
+        # too, with the request's tokens: the cache manager then remembers the pages that are full now, for requests
+        # that share the prefix (ginfer/engine/block_manager.cc:98-108 registers a block as soon as it is full).
+        for rid in reserved_here:
+            cache.commit(rid)
         return logits
 
     def release(self, request_id):
@@ -425,6 +419,25 @@ class ModelRunner:
         out = np.full((table.shape[0], width), -1, dtype=np.int32)
         out[:, :table.shape[1]] = table
         return out
+
+
+def reserve_for_step(cache, entries, max_model_len, reserved):
+    """Cache pages for a step's entries, as far as the caller has not reserved them: a request that the cache does not
+    know is admitted, and tokens that are not reserved yet are (all of an entry's or none).  The requests whose tokens
+    were reserved here are appended to `reserved` as they are, so that the caller can undo them if the step fails, and
+    commit them (only them) when it is launched."""
+    for e in entries:
+        if not cache.has(e.request_id):
+            cache.admit(e.request_id)
+        if cache.pending(e.request_id) == 0:
+            if cache.length(e.request_id) + len(e.tokens) > max_model_len:
+                raise ValueError("request %r would grow to %d tokens, beyond max_model_len %d"
+                                 % (e.request_id, cache.length(e.request_id) + len(e.tokens), max_model_len))
+            cache.append(e.request_id, len(e.tokens))
+            reserved.append(e.request_id)
+        elif cache.pending(e.request_id) != len(e.tokens):
+            raise ValueError("request %r has %d tokens reserved but brings %d"
+                             % (e.request_id, cache.pending(e.request_id), len(e.tokens)))
 
 
 def pad_step(host, t_pad, e_pad, width):

@@ -206,6 +206,48 @@ def test_requests_that_share_a_prefix_share_its_pages(folders, sharp_folders, dt
                                    num_kvcache_blocks=20)).runner.cache.prefix_caching
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_late_request_finds_the_pages_of_a_request_that_is_still_running(sharp_folders, dtype):
+    """Full pages are remembered when they are committed (ginfer/engine/block_manager.cc:98-108), so a request that
+    shares 48 tokens with one that is still decoding starts behind them: 48 tokens found at the moment it is admitted,
+    the same when the first request has finished before, none with sharing off, and the same tokens in all three."""
+    from ginfer_amd import Engine, EngineConfig, SamplingParams
+    folder = sharp_folders["B"]
+    vocab = H.TINY["B"][0]["vocab_size"]
+    first = H.random_tokens(50, vocab, 1300)
+    late = first[:48] + H.random_tokens(7, vocab, 1301)
+    tokens, found = {}, {}
+    for case, (share, first_outputs) in dict(running=(True, 40), finished=(True, 3), alone=(False, 40)).items():
+        eng = Engine(EngineConfig(model_path=folder, dtype=dtype, max_num_batched_tokens=64, max_num_seqs=4, max_seq_len=256,
+                                  kvcache_block_size=8, num_kvcache_blocks=60, enable_prefix_caching=share))
+        a = eng.add_request(first, SamplingParams(max_tokens=first_outputs, ignore_eos=True))
+        done = {}
+        for _ in range(8):
+            if eng.has_unfinished():
+                for o in eng.step():
+                    done[o.request_id] = o
+        assert (a in done) == (case == "finished")
+        before = eng.runner.cache.prefix_hit_tokens
+        b = eng.add_request(late, SamplingParams(max_tokens=6, ignore_eos=True))
+        while b not in done:
+            for o in eng.step():
+                done[o.request_id] = o
+            if case == "running" and "at_admission" not in found and eng.runner.cache.has(b):
+                # the first request is still running when the late one has got its pages
+                found["at_admission"] = (eng.runner.cache.prefix_hit_tokens - before, eng.runner.cache.has(a))
+        found[case] = eng.runner.cache.prefix_hit_tokens - before
+        while eng.has_unfinished():
+            for o in eng.step():
+                done[o.request_id] = o
+        eng.runner.cache.check()
+        tokens[case] = (done[a].token_ids[:3], done[b].token_ids)
+        _greedy_as_plain(folder, [late], [done[b]], dtype)
+        del eng
+    assert found == dict(at_admission=(48, True), running=48, finished=48, alone=0)
+    if dtype == "float32":
+        assert tokens["running"] == tokens["finished"] == tokens["alone"]
+
+
 def test_temperature_sampling_matches_plain_with_same_uniforms(folders):
     from ginfer_amd import Engine, EngineConfig, SamplingParams
     from ginfer_amd.sampling import uniform

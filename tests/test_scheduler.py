@@ -309,6 +309,65 @@ def test_a_request_starts_behind_the_prefix_that_the_cache_holds():
     assert all(g.pool.num_free == g.pool.num_pages for g in cache.groups)
 
 
+def run_as_the_engine(sched, cache, seqs, arrivals=None, on_admit=None, max_steps=10000):
+    """The engine's own order of calls around a step, without the device: schedule (which reserves), the runner's
+    bookkeeping for the step's entries (which finds everything reserved and so commits nothing), advance (which commits
+    with the requests' tokens), then the tokens are absorbed.  arrivals: {step number: sequence added before that step}."""
+    from ginfer_amd.engine.runner import reserve_for_step, StepEntry
+    for s in seqs:
+        sched.add(s)
+    done, steps = [], 0
+    while not sched.is_finished() or (arrivals and any(k >= steps for k in arrivals)):
+        if arrivals and steps in arrivals:
+            sched.add(arrivals[steps])
+        hits_before = cache.prefix_hit_tokens
+        batch = sched.schedule()
+        if on_admit:
+            on_admit(steps, batch, cache.prefix_hit_tokens - hits_before)
+        entries = [StepEntry(b.seq.request_id, b.seq.token_ids[b.seq.num_computed:b.seq.num_computed + b.num_tokens], [])
+                   for b in batch]
+        reserved = []
+        reserve_for_step(cache, entries, sched.max_model_len, reserved)
+        assert reserved == []                    # the scheduler had reserved every token
+        for rid in reserved:
+            cache.commit(rid)
+        sched.advance(batch)
+        cache.check()
+        done += sched.absorb(batch, [fake_token(b.seq.token_ids) for b in batch if b.samples], now=float(steps))
+        cache.check()
+        steps += 1
+        assert steps < max_steps
+    return done
+
+
+@pytest.mark.parametrize("finished_first", [False, True])
+def test_a_request_finds_the_pages_of_a_request_that_is_still_running(finished_first):
+    """Pages are remembered as soon as they are full and committed (ginfer/engine/block_manager.cc:98-108), not when
+    their request ends: a request that arrives while the first one still decodes starts behind the 48 tokens that
+    the two have in common."""
+    sched, cache = make(num_pages=64, page_size=8, budget=64, prefix_caching=True)
+    a = seq(0, 50, max_tokens=3 if finished_first else 30)
+    b = Sequence(1, a.token_ids[:48] + [901, 902, 903], 51, SamplingParams(max_tokens=4))
+    seen = {}
+
+    def on_admit(step, batch, hits):
+        for sc in batch:
+            if sc.seq is b and b.request_id not in seen:
+                seen[b.request_id] = (hits, sc.seq.num_computed, sc.num_tokens, a.state)
+    done = run_as_the_engine(sched, cache, [a], arrivals={6: b}, on_admit=on_admit)
+    hits, behind, ran, state_of_a = seen[1]
+    assert (hits, behind, ran) == (48, 48, 3)
+    assert state_of_a is (State.FINISHED if finished_first else State.RUNNING)
+    assert {s.request_id: s.token_ids for s in done} == {0: expected(a), 1: expected(b)}
+    # without sharing nothing is found
+    sched, cache = make(num_pages=64, page_size=8, budget=64, prefix_caching=False)
+    a = seq(0, 50, max_tokens=30)
+    b = Sequence(1, a.token_ids[:48] + [901, 902, 903], 51, SamplingParams(max_tokens=4))
+    seen.clear()
+    run_as_the_engine(sched, cache, [a], arrivals={6: b}, on_admit=on_admit)
+    assert seen[1][:3] == (0, 0, 51)
+
+
 def test_an_evicted_request_finds_its_own_pages_again():
     sched, cache = make(num_pages=8, page_size=4, max_num_seqs=2, budget=32, prefix_caching=True)
     a, b = seq(0, 9, max_tokens=12), seq(1, 9, max_tokens=12)
