@@ -99,8 +99,9 @@ class CacheGroup:
 class CacheManager:
     def __init__(self, cache_specs, page_size, num_pages, max_requests, prefix_caching=False):
         """cache_specs: per schedule entry KVCacheSpec | StateSpec | None (None: keeps nothing, or reads
-        another entry's cache).  num_pages: pages of every group's pool.  prefix_caching: requests admitted with
-        their tokens share the pages of a known prefix."""
+        another entry's cache).  num_pages: pages of every group's pool, or a list with one count per group (in the
+        order of `group_specs(cache_specs)`; a group with a window needs few, see `plan_pages`).  prefix_caching:
+        requests admitted with their tokens share the pages of a known prefix."""
         if prefix_caching and not self.supports_prefix_caching(cache_specs):
             raise ValueError("prefixes cannot be shared in a model with a window or with per-request state")
         self.prefix_caching = bool(prefix_caching)
@@ -109,18 +110,24 @@ class CacheManager:
             raise ValueError("page_size must be positive")
         self.page_size, self.max_requests = int(page_size), int(max_requests)
         self.cache_specs = list(cache_specs)
-        by_key: Dict[KVCacheSpec, List[int]] = {}
-        for i, s in enumerate(self.cache_specs):
-            if isinstance(s, KVCacheSpec):
-                by_key.setdefault(s, []).append(i)
-        self.groups = [CacheGroup(k, v, num_pages, self.page_size) for k, v in by_key.items()]
+        by_key = self.group_specs(self.cache_specs)
+        if isinstance(num_pages, (list, tuple)):
+            if len(num_pages) != len(by_key):
+                raise ValueError("%d page counts for %d cache groups" % (len(num_pages), len(by_key)))
+            counts = [int(n) for n in num_pages]
+        else:
+            counts = [int(num_pages)] * len(by_key)
+        self.groups = [CacheGroup(k, v, n, self.page_size) for (k, v), n in zip(by_key.items(), counts)]
         self.group_of = {}               # schedule entry -> (group index, index inside the group)
         for gi, g in enumerate(self.groups):
             for j, e in enumerate(g.entries):
                 self.group_of[e] = (gi, j)
         self.state_entries = [i for i, s in enumerate(self.cache_specs) if isinstance(s, StateSpec)]
         self.slots = SlotPool(self.max_requests)
-        self.state_tensors = {}          # schedule entry -> device tensor [max_requests, *shape]
+        # one more slot than requests: the rows that pad a recorded step read and write the state of this slot, which
+        # no request ever holds
+        self.pad_slot = self.max_requests
+        self.state_tensors = {}          # schedule entry -> device tensor [max_requests + 1, *shape]
         self.requests: Dict[object, _Request] = {}
         # host mirrors for building a step without a Python loop per request: per group the block tables
         # by state slot (int32, -1 where there is no page), and the lengths by state slot
@@ -129,15 +136,62 @@ class CacheManager:
         self._any_window = any(g.window is not None for g in self.groups)
 
     @staticmethod
+    def group_specs(cache_specs):
+        """{KVCacheSpec: [schedule entries]} in the order in which the groups are made."""
+        by_key: Dict[KVCacheSpec, List[int]] = {}
+        for i, s in enumerate(cache_specs):
+            if isinstance(s, KVCacheSpec):
+                by_key.setdefault(s, []).append(i)
+        return by_key
+
+    @staticmethod
+    def window_pages(window, page_size, max_requests, max_step_tokens, max_model_len):
+        """Pages that a group with this window can hold at most.  Between steps a request holds the pages of positions
+        [length - window + 1, length), at most (window - 1) // page + 2 of them (`commit` gives the others back); while it
+        runs n tokens of a step it holds those of [length - window + 1, length + n), at most ceil(n / page) + 1 more; over
+        the requests of a step the n add up to the step's token budget.  Never more than all keys of every request."""
+        per_request_all = -(-max_model_len // page_size)
+        per_request = min((window - 1) // page_size + 3, per_request_all)
+        return min(max_requests * per_request + -(-max_step_tokens // page_size), max_requests * per_request_all)
+
+    @classmethod
+    def plan_pages(cls, cache_specs, page_size, element_size, pool_bytes, max_requests, max_step_tokens, max_model_len):
+        """Page counts per group for a pool of pool_bytes: a group with a window gets what it can ever hold
+        (`window_pages`), the groups that keep all keys share the rest alike (every one of them holds the same number
+        of pages per token).  Raises if the bytes do not give every group a page."""
+        groups = cls.group_specs(cache_specs)
+        if not groups:
+            return []
+        page_bytes = [len(entries) * 2 * spec.num_kv_heads * page_size * spec.head_dim * element_size
+                      for spec, entries in groups.items()]
+        counts, left = [None] * len(groups), int(pool_bytes)
+        for gi, spec in enumerate(groups):
+            if spec.window is not None:
+                counts[gi] = cls.window_pages(spec.window, page_size, max_requests, max_step_tokens, max_model_len)
+                left -= counts[gi] * page_bytes[gi]
+        rest = [gi for gi, c in enumerate(counts) if c is None]
+        if rest:
+            per = left // sum(page_bytes[gi] for gi in rest) if left > 0 else 0
+            for gi in rest:
+                counts[gi] = per
+        elif left < 0:       # windows only and too little memory: shrink them alike
+            total = sum(c * b for c, b in zip(counts, page_bytes))
+            counts = [c * int(pool_bytes) // total for c in counts]
+        if min(counts) < 1:
+            raise RuntimeError("no memory left for the cache: %d bytes give the groups %s pages (a page of each takes %s bytes)"
+                               % (pool_bytes, counts, page_bytes))
+        return counts
+
+    @staticmethod
     def supports_prefix_caching(cache_specs):
         return (any(isinstance(s, KVCacheSpec) for s in cache_specs)
                 and not any(isinstance(s, StateSpec) or (isinstance(s, KVCacheSpec) and s.window is not None)
                             for s in cache_specs))
 
     # ---- device memory
-    def bytes_per_page(self, element_size):
-        return sum(len(g.entries) * 2 * g.spec.num_kv_heads * self.page_size * g.spec.head_dim * element_size
-                   for g in self.groups)
+    def pool_bytes(self, element_size):
+        return sum(g.pool.num_pages * len(g.entries) * 2 * g.spec.num_kv_heads * self.page_size * g.spec.head_dim
+                   * element_size for g in self.groups)
 
     def allocate_device(self, dtype, device):
         import torch
@@ -146,7 +200,7 @@ class CacheManager:
                                     g.spec.num_kv_heads * self.page_size * g.spec.head_dim), dtype=dtype, device=device)
         for e in self.state_entries:
             s = self.cache_specs[e]
-            self.state_tensors[e] = torch.zeros((self.max_requests,) + tuple(s.shape), dtype=s.dtype, device=device)
+            self.state_tensors[e] = torch.zeros((self.max_requests + 1,) + tuple(s.shape), dtype=s.dtype, device=device)
 
     def kv_views(self, entry):
         """(k_pages [pages, nkv, page_size, hd], v_pages [pages, nkv, hd, page_size]) of a schedule entry."""
@@ -343,6 +397,22 @@ class CacheManager:
         self._length_np[req.slot] = req.length
         if self.prefix_caching and token_ids is not None:
             self._remember(req, token_ids)
+        if self._any_window:
+            # what lies behind the window of the next token goes back now: whoever takes such a page writes it in a
+            # later step, behind this step's reads in stream order.  Between steps a request then holds the pages of
+            # one window only, which is what `window_pages` counts on.
+            for gi, g in enumerate(self.groups):
+                if g.window is None:
+                    continue
+                table = req.tables[gi]
+                first = min(g.first_needed_block(req.length), len(table))
+                give = [i for i in range(req.gone[gi], first) if table[i] >= 0]
+                if give:
+                    g.pool.give_back([table[i] for i in give])
+                    for i in give:
+                        table[i] = -1
+                    self._mirror_table(gi, req, give)
+                req.gone[gi] = max(req.gone[gi], first)
 
     def release(self, rid, token_ids=None):
         """The request ends (or is evicted): every page and its slot go back, the pages of its end first, so

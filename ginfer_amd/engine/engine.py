@@ -22,7 +22,9 @@ class EngineConfig:
     max_seq_len: int = 4096               # longest sequence (prompt + output) a request may reach
     gpu_memory_utilization: float = 0.9   # share of the free device memory that becomes cache pages
     kvcache_block_size: int = 16          # tokens per cache page
-    num_kvcache_blocks: Optional[int] = None   # pages per cache group; None: from free memory
+    # pages per cache group; None: from the memory that is free with the weights loaded, times gpu_memory_utilization;
+    # groups of layers with a window then get only what a window can hold, the others share the rest
+    num_kvcache_blocks: Optional[int] = None
     pipeline_decode: bool = True          # launch a decode step before the tokens of the step before it are read
     # requests share the cache pages of a common prefix (ginfer/engine/block_manager.cc:63-110, where it cannot be
     # switched off).  None: wherever the model allows it (no window, no per-request state); True: or refuse
@@ -57,6 +59,7 @@ class Engine:
         self.runner = ModelRunner(config.model_path, dtype=config.dtype, page_size=config.kvcache_block_size,
                                   num_pages=config.num_kvcache_blocks, max_requests=config.max_num_seqs,
                                   max_model_len=config.max_seq_len,
+                                  max_num_batched_tokens=config.max_num_batched_tokens,
                                   gpu_memory_utilization=config.gpu_memory_utilization,
                                   prefix_caching=config.enable_prefix_caching,
                                   graph_mixed_steps=config.graph_mixed_steps,

@@ -44,10 +44,12 @@ def require_gpu():
 class ModelRunner:
     def __init__(self, model_path, dtype="bfloat16", page_size=16, num_pages=None, max_requests=64,
                  max_model_len=None, gpu_memory_utilization=0.9, device=None, config=None, use_graphs=True,
-                 prefix_caching=False, random_seed=None, graph_mixed_steps=True):
+                 prefix_caching=False, random_seed=None, graph_mixed_steps=True, max_num_batched_tokens=None):
         """model_path: a folder with config.json and the weights.  With model_path None, `config` (a typed
         configuration) and `random_seed` make a model whose weights are drawn on the device, for shapes too
-        large to pass through a file."""
+        large to pass through a file.  num_pages: pages of every cache group (or a list, one count per group);
+        None: from the memory that is free once the weights are loaded and the largest step (max_num_batched_tokens
+        tokens, max_requests requests) has run, times gpu_memory_utilization."""
         self.device = device or require_gpu()
         if dtype not in DTYPES:
             raise ValueError("dtype must be one of %s, got %r" % (sorted(DTYPES), dtype))
@@ -67,19 +69,13 @@ class ModelRunner:
         else:
             load_weights(self.model, model_path, self.device)
         self.page_size = int(page_size)
+        self.max_requests = int(max_requests)
+        self.max_step_tokens = int(min(max_num_batched_tokens or 2048, self.max_model_len))
         specs = self.model.cache_specs()
-        if num_pages is None:
-            num_pages = self._pages_from_free_memory(specs, gpu_memory_utilization)
         if prefix_caching is None:       # where the model allows it
             prefix_caching = CacheManager.supports_prefix_caching(specs)
-        self.cache = CacheManager(specs, self.page_size, int(num_pages), int(max_requests), prefix_caching=prefix_caching)
-        self.cache.allocate_device(self.dtype, self.device)
-        self._owner_of = [i if e.cache_of is None else e.cache_of for i, e in enumerate(self.model.schedule)]
-        self._buffers = _BufferCache(len(self.cache.groups), self.device)
-        self.use_graphs = bool(use_graphs) and self.model.capturable()
-        self._graphs, self._graph_seen = {}, {}
         self.graph_mixed_steps = bool(graph_mixed_steps)
-        self._padded_buffers = {}
+        self._graphs, self._graph_seen, self._padded_buffers = {}, {}, {}
         self._graph_budget, self._graph_bytes, self._graph_bytes_seen = None, 0, {}
         # Padding pays while the host's launches (~5 ms a step) outlast the device's work on the padded rows, which may
         # be twice the step's own: with some 1e15 operations a second that is rows * weights < ~1.5e12 (512 rows for a
@@ -89,19 +85,61 @@ class ModelRunner:
         # how steps ran: launched kernel by kernel, replayed as a recorded decode step, replayed as a recorded step
         # with prompt portions; and how many steps were recorded
         self.counts = dict(launched=0, replayed_decode=0, replayed_padded=0, recorded=0, recording_seconds=0.0)
+        self.use_graphs = False          # nothing is recorded while the pool is being planned
+        self.memory_plan = None
+        if num_pages is None:
+            num_pages = self._plan_pool(specs, float(gpu_memory_utilization))
+            self.counts["launched"] = 0
+        self._install_cache(specs, num_pages, prefix_caching)
+        self.use_graphs = bool(use_graphs) and self.model.capturable()
 
-    def _pages_from_free_memory(self, specs, utilization):
-        """Pages = free device memory (after the weights are resident) * utilization / bytes per page, the
-        reference's sizing (ginfer/engine/model_runner.cc:52-70)."""
-        probe = CacheManager(specs, self.page_size, 0, 1)
-        per_page = probe.bytes_per_page(torch.empty(0, dtype=self.dtype).element_size())
-        if per_page == 0:
+    def _install_cache(self, specs, num_pages, prefix_caching):
+        self.cache = CacheManager(specs, self.page_size, num_pages, self.max_requests, prefix_caching=prefix_caching)
+        self.cache.allocate_device(self.dtype, self.device)
+        self._owner_of = [i if e.cache_of is None else e.cache_of for i, e in enumerate(self.model.schedule)]
+        self._buffers = _BufferCache(len(self.cache.groups), self.device)
+
+    def _plan_pool(self, specs, utilization):
+        """Page counts per cache group from the device's memory, in the reference's order (ginfer/model/model.cc:48-120
+        makes the scratch memory first, ginfer/engine/model_runner.cc:52-70 then sizes the pool from what is free):
+        the largest step runs once over a small pool of its own, which tells what activations, logits and the library's
+        workspace take at their peak; the pool is free memory x utilization, and a utilization that leaves less than
+        that peak beside the pool is refused.  Groups with a window get what they can ever hold, the groups that keep
+        all keys share the rest (`CacheManager.plan_pages`)."""
+        if not 0.0 < utilization <= 1.0:
+            raise ValueError("gpu_memory_utilization must lie in (0, 1], got %r" % (utilization,))
+        esize = torch.empty(0, dtype=self.dtype).element_size()
+        if not CacheManager.group_specs(specs):
             return 0
-        free, _ = torch.cuda.mem_get_info(self.device)
-        pages = int(free * utilization) // per_page
-        if pages < 1:
-            raise RuntimeError("no memory left for the cache: %d bytes free, a page takes %d" % (free, per_page))
-        return pages
+        T, R, ps = self.max_step_tokens, self.max_requests, self.page_size
+        # the largest step over a pool that just holds it: one portion of T tokens, then one token of R requests
+        probe_pages = -(-T // ps) + R + 1
+        self._install_cache(specs, probe_pages, False)
+        torch.cuda.synchronize(self.device)
+        resident = torch.cuda.memory_allocated(self.device)
+        torch.cuda.reset_peak_memory_stats(self.device)
+        try:
+            self.step([StepEntry(("probe", 0), [0] * T, [T - 1])])
+            self.release(("probe", 0))
+            self.step([StepEntry(("probe", r), [0], [0]) for r in range(R)])
+            for r in range(R):
+                self.release(("probe", r))
+            torch.cuda.synchronize(self.device)
+        finally:
+            peak = torch.cuda.max_memory_allocated(self.device) - resident
+            del self.cache, self._buffers
+            torch.cuda.empty_cache()
+        free, total = torch.cuda.mem_get_info(self.device)
+        pool = int(free * utilization)
+        need = int(peak * 1.1) + (64 << 20)          # the step's own peak, a tenth more, and the allocator's rounding
+        if free - pool < need:
+            raise ValueError("gpu_memory_utilization %.3f leaves %d MB beside the cache, but a step of %d tokens and %d "
+                             "requests takes up to %d MB: at most %.3f fits (%d MB are free with the weights loaded)"
+                             % (utilization, (free - pool) >> 20, T, R, need >> 20, max(0.0, (free - need) / free),
+                                free >> 20))
+        counts = CacheManager.plan_pages(specs, ps, esize, pool, R, T, self.max_model_len)
+        self.memory_plan = dict(free_bytes=int(free), pool_bytes=pool, step_peak_bytes=int(peak), pages=list(counts))
+        return counts
 
     @property
     def vocab_size(self):
@@ -364,7 +402,7 @@ class ModelRunner:
         return ctx
 
     def _pad(self, host, t_pad, e_pad, width):
-        return pad_step(host, t_pad, e_pad, width)
+        return pad_step(host, t_pad, e_pad, width, self.cache.pad_slot)
 
     def _capture_padded(self, key, host):
         _, t_pad, e_pad, bucket = key
@@ -373,13 +411,7 @@ class ModelRunner:
                            n_tiles=self._padded_tiles(t_pad, e_pad))
         ctx = self._padded_context(host, buf, t_pad, e_pad, width, bucket)
         extra = dict(ctx.extra)
-        side = torch.cuda.Stream()
-        side.wait_stream(torch.cuda.current_stream())
-        with torch.cuda.stream(side):
-            self.model.forward(ctx)          # outside the graph first: libraries load, the allocator settles
-        torch.cuda.current_stream().wait_stream(side)
-        torch.cuda.synchronize()
-        self.counts["recorded"] += 1
+        self._run_once_unrecorded(ctx)
         graph = torch.cuda.CUDAGraph()
         ctx.extra = extra
         with torch.cuda.graph(graph):
@@ -397,13 +429,7 @@ class ModelRunner:
         buf = _StepBuffers(E, E, E, width, E, len(self.cache.groups), self.device)
         padded = dict(host, width=width, tables=[self._widen(t, width) for t in host["tables"]])
         ctx = self._context(padded, buf)
-        side = torch.cuda.Stream()
-        side.wait_stream(torch.cuda.current_stream())
-        with torch.cuda.stream(side):
-            self.model.forward(ctx)          # warm-up outside the graph: libraries load, allocator settles
-        torch.cuda.current_stream().wait_stream(side)
-        torch.cuda.synchronize()
-        self.counts["recorded"] += 1
+        self._run_once_unrecorded(ctx)
         graph = torch.cuda.CUDAGraph()
         ctx.extra = {"decode_info": buf.dev["decode_info"], "decode_span": bucket}
         with torch.cuda.graph(graph):
@@ -411,6 +437,22 @@ class ModelRunner:
         g = dict(graph=graph, buf=_GraphBuffers(buf, width, self._widen), logits=logits, ctx=ctx)
         self._graphs[key] = g
         return g
+
+    def _run_once_unrecorded(self, ctx):
+        """Before a step is recorded it runs once outside the graph, on a stream of its own: libraries load what they
+        need, the allocator settles.  The step itself is the replay that follows, so this run must leave nothing
+        behind: keys and values it writes are written again by the replay, the same ones into the same places, and
+        per-request state, which a second run would advance twice, is put back as it was."""
+        saved = {e: t.clone() for e, t in self.cache.state_tensors.items()}
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            self.model.forward(ctx)
+        torch.cuda.current_stream().wait_stream(side)
+        for e, t in saved.items():
+            self.cache.state_tensors[e].copy_(t)
+        torch.cuda.synchronize()
+        self.counts["recorded"] += 1
 
     @staticmethod
     def _widen(table, width):
@@ -440,9 +482,10 @@ def reserve_for_step(cache, entries, max_model_len, reserved):
                              % (e.request_id, cache.pending(e.request_id), len(e.tokens)))
 
 
-def pad_step(host, t_pad, e_pad, width):
+def pad_step(host, t_pad, e_pad, width, pad_slot):
     """The host arrays of a step laid into t_pad token rows and e_pad + 1 entries: the step's own come first, the
-    rest is padding (see ModelRunner._run_padded).  Tables are `width` wide."""
+    rest is padding (see ModelRunner._run_padded).  Tables are `width` wide.  pad_slot: the state slot of the entries
+    that are padding, one that no request holds (a mixer with state of its own reads and writes it for them)."""
     from ..kernels import ops
     T, E = host["T"], host["E"]
     dummy, entries = e_pad, e_pad + 1
@@ -474,7 +517,7 @@ def pad_step(host, t_pad, e_pad, width):
                 ent=grown(host["ent"], t_pad, dummy), cu=cu, q_start=grown(host["q_start"], entries, 0), q_len=q_len,
                 rows=grown(host["rows"], e_pad, 0), width=width, tables=tables,
                 slot_maps=[grown(sm, t_pad, -1) for sm in host["slot_maps"]],
-                state_slots=grown(host["state_slots"], entries, 0), decode_info=info, tiles=tile_arr)
+                state_slots=grown(host["state_slots"], entries, pad_slot), decode_info=info, tiles=tile_arr)
 
 
 def _context_bucket(max_kv):

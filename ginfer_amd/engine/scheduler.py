@@ -55,12 +55,17 @@ class Scheduler:
         if seq.num_prompt_tokens + 1 > self.max_model_len:
             raise ValueError("request %r: prompt of %d tokens leaves no room under max_model_len %d"
                              % (seq.request_id, seq.num_prompt_tokens, self.max_model_len))
-        need = -(-min(total, self.max_model_len) // self.cache.page_size)
+        ps = self.cache.page_size
+        grown = min(total, self.max_model_len)
         for gi, g in enumerate(self.cache.groups):
-            if g.window is None and need > g.pool.num_pages:
-                raise ValueError("request %r can grow to %d tokens (%d pages) but the cache has %d pages; "
-                                 "it could never finish" % (seq.request_id, min(total, self.max_model_len), need,
-                                                            g.pool.num_pages))
+            need = -(-grown // ps)
+            if g.window is not None:         # token by token a window holds the pages of `window` positions, one more at most
+                need = min(need, -(-g.window // ps) + 1)
+            if need > g.pool.num_pages:
+                raise ValueError("request %r can grow to %d tokens (%d pages%s) but cache group %d has %d pages; "
+                                 "it could never finish" % (seq.request_id, grown, need,
+                                                            "" if g.window is None else " of a window of %d" % g.window,
+                                                            gi, g.pool.num_pages))
         seq.state = State.WAITING
         self.waiting.append(seq)
 

@@ -58,7 +58,7 @@ def test_groups_by_need():
     m = CacheManager([FULL, WIN, None, FULL, StateSpec((8,), torch.float32), WIN], page_size=8, num_pages=10, max_requests=3)
     assert [(g.spec, g.entries) for g in m.groups] == [(FULL, [0, 3]), (WIN, [1, 5])]
     assert m.group_of == {0: (0, 0), 3: (0, 1), 1: (1, 0), 5: (1, 1)} and m.state_entries == [4]
-    assert m.bytes_per_page(2) == 4 * 2 * 2 * 8 * 16 * 2
+    assert m.pool_bytes(2) == 10 * 4 * 2 * 2 * 8 * 16 * 2
 
 
 def test_append_commit_release_and_reuse():
@@ -95,9 +95,11 @@ def test_window_gives_pages_back():
     m = CacheManager([FULL, WIN], page_size=8, num_pages=8, max_requests=1)
     m.admit("a")
     m.append("a", 30)
+    assert m.table("a", 1) == [0, 1, 2, 3]                  # while the step runs, its first query needs block 0
     m.commit("a")
-    assert m.table("a", 1) == [0, 1, 2, 3]
-    # the next token sits at 30 and sees positions 11..30: block 0 (positions 0..7) is behind the window
+    # the next token sits at 30 and sees positions 11..30: block 0 (positions 0..7) is behind the window and goes back
+    # as soon as the 30 tokens are committed
+    assert m.table("a", 1) == [-1, 1, 2, 3] and m.groups[1].pool.num_free == 8 - 3
     m.append("a", 1)
     m.commit("a")
     assert m.table("a", 1) == [-1, 1, 2, 3] and m.table("a", 0) == [0, 1, 2, 3]
@@ -300,3 +302,54 @@ def test_random_orders_with_shared_prefixes(seed):
     m.check()
     assert all(g.pool.num_free == g.pool.num_pages for g in m.groups) and m.slots.num_free == 4
     assert hits > 0 and hits == m.prefix_hit_tokens
+
+
+# ---- how a pool is shared out among groups
+
+def test_a_group_with_a_window_gets_what_a_window_can_hold_and_the_rest_goes_to_all_keys():
+    specs = [FULL, WIN, FULL, WIN, None]
+    ps, esize, requests, step, longest = 16, 2, 8, 256, 4096
+    page_full = 2 * 2 * FULL.num_kv_heads * ps * FULL.head_dim * esize       # two entries, keys and values
+    page_win = 2 * 2 * WIN.num_kv_heads * ps * WIN.head_dim * esize
+    pool = 64 << 20
+    counts = CacheManager.plan_pages(specs, ps, esize, pool, requests, step, longest)
+    w = CacheManager.window_pages(WIN.window, ps, requests, step, longest)
+    assert w == requests * ((WIN.window - 1) // ps + 3) + step // ps
+    assert counts == [(pool - w * page_win) // page_full, w]
+    assert counts[0] * page_full > 0.9 * pool                 # nearly all of the pool keeps all keys
+    m = CacheManager(specs, ps, counts, requests)
+    assert [g.pool.num_pages for g in m.groups] == counts and m.pool_bytes(esize) <= pool
+    # a window as long as the longest request is worth no more than all keys
+    assert CacheManager.window_pages(10 ** 6, ps, requests, step, longest) == requests * (longest // ps)
+    # windows only: each gets what it can hold; too little memory: refused
+    assert CacheManager.plan_pages([WIN, WIN], ps, esize, pool, requests, step, longest) == [w]
+    with pytest.raises(RuntimeError, match="no memory left"):
+        CacheManager.plan_pages(specs, ps, esize, w * page_win + page_full - 1, requests, step, longest)
+    with pytest.raises(ValueError, match="page counts"):
+        CacheManager(specs, ps, [4], requests)
+
+
+def test_every_step_fits_the_pages_planned_for_a_window():
+    """Whatever portions the requests of a step run, a group with a window never holds more pages than were planned."""
+    import random
+    ps, requests, step, longest = 8, 4, 40, 400
+    win = KVCacheSpec(1, 16, 20)
+    pages = CacheManager.window_pages(win.window, ps, requests, step, longest)
+    m = CacheManager([win], ps, pages, requests)
+    rng = random.Random(3)
+    for r in range(requests):
+        m.admit(r)
+    for _ in range(300):
+        budget = step
+        for r in rng.sample(range(requests), requests):
+            n = min(rng.choice([1, 1, 2, 7, 19, 40]), budget, longest - m.length(r))
+            if n > 0:
+                m.append(r, n)            # never raises OutOfPages
+                budget -= n
+        for r in range(requests):
+            if m.pending(r):
+                m.commit(r)
+            if m.length(r) >= longest:
+                m.release(r)
+                m.admit(r)
+        m.check()

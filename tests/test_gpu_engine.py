@@ -826,3 +826,42 @@ def test_recorded_steps_with_prompt_portions(folders, sharp_folders, name, dtype
     for (rid, p), row in got[True].items():
         err = float(np.abs(row.astype(np.float64) - refs[rid][p]).max() / np.abs(refs[rid]).max())
         assert np.isfinite(row).all() and err <= H.TOL[dtype], "%s %s: request %s position %d: error %.3g" % (name, dtype, rid, p, err)
+
+
+def test_the_pool_is_planned_from_free_memory_after_the_largest_step(folders, monkeypatch):
+    """The pool is sized from what is free once the weights are loaded and the largest step has run (the order of
+    ginfer/engine/model_runner.cc:52-70); layers with a window get the pages a window can hold and nearly all of the
+    pool keeps all keys; a utilization that leaves the largest step no room is refused."""
+    from ginfer_amd import ModelRunner, Engine, EngineConfig, SamplingParams
+    from ginfer_amd.cache import CacheManager
+    real = torch.cuda.mem_get_info
+    monkeypatch.setattr(torch.cuda, "mem_get_info", lambda *a, **k: (64 << 20, real(*a, **k)[1]))     # as if 64 MB were free
+    # the largest step's own needs come to more than the 10 % of 64 MB: refused, and the message says what would fit
+    with pytest.raises(ValueError, match="gpu_memory_utilization 0.999 leaves"):
+        ModelRunner(folders["C"], dtype="bfloat16", page_size=16, max_requests=4, max_model_len=384,
+                    max_num_batched_tokens=128, gpu_memory_utilization=0.999)
+    monkeypatch.setattr(torch.cuda, "mem_get_info", lambda *a, **k: (1 << 30, real(*a, **k)[1]))      # as if 1 GB were free
+    r = ModelRunner(folders["C"], dtype="bfloat16", page_size=16, max_requests=4, max_model_len=384,
+                    max_num_batched_tokens=128, gpu_memory_utilization=0.5)
+    plan = r.memory_plan
+    assert plan["free_bytes"] == 1 << 30 and plan["pool_bytes"] == 1 << 29 and plan["step_peak_bytes"] > 0
+    groups = r.cache.groups
+    assert [g.pool.num_pages for g in groups] == plan["pages"]
+    all_keys = [g for g in groups if g.window is None]
+    windowed = [g for g in groups if g.window is not None]
+    assert len(all_keys) == 1 and len(windowed) == 1           # layer 0 keeps all keys, layers 1 to 3 a window of 40
+    assert windowed[0].pool.num_pages == CacheManager.window_pages(40, 16, 4, 128, 384) == 4 * (39 // 16 + 3) + 8
+    per_page = lambda g: len(g.entries) * 2 * g.spec.num_kv_heads * 16 * g.spec.head_dim * 2
+    assert all_keys[0].pool.num_pages * per_page(all_keys[0]) > 0.9 * plan["pool_bytes"]
+    assert r.cache.pool_bytes(2) <= plan["pool_bytes"]
+    del r
+    monkeypatch.undo()
+    torch.cuda.empty_cache()
+    # through the engine, with pages from free memory: requests longer than the window, tokens as the plain model's
+    eng = Engine(EngineConfig(model_path=folders["C"], dtype="float32", max_num_batched_tokens=48, max_num_seqs=3,
+                              max_seq_len=200, gpu_memory_utilization=0.05))
+    prompts = [H.random_tokens(n, 777, 40 + n) for n in (90, 7, 130)]
+    outs = eng.generate(prompts, SamplingParams(max_tokens=12, ignore_eos=True))
+    _greedy_as_plain(folders["C"], prompts, outs, "float32")
+    eng.runner.cache.check()
+    assert all(g.pool.num_free == g.pool.num_pages for g in eng.runner.cache.groups)

@@ -309,6 +309,115 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped(tmp_path):
             assert err < 1e-4, "request %s position %d: %.3g" % (rid, p, err)
 
 
+def _register_recordable_toy():
+    """The toy running mean again, written so that its forward may be recorded into a HIP graph: it reads everything
+    that changes from step to step from the step's device arrays (entries' first rows, their requests' lengths, the state
+    slots) and launches the same operations whatever the batch is.  Entries that are padding read and write whatever
+    state slot they are given."""
+    from ginfer_amd.config import register_architecture, PartSpec, LayerSpec, ScheduleEntry, ModelSpec
+    from ginfer_amd.parts import register_mixer, Part, StateSpec
+    from ginfer_amd.weights import WeightSpec
+
+    @register_mixer("toy_running_mean_recordable")
+    class RecordableRunningMean(Part):
+        capturable = True
+
+        def __init__(self, hidden_size, dtype, device):
+            self.H, self.dtype, self.device = hidden_size, dtype, device
+
+        def cache_spec(self):
+            return StateSpec((self.H + 1,), torch.float32)
+
+        def weight_specs(self):
+            return {"mix.weight": WeightSpec((self.H, self.H))}
+
+        def bind_weights(self, t):
+            self.w = t["mix.weight"]
+
+        def forward(self, x, step, cache):
+            T, H = x.shape[0], self.H
+            ent = step.token_entry.long()
+            cu = step.cu_tokens.long()
+            fresh = (step.q_start == 0)[:, None]
+            before = torch.where(fresh, torch.zeros_like(cache.state[cache.slots]), cache.state[cache.slots])   # [entries, H + 1]
+            sums0 = torch.cat([torch.zeros((1, H), dtype=torch.float32, device=x.device), torch.cumsum(x.float(), dim=0)])
+            rows = torch.arange(T, device=x.device)
+            sums = before[ent, :H] + sums0[rows + 1] - sums0[cu[ent]]
+            counts = before[ent, H] + (rows - cu[ent] + 1).float()
+            last = torch.clamp(cu[1:] - 1, min=0)            # an entry without tokens (padding) names some row: its slot is the padding's
+            after = torch.cat([sums[last], counts[last][:, None]], dim=1)
+            cache.state.index_copy_(0, cache.slots, after)
+            return ((sums / counts[:, None]).to(self.dtype) @ self.w.t())
+
+    @register_architecture("ToyRecordableStateLM")
+    @dataclass
+    class ToyRecordableConfig:
+        hidden_size: int = 48
+        vocab_size: int = 211
+        architecture = "ToyRecordableStateLM"
+
+        @classmethod
+        def from_dict(cls, d):
+            return cls(d["hidden_size"], d["vocab_size"])
+
+        def to_dict(self):
+            return dict(architectures=["ToyRecordableStateLM"], hidden_size=self.hidden_size, vocab_size=self.vocab_size)
+
+        def model_spec(self):
+            Hd = self.hidden_size
+            norm = PartSpec("rmsnorm", dict(size=Hd, eps=1e-5))
+            pos = PartSpec("rope_neox", dict(theta=1e4, rotary_dim=16, max_positions=256))
+            attn = PartSpec("attention", dict(hidden_size=Hd, num_heads=3, num_kv_heads=1, head_dim=16, qkv_bias=True,
+                                              out_bias=False, window=None, position=pos, scale=None))
+            toy = PartSpec("toy_running_mean_recordable", dict(hidden_size=Hd))
+            ffn = PartSpec("swiglu", dict(hidden_size=Hd, intermediate_size=80))
+            layers = [LayerSpec("model.layers.%d" % i, m, ffn, norm, norm) for i, m in enumerate([attn, toy, attn])]
+            schedule = [ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(2, cache_of=0), ScheduleEntry(1)]
+            return ModelSpec(hidden_size=Hd, vocab_size=self.vocab_size, layers=layers, schedule=schedule,
+                             embedding=PartSpec("embedding", dict(vocab_size=self.vocab_size, hidden_size=Hd)),
+                             final_norm=norm, head=PartSpec("lm_head", dict(vocab_size=self.vocab_size, hidden_size=Hd,
+                                                                            tied=True)),
+                             max_positions=256, eos_token_ids=[0])
+    return ToyRecordableConfig
+
+
+def test_state_of_a_live_request_survives_the_padding_of_recorded_steps(tmp_path):
+    """A mixer with state of its own whose forward may be recorded: steps with prompt portions are laid into recorded
+    steps of padded sizes, whose padding entries read and write a state slot of their own, never the slot of a live
+    request (the first request here holds slot 0 all along).  Same weights and plain statement as the toy above."""
+    from ginfer_amd import ModelRunner, write_random_model
+    Toy = _register_recordable_toy()
+    folder = write_random_model(str(tmp_path / "toy"), Toy(), seed=4, dtype="float32")
+    reqs = {"a": H.random_tokens(60, 211, 1), "b": H.random_tokens(23, 211, 2), "c": H.random_tokens(37, 211, 3),
+            "d": H.random_tokens(18, 211, 4)}
+    runner = ModelRunner(folder, dtype="float32", page_size=8, num_pages=24, max_requests=3)
+    assert runner.use_graphs and runner.cache.pad_slot == 3
+    assert all(t.shape[0] == 4 for t in runner.cache.state_tensors.values())
+    refs = {rid: _toy_plain(folder, ids) for rid, ids in reqs.items()}
+    # "a" trickles along two tokens a step (slot 0) while the others come and go in portions: every step is padded
+    steps, at = [], {"a": 0}
+    others = [("b", (9, 14)), ("c", (20, 17)), ("d", (5, 13))]
+    for rid, cuts in others:
+        o = 0
+        for n in cuts:
+            a0 = at["a"]
+            # few wanted places: a recorded step returns at most as many rows as it has entries
+            steps.append(dict(entries=[dict(id="a", tokens=reqs["a"][a0:a0 + 2], want=[1]),
+                                       dict(id=rid, tokens=reqs[rid][o:o + n], want=[0, n - 1])],
+                              end=[rid] if o + n == len(reqs[rid]) else []))
+            at["a"] += 2
+            o += n
+    for rounds in range(3):          # shapes seen a second time are recorded, a third time replayed
+        got = H.run_steps(runner, steps)
+        runner.release("a")
+        runner.cache.check()
+        for (rid, p), row in got.items():
+            ref = refs[rid]
+            err = np.abs(row - ref[p]).max() / np.abs(ref).max()
+            assert err < 1e-4, "round %d: request %s position %d: %.3g" % (rounds, rid, p, err)
+    assert runner.counts["replayed_padded"] > 0, runner.counts
+
+
 def _register_routed_toy():
     """A second toy architecture defined here, in the test: a feed-forward that routes every token to one of
     three experts (router logits in 32-bit), in one layer only, beside the package's dense one in the other; and

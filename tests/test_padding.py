@@ -34,7 +34,7 @@ def test_a_step_laid_into_padded_sizes(q_len, q_start):
     host = host_arrays(q_len, q_start)
     T, E = host["T"], host["E"]
     t_pad, e_pad, width = 64, 8, 16
-    p = pad_step(host, t_pad, e_pad, width)
+    p = pad_step(host, t_pad, e_pad, width, pad_slot=99)
     dummy = e_pad
     # sizes
     assert p["T"] == t_pad and p["E"] == e_pad + 1 and p["width"] == width

@@ -443,3 +443,19 @@ def test_abort_gives_everything_back_wherever_the_request_stands():
     sched2.abort(5)
     assert sched2.absorb(batch, [123]) == [] and b.num_output_tokens == 0 and sched2.is_finished()
     cache2.check()
+
+
+def test_a_window_smaller_than_its_pool_needs_is_refused_when_the_request_is_added():
+    # a window of 40 with pages of 16 holds up to 4 pages token by token: 3 pages could never do
+    sched, cache = make(num_pages=3, page_size=16, window=40, max_model_len=512)
+    with pytest.raises(ValueError, match="window of 40"):
+        sched.add(seq(0, 100, max_tokens=50))
+    sched, cache = make(num_pages=4, page_size=16, window=40, max_model_len=512)
+    a = seq(0, 100, max_tokens=50)
+    done, _ = run(sched, cache, [a])
+    assert done[0].token_ids == expected(a)
+    # a short request needs no more than its own length
+    sched, cache = make(num_pages=2, page_size=16, window=40, max_model_len=512)
+    b = seq(1, 20, max_tokens=10)
+    done, _ = run(sched, cache, [b])
+    assert done[0].token_ids == expected(b)
