@@ -12,7 +12,7 @@ from dataclasses import dataclass, field, asdict
 from typing import List, Optional
 
 from .registry import register_architecture, ConfigError
-from .spec import PartSpec, LayerSpec, ScheduleEntry, ModelSpec
+from .spec import PartSpec, prenorm_layer, ScheduleEntry, ModelSpec
 
 _REQUIRED = ("num_hidden_layers", "vocab_size", "max_position_embeddings", "num_attention_heads",
              "num_key_value_heads", "hidden_size", "intermediate_size")
@@ -137,9 +137,8 @@ class Qwen2Config:
                 scale=None))
             ffn = PartSpec("swiglu", dict(hidden_size=self.hidden_size,
                                           intermediate_size=self.intermediate_size))
-            layers.append(LayerSpec(prefix="model.layers.%d" % i, mixer=mixer, feed_forward=ffn,
-                                    mixer_norm=norm, feed_forward_norm=norm,
-                                    arrangement="prenorm"))
+            layers.append(prenorm_layer("model.layers.%d" % i, mixer=mixer, feed_forward=ffn,
+                                        mixer_norm=norm, feed_forward_norm=norm))
         spec = ModelSpec(
             hidden_size=self.hidden_size, vocab_size=self.vocab_size, layers=layers,
             schedule=[ScheduleEntry(i) for i in range(self.num_hidden_layers)],

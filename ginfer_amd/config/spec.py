@@ -1,8 +1,8 @@
 """What a model is made of, as data.
 
 An architecture's typed configuration turns into a `ModelSpec`: one `LayerSpec` per layer, each
-naming its mixer, feed-forward and norm by registry kind with every size and constant as a
-parameter, and a `schedule` that lists the order in which layers run.  The builder in
+naming its parts (mixer, feed-forward, norms, whatever roles its arrangement has) by registry kind with
+every size and constant as a parameter, and a `schedule` that lists the order in which layers run.  The builder in
 `ginfer_amd.parts.model` reads nothing but this; no part ever sees the architecture's name.
 """
 from dataclasses import dataclass, field
@@ -31,17 +31,29 @@ def _freeze(v):
 
 @dataclass
 class LayerSpec:
-    """One block: how mixer, feed-forward and norms are arranged, and the prefix of its tensors."""
+    """One block: its parts by role, how they are arranged around the residual stream, and the prefix of its tensors.
+    Which roles a block has is the arrangement's matter (`roles` of the registered arrangement class: role -> family of
+    parts, e.g. {"mixer": "mixer", "feed_forward": "feed_forward", "mixer_norm": "norm", ...}); a layer names exactly
+    those.  `names` gives each role the prefix of its tensors inside the layer, as the checkpoint spells it (a role
+    that is not listed is spelt as the role itself)."""
     prefix: str
-    mixer: PartSpec
-    feed_forward: PartSpec
-    mixer_norm: PartSpec
-    feed_forward_norm: PartSpec
+    parts: Dict[str, PartSpec]
     arrangement: str = "prenorm"
-    # tensor-name prefix of each part inside the layer, as the checkpoint spells it
-    names: Dict[str, str] = field(default_factory=lambda: dict(
-        mixer="self_attn", feed_forward="mlp", mixer_norm="input_layernorm",
-        feed_forward_norm="post_attention_layernorm"))
+    names: Dict[str, str] = field(default_factory=dict)
+
+    def name_of(self, role):
+        return self.names.get(role, role)
+
+
+def prenorm_layer(prefix, mixer, feed_forward, mixer_norm, feed_forward_norm, names=None):
+    """The usual block of four parts (norm, mixer, norm, feed-forward) with the tensor names that checkpoints of this
+    family of models use."""
+    spelt = dict(mixer="self_attn", feed_forward="mlp", mixer_norm="input_layernorm",
+                 feed_forward_norm="post_attention_layernorm")
+    spelt.update(names or {})
+    return LayerSpec(prefix=prefix, parts=dict(mixer=mixer, feed_forward=feed_forward, mixer_norm=mixer_norm,
+                                               feed_forward_norm=feed_forward_norm),
+                     arrangement="prenorm", names=spelt)
 
 
 @dataclass

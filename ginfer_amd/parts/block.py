@@ -3,8 +3,35 @@ from ..kernels import ops
 from .registry import register_arrangement
 
 
+class Arrangement:
+    """How a layer's parts sit around the residual stream.  A kind of arrangement says which roles it has and of which
+    family each is (`roles`: role -> "mixer" | "feed_forward" | "norm"); the model builds the parts that a layer names
+    for exactly these roles and hands them over as a dictionary.  Every part becomes an attribute under its role's
+    name.  forward(residual float32 [T, H], delta, step, cache) takes the output of the block before as a pending
+    `delta` (it is added to the residual by the first norm that runs) and returns its own last output as the next one.
+    cache_spec(): what one run of the block keeps per request; the mixer's, unless the kind says otherwise."""
+
+    roles = {}
+
+    def __init__(self, parts):
+        self._parts = dict(parts)
+        for role, part in self._parts.items():
+            setattr(self, role, part)
+
+    def parts(self):
+        """(role, part) pairs; the roles are what `LayerSpec.names` gives tensor prefixes for."""
+        return list(self._parts.items())
+
+    def cache_spec(self):
+        mixer = self._parts.get("mixer")
+        return mixer.cache_spec() if mixer is not None else None
+
+    def forward(self, residual, delta, step, cache):
+        raise NotImplementedError
+
+
 @register_arrangement("prenorm")
-class PreNormBlock:
+class PreNormBlock(Arrangement):
     """n = norm1(x); h = x + mixer(n); n = norm2(h); x = h + feed_forward(n)
     (ginfer/core/layer/transformer/encoder.cc:33-39).  The residual stream is kept in 32-bit and every add
     is fused into the norm that follows it, so a block takes the previous block's output as a pending
@@ -15,16 +42,13 @@ class PreNormBlock:
     given the first norm of the block that runs next (`into_norm`), if that block says `takes_folded_input()`;
     it then returns ops.ScaledRows in place of its delta, and the next block skips its first norm."""
 
-    def __init__(self, mixer, feed_forward, mixer_norm, feed_forward_norm):
-        self.mixer, self.feed_forward = mixer, feed_forward
-        self.mixer_norm, self.feed_forward_norm = mixer_norm, feed_forward_norm
+    roles = {"mixer": "mixer", "feed_forward": "feed_forward", "mixer_norm": "norm", "feed_forward_norm": "norm"}
+
+    def __init__(self, parts):
+        super().__init__(parts)
+        mixer, feed_forward, feed_forward_norm = self.mixer, self.feed_forward, self.feed_forward_norm
         self.folds = (getattr(mixer, "folds_norm", False) and getattr(feed_forward, "takes_scaled_rows", False)
                       and getattr(feed_forward_norm, "foldable", False))
-
-    def parts(self):
-        """(role, part): the roles are the keys of `LayerSpec.names`, which gives each its tensor prefix."""
-        return [("mixer", self.mixer), ("feed_forward", self.feed_forward), ("mixer_norm", self.mixer_norm),
-                ("feed_forward_norm", self.feed_forward_norm)]
 
     @property
     def folds_output(self):
@@ -53,9 +77,10 @@ class PreNormBlock:
         return self.feed_forward.forward(a)
 
 
-def whole(delta, norm):
+def whole(delta, norm=None):
     """A mixer or feed-forward may hand on float32 partial sums [parts, T, H] of a K-split product.  A norm
-    that says `accepts_partial_sums` adds them up itself; for any other they are added up here."""
+    that says `accepts_partial_sums` adds them up itself; for any other (or for none) they are added up here."""
     if delta is not None and delta.dim() == 3 and not getattr(norm, "accepts_partial_sums", False):
-        return delta.sum(dim=0).to(norm.dtype)
+        total = delta.sum(dim=0)
+        return total.to(norm.dtype) if norm is not None else total
     return delta

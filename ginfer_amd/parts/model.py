@@ -68,12 +68,13 @@ class DecoderModel:
         self.final_norm = registry.lookup("norm", spec.final_norm.kind)(**spec.final_norm.params, **kw)
         self.head = registry.lookup("head", spec.head.kind)(**spec.head.params, **kw)
         self.blocks = []
-        for ls in spec.layers:
-            mixer = self._build("mixer", ls.mixer)
-            ffn = self._build("feed_forward", ls.feed_forward)
-            n1 = self._build("norm", ls.mixer_norm)
-            n2 = self._build("norm", ls.feed_forward_norm)
-            self.blocks.append(registry.lookup("arrangement", ls.arrangement)(mixer, ffn, n1, n2))
+        for i, ls in enumerate(spec.layers):
+            arrangement = registry.lookup("arrangement", ls.arrangement)
+            roles = arrangement.roles        # role -> family of parts
+            if set(ls.parts) != set(roles):
+                raise ValueError("layer %d: arrangement %r has the roles %s, the layer names %s"
+                                 % (i, ls.arrangement, sorted(roles), sorted(ls.parts)))
+            self.blocks.append(arrangement({role: self._build(roles[role], ls.parts[role]) for role in roles}))
         self.schedule = list(spec.schedule)
         # per run of the schedule: the first norm of the block that runs next, where this run's block can fold it
         # into its own last product and that block takes its input so (a matter of speed only)
@@ -102,7 +103,7 @@ class DecoderModel:
                (names["head"], self.head)]
         for ls, block in zip(self.spec.layers, self.blocks):
             for role, part in block.parts():
-                out.append((ls.prefix + "." + ls.names[role], part))
+                out.append((ls.prefix + "." + ls.name_of(role), part))
         return out
 
     def weight_specs(self):
@@ -145,7 +146,7 @@ class DecoderModel:
         another entry's cache."""
         out = []
         for e in self.schedule:
-            out.append(None if e.cache_of is not None else self.blocks[e.layer].mixer.cache_spec())
+            out.append(None if e.cache_of is not None else self.blocks[e.layer].cache_spec())
         return out
 
     # ---- forward

@@ -57,15 +57,15 @@ def test_no_size_stands_in_code():
         assert len(spec.layers) == d["num_hidden_layers"] == len(spec.schedule)
         hd = d.get("head_dim") or d["hidden_size"] // d["num_attention_heads"]
         for i, layer in enumerate(spec.layers):
-            m, f = layer.mixer.params, layer.feed_forward.params
+            m, f = layer.parts["mixer"].params, layer.parts["feed_forward"].params
             assert (m["num_heads"], m["num_kv_heads"], m["head_dim"]) == (d["num_attention_heads"], d["num_key_value_heads"], hd)
             assert m["position"].params["theta"] == d["rope_theta"] and m["position"].params["rotary_dim"] == hd
-            assert f["intermediate_size"] == d["intermediate_size"] and layer.mixer_norm.params["eps"] == d["rms_norm_eps"]
+            assert f["intermediate_size"] == d["intermediate_size"] and layer.parts["mixer_norm"].params["eps"] == d["rms_norm_eps"]
             assert m["qkv_bias"] is True and m["out_bias"] is False     # ginfer/model/qwen2.cc:15-17
         assert spec.head.params["tied"] == d["tie_word_embeddings"] and spec.vocab_size == d["vocab_size"]
     c = config_from_dict(H.TINY_C)
-    assert [l.mixer.params["window"] for l in c.model_spec().layers] == [None, 40, 40, 40]
-    assert [l.mixer.params["window"] for l in config_from_dict(H.TINY_A).model_spec().layers] == [None, None]
+    assert [l.parts["mixer"].params["window"] for l in c.model_spec().layers] == [None, 40, 40, 40]
+    assert [l.parts["mixer"].params["window"] for l in config_from_dict(H.TINY_A).model_spec().layers] == [None, None]
     assert config_from_dict(H.TINY_B).eos_token_ids == [998, 999]
 
 

@@ -158,7 +158,8 @@ def test_block_folds_the_norm_between_mixer_and_feed_forward(T):
         part.bind_weights({n: ((1 + rnd(sp.shape, 10 * k + i, 0.1)) if n == "weight" and part in norms
                                else rnd(sp.shape, 10 * k + i, 0.15)).to(dtype).to(dev())
                            for i, (n, sp) in enumerate(part.weight_specs().items())})
-    block = lookup("arrangement", "prenorm")(mixer, ff, norms[0], norms[1])
+    block = lookup("arrangement", "prenorm")(dict(mixer=mixer, feed_forward=ff, mixer_norm=norms[0],
+                                                  feed_forward_norm=norms[1]))
     assert block.folds
     seen = []
     inner = mixer.forward
@@ -196,7 +197,7 @@ def _register_toy():
     """A toy architecture defined here, in the test: blocks whose mixer keeps a running sum of its
     inputs per request (state of fixed size, no pages) between blocks with attention, a layer that runs
     twice and a run that reads another run's keys and values."""
-    from ginfer_amd.config import register_architecture, PartSpec, LayerSpec, ScheduleEntry, ModelSpec
+    from ginfer_amd.config import register_architecture, PartSpec, LayerSpec, prenorm_layer, ScheduleEntry, ModelSpec
     from ginfer_amd.parts import register_mixer, Part, StateSpec
     from ginfer_amd.weights import WeightSpec
 
@@ -255,7 +256,7 @@ def _register_toy():
                                               out_bias=False, window=None, position=pos, scale=None))
             toy = PartSpec("toy_running_mean", dict(hidden_size=Hd))
             ffn = PartSpec("swiglu", dict(hidden_size=Hd, intermediate_size=80))
-            layers = [LayerSpec("model.layers.%d" % i, m, ffn, norm, norm) for i, m in enumerate([attn, toy, attn])]
+            layers = [prenorm_layer("model.layers.%d" % i, m, ffn, norm, norm) for i, m in enumerate([attn, toy, attn])]
             # layer 0, the toy layer, layer 2 reading run 0's cache, the toy layer again (a second state)
             schedule = [ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(2, cache_of=0), ScheduleEntry(1)]
             return ModelSpec(hidden_size=Hd, vocab_size=self.vocab_size, layers=layers, schedule=schedule,
@@ -314,7 +315,7 @@ def _register_recordable_toy():
     that changes from step to step from the step's device arrays (entries' first rows, their requests' lengths, the state
     slots) and launches the same operations whatever the batch is.  Entries that are padding read and write whatever
     state slot they are given."""
-    from ginfer_amd.config import register_architecture, PartSpec, LayerSpec, ScheduleEntry, ModelSpec
+    from ginfer_amd.config import register_architecture, PartSpec, LayerSpec, prenorm_layer, ScheduleEntry, ModelSpec
     from ginfer_amd.parts import register_mixer, Part, StateSpec
     from ginfer_amd.weights import WeightSpec
 
@@ -371,7 +372,7 @@ def _register_recordable_toy():
                                               out_bias=False, window=None, position=pos, scale=None))
             toy = PartSpec("toy_running_mean_recordable", dict(hidden_size=Hd))
             ffn = PartSpec("swiglu", dict(hidden_size=Hd, intermediate_size=80))
-            layers = [LayerSpec("model.layers.%d" % i, m, ffn, norm, norm) for i, m in enumerate([attn, toy, attn])]
+            layers = [prenorm_layer("model.layers.%d" % i, m, ffn, norm, norm) for i, m in enumerate([attn, toy, attn])]
             schedule = [ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(2, cache_of=0), ScheduleEntry(1)]
             return ModelSpec(hidden_size=Hd, vocab_size=self.vocab_size, layers=layers, schedule=schedule,
                              embedding=PartSpec("embedding", dict(vocab_size=self.vocab_size, hidden_size=Hd)),
@@ -418,12 +419,142 @@ def test_state_of_a_live_request_survives_the_padding_of_recorded_steps(tmp_path
     assert runner.counts["replayed_padded"] > 0, runner.counts
 
 
+def _register_toy_arrangements():
+    """Two arrangements of a block that the package does not have, registered here: one with two more norms (on the
+    mixer's and on the feed-forward's output, before each is added to the residual stream), and one with a single norm
+    whose rows go to mixer and feed-forward side by side.  A toy architecture uses one of each kind and a usual block
+    between them; tensor names are the roles' own where the layer gives none."""
+    from ginfer_amd.config import register_architecture, PartSpec, LayerSpec, prenorm_layer, ScheduleEntry, ModelSpec
+    from ginfer_amd.parts import register_arrangement
+    from ginfer_amd.parts.block import Arrangement, whole
+
+    @register_arrangement("toy_sandwich")
+    class Sandwich(Arrangement):
+        """h = x + post_mixer_norm(mixer(mixer_norm(x))); x = h + post_feed_forward_norm(feed_forward(feed_forward_norm(h)))"""
+        roles = {"mixer": "mixer", "feed_forward": "feed_forward", "mixer_norm": "norm", "post_mixer_norm": "norm",
+                 "feed_forward_norm": "norm", "post_feed_forward_norm": "norm"}
+
+        def forward(self, residual, delta, step, cache):
+            n = self.mixer_norm.forward(residual, whole(delta, self.mixer_norm))
+            a = whole(self.mixer.forward(n, step, cache))
+            a = self.post_mixer_norm.forward(a.float().contiguous())          # a norm over a branch: nothing is added
+            n = self.feed_forward_norm.forward(residual, a)
+            f = whole(self.feed_forward.forward(n))
+            return self.post_feed_forward_norm.forward(f.float().contiguous())
+
+    @register_arrangement("toy_parallel")
+    class Parallel(Arrangement):
+        """n = norm(x); x = x + mixer(n) + feed_forward(n)"""
+        roles = {"mixer": "mixer", "feed_forward": "feed_forward", "norm": "norm"}
+
+        def forward(self, residual, delta, step, cache):
+            n = self.norm.forward(residual, whole(delta, self.norm))
+            a = whole(self.mixer.forward(n, step, cache))
+            f = whole(self.feed_forward.forward(n))
+            return (a.float() + f.float()).to(n.dtype)
+
+    @register_architecture("ToyArrangedLM")
+    @dataclass
+    class ToyArrangedConfig:
+        hidden_size: int = 56
+        vocab_size: int = 157
+        architecture = "ToyArrangedLM"
+
+        @classmethod
+        def from_dict(cls, d):
+            return cls(d["hidden_size"], d["vocab_size"])
+
+        def to_dict(self):
+            return dict(architectures=["ToyArrangedLM"], hidden_size=self.hidden_size, vocab_size=self.vocab_size)
+
+        def model_spec(self):
+            Hd = self.hidden_size
+            norm = PartSpec("rmsnorm", dict(size=Hd, eps=1e-5))
+            pos = PartSpec("rope_neox", dict(theta=1e4, rotary_dim=16, max_positions=128))
+            attn = PartSpec("attention", dict(hidden_size=Hd, num_heads=4, num_kv_heads=2, head_dim=16, qkv_bias=True,
+                                              out_bias=False, window=None, position=pos, scale=None))
+            ffn = PartSpec("swiglu", dict(hidden_size=Hd, intermediate_size=72))
+            layers = [
+                LayerSpec("model.layers.0", dict(mixer=attn, feed_forward=ffn, mixer_norm=norm, post_mixer_norm=norm,
+                                                 feed_forward_norm=norm, post_feed_forward_norm=norm),
+                          arrangement="toy_sandwich", names=dict(mixer="self_attn", feed_forward="mlp")),
+                prenorm_layer("model.layers.1", attn, ffn, norm, norm),
+                LayerSpec("model.layers.2", dict(mixer=attn, feed_forward=ffn, norm=norm), arrangement="toy_parallel",
+                          names=dict(mixer="self_attn", feed_forward="mlp", norm="shared_layernorm")),
+            ]
+            return ModelSpec(hidden_size=Hd, vocab_size=self.vocab_size, layers=layers,
+                             schedule=[ScheduleEntry(i) for i in range(3)],
+                             embedding=PartSpec("embedding", dict(vocab_size=self.vocab_size, hidden_size=Hd)),
+                             final_norm=norm, head=PartSpec("lm_head", dict(vocab_size=self.vocab_size, hidden_size=Hd,
+                                                                            tied=False)),
+                             max_positions=128, eos_token_ids=[0])
+    return ToyArrangedConfig
+
+
+def _toy_arranged_plain(folder, ids):
+    w = pm.read_weights(folder)
+    T = len(ids)
+    cfg = dict(num_attention_heads=4, num_key_value_heads=2, head_dim=16)
+    sin, cos = pm.rope_tables(1e4, 16, T)
+    pos = list(range(T))
+    x = pm.embedding(w["model.embed_tokens.weight"], ids)
+    norm = lambda v, name: pm.rms_norm(v, w[name + ".weight"], 1e-5)
+    p = "model.layers.0"
+    a, _ = pm.attention_block(norm(x, p + ".mixer_norm"), w, p + ".self_attn", cfg, pos, sin, cos, None)
+    h = x + norm(a, p + ".post_mixer_norm")
+    x = h + norm(pm.feed_forward(norm(h, p + ".feed_forward_norm"), w, p + ".mlp"), p + ".post_feed_forward_norm")
+    p = "model.layers.1"
+    a, _ = pm.attention_block(norm(x, p + ".input_layernorm"), w, p + ".self_attn", cfg, pos, sin, cos, None)
+    h = x + a
+    x = h + pm.feed_forward(norm(h, p + ".post_attention_layernorm"), w, p + ".mlp")
+    p = "model.layers.2"
+    n = norm(x, p + ".shared_layernorm")
+    a, _ = pm.attention_block(n, w, p + ".self_attn", cfg, pos, sin, cos, None)
+    x = x + a + pm.feed_forward(n, w, p + ".mlp")
+    return pm.linear(norm(x, "model.norm"), w["lm_head.weight"]).float().numpy()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_arrangements_with_other_roles_are_registered_built_and_stepped(tmp_path, dtype):
+    """A layer is a dictionary of parts by role, and which roles there are is the arrangement's matter: blocks with six
+    parts and with three, defined here, are built from the configuration, loaded by their own tensor names and stepped
+    whole, in portions and mixed (recorded steps included) against their plain statement."""
+    from ginfer_amd import ModelRunner, write_random_model, config_from_folder
+    from ginfer_amd.config import LayerSpec, PartSpec
+    from ginfer_amd.parts import build_model
+    Toy = _register_toy_arrangements()
+    folder = write_random_model(str(tmp_path / "arranged"), Toy(), seed=12, dtype="float32", std_scale=4.0)
+    assert type(config_from_folder(folder)).__name__ == "ToyArrangedConfig"
+    runner = ModelRunner(folder, dtype=dtype, page_size=8, num_pages=24, max_requests=3)
+    names = set(runner.model.weight_specs())
+    assert {"model.layers.0.post_mixer_norm.weight", "model.layers.0.post_feed_forward_norm.weight",
+            "model.layers.2.shared_layernorm.weight", "model.layers.1.input_layernorm.weight"} <= names
+    assert "model.layers.2.feed_forward_norm.weight" not in names
+    assert [type(b).__name__ for b in runner.model.blocks] == ["Sandwich", "PreNormBlock", "Parallel"]
+    reqs = {"a": H.random_tokens(45, 157, 21), "b": H.random_tokens(18, 157, 22), "c": H.random_tokens(31, 157, 23)}
+    refs = {rid: _toy_arranged_plain(folder, ids) for rid, ids in reqs.items()}
+    for steps in (H.steps_whole(reqs), H.steps_last_decoded(reqs, last=12), H.steps_portions(reqs, sizes=(7, 2, 13)),
+                  H.steps_mixed(reqs, max_live=3, seed=2), H.steps_mixed(reqs, max_live=3, seed=2)):
+        got = H.run_steps(runner, steps)
+        runner.cache.check()
+        for (rid, p), row in got.items():
+            ref = refs[rid]
+            err = np.abs(row - ref[p]).max() / np.abs(ref).max()
+            assert err <= (1e-4 if dtype == "float32" else H.TOL[dtype]), "request %s position %d: %.3g" % (rid, p, err)
+    # a layer that names other roles than its arrangement has is refused with both lists
+    spec = Toy().model_spec()
+    spec.layers[2] = LayerSpec("model.layers.2", dict(spec.layers[2].parts, extra_norm=PartSpec("rmsnorm", dict(size=56, eps=1e-5))),
+                               arrangement="toy_parallel")
+    with pytest.raises(ValueError, match="extra_norm"):
+        build_model(spec, torch.float32, dev())
+
+
 def _register_routed_toy():
     """A second toy architecture defined here, in the test: a feed-forward that routes every token to one of
     three experts (router logits in 32-bit), in one layer only, beside the package's dense one in the other; and
     a position encoding of its own (rotation by a fraction of the position), used by one layer's attention while
     the other keeps the package's.  None of it touches the package's files."""
-    from ginfer_amd.config import register_architecture, PartSpec, LayerSpec, ScheduleEntry, ModelSpec
+    from ginfer_amd.config import register_architecture, PartSpec, LayerSpec, prenorm_layer, ScheduleEntry, ModelSpec
     from ginfer_amd.parts import register_feed_forward, register_position, Part
     from ginfer_amd.weights import WeightSpec
 
@@ -498,8 +629,8 @@ def _register_routed_toy():
                                                   out_bias=False, window=None, position=pos, scale=None))
             dense = PartSpec("swiglu", dict(hidden_size=Hd, intermediate_size=56))
             routed = PartSpec("toy_one_of_n", dict(hidden_size=Hd, intermediate_size=24, num_experts=3))
-            layers = [LayerSpec("model.layers.0", attn(slow), routed, norm, norm),
-                      LayerSpec("model.layers.1", attn(rope), dense, norm, norm)]
+            layers = [prenorm_layer("model.layers.0", attn(slow), routed, norm, norm),
+                      prenorm_layer("model.layers.1", attn(rope), dense, norm, norm)]
             return ModelSpec(hidden_size=Hd, vocab_size=self.vocab_size, layers=layers,
                              schedule=[ScheduleEntry(0), ScheduleEntry(1)],
                              embedding=PartSpec("embedding", dict(vocab_size=self.vocab_size, hidden_size=Hd)),
