@@ -2,6 +2,7 @@
 // g = gu[t, i], u = gu[t, I + i].  32-bit arithmetic, one rounding.
 // Formula: ginfer/core/op/kernels/cuda/swiglu_kernel.cu:24-27 (which skips a tail of numel % 8).
 #include "common.cuh"
+#include "ginfer_amd.h"   // the entry points below are checked against their declarations
 
 template <typename T>
 __global__ void silu_mul_kernel(T* __restrict__ out, const T* __restrict__ gu, int64_t tokens,

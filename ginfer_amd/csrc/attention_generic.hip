@@ -14,6 +14,7 @@
 // cut into steps, whatever else is in the batch and wherever its pages lie.  Head h reads kv head
 // h / (nh / nkv) (:439-450).  Keys are fetched through block_table[entry][c / page_size].
 #include "common.cuh"
+#include "ginfer_amd.h"   // the entry points below are checked against their declarations
 
 #define MAX_HD 256
 

@@ -29,6 +29,7 @@
 // once per wavefront, and the heads of a group that run side by side hit the same lines in the vector cache.
 // The second prefill kernel (head sizes 64, 128, 256) has one wavefront load each tile into LDS for all heads.
 #include "common.cuh"
+#include "ginfer_amd.h"   // the entry points below are checked against their declarations
 
 #ifndef HEAD_DIM
 #error "compile with -DHEAD_DIM=<head size>"

@@ -3,6 +3,7 @@
 // Formula: ginfer/core/op/kernels/cuda/embedding_kernel.cu:16-24 (which copies in the table's
 // dtype and drops a tail of H % 8 elements; here every element is copied).
 #include "common.cuh"
+#include "ginfer_amd.h"   // the entry points below are checked against their declarations
 
 template <typename T>
 __global__ void embedding_gather_kernel(float* __restrict__ out, const T* __restrict__ table,

@@ -10,6 +10,7 @@
 // that it also serves bfloat16 operands (the kernel tests' oracle and the fallback for shapes the
 // matrix-core kernels refuse).
 #include "common.cuh"
+#include "ginfer_amd.h"   // the entry points below are checked against their declarations
 
 #define TM 64
 #define TN 64

@@ -13,6 +13,7 @@
 // [k + 16g, k + 16g + 16) of every 64-element step as two products, so that the four lanes of a row read
 // 128 consecutive bytes.
 #include "common.cuh"
+#include "ginfer_amd.h"   // the entry points below are checked against their declarations
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
@@ -287,19 +288,7 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(TC* __restrict_
   }
 }
 
-// What ga_gemm_skinny takes beside the product itself; all null or zero for a plain product.
-struct GaSkinnyNorm {
-  const float* in_sumsq;   // [M][in_parts]: the rows of A are (h * g) of a norm whose sums these are
-  int in_parts;
-  float inv_width, eps;
-  float* residual;         // [M][N], row stride ldr: the product is added to it (C is not written)
-  int64_t ldr;
-  const void* gain;        // [N] of the norm that follows
-  int gain_f32;
-  void* scaled;            // bfloat16 [M][N], row stride lds
-  int64_t lds;
-  float* out_sumsq;        // [M][ga_skinny_norm_parts(M, N)]
-};
+// GaSkinnyNorm, what ga_gemm_skinny takes beside the product itself, is declared in ginfer_amd.h.
 
 // Tiles of a product of M rows when the caller leaves the choice to the library: packed where they can be and
 // full tiles would make fewer than 192 workgroups.  Measured on MI355X: a third faster where a product has few

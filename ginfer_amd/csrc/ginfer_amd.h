@@ -7,7 +7,7 @@
 // are raw 16-bit patterns.  Nothing here allocates device memory: scratch memory is the caller's (or, for
 // ga_sample_rows_static, a static array of the library).
 //
-// The declarations repeat the definitions' parameter lists; tests/test_config.py compares the two.
+// Every source includes this header, so the compiler checks each definition against its declaration.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -87,6 +87,10 @@ int ga_attn_prefill(void* out, int64_t out_stride, const void* q, int64_t q_stri
                     const void* v_pages, const void* block_table, int table_width, const void* tiles, int n_tiles,
                     int tile_rows, int nh, int nkv, int page_size, int window, float scale, int fill_workgroups,
                     hipStream_t stream);
+
+// ---- random_fill.hip: out[i] = mean + std * normal(key, i) for n elements, float or bfloat16: the counter-based
+// generator of random_normal.h, which gives the host library (host/random_fill_host.cpp) the same bits
+int ga_random_normal_fill(void* out, int64_t n, uint64_t key, float mean, float std, int is_bf16, hipStream_t stream);
 
 // ---- sampling.hip: out int32 [rows]: argmax (lowest index among equals) where temperature is null or 0, else one
 // draw from softmax(logits / temperature) by the given uniform number; scratch: ga_sample_scratch_floats floats

@@ -12,6 +12,7 @@
 // load).  The slot of token t is slot_mapping[t] = page * page_size + slot_in_page, or -1 to write
 // nothing for that token.
 #include "common.cuh"
+#include "ginfer_amd.h"   // the entry points below are checked against their declarations
 
 template <typename T>
 __global__ void rope_kv_write_kernel(T* __restrict__ qkv, const int32_t* __restrict__ positions,

@@ -9,6 +9,7 @@
 //     the cut into segments depends on the vocabulary alone, never on the rows beside it.
 // The reference samples greedily only (ginfer/engine/sampling_params.h:5-8).
 #include "common.cuh"
+#include "ginfer_amd.h"   // the entry points below are checked against their declarations
 #include <atomic>
 #include <mutex>
 

@@ -40,6 +40,8 @@ class EngineConfig:
     # steps with prompt portions of up to 512 token rows are laid into recorded steps of padded sizes: their launches
     # would cost the host more than the device works on them
     graph_mixed_steps: bool = True
+    # a tensor in the model folder that the model does not read: an error instead of a warning
+    strict_weights: bool = False
 
 
 @dataclass
@@ -63,6 +65,7 @@ class Engine:
                                   gpu_memory_utilization=config.gpu_memory_utilization,
                                   prefix_caching=config.enable_prefix_caching,
                                   graph_mixed_steps=config.graph_mixed_steps,
+                                  strict_weights=config.strict_weights,
                                   config=config.model_config if config.model_path is None else None,
                                   random_seed=config.random_seed if config.model_path is None else None)
         self.scheduler = Scheduler(self.runner.cache, config.max_num_seqs, config.max_num_batched_tokens,

@@ -44,12 +44,14 @@ def require_gpu():
 class ModelRunner:
     def __init__(self, model_path, dtype="bfloat16", page_size=16, num_pages=None, max_requests=64,
                  max_model_len=None, gpu_memory_utilization=0.9, device=None, config=None, use_graphs=True,
-                 prefix_caching=False, random_seed=None, graph_mixed_steps=True, max_num_batched_tokens=None):
+                 prefix_caching=False, random_seed=None, graph_mixed_steps=True, max_num_batched_tokens=None,
+                 strict_weights=False):
         """model_path: a folder with config.json and the weights.  With model_path None, `config` (a typed
         configuration) and `random_seed` make a model whose weights are drawn on the device, for shapes too
         large to pass through a file.  num_pages: pages of every cache group (or a list, one count per group);
         None: from the memory that is free once the weights are loaded and the largest step (max_num_batched_tokens
-        tokens, max_requests requests) has run, times gpu_memory_utilization."""
+        tokens, max_requests requests) has run, times gpu_memory_utilization.  strict_weights: a tensor in the folder
+        that the model does not read is an error, not a warning."""
         self.device = device or require_gpu()
         if dtype not in DTYPES:
             raise ValueError("dtype must be one of %s, got %r" % (sorted(DTYPES), dtype))
@@ -67,7 +69,7 @@ class ModelRunner:
         if model_path is None:
             bind_random_weights(self.model, int(random_seed), self.device)
         else:
-            load_weights(self.model, model_path, self.device)
+            load_weights(self.model, model_path, self.device, strict=strict_weights)
         self.page_size = int(page_size)
         self.max_requests = int(max_requests)
         self.max_step_tokens = int(min(max_num_batched_tokens or 2048, self.max_model_len))

@@ -24,7 +24,15 @@ ARCH = "gfx950"
 FLAGS = ["--offload-arch=" + ARCH, "-O3", "-std=c++17", "-shared", "-fPIC",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
 MODULES = ("embedding", "norm", "rope_kv", "attention_generic", "attention_mfma", "gemm", "gemm_skinny",
-           "activation", "sampling")
+           "activation", "sampling", "random_fill")
+# flags of single modules: the random-weights generator must round every operation by itself, as the host's twin does
+MODULE_FLAGS = {"random_fill": ["-ffp-contract=off"]}
+# headers beside common.cuh that a module includes (they enter its digest)
+MODULE_HEADERS = {"random_fill": ["random_normal.h"]}
+# plain C++ libraries for the host (no GPU runtime), built with the host compiler from csrc/host/
+HOST_MODULES = ("random_fill_host",)
+HOST_FLAGS = ["-O2", "-std=c++17", "-shared", "-fPIC", "-pthread", "-ffp-contract=off"]
+HOST_HEADERS = {"random_fill_host": ["random_normal.h"]}
 # Modules that are compiled for one value of a parameter (a macro) at a time; build_all() without a
 # list compiles these values, and any other value a model needs is compiled when it is first asked for.
 VARIANTS = {"attention_mfma": [{"HEAD_DIM": hd} for hd in range(16, 257, 16)]}
@@ -61,10 +69,10 @@ def _split(module):
 def _digest(module):
     src, defines, _ = _split(module)
     h = hashlib.sha256()
-    for name in (src + ".hip", "common.cuh"):
+    for name in [src + ".hip", "common.cuh", "ginfer_amd.h"] + MODULE_HEADERS.get(src, []):
         with open(os.path.join(CSRC, name), "rb") as f:
             h.update(f.read())
-    h.update(" ".join(FLAGS).encode())
+    h.update(" ".join(FLAGS + MODULE_FLAGS.get(src, [])).encode())
     h.update(repr(sorted(defines.items())).encode())
     return h.hexdigest()[:16]
 
@@ -118,7 +126,7 @@ def compile_module(module, out_dir=None, quiet=False):
     src, defines, stem = _split(module)
     so = os.path.join(out_dir, "lib%s.so" % stem)
     tmp = so + ".%d.tmp" % os.getpid()
-    cmd = ([hipcc] + FLAGS + ["-D%s=%s" % kv for kv in sorted(defines.items())]
+    cmd = ([hipcc] + FLAGS + MODULE_FLAGS.get(src, []) + ["-D%s=%s" % kv for kv in sorted(defines.items())]
            + ["-I", CSRC, "-o", tmp, os.path.join(CSRC, src + ".hip")])
     module = stem
     env = dict(os.environ)
@@ -148,10 +156,81 @@ def compile_module(module, out_dir=None, quiet=False):
     return so
 
 
+def _host_compiler():
+    for cand in (os.environ.get("CXX"), shutil.which("g++"), shutil.which("c++"), shutil.which("clang++"),
+                 "/opt/rocm/llvm/bin/clang++"):
+        if cand and os.path.isfile(cand if os.path.isabs(cand) else (shutil.which(cand) or "")):
+            return cand if os.path.isabs(cand) else shutil.which(cand)
+    return None
+
+
+def _host_digest(name):
+    h = hashlib.sha256()
+    for path in [os.path.join(CSRC, "host", name + ".cpp")] + [os.path.join(CSRC, x) for x in HOST_HEADERS.get(name, [])]:
+        with open(path, "rb") as f:
+            h.update(f.read())
+    h.update(" ".join(HOST_FLAGS).encode())
+    return h.hexdigest()[:16]
+
+
+def compile_host_module(name, out_dir=None):
+    """Runs the host compiler for one plain C++ library; returns its path."""
+    cxx = _host_compiler()
+    if cxx is None:
+        raise KernelBuildError("no C++ compiler found: cannot build host library %r" % name)
+    out_dir = out_dir or _writable_dir()
+    so = os.path.join(out_dir, "lib%s.so" % name)
+    tmp = so + ".%d.tmp" % os.getpid()
+    proc = subprocess.run([cxx] + HOST_FLAGS + ["-o", tmp, os.path.join(CSRC, "host", name + ".cpp")],
+                          stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if proc.returncode != 0:
+        if os.path.exists(tmp):
+            os.remove(tmp)
+        raise KernelBuildError("%s failed for %s:\n%s" % (cxx, name, proc.stdout))
+    os.replace(tmp, so)
+    with open(os.path.join(out_dir, "%s.stamp" % name), "w") as f:
+        f.write(_host_digest(name))
+    return so
+
+
+def load_host(name):
+    """The ctypes library of a plain C++ host module, built first if it is missing or stale.  Needs no GPU."""
+    with _lock:
+        if name in _loaded:
+            return _loaded[name]
+        if name not in HOST_MODULES:
+            raise KernelBuildError("no host library %r" % name)
+        digest, so = _host_digest(name), None
+        for d in _build_dirs():
+            try:
+                with open(os.path.join(d, "%s.stamp" % name)) as f:
+                    if f.read().strip() == digest and os.path.isfile(os.path.join(d, "lib%s.so" % name)):
+                        so = os.path.join(d, "lib%s.so" % name)
+                        break
+            except OSError:
+                pass
+        if so is None:
+            so = compile_host_module(name)
+        try:
+            lib = ctypes.CDLL(so)
+        except OSError as e:
+            raise KernelBuildError("cannot load host library %s: %s" % (so, e))
+        _loaded[name] = lib
+        return lib
+
+
 def build_all(force=False, modules=None, quiet=False):
-    """Builds every module (in parallel); with force, also those already built."""
+    """Builds every module (in parallel); with force, also those already built.  Without a list of modules the
+    host libraries are built too."""
     from concurrent.futures import ThreadPoolExecutor
     if modules is None:
+        for name in HOST_MODULES:
+            if force:
+                compile_host_module(name)
+                if not quiet:
+                    _say("compiled host library %s" % name)
+            else:
+                load_host(name)
         modules = []
         for m in available_modules():
             modules.extend([(m, v) for v in VARIANTS[m]] if m in VARIANTS else [m])

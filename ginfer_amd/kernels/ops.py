@@ -280,6 +280,18 @@ def sample_rows(logits, temperature=None, uniform=None, out=None):
     return out
 
 
+def random_normal_fill(out, key, mean, std):
+    """out[i] = mean + std * normal(key, i) over out's elements in memory order (float32 or bfloat16, contiguous): the
+    counter-based generator that the host shares, so the same key gives the same bits there."""
+    _dev(out)
+    _need(out.is_contiguous() and out.dtype in (torch.float32, torch.bfloat16), "random fill takes a contiguous float32 or "
+          "bfloat16 tensor")
+    lib = build.load("random_fill")
+    _check(lib.ga_random_normal_fill(_ptr(out), _i64(out.numel()), ctypes.c_uint64(int(key)), _f(mean), _f(std),
+                                     _i(_is_bf16(out.dtype)), _stream()), "random_normal_fill")
+    return out
+
+
 SKINNY_MAX_ROWS = 64
 FOLDED_NORM_MAX_ROWS = 16
 

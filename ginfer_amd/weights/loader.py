@@ -2,7 +2,8 @@
 
 The model says which tensors it expects (`model.weight_specs()`: full name -> `WeightSpec`); the
 file says which it holds.  Every disagreement (missing, unexpected, wrong shape, wrong kind of
-dtype) is collected and raised as ONE error.  Floating tensors are kept in the compute dtype
+dtype) is collected and raised as ONE error; tensors that the model does not read are, by themselves,
+a warning (an error with `strict`).  Floating tensors are kept in the compute dtype
 (bfloat16 or float32); integer tables become int32; a tensor whose spec says `keep_32bit` stays in
 32-bit when the file stores it so.  The reference binds the same names without checking shapes
 (ginfer/model/qwen2.cc:34-46, ginfer/model/loader/safetensor_loader.cc:44-81).
@@ -28,10 +29,14 @@ class WeightError(ValueError):
     pass
 
 
-def check_against(specs, available, where, unread=()):
+def check_against(specs, available, where, unread=(), strict=False):
     """specs: name -> WeightSpec; available: name -> (dtype, shape); unread: names the file may hold
-    although the model reads none of them.  Raises one WeightError that lists everything that is wrong,
-    or returns."""
+    although the model reads none of them.  Raises one WeightError that lists everything that is wrong
+    (missing tensors, unexpected ones, wrong shapes or kinds), or returns the list of unexpected tensors.
+    Tensors that the model does not read are no fault by themselves: the reference looks tensors up by name and
+    never sees the others (ginfer/model/loader/safetensor_loader.cc:44-81), and checkpoints carry such tensors
+    (a rotary table, say).  Where they are all that is wrong they are named in a warning; with `strict` they are
+    an error."""
     missing = [n for n in specs if n not in available]
     unexpected = [n for n in available if n not in specs and n not in unread]
     wrong = []
@@ -45,8 +50,12 @@ def check_against(specs, available, where, unread=()):
             wrong.append("%s: expected a floating tensor, found %s" % (n, dtype))
         elif s.kind == "int" and (dtype.is_floating_point or dtype == torch.bool):
             wrong.append("%s: expected an integer tensor, found %s" % (n, dtype))
-    if not (missing or unexpected or wrong):
-        return
+    if not (missing or wrong) and not (strict and unexpected):
+        if unexpected:
+            import sys
+            sys.stderr.write("[ginfer_amd] warning: %s holds %d tensor(s) that the model does not read: %s\n"
+                             % (where, len(unexpected), ", ".join(sorted(unexpected))))
+        return sorted(unexpected)
     lines = ["weights in %s do not match the model:" % where]
     if missing:
         lines.append("  missing tensors (%d): %s" % (len(missing), ", ".join(sorted(missing))))
@@ -88,13 +97,14 @@ class TensorsOnDemand:
         return sorted(self._names)
 
 
-def load_weights(model, folder, device):
+def load_weights(model, folder, device, strict=False):
     """Reads every tensor the model expects from `folder`, converts, uploads, and hands the
-    dictionary to `model.bind_weights`."""
+    dictionary to `model.bind_weights`.  strict: a tensor in the folder that the model does not read is an error
+    instead of a warning."""
     specs = model.weight_specs()
     files = open_model_files(folder)
     available = {n: f.info(n) for n, f in files.items()}
-    check_against(specs, available, folder, unread=set(getattr(model, "unread_weights", list)()))
+    check_against(specs, available, folder, unread=set(getattr(model, "unread_weights", list)()), strict=strict)
     def fetch(name):
         cpu = files[name].tensor(name)
         dt = target_dtype(specs[name], cpu.dtype, model.dtype)

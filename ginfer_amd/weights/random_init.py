@@ -2,8 +2,9 @@
 a seed.  The reference has no such mode (it loads checkpoints only, ginfer/model/qwen2.cc:28-49).
 
 Matrices, embeddings and biases are drawn from N(0, std); norm gains from 1 + N(0, std), as each
-part's `WeightSpec.init` says.  Every tensor has a generator of its own, seeded by the seed and the
-tensor's name, so a tensor's values do not depend on which other tensors the model has.
+part's `WeightSpec.init` says.  The generator is counter-based: an element is a function of (seed, the
+tensor's name, its index) alone, so a tensor's values do not depend on which other tensors the model has,
+and the same function runs on the host (here) and on the device (`bind_random_weights`), bit for bit.
 """
 import hashlib
 import json
@@ -22,44 +23,51 @@ def _tensor_seed(seed, name):
 
 
 def draw(spec, seed, name, dtype, std_scale=1.0):
-    g = torch.Generator(device="cpu")
-    g.manual_seed(_tensor_seed(seed, name))
+    """One tensor on the host: element i is mean + std * normal(key of (seed, name), i) from the counter-based
+    generator that the device kernel shares (csrc/random_normal.h), rounded once to `dtype`."""
     if spec.kind == "int":
         return torch.zeros(spec.shape, dtype=torch.int32)
     if spec.init == "zeros":
-        t = torch.zeros(spec.shape, dtype=torch.float32)
-    elif spec.init == "ones":
-        t = torch.ones(spec.shape, dtype=torch.float32)
-    else:
-        t = torch.empty(spec.shape, dtype=torch.float32).normal_(0.0, spec.std * std_scale, generator=g)
-        if spec.init == "one_plus_normal":
-            t += 1.0
-        elif spec.init != "normal":
-            raise ValueError("unknown init %r for %s" % (spec.init, name))
+        return torch.zeros(spec.shape, dtype=dtype)
+    if spec.init == "ones":
+        return torch.ones(spec.shape, dtype=dtype)
+    if spec.init not in ("normal", "one_plus_normal"):
+        raise ValueError("unknown init %r for %s" % (spec.init, name))
+    import ctypes
+    from ..kernels import build
+    lib = build.load_host("random_fill_host")
+    t = torch.empty(spec.shape, dtype=torch.float32)
+    rc = lib.ga_random_normal_fill_host(ctypes.c_void_p(t.data_ptr()), ctypes.c_int64(t.numel()),
+                                        ctypes.c_uint64(_tensor_seed(seed, name)),
+                                        ctypes.c_float(1.0 if spec.init == "one_plus_normal" else 0.0),
+                                        ctypes.c_float(spec.std * std_scale), ctypes.c_int(min(16, os.cpu_count() or 1)))
+    if rc != 0:
+        raise RuntimeError("the host's random fill failed for %s (code %d)" % (name, rc))
     return t.to(dtype)
 
 
 def bind_random_weights(model, seed, device, std_scale=1.0):
     """Draws every tensor the model expects on the device and binds it: for shapes too large to pass
-    through a file in reasonable time (a 72B shape is 145 GB).  Same distributions and the same seeding by
-    (seed, tensor name) as `draw`, but the device's generator gives other numbers than the host's: a model
-    made here is not the one `write_random_model` writes for the same seed."""
-    from .loader import TensorsOnDemand
+    through a file in reasonable time (a 72B shape is 145 GB).  Same generator and the same key (seed, tensor name)
+    as `draw`: the model made here holds, bit for bit, what `write_random_model` writes for the same seed in the
+    model's dtype."""
+    from ..kernels import ops
+    from .loader import TensorsOnDemand, target_dtype
     specs = model.weight_specs()
 
     def make(name):
         spec = specs[name]
         if spec.kind == "int":
             return torch.zeros(spec.shape, dtype=torch.int32, device=device)
-        dt = model.dtype                 # as a checkpoint stored in the compute dtype would load
+        dt = target_dtype(spec, model.dtype, model.dtype)       # as a checkpoint stored in the compute dtype would load
         if spec.init in ("zeros", "ones"):
             return torch.full(spec.shape, 0.0 if spec.init == "zeros" else 1.0, dtype=dt, device=device)
         if spec.init not in ("normal", "one_plus_normal"):
             raise ValueError("unknown init %r for %s" % (spec.init, name))
-        g = torch.Generator(device=device)
-        g.manual_seed(_tensor_seed(seed, name))
-        return torch.empty(spec.shape, dtype=dt, device=device).normal_(
-            1.0 if spec.init == "one_plus_normal" else 0.0, spec.std * std_scale, generator=g)
+        out = torch.empty(spec.shape, dtype=dt, device=device)
+        ops.random_normal_fill(out, _tensor_seed(seed, name), 1.0 if spec.init == "one_plus_normal" else 0.0,
+                               spec.std * std_scale)
+        return out
     tensors = TensorsOnDemand(specs, make)
     model.bind_weights(tensors)
     return model

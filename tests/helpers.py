@@ -175,11 +175,14 @@ def run_steps(runner, steps):
     return out
 
 
-def run_trace(model_folder, dtype, steps, out_dir, max_tokens, page_size=16, timeout=600):
+def run_trace(model_folder, dtype, steps, out_dir, max_tokens, page_size=16, timeout=600, seed=None):
     """Drives bin/trace_run as a user would: a subprocess, steps on stdin one at a time, each sent
-    only after the previous `done`.  Returns {(request, position): logits row}."""
-    cmd = [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", str(model_folder), "--dtype", dtype,
-           "--out", str(out_dir), "--max-tokens", str(max_tokens), "--page-size", str(page_size)]
+    only after the previous `done`.  Returns {(request, position): logits row}.  With a seed the program gets the
+    folder's config.json and the seed instead of the folder, and draws the weights itself."""
+    model = ["--model", str(model_folder)] if seed is None else \
+        ["--config", os.path.join(str(model_folder), "config.json"), "--seed", str(seed)]
+    cmd = [sys.executable, os.path.join(ROOT, "bin", "trace_run")] + model + [
+        "--dtype", dtype, "--out", str(out_dir), "--max-tokens", str(max_tokens), "--page-size", str(page_size)]
     proc = subprocess.Popen(cmd, stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True)
     at, out = {}, {}
     vocab = pm.read_config(model_folder)["vocab_size"]

@@ -99,6 +99,17 @@ def test_trace_run_program(folders, tmp_path, dtype, name):
     H.compare_with_plain(got, both, folders[name], H.TOL[dtype], "trace_run %s" % dtype)
 
 
+def test_trace_run_program_from_a_configuration_and_a_seed(tmp_path):
+    """bin/trace_run --config CONFIG.json --seed S draws the weights itself, on the device: the logits are those of
+    the model folder that the host writes for the same seed, which the plain implementation reads."""
+    cfg, seed, page = H.TINY["B"]
+    folder = H.make_model_folder(tmp_path / "b", cfg, 11, "float32")
+    reqs = _requests("B", [50, 21], seed=71)
+    steps = H.steps_portions(reqs, sizes=(9, 2, 30))
+    got = H.run_trace(folder, "float32", steps, tmp_path / "out", H.max_live_tokens(steps), page_size=page, seed=11)
+    H.compare_with_plain(got, reqs, folder, H.TOL["float32"], "trace_run from a seed")
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_long_decoding(folders, dtype):
     """Three hundred tokens one by one after a short prompt, across many page edges."""
@@ -739,8 +750,32 @@ def test_steps_launched_ahead_change_nothing(folders, dtype):
     with_ahead, n_ahead = run(True)
     without, none_ahead = run(False)
     assert n_ahead > 5 and none_ahead == 0
-    assert with_ahead == without
     assert {r for _, r in with_ahead} >= {"eos", "max_tokens"}
+    if dtype == "float32":
+        assert with_ahead == without
+        return
+    # bfloat16: the two runs put other requests side by side in their steps (a step launched ahead admits nobody), and a
+    # product of other row counts rounds otherwise, so a draw that lies on the border between two tokens may fall either
+    # way and the request goes on differently from there.  Every token of either run must be what the plain
+    # implementation draws after the run's own tokens so far, up to the bfloat16 tolerance on the logits (greedy) or
+    # on the token's share of the probability (sampled).
+    from ginfer_amd.sampling import uniform
+    cfg, w = pm.read_config(folders[name]), pm.read_weights(folders[name])
+    settings = ((12, 0.0), (12, 0.0), (25, 0.8), (7, 0.0), (30, 0.0), (1, 0.0), (16, 1.1), (20, 0.0))
+    for what, run_tokens in (("launched ahead", with_ahead), ("one by one", without)):
+        for i, ((toks, reason), (_, temp)) in enumerate(zip(run_tokens, settings)):
+            logits = pm.forward(cfg, w, (prompts[i] + toks)[:-1])
+            for k, tok in enumerate(toks):
+                row = logits[len(prompts[i]) - 1 + k]
+                if temp == 0:
+                    best = int(torch.argmax(row))
+                    assert tok == best or float(row[best] - row[tok]) <= H.TOL[dtype] * float(row.abs().max()), \
+                        "%s: request %d token %d: %d, plain %d" % (what, i, k, tok, best)
+                else:
+                    cdf = torch.cumsum(torch.softmax(row / temp, 0), 0)
+                    lo, hi, u = (float(cdf[tok - 1]) if tok else 0.0), float(cdf[tok]), uniform(7, k)
+                    assert lo - H.TOL[dtype] <= u <= hi + H.TOL[dtype], \
+                        "%s: request %d token %d: %d holds [%.4f, %.4f], the draw is %.4f" % (what, i, k, tok, lo, hi, u)
 
 
 def test_weights_drawn_on_the_device():
@@ -762,6 +797,39 @@ def test_weights_drawn_on_the_device():
     assert torch.equal(outs[0], outs[1]) and not torch.equal(outs[0], outs[2])
     with pytest.raises(ValueError):
         ModelRunner(None, dtype="float32", config=cfg)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_weights_drawn_on_the_device_are_the_bits_the_host_writes(tmp_path, dtype):
+    """One generator for host and device: a model whose weights are drawn on the device holds, tensor by tensor and bit
+    for bit, what the model folder written for the same seed holds, so a model that never passed through a file still
+    has its plain twin; and the device's draws have the distribution that is claimed for them."""
+    from ginfer_amd import ModelRunner, StepEntry, config_from_dict, write_random_model
+    from ginfer_amd.kernels import ops
+    from safetensors import safe_open
+    from scipy import stats
+    cfg = config_from_dict(H.TINY_C)
+    folder = write_random_model(str(tmp_path / "m"), cfg, 7, dtype)
+    drawn = ModelRunner(None, dtype=dtype, page_size=16, num_pages=8, max_requests=2, config=cfg, random_seed=7)
+    loaded = ModelRunner(folder, dtype=dtype, page_size=16, num_pages=8, max_requests=2)
+    for (name, a), (_, b) in zip(drawn.model._named_parts(), loaded.model._named_parts()):
+        tensors = [(k, v) for k, v in vars(a).items() if isinstance(v, torch.Tensor)]
+        assert tensors or not a.weight_specs(), name
+        for k, v in tensors:
+            assert v.dtype == getattr(b, k).dtype and torch.equal(v, getattr(b, k)), "%s.%s differs" % (name, k)
+    ids = H.random_tokens(50, 777, 3)
+    got = drawn.step([StepEntry("a", ids, [49])]).cpu()
+    assert torch.equal(got, loaded.step([StepEntry("a", ids, [49])]).cpu())
+    ref = H.plain_logits(folder, ids)[49]
+    assert H.rel_err(got[0].numpy(), ref) <= H.TOL[dtype]
+    # the draws themselves: a million numbers of one key against the normal distribution, and against the host's
+    x = torch.empty(1 << 20, dtype=torch.float32, device=drawn.device)
+    ops.random_normal_fill(x, 99, 0.5, 0.02)
+    x = x.cpu().double().numpy()
+    assert abs(x.mean() - 0.5) < 1e-4 and abs(x.std() - 0.02) < 1e-4
+    z = (x - 0.5) / 0.02
+    assert stats.kstest(z, "norm").pvalue > 1e-3 and abs((z ** 4).mean() - 3.0) < 0.05 and abs((z ** 3).mean()) < 0.02
+    assert np.abs(np.corrcoef(z[:-1], z[1:])[0, 1]) < 5e-3           # neighbours are not correlated
 
 
 def test_abort_in_the_middle_leaves_the_others_untouched(folders):

@@ -97,6 +97,25 @@ def test_one_error_lists_missing_unexpected_and_wrong(tmp_path):
     assert e.value.missing == ["model.layers.1.mlp.up_proj.weight", "model.norm.weight"]
 
 
+def test_tensors_that_the_model_does_not_read_are_a_warning_or_an_error_when_strict(tmp_path, capsys):
+    """A checkpoint may carry tensors the model never reads (the reference looks tensors up by name and never sees the
+    others, ginfer/model/loader/safetensor_loader.cc:44-81): by themselves they are named in a warning; under
+    `strict` they are the error."""
+    cfg = config_from_dict(H.TINY_A)
+    folder = write_random_model(str(tmp_path / "m"), cfg, 0, "float32")
+    f = SafetensorsFile(os.path.join(folder, "model.safetensors"))
+    tensors = {n: f.tensor(n).clone() for n in f.names()}
+    tensors["model.layers.0.self_attn.rotary_emb.inv_freq"] = torch.zeros(8)
+    write_safetensors(os.path.join(folder, "model.safetensors"), tensors)
+    model = build_model(cfg.model_spec(), torch.float32, None)
+    available = {n: fl.info(n) for n, fl in open_model_files(folder).items()}
+    assert check_against(model.weight_specs(), available, folder, unread=model.unread_weights()) == \
+        ["model.layers.0.self_attn.rotary_emb.inv_freq"]
+    assert "does not read: model.layers.0.self_attn.rotary_emb.inv_freq" in capsys.readouterr().err
+    with pytest.raises(WeightError, match=r"unexpected tensors \(1\): model.layers.0.self_attn.rotary_emb.inv_freq"):
+        check_against(model.weight_specs(), available, folder, unread=model.unread_weights(), strict=True)
+
+
 def test_dtype_rules():
     f32, bf16 = torch.float32, torch.bfloat16
     assert target_dtype(WeightSpec((2,)), f32, bf16) == bf16            # kept in bfloat16
@@ -125,6 +144,26 @@ def test_random_weights_mode(tmp_path):
         d = json.load(fh)
     assert d["torch_dtype"] == "bfloat16" and d["architectures"] == ["Qwen2ForCausalLM"]
     assert config_from_dict(d).num_key_value_heads == 1
+
+
+def test_the_host_generator_is_a_function_of_seed_name_and_index():
+    """Counter-based: a tensor's draws depend on the seed and its name alone, any stretch of it can be drawn by
+    itself, and the numbers are normal (mean, spread, tails, no correlation between neighbours)."""
+    import numpy as np
+    from scipy import stats
+    from ginfer_amd.weights.random_init import draw
+    spec = WeightSpec((1 << 18,))
+    a = draw(spec, 5, "t.weight", torch.float32)
+    assert torch.equal(a, draw(spec, 5, "t.weight", torch.float32))
+    assert not torch.equal(a, draw(spec, 6, "t.weight", torch.float32)) and not torch.equal(a, draw(spec, 5, "u.weight", torch.float32))
+    assert torch.equal(draw(WeightSpec((1000,)), 5, "t.weight", torch.float32), a[:1000])      # a prefix is the same numbers
+    assert torch.equal(draw(spec, 5, "t.weight", torch.bfloat16), a.to(torch.bfloat16))        # one rounding
+    z = a.double().numpy() / 0.02
+    assert abs(z.mean()) < 0.01 and abs(z.std() - 1) < 0.01 and abs((z ** 4).mean() - 3) < 0.1
+    assert stats.kstest(z, "norm").pvalue > 1e-3 and np.abs(z).max() < 6.0
+    assert abs(np.corrcoef(z[:-1], z[1:])[0, 1]) < 0.01
+    g = draw(WeightSpec((4096,), init="one_plus_normal"), 5, "g.weight", torch.float32)
+    assert abs(g.mean().item() - 1) < 2e-3 and abs(g.std().item() - 0.02) < 2e-3
 
 
 def test_sharded_folder(tmp_path):
