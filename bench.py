@@ -4,9 +4,10 @@ on one MI355X, with the achieved fraction of the HBM and matrix-core rooflines.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B] [--context C]
 
-A step is one decode step of the engine's own step function plus sampling: every request of the batch
-gets one token, from the paged cache, and its next token comes back to the host; as in the engine, the next
-step is launched before this step's tokens have been waited for.  Prints ONE JSON line.
+A step is one decode step of the engine: `Engine.step()` on requests that the engine itself has prefilled to the
+context, every request of the batch getting one token from the paged cache, its next token coming back to the
+host; the engine launches the next step before this step's tokens have been waited for.  Prints ONE JSON line;
+`device_ms_per_step` is the device's own time for a step's kernels beside the wall time `ms_per_step`.
 """
 import argparse
 import json
@@ -73,8 +74,7 @@ def main():
         sys.exit(2)
 
     import torch
-    from ginfer_amd import ModelRunner, StepEntry, config_from_dict, write_random_model
-    from ginfer_amd.sampling import Sampler, SamplingParams
+    from ginfer_amd import Engine, EngineConfig, SamplingParams, config_from_dict, write_random_model
 
     shape_name, shape = SHAPES[args.shape]
     full_layers = shape["num_hidden_layers"]
@@ -83,6 +83,8 @@ def main():
     device_weights = args.shape == "72b" or not (args.file_weights or args.model_dir)
     cfg = dict(shape, num_hidden_layers=args.layers)
     weight_bytes, kv_per_token, prefill_flops = model_numbers(cfg, args.layers)
+    if args.dtype == "float32":
+        weight_bytes, kv_per_token = 2 * weight_bytes, 2 * kv_per_token
     tmp = None
     folder = args.model_dir
     if device_weights:
@@ -98,94 +100,92 @@ def main():
     points = sorted({int(p) for p in args.points.split(",") if p} | {args.batch})
     max_b = max(points)
     page = 16
-    ctx_pages = -(-(args.context + 1) // page)
+    ctx_pages = -(-(args.context + 24) // page)
     pages = max_b * ctx_pages + -(-args.prefill_tokens // page) + 8
-    runner = ModelRunner(folder, dtype=args.dtype, page_size=page, num_pages=pages, max_requests=max_b + 1,
-                         max_model_len=max(args.context, args.prefill_tokens) + 8,
-                         config=config_from_dict(cfg) if device_weights else None,
-                         random_seed=0 if device_weights else None)
-    sampler = Sampler(runner.device)
+    # The engine itself is what is timed: requests are added, the scheduler cuts their prompts into steps and reserves
+    # their pages, the runner replays recorded decode steps, the sampler picks, tokens come back to the host every step.
+    engine = Engine(EngineConfig(
+        model_path=folder, model_config=config_from_dict(cfg) if device_weights else None,
+        random_seed=0 if device_weights else None, dtype=args.dtype,
+        max_num_batched_tokens=max(2048, args.prefill_tokens, args.context + max_b), max_num_seqs=max_b,
+        max_seq_len=max(args.context, args.prefill_tokens) + max_b + 24, kvcache_block_size=page, num_kvcache_blocks=pages,
+        enable_prefix_caching=False))
     g = torch.Generator().manual_seed(0)
     vocab = cfg["vocab_size"]
 
     def sync():
         torch.cuda.synchronize()
 
-    # ---- prefill: one prompt of 2,048 tokens, the logits of its last place
+    def finite():
+        if not bool(torch.isfinite(engine.last_logits).all()):
+            sys.exit("bench.py: the step that was just timed made logits that are not finite")
+
+    # ---- prefill: one prompt of 2,048 tokens through Engine.step, up to its first token on the host
     T = args.prefill_tokens
-    prompt = torch.randint(0, vocab, (T,), generator=g).tolist()
     times = []
     for i in range(4):
+        prompt = torch.randint(0, vocab, (T,), generator=g).tolist()
+        engine.add_request(prompt, SamplingParams(max_tokens=1, ignore_eos=True))
         sync()
         t0 = time.perf_counter()
-        logits = runner.step([StepEntry("p", prompt, [T - 1])])
-        sampler.sample(logits, [SamplingParams()], [0])
+        done = engine.step()
         sync()
         times.append(time.perf_counter() - t0)
-        runner.release("p")
+        assert len(done) == 1 and len(done[0].token_ids) == 1 and not engine.has_unfinished()
+        finite()
     prefill_s = min(times[1:])
     peak = PEAK_FLOPS["bf16" if args.dtype == "bfloat16" else "fp32"]
     prefill = {"value": round(T / prefill_s, 1), "tokens": T, "ms": round(prefill_s * 1e3, 3),
                "frac": round(prefill_flops(T) / prefill_s / peak, 4)}
 
-    # ---- decode: B requests whose caches hold a context that ends at --context after the timed steps
+    # ---- decode: B requests whose prompts the engine prefills, so that the timed steps end at --context
     def decode(B, steps, warmup):
-        start = args.context - steps - warmup
-        for b in range(B):
-            runner.cache.admit(("d", b))
-            runner.cache.append(("d", b), start)
-            runner.cache.commit(("d", b))
-        for grp in runner.cache.groups:      # synthetic keys and values stand in for a prefilled context
-            grp.tensor.normal_(0.0, 1.0, generator=None)
-        tokens = torch.randint(0, vocab, (B,), generator=g).tolist()
-        params = [SamplingParams() for _ in range(B)]
-
-        ring = [(torch.empty(B, dtype=torch.int32, pin_memory=True), torch.cuda.Event()) for _ in range(3)]
-        at = [0]
-
-        def launch(tokens=None, device_tokens=None):
-            """One step handed to the device: model, sampling, and the tokens' copy to the host behind it."""
-            ids = tokens if tokens is not None else [0] * B
-            logits = runner.step([StepEntry(("d", b), [ids[b]], [0]) for b in range(B)], borrow=True,
-                                 device_tokens=device_tokens)
-            dev = sampler.sample_on_device(logits, params, [0] * B)
-            host, event = ring[at[0] % len(ring)]
-            at[0] += 1
-            host.copy_(dev, non_blocking=True)
-            event.record()
-            return dev, host, event
-
-        def run(n, tokens):
-            """n steps, as the engine drives them: the next step is launched (its ids taken on the device) before
-            this step's tokens, which come to the host every step, have been waited for."""
-            if n <= 0:
-                return tokens
-            cur = launch(tokens=tokens)
-            for _ in range(n - 1):
-                nxt = launch(device_tokens=cur[0])
-                cur[2].synchronize()
-                tokens = cur[1].tolist()
-                cur = nxt
-            cur[2].synchronize()
-            return cur[1].tolist()
-        tokens = run(warmup, tokens)
+        sched = engine.scheduler
+        # Requests are added one by one, each prompt running whole in one step beside a token for every request added
+        # before it (steps are not launched ahead meanwhile, so it is exactly one step); a request added earlier gets a
+        # shorter prompt by as many tokens as it decodes until the last one is in: all reach the same length.
+        engine.config.pipeline_decode = False
+        params = SamplingParams(max_tokens=steps + warmup + B + 16, ignore_eos=True)
+        ids = []
+        for i in range(B):
+            n = args.context - steps - warmup - (B - 1 - i)
+            ids.append(engine.add_request(torch.randint(0, vocab, (n,), generator=g).tolist(), params))
+            engine.step()
+        assert not sched.waiting and len(sched.running) == B and all(s.decoding and s.remaining == 1 for s in sched.running)
+        engine.config.pipeline_decode = True
+        ahead = engine.stats["steps_launched_ahead"]
+        for _ in range(warmup):
+            engine.step()
         sync()
+        del engine.step_log[:]
         t0 = time.perf_counter()
-        tokens = run(steps, tokens)
+        for _ in range(steps):
+            engine.step()
         sync()
         dt = (time.perf_counter() - t0) / steps
-        mean_ctx = args.context - steps / 2.0
-        for b in range(B):
-            runner.release(("d", b))
-        return dt, mean_ctx
+        finite()
+        log = list(engine.step_log)
+        assert len(log) == steps and all(p == 0 and d == B for _, _, p, d in log), "a timed step was no decode step of %d" % B
+        assert engine.stats["steps_launched_ahead"] - ahead >= steps, "the timed steps were not launched ahead"
+        device_ms = 1e3 * sum(d for _, d, _, _ in log) / steps
+        # tokens of a request in the cache after the last timed step (the step launched ahead of it included)
+        cached = [engine.runner.cache.length(rid) for rid in ids]
+        assert max(cached) - min(cached) <= 1 and abs(max(cached) - args.context) <= 2, cached
+        mean_ctx = sum(cached) / float(B) - steps / 2.0
+        for rid in ids:
+            engine.abort(rid)
+        while engine.has_unfinished():
+            engine.step()
+        return dt, mean_ctx, device_ms
 
     def measured_peaks():
         """What this box reaches with library routines, beside the published peaks that the fractions are quoted on:
         a device copy of 2 GB (bytes read + bytes written per second) and a bfloat16 product of 8192^3."""
-        src = torch.empty(1 << 30, dtype=torch.int16, device=runner.device)
+        dev = engine.runner.device
+        src = torch.empty(1 << 30, dtype=torch.int16, device=dev)
         dst = torch.empty_like(src)
-        a = torch.randn(8192, 8192, device=runner.device).bfloat16()
-        b = torch.randn(8192, 8192, device=runner.device).bfloat16()
+        a = torch.randn(8192, 8192, device=dev).bfloat16()
+        b = torch.randn(8192, 8192, device=dev).bfloat16()
         out = {}
         for name, fn, work in (("copy_GBps", lambda: dst.copy_(src), 2 * src.numel() * 2 / 1e9),
                                ("bf16_product_TFLOPs", lambda: torch.mm(a, b.t()), 2 * 8192 ** 3 / 1e12)):
@@ -202,13 +202,13 @@ def main():
     results = {}
     for B in points:
         results[B] = decode(B, args.steps, args.warmup)
-    dt, mean_ctx = results[args.batch]
+    dt, mean_ctx, device_ms = results[args.batch]
     step_bytes = weight_bytes + args.batch * mean_ctx * kv_per_token
     achieved = step_bytes / dt / 1e9
     out = {
         "metric": "decode tok/s at batch %d (Qwen2 %s shape, context %d)" % (args.batch, args.shape.upper(), args.context),
         "value": round(args.batch / dt, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(dt * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "ms_per_step": round(dt * 1e3, 4), "device_ms_per_step": round(device_ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic tokens, random weights N(0, 0.02)",
         "config": {"model": shape_name, "global_batch": args.batch, "seq_len": args.context,
                    "parallelism": "single-gpu", "layers": args.layers, "layers_full": full_layers,

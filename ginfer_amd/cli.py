@@ -6,6 +6,8 @@ environment variable, the engine settings carry the names of its `engine::Config
 
     python -m ginfer_amd generate  --model-path DIR --prompt-ids 1,2,3 --prompt-ids 4,5 --max-tokens 16
     python -m ginfer_amd benchmark --model-path DIR --num-prompts 256 --prompt-len 512 --max-tokens 128
+    python -m ginfer_amd benchmark --random-config C.json --num-prompts 64 --prompt-len-min 128 --prompt-len-max 2048 \
+                                   --max-tokens 256 --max-num-batched-tokens 2048 --max-num-seqs 64
     python -m ginfer_amd random-weights --config config.json --seed 0 --out DIR
     python -m ginfer_amd generate  --random-config config.json --prompt-ids 1,2,3      (weights drawn on the device)
 """
@@ -108,16 +110,23 @@ def cmd_generate(args):
 
 def cmd_benchmark(args):
     """The reference's EngineTest.Benchmark (ginfer/test/test_engine.cc:57-111): random prompts of one
-    length, a warm-up generate, then the timed one."""
+    length (or of lengths drawn from a range), a warm-up generate, then the timed one.  Reports output and total
+    tokens a second, times to the first and per further token, and every step's wall time beside the device's own
+    time for it (mean, median, 99th percentile, histogram)."""
     engine = _engine(args)
     rng = random.Random(0)
     vocab = min(engine.runner.vocab_size, 10001)
-    prompts = [[rng.randrange(vocab) for _ in range(args.prompt_len)] for _ in range(args.num_prompts)]
+    lo = args.prompt_len if args.prompt_len_min is None else args.prompt_len_min
+    hi = args.prompt_len if args.prompt_len_max is None else args.prompt_len_max
+    if not 1 <= lo <= hi:
+        sys.exit("prompt lengths must satisfy 1 <= --prompt-len-min <= --prompt-len-max")
+    prompts = [[rng.randrange(vocab) for _ in range(rng.randint(lo, hi))] for _ in range(args.num_prompts)]
     args.ignore_eos = True
     # the warm-up has prompts of its own: the timed run finds nothing of its prompts in the cache
-    engine.generate([[rng.randrange(vocab) for _ in range(args.prompt_len)] for _ in range(2)], _params(args, 2))
+    engine.generate([[rng.randrange(vocab) for _ in range(hi)] for _ in range(2)], _params(args, 2))
     for k in engine.stats:
         engine.stats[k] = 0 if isinstance(engine.stats[k], int) else 0.0
+    del engine.step_log[:]
     t0 = time.perf_counter()
     if args.request_rate > 0:
         outs = _generate_as_they_arrive(engine, prompts, _params(args, len(prompts)), args.request_rate, rng)
@@ -127,13 +136,35 @@ def cmd_benchmark(args):
     rep = _report(engine, [], wall)
     total = sum(len(o.prompt_token_ids) + len(o.token_ids) for o in outs)
     rep.update(total_tokens=total, total_tok_s=total / wall, output_tok_s=sum(len(o.token_ids) for o in outs) / wall)
+    log = engine.step_log
+    rep.update(prompt_tokens=sum(len(p) for p in prompts), prompt_len_min=lo, prompt_len_max=hi,
+               device_s=round(sum(d for _, d, _, _ in log), 4))
     for name, values in (("ttft_ms", [o.ttft * 1e3 for o in outs if o.ttft is not None]),
-                         ("tpot_ms", [o.tpot * 1e3 for o in outs if o.tpot is not None])):
+                         ("tpot_ms", [o.tpot * 1e3 for o in outs if o.tpot is not None]),
+                         ("step_wall_ms", [w * 1e3 for w, _, _, _ in log]),
+                         ("step_device_ms", [d * 1e3 for _, d, _, _ in log]),
+                         ("decode_step_wall_ms", [w * 1e3 for w, _, p, d in log if p == 0 and d > 0]),
+                         ("decode_step_device_ms", [dv * 1e3 for _, dv, p, d in log if p == 0 and d > 0])):
         values.sort()
         if values:
             rep[name] = dict(mean=round(sum(values) / len(values), 3), p50=round(values[len(values) // 2], 3),
                              p99=round(values[min(len(values) - 1, int(len(values) * 0.99))], 3))
+    rep["step_wall_ms_histogram"] = _histogram([w * 1e3 for w, _, _, _ in log])
+    rep["step_device_ms_histogram"] = _histogram([d * 1e3 for _, d, _, _ in log])
     print(json.dumps(rep))
+
+
+def _histogram(values_ms):
+    """Counts of steps by time, in bins that double: "<0.5", "0.5-1", "1-2", ... ">=256" (milliseconds)."""
+    edges = [0.5 * 2 ** k for k in range(10)]
+    names = ["<0.5"] + ["%g-%g" % (a, b) for a, b in zip(edges[:-1], edges[1:])] + [">=%g" % edges[-1]]
+    counts = [0] * len(names)
+    for v in values_ms:
+        k = 0
+        while k < len(edges) and v >= edges[k]:
+            k += 1
+        counts[k] += 1
+    return {n: c for n, c in zip(names, counts) if c}
 
 
 def _generate_as_they_arrive(engine, prompts, params, rate, rng):
@@ -179,6 +210,9 @@ def main(argv=None):
     _engine_args(b)
     b.add_argument("--num-prompts", type=int, default=256)
     b.add_argument("--prompt-len", type=int, default=512)
+    b.add_argument("--prompt-len-min", type=int, default=None,
+                   help="with --prompt-len-max: prompt lengths drawn uniformly from this range (default: all --prompt-len)")
+    b.add_argument("--prompt-len-max", type=int, default=None)
     b.add_argument("--request-rate", type=float, default=0.0,
                    help="requests a second arriving while the engine runs (0: all at once, the reference's benchmark)")
     b.set_defaults(fn=cmd_benchmark, max_num_batched_tokens=16384, max_num_seqs=256, max_tokens=128)

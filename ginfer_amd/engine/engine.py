@@ -79,7 +79,12 @@ class Engine:
                              torch.cuda.Event()) for _ in range(4)]
         self._ring_at = 0
         self.stats = dict(prefill_tokens=0, prefill_time=0.0, decode_tokens=0, decode_time=0.0, steps=0,
-                          steps_launched_ahead=0)
+                          steps_launched_ahead=0, device_time=0.0)
+        # one record a step: wall time of Engine.step, the device's own time for the step's kernels (model and sampling,
+        # between two events on the stream) and the step's tokens; the reference accounts wall time only
+        # (ginfer/engine/engine.cc:93-121)
+        self.step_log = []
+        self.last_logits = None          # the logits of the step launched last (a buffer that the next step overwrites)
         if config.warmup:
             self._warm_up()
 
@@ -142,11 +147,15 @@ class Engine:
             s = sc.seq
             toks = [0] if device_tokens is not None else s.token_ids[s.num_computed:s.num_computed + sc.num_tokens]
             entries.append(StepEntry(s.request_id, toks, [sc.num_tokens - 1] if sc.samples else []))
+        began, ended = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        began.record()
         logits = self.runner.step(entries, borrow=True, device_tokens=device_tokens)
+        self.last_logits = logits
         sampling = [sc.seq for sc in scheduled if sc.samples]
         ahead = 1 if device_tokens is not None else 0      # the token before is not in the request's list yet
         tokens = self.sampler.sample_on_device(logits, [s.params for s in sampling],
                                                [s.num_output_tokens + ahead for s in sampling])
+        ended.record()
         arrival = None
         if tokens is not None:               # the copy to the host is queued now, behind this step only
             host, event = self._token_ring[self._ring_at]
@@ -157,7 +166,7 @@ class Engine:
         n_prefill = sum(sc.num_tokens for sc in scheduled if not sc.seq.decoding)   # prompts, and evicted requests fed again
         self.scheduler.advance(scheduled)
         return dict(scheduled=scheduled, tokens=tokens, arrival=arrival, n_prefill=n_prefill,
-                    n_decode=sum(sc.num_tokens for sc in scheduled) - n_prefill)
+                    n_decode=sum(sc.num_tokens for sc in scheduled) - n_prefill, events=(began, ended))
 
     def step(self, on_token=None) -> List[RequestOutput]:
         """One scheduled batch through the model; returns the requests that finished in it.  While every
@@ -201,6 +210,12 @@ class Engine:
         st["decode_tokens"] += n_decode
         st["prefill_time"] += dt * n_prefill / total
         st["decode_time"] += dt * n_decode / total
+        began, ended = cur["events"]
+        if cur["arrival"] is None:
+            ended.synchronize()              # a step that samples nothing: its end has not been waited for yet
+        device_s = began.elapsed_time(ended) * 1e-3
+        st["device_time"] += device_s
+        self.step_log.append((dt, device_s, n_prefill, n_decode))
         return [self._output(s) for s in finished]
 
     @staticmethod
