@@ -13,72 +13,185 @@
 // every reduction in a fixed order, so a token's result is bit-identical however the request was
 // cut into steps, whatever else is in the batch and wherever its pages lie.  Head h reads kv head
 // h / (nh / nkv) (:439-450).  Keys are fetched through block_table[entry][c / page_size].
+//
+// A workgroup holds the wavefronts of `tq` neighbouring tokens of the step and of all query heads of ONE kv head.
+// Tokens of the same request see the same keys, and so do the heads of a kv group: a tile of 64 keys and their values
+// comes from the pages ONCE per workgroup, with consecutive lanes on consecutive elements, into LDS (keys [key][dim],
+// values [dim][key], each row padded by one word so that neither a lane per key nor a lane per dimension meets a bank
+// twice), and every wavefront takes its operands from there.  What a wavefront computes, and in which order it adds,
+// does not depend on what shares the workgroup with it: its dot products run over the dimensions in ascending order,
+// its sums over the keys of a tile likewise, and tiles follow each other in ascending order.
 #include "common.cuh"
 #include "ginfer_amd.h"   // the entry points below are checked against their declarations
 
 #define MAX_HD 256
+#define GA_MAX_WAVES 16
 
-template <typename T>
-__global__ void paged_attention_generic_kernel(
+// VEC elements (16 bytes) of T per load where head size and page size allow it, else one
+template <typename T, int VEC>
+struct VecLoad {
+  float v[VEC];
+  __device__ __forceinline__ void zero() {
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) v[i] = 0.f;
+  }
+  __device__ __forceinline__ void load(const T* p) {
+    if (VEC == 1) {
+      v[0] = Num<T>::ld(p);
+    } else {
+      const uint4 raw = *reinterpret_cast<const uint4*>(p);
+      const T* e = reinterpret_cast<const T*>(&raw);
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) v[i] = Num<T>::ld(e + i);
+    }
+  }
+};
+
+#define GA_BATCH 4         // loads of a thread that are under way at a time
+
+template <typename T, int VEC>
+__global__ __launch_bounds__(64 * GA_MAX_WAVES) void paged_attention_generic_kernel(
     T* __restrict__ out, int64_t out_stride, const T* __restrict__ q, int64_t q_stride,
     const T* __restrict__ k_pages, const T* __restrict__ v_pages,
     const int32_t* __restrict__ block_table, int table_width,
-    const int32_t* __restrict__ token_entry, const int32_t* __restrict__ positions, int nh, int nkv,
-    int hd, int page_size, int window, float scale) {
-  __shared__ float q_s[MAX_HD];
-  __shared__ float p_s[WAVE];
-  const int64_t t = blockIdx.x;
-  const int h = blockIdx.y;
-  const int g = h / (nh / nkv);
-  const int lane = threadIdx.x;
-  const int pos = positions[t];
+    const int32_t* __restrict__ token_entry, const int32_t* __restrict__ positions, int tokens, int nh, int nkv,
+    int hd, int page_size, int window, float scale, int tq, int hpw) {
+  extern __shared__ float lds[];
+  const int group = nh / nkv, head_blocks = (group + hpw - 1) / hpw;     // hpw heads of a kv group to a workgroup
+  const int waves = tq * hpw, threads = waves * WAVE;
+  float* k_s = lds;                              // [64][hd + 1]
+  float* v_s = k_s + WAVE * (hd + 1);            // [hd][64 + 1]
+  float* q_s = v_s + hd * (WAVE + 1);            // [waves][hd]
+  float* p_s = q_s + waves * hd;                 // [waves][64]
+  int32_t* page_s = reinterpret_cast<int32_t*>(p_s + waves * WAVE);     // [64]: the page of every key of the tile, or -1
+  const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
+  const int g = blockIdx.y / head_blocks, hl = (blockIdx.y % head_blocks) * hpw + wave % hpw;
+  const int tl = wave / hpw, h = g * group + hl;                  // the wavefront's token of the workgroup, and head
+  const int64_t t0 = (int64_t)blockIdx.x * tq;
+  const int64_t t = t0 + tl;
+  const bool live = t < tokens && hl < group;
+  const int pos = live ? positions[t] : -1;
   const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
-  const int32_t* bt = block_table + (int64_t)token_entry[t] * table_width;
-  const T* qp = q + t * q_stride + (int64_t)h * hd;
-  for (int d = lane; d < hd; d += WAVE) q_s[d] = Num<T>::ld(qp + d);
-  __syncthreads();
+  if (live) {
+    const T* qp = q + t * q_stride + (int64_t)h * hd;
+    for (int d = lane; d < hd; d += WAVE) q_s[wave * hd + d] = Num<T>::ld(qp + d);
+  }
 
   float m = -INFINITY, l = 0.f;
   float acc[MAX_HD / WAVE];
 #pragma unroll
   for (int i = 0; i < MAX_HD / WAVE; ++i) acc[i] = 0.f;
 
-  for (int tile = (lo / WAVE) * WAVE; tile <= pos; tile += WAVE) {
-    const int c = tile + lane;
-    const bool valid = c >= lo && c <= pos;
-    float s = -INFINITY;
-    if (valid) {
-      const int64_t page = bt[c / page_size];
-      const T* kp = k_pages + ((page * nkv + g) * page_size + (c % page_size)) * hd;
-      float dot = 0.f;
-      for (int d = 0; d < hd; ++d) dot += q_s[d] * Num<T>::ld(kp + d);
-      s = dot * scale;
+  // The workgroup's tokens fall into runs of one request each (a prompt portion: one run; single tokens of several
+  // requests: a run each).  A run's tiles are loaded once and serve every wavefront of the run.
+  int run_begin = 0;
+  while (run_begin < tq && t0 + run_begin < tokens) {
+    const int run_entry = token_entry[t0 + run_begin];
+    int run_end = run_begin, lo_min = 0x7fffffff, pos_max = -1;
+    while (run_end < tq && t0 + run_end < tokens && token_entry[t0 + run_end] == run_entry) {
+      const int p = positions[t0 + run_end];
+      const int l0 = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+      lo_min = l0 < lo_min ? l0 : lo_min;
+      pos_max = p > pos_max ? p : pos_max;
+      ++run_end;
     }
-    const float m_new = fmaxf(m, wave_max(s));   // finite: every tile holds at least one valid key
-    const float p = valid ? expf(s - m_new) : 0.f;
-    const float alpha = expf(m - m_new);         // exp(-inf) = 0 on the first tile
-    l = l * alpha + wave_sum(p);
-    m = m_new;
-    __syncthreads();
-    p_s[lane] = p;
-    __syncthreads();
-    const int j0 = lo > tile ? lo - tile : 0;
-    const int j1 = pos - tile < WAVE - 1 ? pos - tile : WAVE - 1;
-#pragma unroll
-    for (int i = 0; i < MAX_HD / WAVE; ++i) {
-      const int d = lane + i * WAVE;
-      if (d < hd) {
-        float a = acc[i] * alpha;
-        for (int j = j0; j <= j1; ++j) {
-          const int cc = tile + j;
-          const int64_t page = bt[cc / page_size];
-          const T* vp = v_pages + ((page * nkv + g) * hd + d) * page_size + (cc % page_size);
-          a += p_s[j] * Num<T>::ld(vp);
-        }
-        acc[i] = a;
+    const bool mine = live && tl >= run_begin && tl < run_end;
+    const int32_t* bt = block_table + (int64_t)run_entry * table_width;
+    const int first_page = lo_min / page_size, last_page = pos_max / page_size;    // the pages that the run reads
+    for (int tile = (lo_min / WAVE) * WAVE; tile <= pos_max; tile += WAVE) {
+      __syncthreads();                            // the tile before has been read (and q_s is written)
+      if (threadIdx.x < WAVE) {
+        const int pi = (tile + (int)threadIdx.x) / page_size;
+        page_s[threadIdx.x] = (pi >= first_page && pi <= last_page) ? bt[pi] : -1;
       }
+      __syncthreads();
+      // keys: VEC dimensions of one key to a load, consecutive threads on consecutive dimensions
+      {
+        const int per_key = hd / VEC, nvec = WAVE * per_key;
+        for (int base = threadIdx.x; base < nvec; base += threads * GA_BATCH) {
+          VecLoad<T, VEC> r[GA_BATCH];
+          bool ok[GA_BATCH];
+#pragma unroll
+          for (int u = 0; u < GA_BATCH; ++u) {
+            const int v = base + u * threads;
+            const int j = v / per_key, d = (v - j * per_key) * VEC;
+            const int64_t page = v < nvec ? page_s[j] : -1;
+            ok[u] = page >= 0;
+            if (ok[u]) r[u].load(k_pages + ((page * nkv + g) * page_size + ((tile + j) % page_size)) * hd + d);
+          }
+#pragma unroll
+          for (int u = 0; u < GA_BATCH; ++u) {
+            const int v = base + u * threads;
+            const int j = v / per_key, d = (v - j * per_key) * VEC;
+            if (ok[u]) {
+#pragma unroll
+              for (int i = 0; i < VEC; ++i) k_s[j * (hd + 1) + d + i] = r[u].v[i];
+            }
+          }
+        }
+      }
+      // values: VEC keys of one dimension to a load (a page keeps the keys of a dimension side by side)
+      {
+        const int per_dim = WAVE / VEC, nvec = hd * per_dim;
+        for (int base = threadIdx.x; base < nvec; base += threads * GA_BATCH) {
+          VecLoad<T, VEC> r[GA_BATCH];
+          bool ok[GA_BATCH];
+#pragma unroll
+          for (int u = 0; u < GA_BATCH; ++u) {
+            const int v = base + u * threads;
+            const int d = v / per_dim, j = (v - d * per_dim) * VEC;
+            const int64_t page = v < nvec ? page_s[j] : -1;
+            ok[u] = page >= 0;
+            if (ok[u]) r[u].load(v_pages + ((page * nkv + g) * hd + d) * page_size + ((tile + j) % page_size));
+          }
+#pragma unroll
+          for (int u = 0; u < GA_BATCH; ++u) {
+            const int v = base + u * threads;
+            const int d = v / per_dim, j = (v - d * per_dim) * VEC;
+            if (ok[u]) {
+#pragma unroll
+              for (int i = 0; i < VEC; ++i) v_s[d * (WAVE + 1) + j + i] = r[u].v[i];
+            }
+          }
+        }
+      }
+      __syncthreads();
+      if (!mine || tile > pos || tile + WAVE - 1 < lo) continue;      // not a tile of this wavefront's token
+      const int c = tile + lane;
+      const bool valid = c >= lo && c <= pos;
+      float s = -INFINITY;
+      if (valid) {
+        const float* kr = k_s + lane * (hd + 1);
+        const float* qr = q_s + wave * hd;
+        float dot = 0.f;
+        for (int d = 0; d < hd; ++d) dot += qr[d] * kr[d];
+        s = dot * scale;
+      }
+      const float m_new = fmaxf(m, wave_max(s));   // finite: every tile holds at least one valid key
+      const float p = valid ? expf(s - m_new) : 0.f;
+      const float alpha = expf(m - m_new);         // exp(-inf) = 0 on the first tile
+      l = l * alpha + wave_sum(p);
+      m = m_new;
+      p_s[wave * WAVE + lane] = p;                 // read by this wavefront alone: LDS keeps a wavefront's order
+      __builtin_amdgcn_wave_barrier();
+      const int j0 = lo > tile ? lo - tile : 0;
+      const int j1 = pos - tile < WAVE - 1 ? pos - tile : WAVE - 1;
+      const float* pr = p_s + wave * WAVE;
+#pragma unroll
+      for (int i = 0; i < MAX_HD / WAVE; ++i) {
+        const int d = lane + i * WAVE;
+        if (d < hd) {
+          const float* vr = v_s + d * (WAVE + 1);
+          float a = acc[i] * alpha;
+          for (int j = j0; j <= j1; ++j) a += pr[j] * vr[j];
+          acc[i] = a;
+        }
+      }
+      __builtin_amdgcn_wave_barrier();
     }
+    run_begin = run_end;
   }
+  if (!live) return;
   T* op = out + t * out_stride + (int64_t)h * hd;
   const float inv = 1.0f / l;
 #pragma unroll
@@ -90,28 +203,47 @@ __global__ void paged_attention_generic_kernel(
 
 // out: [T, nh*hd] (row stride out_stride elements); q: rows of stride q_stride (the fused q|k|v
 // buffer); k_pages: [pages, nkv, page_size, hd]; v_pages: [pages, nkv, hd, page_size]; block_table: [entries, table_width];
-// token_entry, positions: [T].
+// token_entry, positions: [T].  tokens_per_workgroup: how many neighbouring tokens of the step share a workgroup and,
+// where they are of one request, its tiles of keys and values (1 for steps of single tokens; 0: the library chooses);
+// a token's result does not depend on it.
 extern "C" int ga_paged_attention_generic(void* out, int64_t out_stride, const void* q,
                                           int64_t q_stride, const void* k_pages,
                                           const void* v_pages, const void* block_table,
                                           int table_width, const void* token_entry,
                                           const void* positions, int tokens, int nh, int nkv, int hd,
                                           int page_size, int window, float scale, int is_bf16,
-                                          hipStream_t stream) {
+                                          int tokens_per_workgroup, hipStream_t stream) {
   if (tokens <= 0) return 0;
-  if (hd > MAX_HD || hd <= 0 || nkv <= 0 || nh % nkv != 0) return -1;
-  dim3 grid(tokens, nh), block(WAVE);
-  if (is_bf16)
-    hipLaunchKernelGGL(paged_attention_generic_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)out,
-                       out_stride, (const bf16_t*)q, q_stride, (const bf16_t*)k_pages,
-                       (const bf16_t*)v_pages, (const int32_t*)block_table, table_width,
-                       (const int32_t*)token_entry, (const int32_t*)positions, nh, nkv, hd,
-                       page_size, window, scale);
-  else
-    hipLaunchKernelGGL(paged_attention_generic_kernel<float>, grid, block, 0, stream, (float*)out,
-                       out_stride, (const float*)q, q_stride, (const float*)k_pages,
-                       (const float*)v_pages, (const int32_t*)block_table, table_width,
-                       (const int32_t*)token_entry, (const int32_t*)positions, nh, nkv, hd,
-                       page_size, window, scale);
+  if (hd > MAX_HD || hd <= 0 || nkv <= 0 || nh % nkv != 0 || page_size <= 0) return -1;
+  const int group = nh / nkv;
+  const int hpw = group < GA_MAX_WAVES ? group : GA_MAX_WAVES, head_blocks = (group + hpw - 1) / hpw;
+  int tq = tokens_per_workgroup > 0 ? tokens_per_workgroup : 4;
+  if (tq * hpw > GA_MAX_WAVES) tq = GA_MAX_WAVES / hpw;
+  if (tq > tokens) tq = tokens;
+  const int waves = tq * hpw;
+  const size_t lds = sizeof(float) * ((size_t)WAVE * (hd + 1) + (size_t)hd * (WAVE + 1) + (size_t)waves * hd + (size_t)waves * WAVE)
+                     + sizeof(int32_t) * WAVE;
+  if ((int64_t)nkv * head_blocks > 65535) return -3;
+  dim3 grid((tokens + tq - 1) / tq, nkv * head_blocks), block(WAVE * waves);
+  // 16-byte loads where a key's dimensions and a page's keys come in whole vectors at 16-byte addresses
+  const int vec = is_bf16 ? 8 : 4;
+  const bool wide = hd % vec == 0 && page_size % vec == 0 && WAVE % page_size == 0 &&
+                    ((uintptr_t)k_pages % 16 == 0) && ((uintptr_t)v_pages % 16 == 0);
+#define LAUNCH(TT, VV)                                                                                               \
+  do {                                                                                                               \
+    const void* fn = (const void*)paged_attention_generic_kernel<TT, VV>;                                            \
+    if (lds > 48 * 1024 && hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) \
+      return -4;                                                                                                     \
+    hipLaunchKernelGGL((paged_attention_generic_kernel<TT, VV>), grid, block, lds, stream, (TT*)out, out_stride,     \
+                       (const TT*)q, q_stride, (const TT*)k_pages, (const TT*)v_pages, (const int32_t*)block_table,  \
+                       table_width, (const int32_t*)token_entry, (const int32_t*)positions, tokens, nh, nkv, hd,      \
+                       page_size, window, scale, tq, hpw);                                                           \
+  } while (0)
+  if (is_bf16) {
+    if (wide) LAUNCH(bf16_t, 8); else LAUNCH(bf16_t, 1);
+  } else {
+    if (wide) LAUNCH(float, 4); else LAUNCH(float, 1);
+  }
+#undef LAUNCH
   return GA_CHECK_LAUNCH();
 }

@@ -210,10 +210,12 @@ def _check_attention_operands(q, k_pages, v_pages, block_table, token_entry, pos
 
 
 def paged_attention_generic(q, k_pages, v_pages, block_table, token_entry, positions, num_heads, num_kv_heads,
-                            head_dim, scale, window=None, out=None):
+                            head_dim, scale, window=None, out=None, tokens_per_workgroup=0):
     """q: rows of the fused projection ([T, >= nh*hd]; the first nh*hd columns are the queries).
     Token t attends to the keys of request token_entry[t] at positions
-    [max(0, p - window + 1), p], p = positions[t].  Returns [T, nh*hd]."""
+    [max(0, p - window + 1), p], p = positions[t].  Returns [T, nh*hd].  tokens_per_workgroup: how many neighbouring
+    tokens share a workgroup and (where they are of one request) its tiles of keys and values; 1 suits steps of
+    single tokens, 0 leaves it to the library; no token's result depends on it."""
     T = _check_attention_operands(q, k_pages, v_pages, block_table, token_entry, positions, num_heads,
                                   num_kv_heads, head_dim)
     _need(0 < head_dim <= 256,
@@ -227,7 +229,7 @@ def paged_attention_generic(q, k_pages, v_pages, block_table, token_entry, posit
         _ptr(out), _i64(out.stride(0)), _ptr(q), _i64(q.stride(0)), _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
         _i(block_table.shape[1]), _ptr(token_entry), _ptr(positions), _i(T), _i(num_heads), _i(num_kv_heads),
         _i(head_dim), _i(k_pages.shape[2]), _i(int(window) if window else 0), _f(scale), _i(_is_bf16(q.dtype)),
-        _stream()), "paged_attention_generic")
+        _i(int(tokens_per_workgroup)), _stream()), "paged_attention_generic")
     return out
 
 
@@ -612,4 +614,5 @@ def paged_attention(q, k_pages, v_pages, block_table, step, num_heads, num_kv_he
         return paged_attention_mfma(q, k_pages, v_pages, block_table, step, num_heads, num_kv_heads, head_dim, scale,
                                     window)
     return paged_attention_generic(q, k_pages, v_pages, block_table, step.token_entry, step.positions, num_heads,
-                                   num_kv_heads, head_dim, scale, window)
+                                   num_kv_heads, head_dim, scale, window,
+                                   tokens_per_workgroup=1 if step.max_q_len == 1 else 0)
