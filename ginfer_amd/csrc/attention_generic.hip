@@ -17,8 +17,8 @@
 // A workgroup holds the wavefronts of `tq` neighbouring tokens of the step and of all query heads of ONE kv head.
 // Tokens of the same request see the same keys, and so do the heads of a kv group: a tile of 64 keys and their values
 // comes from the pages ONCE per workgroup, with consecutive lanes on consecutive elements, into LDS (keys [key][dim],
-// values [dim][key], each row padded by one word so that neither a lane per key nor a lane per dimension meets a bank
-// twice), and every wavefront takes its operands from there.  What a wavefront computes, and in which order it adds,
+// values [dim][key], each row padded by four words so that rows stay 16-byte aligned and neither a lane per key nor a
+// lane per dimension meets a bank twice), and every wavefront takes its operands from there.  What a wavefront computes, and in which order it adds,
 // does not depend on what shares the workgroup with it: its dot products run over the dimensions in ascending order,
 // its sums over the keys of a tile likewise, and tiles follow each other in ascending order.
 #include "common.cuh"
@@ -26,6 +26,8 @@
 
 #define MAX_HD 256
 #define GA_MAX_WAVES 16
+#define KPAD 4              // floats that pad a row of keys in LDS: rows stay 16-byte aligned, lanes on different banks
+#define VS (WAVE + 4)       // a row of values in LDS, in floats
 
 // VEC elements (16 bytes) of T per load where head size and page size allow it, else one
 template <typename T, int VEC>
@@ -47,7 +49,7 @@ struct VecLoad {
   }
 };
 
-#define GA_BATCH 4         // loads of a thread that are under way at a time
+#define GA_BATCH 4         // loads of keys, and as many of values, that a thread has under way at a time
 
 template <typename T, int VEC>
 __global__ __launch_bounds__(64 * GA_MAX_WAVES) void paged_attention_generic_kernel(
@@ -59,9 +61,10 @@ __global__ __launch_bounds__(64 * GA_MAX_WAVES) void paged_attention_generic_ker
   extern __shared__ float lds[];
   const int group = nh / nkv, head_blocks = (group + hpw - 1) / hpw;     // hpw heads of a kv group to a workgroup
   const int waves = tq * hpw, threads = waves * WAVE;
-  float* k_s = lds;                              // [64][hd + 1]
-  float* v_s = k_s + WAVE * (hd + 1);            // [hd][64 + 1]
-  float* q_s = v_s + hd * (WAVE + 1);            // [waves][hd]
+  const int ks = hd + KPAD;                      // a key's row in LDS, in floats
+  float* k_s = lds;                              // [64][hd + KPAD]
+  float* v_s = k_s + WAVE * ks;                  // [hd][64 + VPAD]
+  float* q_s = v_s + hd * VS;                    // [waves][hd]
   float* p_s = q_s + waves * hd;                 // [waves][64]
   int32_t* page_s = reinterpret_cast<int32_t*>(p_s + waves * WAVE);     // [64]: the page of every key of the tile, or -1
   const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
@@ -98,60 +101,57 @@ __global__ __launch_bounds__(64 * GA_MAX_WAVES) void paged_attention_generic_ker
     const bool mine = live && tl >= run_begin && tl < run_end;
     const int32_t* bt = block_table + (int64_t)run_entry * table_width;
     const int first_page = lo_min / page_size, last_page = pos_max / page_size;    // the pages that the run reads
+    // the page of every key of a tile, asked for one tile ahead
+    auto tile_page = [&](int tile) -> int32_t {
+      if (threadIdx.x >= WAVE || tile > pos_max) return -1;
+      const int pi = (tile + (int)threadIdx.x) / page_size;
+      return (pi >= first_page && pi <= last_page) ? bt[pi] : -1;
+    };
+    int32_t my_page = tile_page((lo_min / WAVE) * WAVE);
+    const int per_key = hd / VEC, per_dim = WAVE / VEC, nvec = WAVE * per_key;       // as many vectors of values as of keys
     for (int tile = (lo_min / WAVE) * WAVE; tile <= pos_max; tile += WAVE) {
       __syncthreads();                            // the tile before has been read (and q_s is written)
-      if (threadIdx.x < WAVE) {
-        const int pi = (tile + (int)threadIdx.x) / page_size;
-        page_s[threadIdx.x] = (pi >= first_page && pi <= last_page) ? bt[pi] : -1;
-      }
+      if (threadIdx.x < WAVE) page_s[threadIdx.x] = my_page;
       __syncthreads();
-      // keys: VEC dimensions of one key to a load, consecutive threads on consecutive dimensions
-      {
-        const int per_key = hd / VEC, nvec = WAVE * per_key;
-        for (int base = threadIdx.x; base < nvec; base += threads * GA_BATCH) {
-          VecLoad<T, VEC> r[GA_BATCH];
-          bool ok[GA_BATCH];
+      my_page = tile_page(tile + WAVE);           // on its way while this tile is loaded and multiplied
+      // keys: VEC dimensions of one key to a load, consecutive threads on consecutive dimensions; values: VEC keys of
+      // one dimension to a load (a page keeps the keys of a dimension side by side).  A batch of both is under way
+      // before the first of it is put into LDS.
+      for (int base = threadIdx.x; base < nvec; base += threads * GA_BATCH) {
+        VecLoad<T, VEC> rk[GA_BATCH], rv[GA_BATCH];
+        bool okk[GA_BATCH], okv[GA_BATCH];
 #pragma unroll
-          for (int u = 0; u < GA_BATCH; ++u) {
-            const int v = base + u * threads;
-            const int j = v / per_key, d = (v - j * per_key) * VEC;
-            const int64_t page = v < nvec ? page_s[j] : -1;
-            ok[u] = page >= 0;
-            if (ok[u]) r[u].load(k_pages + ((page * nkv + g) * page_size + ((tile + j) % page_size)) * hd + d);
-          }
+        for (int u = 0; u < GA_BATCH; ++u) {
+          const int v = base + u * threads;
+          const int j = v / per_key, d = (v - j * per_key) * VEC;
+          const int64_t page = v < nvec ? page_s[j] : -1;
+          okk[u] = page >= 0;
+          if (okk[u]) rk[u].load(k_pages + ((page * nkv + g) * page_size + ((tile + j) % page_size)) * hd + d);
+        }
 #pragma unroll
-          for (int u = 0; u < GA_BATCH; ++u) {
-            const int v = base + u * threads;
-            const int j = v / per_key, d = (v - j * per_key) * VEC;
-            if (ok[u]) {
+        for (int u = 0; u < GA_BATCH; ++u) {
+          const int v = base + u * threads;
+          const int d = v / per_dim, j = (v - d * per_dim) * VEC;
+          const int64_t page = v < nvec ? page_s[j] : -1;
+          okv[u] = page >= 0;
+          if (okv[u]) rv[u].load(v_pages + ((page * nkv + g) * hd + d) * page_size + ((tile + j) % page_size));
+        }
 #pragma unroll
-              for (int i = 0; i < VEC; ++i) k_s[j * (hd + 1) + d + i] = r[u].v[i];
-            }
+        for (int u = 0; u < GA_BATCH; ++u) {
+          const int v = base + u * threads;
+          const int j = v / per_key, d = (v - j * per_key) * VEC;
+          if (okk[u]) {
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) k_s[j * ks + d + i] = rk[u].v[i];
           }
         }
-      }
-      // values: VEC keys of one dimension to a load (a page keeps the keys of a dimension side by side)
-      {
-        const int per_dim = WAVE / VEC, nvec = hd * per_dim;
-        for (int base = threadIdx.x; base < nvec; base += threads * GA_BATCH) {
-          VecLoad<T, VEC> r[GA_BATCH];
-          bool ok[GA_BATCH];
 #pragma unroll
-          for (int u = 0; u < GA_BATCH; ++u) {
-            const int v = base + u * threads;
-            const int d = v / per_dim, j = (v - d * per_dim) * VEC;
-            const int64_t page = v < nvec ? page_s[j] : -1;
-            ok[u] = page >= 0;
-            if (ok[u]) r[u].load(v_pages + ((page * nkv + g) * hd + d) * page_size + ((tile + j) % page_size));
-          }
+        for (int u = 0; u < GA_BATCH; ++u) {
+          const int v = base + u * threads;
+          const int d = v / per_dim, j = (v - d * per_dim) * VEC;
+          if (okv[u]) {
 #pragma unroll
-          for (int u = 0; u < GA_BATCH; ++u) {
-            const int v = base + u * threads;
-            const int d = v / per_dim, j = (v - d * per_dim) * VEC;
-            if (ok[u]) {
-#pragma unroll
-              for (int i = 0; i < VEC; ++i) v_s[d * (WAVE + 1) + j + i] = r[u].v[i];
-            }
+            for (int i = 0; i < VEC; ++i) v_s[d * VS + j + i] = rv[u].v[i];
           }
         }
       }
@@ -161,10 +161,21 @@ __global__ __launch_bounds__(64 * GA_MAX_WAVES) void paged_attention_generic_ker
       const bool valid = c >= lo && c <= pos;
       float s = -INFINITY;
       if (valid) {
-        const float* kr = k_s + lane * (hd + 1);
+        const float* kr = k_s + lane * ks;
         const float* qr = q_s + wave * hd;
         float dot = 0.f;
-        for (int d = 0; d < hd; ++d) dot += qr[d] * kr[d];
+        int d = 0;
+        if ((hd & 3) == 0) {                      // four dimensions to an LDS read; the sum keeps its order
+          for (; d < hd; d += 4) {
+            const float4 qq = *reinterpret_cast<const float4*>(qr + d);
+            const float4 kk = *reinterpret_cast<const float4*>(kr + d);
+            dot = __builtin_fmaf(qq.x, kk.x, dot);
+            dot = __builtin_fmaf(qq.y, kk.y, dot);
+            dot = __builtin_fmaf(qq.z, kk.z, dot);
+            dot = __builtin_fmaf(qq.w, kk.w, dot);
+          }
+        }
+        for (; d < hd; ++d) dot = __builtin_fmaf(qr[d], kr[d], dot);
         s = dot * scale;
       }
       const float m_new = fmaxf(m, wave_max(s));   // finite: every tile holds at least one valid key
@@ -181,9 +192,19 @@ __global__ __launch_bounds__(64 * GA_MAX_WAVES) void paged_attention_generic_ker
       for (int i = 0; i < MAX_HD / WAVE; ++i) {
         const int d = lane + i * WAVE;
         if (d < hd) {
-          const float* vr = v_s + d * (WAVE + 1);
+          const float* vr = v_s + d * VS;
           float a = acc[i] * alpha;
-          for (int j = j0; j <= j1; ++j) a += pr[j] * vr[j];
+          int j = j0;
+          for (; j <= j1 && (j & 3); ++j) a = __builtin_fmaf(pr[j], vr[j], a);
+          for (; j + 3 <= j1; j += 4) {            // four keys to an LDS read, added in ascending order
+            const float4 pp = *reinterpret_cast<const float4*>(pr + j);
+            const float4 vv = *reinterpret_cast<const float4*>(vr + j);
+            a = __builtin_fmaf(pp.x, vv.x, a);
+            a = __builtin_fmaf(pp.y, vv.y, a);
+            a = __builtin_fmaf(pp.z, vv.z, a);
+            a = __builtin_fmaf(pp.w, vv.w, a);
+          }
+          for (; j <= j1; ++j) a = __builtin_fmaf(pr[j], vr[j], a);
           acc[i] = a;
         }
       }
@@ -221,7 +242,7 @@ extern "C" int ga_paged_attention_generic(void* out, int64_t out_stride, const v
   if (tq * hpw > GA_MAX_WAVES) tq = GA_MAX_WAVES / hpw;
   if (tq > tokens) tq = tokens;
   const int waves = tq * hpw;
-  const size_t lds = sizeof(float) * ((size_t)WAVE * (hd + 1) + (size_t)hd * (WAVE + 1) + (size_t)waves * hd + (size_t)waves * WAVE)
+  const size_t lds = sizeof(float) * ((size_t)WAVE * (hd + KPAD) + (size_t)hd * VS + (size_t)waves * hd + (size_t)waves * WAVE)
                      + sizeof(int32_t) * WAVE;
   if ((int64_t)nkv * head_blocks > 65535) return -3;
   dim3 grid((tokens + tq - 1) / tq, nkv * head_blocks), block(WAVE * waves);
