@@ -21,6 +21,7 @@ import torch
 from ..cache import CacheManager
 from ..config import config_from_folder
 from ..kernels import build
+from ..kernels.tuning import TUNING
 from ..parts.base import KVCacheSpec, StateSpec
 from ..parts.model import build_model, StepContext, KVView, StateView
 from ..weights import load_weights, bind_random_weights
@@ -83,7 +84,7 @@ class ModelRunner:
         # be twice the step's own: with some 1e15 operations a second that is rows * weights < ~1.5e12 (512 rows for a
         # 1.5B model, 128 for a 7B one, none for a 72B one)
         weights = sum(int(np.prod(ws.shape)) for ws in self.model.weight_specs().values())
-        self._padded_max_rows = min(MIXED_GRAPH_MAX_TOKENS, int(1.5e12 // max(weights, 1)))
+        self._padded_max_rows = min(TUNING.mixed_graph_max_tokens, int(TUNING.padded_rows_times_weights // max(weights, 1)))
         # how steps ran: launched kernel by kernel, replayed as a recorded decode step, replayed as a recorded step
         # with prompt portions; and how many steps were recorded
         self.counts = dict(launched=0, replayed_decode=0, replayed_padded=0, recorded=0, recording_seconds=0.0)
@@ -534,7 +535,6 @@ def _context_bucket(max_kv):
 GRAPH_MAX_ROWS = 256     # decode batches up to this many requests are recorded
 GRAPH_AFTER = 2          # a batch shape is recorded the second time it is seen
 GRAPH_KEEP = 128         # recorded shapes kept at a time (least recently used goes first)
-MIXED_GRAPH_MAX_TOKENS = 512    # steps with prompt portions are recorded up to this many token rows (padding included)
 
 
 class _StepBuffers:

@@ -10,6 +10,7 @@ import ctypes
 import torch
 
 from . import build
+from .tuning import TUNING
 
 _vp = ctypes.c_void_p
 _i = ctypes.c_int
@@ -480,13 +481,6 @@ def qkv_rope_skinny(x, w, bias, positions, cos, sin, slot_mapping, k_pages, v_pa
 # ----------------------------------------------------------------------------- attention on the matrix cores
 
 MFMA_HEAD_DIMS = tuple(range(16, 257, 16))
-_DECODE_TARGET_WORKGROUPS = 256       # four wavefronts each, one workgroup per compute unit: measured best on MI355X
-_MIN_SPLIT_KEYS = 128                 # one tile of 32 keys for each wavefront of a workgroup
-_MAX_SPLITS = 256
-PREFILL_WIDE_TILES_FROM = 1024        # tokens in a step from which prompt rows go 32 to a wavefront
-# workgroups that fill the chip: heads of a kv group go side by side into a prefill workgroup only while the step
-# still makes this many workgroups
-PREFILL_FILL_WORKGROUPS = 256
 
 
 def attention_mfma_supported(dtype, head_dim, page_size):
@@ -512,7 +506,7 @@ def plan_rows(q_len, q_start, tile_rows):
     return decode_rows, decode_pos, decode_entries, tiles
 
 
-PLAN_TILE_ROWS = 16       # rows of a prompt portion per wavefront in steps of fewer than PREFILL_WIDE_TILES_FROM tokens
+PLAN_TILE_ROWS = 16       # rows of a prompt portion per wavefront in steps of fewer than TUNING.prefill_wide_tiles_from tokens
 
 
 def _attention_plan(step, tile_rows, device):
@@ -556,7 +550,8 @@ def _decode_splits(plan, window, nkv, head_blocks):
             lo = max(0, pos - window + 1) if window else 0
             span = max(span, pos + 1 - (lo // 32) * 32)
     per_split = plan["n_decode"] * nkv * head_blocks
-    splits = max(1, min(_DECODE_TARGET_WORKGROUPS // max(per_split, 1), -(-span // _MIN_SPLIT_KEYS), _MAX_SPLITS))
+    splits = max(1, min(TUNING.decode_target_workgroups // max(per_split, 1), -(-span // TUNING.decode_min_split_keys),
+                        TUNING.decode_max_splits))
     split_keys = -(-(-(-span // splits)) // 32) * 32
     return split_keys, -(-span // split_keys)
 
@@ -580,7 +575,7 @@ def paged_attention_mfma(q, k_pages, v_pages, block_table, step, num_heads, num_
     lib = build.load("attention_mfma", {"HEAD_DIM": head_dim})
     _need(lib.ga_attn_head_dim() == head_dim, "attention library was built for another head size")
     # rows of a prompt portion per wavefront: 32 where the kernel has it and the step is long, else 16
-    wide = T >= PREFILL_WIDE_TILES_FROM
+    wide = T >= TUNING.prefill_wide_tiles_from
     tile_rows = lib.ga_attn_prefill_max_tile_rows() if wide else 16
     plan = _attention_plan(step, tile_rows, q.device)
     _need(sum(step.host_q_len) == T, "the step's entries do not add up to its tokens")
@@ -602,7 +597,7 @@ def paged_attention_mfma(q, k_pages, v_pages, block_table, step, num_heads, num_
         _check(lib.ga_attn_prefill(
             _ptr(out), _i64(out.stride(0)), _ptr(q), _i64(q.stride(0)), _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
             _i(block_table.shape[1]), _ptr(plan["tiles"]), _i(plan["n_tiles"]), _i(tile_rows), _i(num_heads), _i(num_kv_heads),
-            _i(page_size), _i(w), _f(scale), _i(PREFILL_FILL_WORKGROUPS), _stream()), "attn_prefill")
+            _i(page_size), _i(w), _f(scale), _i(TUNING.prefill_fill_workgroups), _stream()), "attn_prefill")
     return out
 
 

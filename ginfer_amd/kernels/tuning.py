@@ -1,0 +1,73 @@
+"""Where a step's work goes: every threshold by which a part or a kernel dispatcher chooses between two ways of doing
+the same thing lives here, in one table, with what it was measured on.  They decide speed only, never results (beyond
+rounding in bfloat16): any setting gives right answers.  The values were measured on one MI355X (256 compute units) at
+the layer sizes of a 1.5B and a 7B model; a model of other sizes may want others:
+
+    from ginfer_amd.kernels.tuning import TUNING
+    TUNING.library_from_rows = 32                       # for the process
+    GINFER_AMD_TUNING='{"library_from_rows": 32}'       # or from the environment, as JSON
+
+Nothing else in the package holds such a number.
+"""
+import json
+import os
+from dataclasses import dataclass, fields
+
+
+@dataclass
+class Tuning:
+    # ---- bfloat16 products (parts/linear.py).  Up to 64 rows the package's weight-streaming kernel can take a product,
+    # beyond that only the BLAS library.
+    # From more rows than this, products with at least `library_min_out_features` output columns (gate-up, the head) go
+    # to the library: the streaming kernel re-reads the rows once per 64 columns.
+    library_from_rows: int = 16
+    library_min_out_features: int = 4096
+    # With more than 16 rows and at least this many output columns the streaming kernel takes four tiles of the weight
+    # per wavefront, which halves the re-reading of the rows.
+    four_tiles_min_out_features: int = 4096
+    # A product whose consumer can add partial sums splits a K of at least `split_k_min_in_features` over workgroups
+    # (a shorter K only in two parts); at most `max_split_k_parts` parts.
+    split_k_from: int = 4096
+    split_k_min_in_features: int = 1024
+    max_split_k_parts: int = 16
+    # A product that folds the norm after it cannot split K over workgroups.  With a K of `split_k_from` or more it still
+    # folds up to this many rows (packed tiles fill the chip), and beyond only if its full tiles make at least
+    # `fold_min_workgroups` workgroups.
+    fold_long_k_up_to_rows: int = 8
+    fold_min_workgroups: int = 192
+    # The library's product of 65 to 256 rows with a K of at least `split_k_from` and at most this many output columns
+    # is cut into pieces of K side by side (a batched product): one product leaves a quarter of the chip idle.
+    library_split_min_rows: int = 65
+    library_split_max_rows: int = 256
+    library_split_max_out_features: int = 4096
+    # The gate-up product lies transposed (weights as the library's first operand) for row counts from this on that
+    # are a multiple of it: the library's tiles then fit the rows.
+    transposed_gate_up_row_multiple: int = 256
+    # ---- the fused q|k|v projection + rotation + cache write (parts/attention.py): from more rows than this and a K
+    # of at least that, the library's product followed by the rotation kernel is faster (the fused kernel cannot split K).
+    fused_qkv_up_to_rows: int = 16
+    fused_qkv_unless_in_features: int = 3072
+    # ---- attention on the matrix cores (kernels/ops.py)
+    decode_target_workgroups: int = 256      # key splits are chosen so that a decode step makes about this many workgroups
+    decode_min_split_keys: int = 128         # one tile of 32 keys for each wavefront of a workgroup
+    decode_max_splits: int = 256
+    prefill_wide_tiles_from: int = 1024      # tokens in a step from which prompt rows go 32 to a wavefront
+    # heads of a kv group go side by side into a prefill workgroup only while the step still makes this many workgroups
+    prefill_fill_workgroups: int = 256
+    # ---- recorded steps (engine/runner.py): steps with prompt portions are laid into recorded steps of padded sizes up
+    # to `mixed_graph_max_tokens` rows, fewer for large models: padding pays while rows x weights stays under what the
+    # device does in the time the host needs to launch a step kernel by kernel.
+    mixed_graph_max_tokens: int = 512
+    padded_rows_times_weights: float = 1.5e12
+
+    def update(self, values):
+        known = {f.name: f.type for f in fields(self)}
+        for k, v in values.items():
+            if k not in known:
+                raise KeyError("no tuning value %r (known: %s)" % (k, ", ".join(sorted(known))))
+            setattr(self, k, type(getattr(self, k))(v))
+
+
+TUNING = Tuning()
+if os.environ.get("GINFER_AMD_TUNING"):
+    TUNING.update(json.loads(os.environ["GINFER_AMD_TUNING"]))

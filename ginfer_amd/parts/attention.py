@@ -4,6 +4,7 @@ import math
 import torch
 
 from ..kernels import ops
+from ..kernels.tuning import TUNING
 from ..weights.loader import WeightSpec
 from .base import Part, KVCacheSpec
 from .linear import linear, linear_into_norm
@@ -15,7 +16,7 @@ def _library_then_rotation_is_faster(rows, in_features):
     MI355X at a 7B model's sizes (K 3584, 4608 outputs): from 17 rows on the BLAS library's product followed by
     the rotation kernel is faster (32 rows: 17.6 us against 20.6; 64 rows: 23.4 against 28.1); at a 1.5B model's
     (K 1536) the fused kernel stays ahead or level up to 64 rows."""
-    return rows > 16 and in_features >= 3072
+    return rows > TUNING.fused_qkv_up_to_rows and in_features >= TUNING.fused_qkv_unless_in_features
 
 
 @register_mixer("attention")

@@ -9,14 +9,7 @@ these calls are checked bit for bit against eager steps in the tests."""
 import torch
 
 from ..kernels import ops
-
-
-# from this many input features on, a product is "long": a folded norm gives way to a split over workgroups
-SPLIT_K_FROM = 4096
-MAX_SPLIT_K_PARTS = 16
-# a folded norm keeps K within a workgroup; measured on MI355X, a product with a long K and fewer than 192
-# workgroups of full tiles still gains from folding while its tiles are packed (up to 8 rows)
-FOLD_LONG_K_UP_TO_ROWS = 8
+from ..kernels.tuning import TUNING      # every threshold below is a field of this table, with what it was measured on
 
 
 def linear(x, weight, bias=None, out_dtype=None, parts_ok=False):
@@ -32,11 +25,11 @@ def linear(x, weight, bias=None, out_dtype=None, parts_ok=False):
         # 16-row tile of W per wavefront streams best; beyond, four tiles halve the re-reading of x; a
         # long K is split over workgroups where the consumer can add the parts
         many = x.shape[0] > 16
-        if parts_ok and out_dtype is None and x.shape[1] >= 1024:
+        if parts_ok and out_dtype is None and x.shape[1] >= TUNING.split_k_min_in_features:
             nt, splits = _split_plan(x.shape[0], weight.shape[0], x.shape[1])
             if splits > 1:
                 return ops.gemm_skinny(x, weight, bias, out_dtype=torch.float32, nt=nt, grid_splits=splits)
-        return ops.gemm_skinny(x, weight, bias, out_dtype=out_dtype, nt=4 if (many and weight.shape[0] >= 4096) else 1)
+        return ops.gemm_skinny(x, weight, bias, out_dtype=out_dtype, nt=4 if (many and weight.shape[0] >= TUNING.four_tiles_min_out_features) else 1)
     if parts_ok and out_dtype is None and bias is None:
         parts = _library_split(x.shape[0], weight.shape[0], x.shape[1])
         if parts > 1:
@@ -65,11 +58,11 @@ def _split_plan(rows, out_features, in_features):
     23 us).  That gives 10 parts at 64 rows and 5 at 8 for the 1.5B shape's down projection, 4 for the 7B
     shape's; a product with a short K and few columns keeps 2 parts."""
     steps = -(-in_features // 64)
-    cap = max(1, min(MAX_SPLIT_K_PARTS, steps // 8))       # parts that leave every wavefront a step
+    cap = max(1, min(TUNING.max_split_k_parts, steps // 8))       # parts that leave every wavefront a step
     tiles4 = -(-out_features // 64)
     if rows > 16 and tiles4 * cap >= 192:
         return 4, _nearest_divisor(steps, 256.0 / tiles4, cap)
-    if in_features < SPLIT_K_FROM:
+    if in_features < TUNING.split_k_from:
         return 1, min(2, cap)
     return 1, _nearest_divisor(steps, 512.0 / -(-out_features // 16), cap)
 
@@ -86,17 +79,15 @@ def _nearest_divisor(n, target, cap):
 def _library_is_faster(rows, out_features):
     """Measured on MI355X: from 17 rows on, products with a wide output (the gate-up product, the head) run
     faster in the BLAS library than in the weight-streaming kernel, which re-reads x once per 64 outputs."""
-    return rows > LIBRARY_FROM_ROWS and out_features >= 4096
-
-
-LIBRARY_FROM_ROWS = 16
+    return rows > TUNING.library_from_rows and out_features >= TUNING.library_min_out_features
 
 
 def _library_split(rows, out_features, in_features):
     """Into how many pieces of K the library's product is cut.  Measured on MI355X: with up to 256 rows, few
     output columns and a long K (the down projection of a busy decode step) the library's single product leaves
     a quarter of the chip idle and takes 31 us where five pieces side by side take 23."""
-    if not (64 < rows <= 256 and in_features >= SPLIT_K_FROM and out_features <= 4096):
+    if not (TUNING.library_split_min_rows <= rows <= TUNING.library_split_max_rows and in_features >= TUNING.split_k_from
+            and out_features <= TUNING.library_split_max_out_features):
         return 1
     for parts in (5, 4, 2):
         if in_features % parts == 0 and (in_features // parts) % 8 == 0:
@@ -111,7 +102,8 @@ def linear_into_norm(x, weight, bias, residual, norm):
     root-mean-square norm with a gain): the caller then takes the ordinary way."""
     if not getattr(norm, "foldable", False) or x.dtype != torch.bfloat16 or residual is None:
         return None
-    if x.shape[1] >= SPLIT_K_FROM and x.shape[0] > FOLD_LONG_K_UP_TO_ROWS and weight.shape[0] < 16 * 192:
+    if (x.shape[1] >= TUNING.split_k_from and x.shape[0] > TUNING.fold_long_k_up_to_rows
+            and weight.shape[0] < 16 * TUNING.fold_min_workgroups):
         return None      # a long K and few columns: the split over workgroups is worth more than the folded norm
     if not ops.folded_norm_supported(x, weight, residual, norm.weight):
         return None
@@ -137,5 +129,6 @@ def _transposed_product_is_faster(x, weight):
     256 (the portions that a token budget of 2,048 cuts) the library's tiles fit the rows when the weights are its
     first operand: level to 15 % faster (2,048 rows of the 1.5B shape: 115 -> 98 us; 256 rows, a decode step of 256
     requests: 3 to 8 %); with other row counts it is up to 20 % slower, so they keep the usual product."""
-    return (x.dtype == torch.bfloat16 and x.shape[0] >= 256 and x.shape[0] % 256 == 0 and x.is_contiguous()
+    every = TUNING.transposed_gate_up_row_multiple
+    return (x.dtype == torch.bfloat16 and x.shape[0] >= every and x.shape[0] % every == 0 and x.is_contiguous()
             and weight.shape[0] % 16 == 0 and x.shape[1] % 8 == 0)

@@ -129,3 +129,22 @@ def test_header_declares_every_entry_point_as_it_is_defined():
     assert defined and set(defined) == set(declared), (sorted(set(defined) ^ set(declared)))
     for name in defined:
         assert defined[name] == declared[name], "%s: defined %s, declared %s" % (name, defined[name], declared[name])
+
+
+def test_dispatch_thresholds_live_in_one_table():
+    import os
+    """Every threshold that chooses between two ways of doing the same work is a field of kernels/tuning.py; values can
+    be set for the process or from the environment, unknown names are refused."""
+    import json
+    import subprocess
+    import sys
+    from ginfer_amd.kernels.tuning import Tuning, TUNING
+    t = Tuning()
+    t.update({"library_from_rows": 32, "padded_rows_times_weights": 2e12})
+    assert t.library_from_rows == 32 and t.padded_rows_times_weights == 2e12 and TUNING.library_from_rows == 16
+    with pytest.raises(KeyError, match="no tuning value"):
+        t.update({"library_from_row": 1})
+    out = subprocess.run([sys.executable, "-c", "from ginfer_amd.kernels.tuning import TUNING; print(TUNING.decode_max_splits)"],
+                         env=dict(os.environ, GINFER_AMD_TUNING=json.dumps({"decode_max_splits": 64})), capture_output=True,
+                         text=True, cwd=os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+    assert out.stdout.strip() == "64", out.stderr

@@ -407,7 +407,7 @@ MFMA_SEQS = ATTN_SEQS + [[(1, 31), (1, 32), (1, 33), (1, 64), (1, 65)], [(31, 31
 @pytest.mark.parametrize("seqs", MFMA_SEQS)
 def test_paged_attention_mfma(nh, nkv, hd, seqs, wide, monkeypatch):
     from ginfer_amd.kernels import ops
-    monkeypatch.setattr(ops, "PREFILL_WIDE_TILES_FROM", 0 if wide else 1 << 30)    # 32 or 16 rows to a wavefront
+    monkeypatch.setattr(ops.TUNING, "prefill_wide_tiles_from", 0 if wide else 1 << 30)    # 32 or 16 rows to a wavefront
     if wide and max(q for q, _ in seqs) == 1:
         pytest.skip("no prompt rows in this case")
     if sum(kv for _, kv in seqs) * nkv * hd > 3e6 and (nh, nkv, hd) not in ((12, 2, 128), (6, 1, 32)):
@@ -430,8 +430,8 @@ def test_paged_attention_mfma_heads_side_by_side(nh, nkv, hd, seqs, wide, monkey
     groups of 2 to 7 heads with one or two streams of tiles, page sizes of 8 to 64, portions that start inside a
     sequence), beside a head size that it is not built for."""
     from ginfer_amd.kernels import ops
-    monkeypatch.setattr(ops, "PREFILL_WIDE_TILES_FROM", 0 if wide else 1 << 30)
-    monkeypatch.setattr(ops, "PREFILL_FILL_WORKGROUPS", 1)
+    monkeypatch.setattr(ops.TUNING, "prefill_wide_tiles_from", 0 if wide else 1 << 30)
+    monkeypatch.setattr(ops.TUNING, "prefill_fill_workgroups", 1)
     for ps in (16, 8, 32, 64):
         a, ref, _ = _paged_case(seqs, nh, nkv, hd, ps, torch.bfloat16, seed=hd + ps)
         out = ops.paged_attention_mfma(a["q"], a["k_pages"], a["v_pages"], a["block_table"], _Step(seqs, a), nh, nkv, hd,
@@ -443,8 +443,8 @@ def test_paged_attention_mfma_heads_side_by_side(nh, nkv, hd, seqs, wide, monkey
 @pytest.mark.parametrize("window", [1, 5, 16, 40, 64, 100])
 def test_paged_attention_mfma_heads_side_by_side_window(window, wide, monkeypatch):
     from ginfer_amd.kernels import ops
-    monkeypatch.setattr(ops, "PREFILL_WIDE_TILES_FROM", 0 if wide else 1 << 30)
-    monkeypatch.setattr(ops, "PREFILL_FILL_WORKGROUPS", 1)
+    monkeypatch.setattr(ops.TUNING, "prefill_wide_tiles_from", 0 if wide else 1 << 30)
+    monkeypatch.setattr(ops.TUNING, "prefill_fill_workgroups", 1)
     nh, nkv, hd = 6, 2, 64
     seqs = [(30, 90), (7, 7), (50, 130), (200, 330), (1, 2000)]
     for ps in (16, 8):
@@ -459,8 +459,8 @@ def test_paged_attention_mfma_heads_side_by_side_window(window, wide, monkeypatc
                                    "last", "window_edge", "behind_window"])
 def test_paged_attention_mfma_heads_side_by_side_finds_one_far_key(where, wide, monkeypatch):
     from ginfer_amd.kernels import ops
-    monkeypatch.setattr(ops, "PREFILL_WIDE_TILES_FROM", 0 if wide else 1 << 30)
-    monkeypatch.setattr(ops, "PREFILL_FILL_WORKGROUPS", 1)
+    monkeypatch.setattr(ops.TUNING, "prefill_wide_tiles_from", 0 if wide else 1 << 30)
+    monkeypatch.setattr(ops.TUNING, "prefill_fill_workgroups", 1)
     nh, nkv, hd, ps = 6, 2, 64, 16
     kv = 300
     window = 100 if "window" in where else None
@@ -483,7 +483,7 @@ def test_paged_attention_mfma_heads_side_by_side_finds_one_far_key(where, wide, 
 def test_paged_attention_mfma_every_head_size(hd, wide, monkeypatch):
     """Head sizes in steps of 16 up to 256, each with a group of 3 heads: portions of prompts beside single tokens."""
     from ginfer_amd.kernels import ops
-    monkeypatch.setattr(ops, "PREFILL_WIDE_TILES_FROM", 0 if wide else 1 << 30)
+    monkeypatch.setattr(ops.TUNING, "prefill_wide_tiles_from", 0 if wide else 1 << 30)
     seqs = [(1, 130), (37, 101), (64, 64), (1, 17), (2, 300)]
     a, ref, _ = _paged_case(seqs, 6, 2, hd, 16, torch.bfloat16, seed=hd)
     out = ops.paged_attention_mfma(a["q"], a["k_pages"], a["v_pages"], a["block_table"], _Step(seqs, a), 6, 2, hd,
@@ -495,7 +495,7 @@ def test_paged_attention_mfma_every_head_size(hd, wide, monkeypatch):
 @pytest.mark.parametrize("window", [1, 5, 16, 40, 64, 100])
 def test_paged_attention_mfma_window(window, wide, monkeypatch):
     from ginfer_amd.kernels import ops
-    monkeypatch.setattr(ops, "PREFILL_WIDE_TILES_FROM", 0 if wide else 1 << 30)
+    monkeypatch.setattr(ops.TUNING, "prefill_wide_tiles_from", 0 if wide else 1 << 30)
     nh, nkv, hd, ps = 6, 3, 48, 16
     seqs = [(1, 200), (30, 90), (7, 7), (1, window), (1, window + 1), (50, 130), (1, 2000)]
     a, ref, _ = _paged_case(seqs, nh, nkv, hd, ps, torch.bfloat16, seed=window, window=window)
@@ -509,7 +509,7 @@ def test_paged_attention_mfma_window(window, wide, monkeypatch):
                                    "last", "window_edge", "behind_window"])
 def test_paged_attention_mfma_finds_one_far_key(where, wide, monkeypatch):
     from ginfer_amd.kernels import ops
-    monkeypatch.setattr(ops, "PREFILL_WIDE_TILES_FROM", 0 if wide else 1 << 30)
+    monkeypatch.setattr(ops.TUNING, "prefill_wide_tiles_from", 0 if wide else 1 << 30)
     nh, nkv, hd, ps = 4, 2, 32, 16
     kv = 300
     window = 100 if "window" in where else None

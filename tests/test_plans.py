@@ -8,8 +8,8 @@ def test_parts_divide_the_steps_of_k_and_leave_every_wavefront_work():
             for k in (64, 520, 1536, 3584, 8960, 18944, 29568):
                 nt, parts = L._split_plan(rows, n, k)
                 steps = -(-k // 64)
-                assert nt in (1, 4) and 1 <= parts <= L.MAX_SPLIT_K_PARTS
-                assert parts == 1 or (steps % parts == 0 or k < L.SPLIT_K_FROM) and parts * 8 <= max(steps, 8)
+                assert nt in (1, 4) and 1 <= parts <= L.TUNING.max_split_k_parts
+                assert parts == 1 or (steps % parts == 0 or k < L.TUNING.split_k_from) and parts * 8 <= max(steps, 8)
                 assert nt == 1 or rows > 16
 
 
