@@ -40,6 +40,9 @@ class Tuning:
     library_split_min_rows: int = 65
     library_split_max_rows: int = 256
     library_split_max_out_features: int = 4096
+    # The same for the rows of prompt portions up to this many, in four pieces (the float32 parts cost the norm that
+    # adds them more to read, so the gain is smaller and ends at 4,096 rows).
+    library_split_portion_max_rows: int = 2048
     # The gate-up product lies transposed (weights as the library's first operand) for row counts from this on that
     # are a multiple of it: the library's tiles then fit the rows.
     transposed_gate_up_row_multiple: int = 256

@@ -85,11 +85,19 @@ def _library_is_faster(rows, out_features):
 def _library_split(rows, out_features, in_features):
     """Into how many pieces of K the library's product is cut.  Measured on MI355X: with up to 256 rows, few
     output columns and a long K (the down projection of a busy decode step) the library's single product leaves
-    a quarter of the chip idle and takes 31 us where five pieces side by side take 23."""
-    if not (TUNING.library_split_min_rows <= rows <= TUNING.library_split_max_rows and in_features >= TUNING.split_k_from
-            and out_features <= TUNING.library_split_max_out_features):
+    a quarter of the chip idle and takes 31 us where five pieces side by side take 23.  A prompt portion's rows
+    gain less, while the float32 parts cost the norm more to read: four pieces take the down projection of the 1.5B
+    shape and the norm after it from 50.7 to 39.0 us at 1,024 rows and from 76.0 to 69.8 at 2,048 (the library's one
+    product makes 264 tiles for 256 compute units there); at 4,096 rows nothing is gained."""
+    if not (in_features >= TUNING.split_k_from and out_features <= TUNING.library_split_max_out_features):
         return 1
-    for parts in (5, 4, 2):
+    if TUNING.library_split_min_rows <= rows <= TUNING.library_split_max_rows:
+        tries = (5, 4, 2)
+    elif TUNING.library_split_max_rows < rows <= TUNING.library_split_portion_max_rows:
+        tries = (4, 2)
+    else:
+        return 1
+    for parts in tries:
         if in_features % parts == 0 and (in_features // parts) % 8 == 0:
             return parts
     return 1
