@@ -154,7 +154,8 @@ class Engine:
         sampling = [sc.seq for sc in scheduled if sc.samples]
         ahead = 1 if device_tokens is not None else 0      # the token before is not in the request's list yet
         tokens = self.sampler.sample_on_device(logits, [s.params for s in sampling],
-                                               [s.num_output_tokens + ahead for s in sampling])
+                                               [s.num_output_tokens + ahead for s in sampling],
+                                               [s.request_id for s in sampling])
         ended.record()
         arrival = None
         if tokens is not None:               # the copy to the host is queued now, behind this step only

@@ -1,5 +1,5 @@
 from .params import SamplingParams
-from .rng import uniform
+from .rng import uniform, request_seed
 from .sampler import Sampler
 
-__all__ = ["SamplingParams", "uniform", "Sampler"]
+__all__ = ["SamplingParams", "uniform", "request_seed", "Sampler"]

@@ -9,7 +9,9 @@ class SamplingParams:
     max_tokens: int = 64
     ignore_eos: bool = False
     temperature: float = 0.0          # 0: greedy (argmax, lowest index among equals)
-    seed: int = 0                     # with temperature: the n-th output token uses uniform(seed, n)
+    # with temperature: the n-th output token uses uniform(seed, n); None: a seed of the request's own (its id is the
+    # key), so that two requests with the same settings do not draw the same numbers
+    seed: Optional[int] = None
     stop_token_ids: Optional[List[int]] = None   # None: the configuration's end-of-sequence ids
 
     def validate(self):

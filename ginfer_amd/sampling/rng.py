@@ -17,3 +17,8 @@ def uniform(seed, n):
     """A float32-exact number in [0, 1) for output position n of a request with this seed."""
     z = _mix(_mix(seed & _MASK) ^ ((n + 1) * 0xD1342543DE82EF95 & _MASK))
     return (z >> 40) / float(1 << 24)
+
+
+def request_seed(request_id):
+    """The seed of a request that names none: a function of its id alone."""
+    return _mix((int(request_id) & _MASK) ^ 0xA0761D6478BD642F)

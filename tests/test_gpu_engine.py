@@ -259,6 +259,29 @@ def test_a_late_request_finds_the_pages_of_a_request_that_is_still_running(sharp
         assert tokens["running"] == tokens["finished"] == tokens["alone"]
 
 
+def test_requests_without_a_seed_draw_from_streams_of_their_own(folders):
+    """Two requests with the same prompt and the same sampling settings, no seed named: each draws from the stream of
+    its own id, so their tokens differ (and each is what the plain sampler draws with that stream's numbers); with a
+    seed named, both give the same tokens."""
+    from ginfer_amd import Engine, EngineConfig, SamplingParams
+    from ginfer_amd.sampling import uniform, request_seed
+    folder = folders["B"]
+    prompt = H.random_tokens(20, 1000, 77)
+    eng = Engine(EngineConfig(model_path=folder, dtype="float32", max_num_batched_tokens=64, max_num_seqs=4, max_seq_len=128,
+                              kvcache_block_size=8, num_kvcache_blocks=40, enable_prefix_caching=False))
+    outs = eng.generate([prompt, prompt], SamplingParams(max_tokens=16, temperature=1.0, ignore_eos=True))
+    assert outs[0].token_ids != outs[1].token_ids
+    cfg, w = pm.read_config(folder), pm.read_weights(folder)
+    for o in outs:
+        logits = pm.forward(cfg, w, (prompt + o.token_ids)[:-1])
+        for k, tok in enumerate(o.token_ids):
+            row, u = logits[len(prompt) - 1 + k], uniform(request_seed(o.request_id), k)
+            want = pm.sample_token(row, 1.0, u)
+            assert want == tok or _is_a_tie(row, 1.0, u, tok, want)
+    same = eng.generate([prompt, prompt], SamplingParams(max_tokens=16, temperature=1.0, ignore_eos=True, seed=3))
+    assert same[0].token_ids == same[1].token_ids
+
+
 def test_temperature_sampling_matches_plain_with_same_uniforms(folders):
     from ginfer_amd import Engine, EngineConfig, SamplingParams
     from ginfer_amd.sampling import uniform

@@ -21,7 +21,10 @@ def test_measured_shapes_keep_their_plans():
     assert L._split_plan(64, 3584, 18944) == (4, 4)
     assert L._split_plan(64, 3584, 3584) == (4, 4)
     assert L._library_split(256, 1536, 8960) == 5 and L._library_split(64, 1536, 8960) == 1
-    assert L._library_split(256, 17920, 1536) == 1 and L._library_split(512, 1536, 8960) == 1
+    assert L._library_split(256, 17920, 1536) == 1
+    # the rows of prompt portions: four pieces up to 2,048 rows, one product beyond
+    assert L._library_split(512, 1536, 8960) == 4 and L._library_split(2048, 1536, 8960) == 4
+    assert L._library_split(4096, 1536, 8960) == 1 and L._library_split(2048, 1536, 1536) == 1
 
 
 def test_nearest_divisor():

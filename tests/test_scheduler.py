@@ -172,6 +172,11 @@ def test_uniform_numbers_are_a_function_of_seed_and_place():
     us = [uniform(3, n) for n in range(1000)]
     assert all(0.0 <= u < 1.0 for u in us) and len(set(us)) > 990
     assert us == [uniform(3, n) for n in range(1000)] and uniform(4, 0) != uniform(3, 0)
+    # a request that names no seed draws from a stream of its own: a function of its id, different for every request
+    from ginfer_amd.sampling import request_seed
+    seeds = [request_seed(i) for i in range(1000)]
+    assert len(set(seeds)) == 1000 and seeds == [request_seed(i) for i in range(1000)]
+    assert SamplingParams().seed is None
     assert abs(sum(us) / 1000 - 0.5) < 0.05
     import numpy as np
     assert all(float(np.float32(u)) == u for u in us)          # exact in 32-bit
