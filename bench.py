@@ -68,6 +68,8 @@ def main():
     ap.add_argument("--no-engine-warmup", action="store_true",
                     help="the engine does not run its warm-up steps when it starts (for kernel profiles: fewer calls that "
                          "are not the measurement's)")
+    ap.add_argument("--autotune", action="store_true",
+                    help="the engine times the plans of its products before it records a step (EngineConfig.autotune)")
     ap.add_argument("--file-weights", action="store_true",
                     help="write the random weights into a model folder and load them from there, instead of drawing them "
                          "on the device (not for 72b: 145 GB)")
@@ -112,7 +114,7 @@ def main():
         random_seed=0 if device_weights else None, dtype=args.dtype,
         max_num_batched_tokens=max(2048, args.prefill_tokens, args.context + max_b), max_num_seqs=max_b,
         max_seq_len=max(args.context, args.prefill_tokens) + max_b + 24, kvcache_block_size=page, num_kvcache_blocks=pages,
-        enable_prefix_caching=False, warmup=not args.no_engine_warmup))
+        enable_prefix_caching=False, warmup=not args.no_engine_warmup, autotune=args.autotune))
     g = torch.Generator().manual_seed(0)
     vocab = cfg["vocab_size"]
 

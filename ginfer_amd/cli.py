@@ -44,6 +44,9 @@ def _engine_args(p):
                    help="steps with prompt portions are launched kernel by kernel, never replayed from a recording")
     p.add_argument("--strict-weights", action="store_true",
                    help="a tensor in the model folder that the model does not read is an error, not a warning")
+    p.add_argument("--autotune", action="store_true",
+                   help="time the plans of a step's products on this model's weights before the step is recorded, and "
+                        "keep the fastest (a second or so per number of rows, once)")
     p.add_argument("--no-prefix-caching", action="store_true",
                    help="requests do not share the cache pages of a common prefix")
 
@@ -63,7 +66,7 @@ def _engine(args):
         max_num_seqs=args.max_num_seqs, max_seq_len=args.max_seq_len,
         gpu_memory_utilization=args.gpu_memory_utilization, kvcache_block_size=args.kvcache_block_size,
         num_kvcache_blocks=args.num_kvcache_blocks, pipeline_decode=not args.no_pipeline_decode,
-        graph_mixed_steps=not args.no_graph_mixed_steps, strict_weights=args.strict_weights,
+        graph_mixed_steps=not args.no_graph_mixed_steps, strict_weights=args.strict_weights, autotune=args.autotune,
         enable_prefix_caching=False if args.no_prefix_caching else None))
 
 

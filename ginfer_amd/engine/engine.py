@@ -42,6 +42,9 @@ class EngineConfig:
     graph_mixed_steps: bool = True
     # a tensor in the model folder that the model does not read: an error instead of a warning
     strict_weights: bool = False
+    # before a step of some number of rows is recorded, the products that can be done in several ways are timed in
+    # each, on this model's own weights, and the fastest kept (a second or so per number of rows, once)
+    autotune: bool = False
 
 
 @dataclass
@@ -65,7 +68,7 @@ class Engine:
                                   gpu_memory_utilization=config.gpu_memory_utilization,
                                   prefix_caching=config.enable_prefix_caching,
                                   graph_mixed_steps=config.graph_mixed_steps,
-                                  strict_weights=config.strict_weights,
+                                  strict_weights=config.strict_weights, autotune=config.autotune,
                                   config=config.model_config if config.model_path is None else None,
                                   random_seed=config.random_seed if config.model_path is None else None)
         self.scheduler = Scheduler(self.runner.cache, config.max_num_seqs, config.max_num_batched_tokens,

@@ -11,6 +11,7 @@ Steps whose shapes come again are recorded into HIP graphs and replayed: steps o
 number of requests, short steps with prompt portions laid into padded sizes (`_run_padded`); all side inputs of
 a recorded step live in one static buffer that every replay refills.
 """
+import os
 import time
 from dataclasses import dataclass, field
 from typing import List, Sequence
@@ -20,7 +21,7 @@ import torch
 
 from ..cache import CacheManager
 from ..config import config_from_folder
-from ..kernels import build
+from ..kernels import autotune, build
 from ..kernels.tuning import TUNING
 from ..parts.base import KVCacheSpec, StateSpec
 from ..parts.model import build_model, StepContext, KVView, StateView
@@ -46,13 +47,15 @@ class ModelRunner:
     def __init__(self, model_path, dtype="bfloat16", page_size=16, num_pages=None, max_requests=64,
                  max_model_len=None, gpu_memory_utilization=0.9, device=None, config=None, use_graphs=True,
                  prefix_caching=False, random_seed=None, graph_mixed_steps=True, max_num_batched_tokens=None,
-                 strict_weights=False):
+                 strict_weights=False, autotune=False):
         """model_path: a folder with config.json and the weights.  With model_path None, `config` (a typed
         configuration) and `random_seed` make a model whose weights are drawn on the device, for shapes too
         large to pass through a file.  num_pages: pages of every cache group (or a list, one count per group);
         None: from the memory that is free once the weights are loaded and the largest step (max_num_batched_tokens
         tokens, max_requests requests) has run, times gpu_memory_utilization.  strict_weights: a tensor in the folder
-        that the model does not read is an error, not a warning."""
+        that the model does not read is an error, not a warning.  autotune: before a step of some number of rows is
+        recorded, the products that can be done in several ways are timed in each and the fastest kept
+        (kernels/autotune.py); takes a second or so per number of rows, once."""
         self.device = device or require_gpu()
         if dtype not in DTYPES:
             raise ValueError("dtype must be one of %s, got %r" % (sorted(DTYPES), dtype))
@@ -78,6 +81,7 @@ class ModelRunner:
         if prefix_caching is None:       # where the model allows it
             prefix_caching = CacheManager.supports_prefix_caching(specs)
         self.graph_mixed_steps = bool(graph_mixed_steps)
+        self.autotune = bool(autotune)
         self._graphs, self._graph_seen, self._padded_buffers = {}, {}, {}
         self._graph_budget, self._graph_bytes, self._graph_bytes_seen = None, 0, {}
         # Padding pays while the host's launches (~5 ms a step) outlast the device's work on the padded rows, which may
@@ -413,10 +417,8 @@ class ModelRunner:
         buf = _StepBuffers(t_pad, e_pad + 1, e_pad, width, e_pad, len(self.cache.groups), self.device,
                            n_tiles=self._padded_tiles(t_pad, e_pad))
         ctx = self._padded_context(host, buf, t_pad, e_pad, width, bucket)
-        extra = dict(ctx.extra)
-        self._run_once_unrecorded(ctx)
+        self._settle(ctx, dict(ctx.extra))
         graph = torch.cuda.CUDAGraph()
-        ctx.extra = extra
         with torch.cuda.graph(graph):
             logits = self.model.forward(ctx)
         g = dict(graph=graph, buf=buf, logits=logits, ctx=ctx, width=width)
@@ -432,16 +434,31 @@ class ModelRunner:
         buf = _StepBuffers(E, E, E, width, E, len(self.cache.groups), self.device)
         padded = dict(host, width=width, tables=[self._widen(t, width) for t in host["tables"]])
         ctx = self._context(padded, buf)
-        self._run_once_unrecorded(ctx)
+        self._settle(ctx, {"decode_info": buf.dev["decode_info"], "decode_span": bucket})
         graph = torch.cuda.CUDAGraph()
-        ctx.extra = {"decode_info": buf.dev["decode_info"], "decode_span": bucket}
         with torch.cuda.graph(graph):
             logits = self.model.forward(ctx)
         g = dict(graph=graph, buf=_GraphBuffers(buf, width, self._widen), logits=logits, ctx=ctx)
         self._graphs[key] = g
         return g
 
-    def _run_once_unrecorded(self, ctx):
+    def _settle(self, ctx, extra):
+        """What precedes the recording of a step: with autotune, a run in which the products report themselves and the
+        timing of their plans; then the run that warms up what the recording will call.  Every run starts from the
+        same `extra` (a run leaves its plans of rows and tiles there)."""
+        if self.autotune:
+            ctx.extra = dict(extra)
+            with autotune.collecting() as seen:
+                self._run_once_unrecorded(ctx, count=False)
+            t0 = time.perf_counter()
+            self.counts["autotuned_keys"] = self.counts.get("autotuned_keys", 0) + autotune.tune(
+                seen, self.device, verbose=bool(os.environ.get("GINFER_AMD_AUTOTUNE_VERBOSE")))
+            self.counts["autotune_seconds"] = round(self.counts.get("autotune_seconds", 0.0) + time.perf_counter() - t0, 3)
+        ctx.extra = dict(extra)
+        self._run_once_unrecorded(ctx)
+        ctx.extra = dict(extra)
+
+    def _run_once_unrecorded(self, ctx, count=True):
         """Before a step is recorded it runs once outside the graph, on a stream of its own: libraries load what they
         need, the allocator settles.  The step itself is the replay that follows, so this run must leave nothing
         behind: keys and values it writes are written again by the replay, the same ones into the same places, and
@@ -455,7 +472,8 @@ class ModelRunner:
         for e, t in saved.items():
             self.cache.state_tensors[e].copy_(t)
         torch.cuda.synchronize()
-        self.counts["recorded"] += 1
+        if count:
+            self.counts["recorded"] += 1
 
     @staticmethod
     def _widen(table, width):

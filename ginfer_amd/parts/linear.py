@@ -8,7 +8,7 @@ the products with a wide output, where it was measured faster; replays of record
 these calls are checked bit for bit against eager steps in the tests."""
 import torch
 
-from ..kernels import ops
+from ..kernels import autotune, ops
 from ..kernels.tuning import TUNING      # every threshold below is a field of this table, with what it was measured on
 
 
@@ -20,26 +20,54 @@ def linear(x, weight, bias=None, out_dtype=None, parts_ok=False):
         return ops.gemm_skinny(x, weight, bias, out_dtype=out_dtype, nt=1)
     if x.dtype == torch.float32:
         return ops.gemm_nt(x, weight, bias)
-    if ops.gemm_skinny_supported(x, weight) and not _library_is_faster(x.shape[0], weight.shape[0]):
+    float32_out = out_dtype == torch.float32
+    skinny_ok = ops.gemm_skinny_supported(x, weight)
+    plan = None
+    if autotune.active():
+        key = ("linear", autotune.rows_class(x.shape[0]), weight.shape[0], x.shape[1], bias is not None, float32_out,
+               bool(parts_ok), skinny_ok)
+        plan = autotune.choose(key, (weight, bias))
+    if plan is None:
+        plan = linear_plan(x.shape[0], weight.shape[0], x.shape[1], bias is not None, float32_out, parts_ok, skinny_ok)
+    return run_linear_plan(plan, x, weight, bias, out_dtype)
+
+
+def linear_plan(rows, out_features, in_features, has_bias, float32_out, parts_ok, skinny_ok):
+    """The way a bfloat16 product is done, by the rules: ("skinny", tiles of W per wavefront, parts of K) for the
+    package's weight-streaming kernel, ("library", pieces of K) for the BLAS library.  More than one part or piece
+    means float32 partial sums [parts, M, N] for the consumer to add."""
+    may_split = parts_ok and not float32_out
+    if skinny_ok and not _library_is_faster(rows, out_features):
         # tilings measured on MI355X (graph replays, weights not cache-resident): up to 16 rows one
         # 16-row tile of W per wavefront streams best; beyond, four tiles halve the re-reading of x; a
         # long K is split over workgroups where the consumer can add the parts
-        many = x.shape[0] > 16
-        if parts_ok and out_dtype is None and x.shape[1] >= TUNING.split_k_min_in_features:
-            nt, splits = _split_plan(x.shape[0], weight.shape[0], x.shape[1])
+        if may_split and in_features >= TUNING.split_k_min_in_features:
+            nt, splits = _split_plan(rows, out_features, in_features)
             if splits > 1:
-                return ops.gemm_skinny(x, weight, bias, out_dtype=torch.float32, nt=nt, grid_splits=splits)
-        return ops.gemm_skinny(x, weight, bias, out_dtype=out_dtype, nt=4 if (many and weight.shape[0] >= TUNING.four_tiles_min_out_features) else 1)
-    if parts_ok and out_dtype is None and bias is None:
-        parts = _library_split(x.shape[0], weight.shape[0], x.shape[1])
+                return ("skinny", nt, splits)
+        return ("skinny", 4 if (rows > 16 and out_features >= TUNING.four_tiles_min_out_features) else 1, 1)
+    if may_split and not has_bias:
+        parts = _library_split(rows, out_features, in_features)
         if parts > 1:
-            # the library, once, over `parts` pieces of K side by side (a batched product over views of x and
-            # the weight): float32 partial sums for the norm that follows, and work for all of the chip
-            M, K = x.shape
-            kc = K // parts
-            xv = x.as_strided((parts, M, kc), (kc, x.stride(0), 1))
-            wv = weight.as_strided((parts, kc, weight.shape[0]), (kc, 1, K))
-            return torch.bmm(xv, wv, out_dtype=torch.float32)
+            return ("library", parts)
+    return ("library", 1)
+
+
+def run_linear_plan(plan, x, weight, bias, out_dtype):
+    if plan[0] == "skinny":
+        _, nt, splits = plan
+        if splits > 1:
+            return ops.gemm_skinny(x, weight, bias, out_dtype=torch.float32, nt=nt, grid_splits=splits)
+        return ops.gemm_skinny(x, weight, bias, out_dtype=out_dtype, nt=nt)
+    _, parts = plan
+    if parts > 1:
+        # the library, once, over `parts` pieces of K side by side (a batched product over views of x and
+        # the weight): float32 partial sums for the norm that follows, and work for all of the chip
+        M, K = x.shape
+        kc = K // parts
+        xv = x.as_strided((parts, M, kc), (kc, x.stride(0), 1))
+        wv = weight.as_strided((parts, kc, weight.shape[0]), (kc, 1, K))
+        return torch.bmm(xv, wv, out_dtype=torch.float32)
     if out_dtype == torch.float32:
         y = torch.mm(x, weight.t(), out_dtype=torch.float32)
         if bias is not None:
@@ -48,6 +76,53 @@ def linear(x, weight, bias=None, out_dtype=None, parts_ok=False):
     if bias is not None:
         return torch.addmm(bias, x, weight.t())
     return torch.mm(x, weight.t())
+
+
+def linear_candidates(key):
+    """Every plan that does the product of an autotune key; the plan by the rules first."""
+    _, rows, out_features, in_features, has_bias, float32_out, parts_ok, skinny_ok = key
+    plans = [linear_plan(rows, out_features, in_features, has_bias, float32_out, parts_ok, skinny_ok)]
+
+    def add(plan):
+        if plan not in plans:
+            plans.append(plan)
+
+    may_split = parts_ok and not float32_out
+    if skinny_ok:
+        tiles = (1, 4) if rows > 16 else (1,)
+        for nt in tiles:
+            add(("skinny", nt, 1))
+        if may_split and in_features >= TUNING.split_k_min_in_features:
+            steps = -(-in_features // 64)
+            for parts in (2, 3, 4, 5, 6, 7, 8, 10, 12, 14, 16):
+                if parts <= min(TUNING.max_split_k_parts, steps // 8) and steps % parts == 0:
+                    for nt in tiles:
+                        add(("skinny", nt, parts))
+    add(("library", 1))
+    if may_split and not has_bias:
+        for parts in (2, 3, 4, 5, 7, 8, 10, 14, 16):
+            if in_features % parts == 0 and (in_features // parts) % 8 == 0 and in_features // parts >= 512:
+                add(("library", parts))
+    return plans
+
+
+def _linear_timing(key, operands, device):
+    """For the tuner: the product on random rows, followed, where it may come in parts, by the norm that adds them
+    (more parts cost that norm more to read)."""
+    _, rows, out_features, in_features, _, float32_out, parts_ok, _ = key
+    x = (torch.randn((rows, in_features), device=device) * 0.5).to(torch.bfloat16)
+    residual = torch.zeros((rows, out_features), dtype=torch.float32, device=device) if parts_ok else None
+    gain = torch.ones((out_features,), dtype=torch.bfloat16, device=device) if parts_ok else None
+
+    def run(plan, i):
+        weight, bias = operands[i]
+        y = run_linear_plan(plan, x, weight, bias, torch.float32 if float32_out else None)
+        if parts_ok:
+            ops.add_rmsnorm(residual, y, gain, 1e-6, torch.bfloat16)
+    return run
+
+
+autotune.register_kind("linear", linear_candidates, _linear_timing)
 
 
 def _split_plan(rows, out_features, in_features):
@@ -123,20 +198,64 @@ def gated_linear(x, weight_gate_up):
     ops.ScaledRows."""
     if isinstance(x, ops.ScaledRows):
         return ops.gemm_skinny(x, weight_gate_up, gated=True)
-    if (x.dtype == torch.bfloat16 and ops.gemm_skinny_supported(x, weight_gate_up)
-            and not _library_is_faster(x.shape[0], weight_gate_up.shape[0])):
+    skinny_ok = x.dtype == torch.bfloat16 and ops.gemm_skinny_supported(x, weight_gate_up)
+    transposable = _transposable(x, weight_gate_up)
+    plan = None
+    if autotune.active() and x.dtype == torch.bfloat16:
+        key = ("gated", autotune.rows_class(x.shape[0]), weight_gate_up.shape[0], x.shape[1], skinny_ok, transposable)
+        plan = autotune.choose(key, (weight_gate_up,))
+    if plan is None:
+        plan = gated_plan(x.shape[0], weight_gate_up.shape[0], skinny_ok, transposable)
+    return run_gated_plan(plan, x, weight_gate_up)
+
+
+def gated_plan(rows, out_features, skinny_ok, transposable):
+    """By the rules: ("skinny",) the weight-streaming kernel with the activation in its epilogue; ("transposed",) the
+    library with the weights as its first operand, which leaves the product transposed, [2I, M], and the activation on
+    that; ("library",) the usual product and the activation."""
+    if skinny_ok and not _library_is_faster(rows, out_features):
+        return ("skinny",)
+    if transposable and _transposed_product_is_faster(rows):
+        return ("transposed",)
+    return ("library",)
+
+
+def run_gated_plan(plan, x, weight_gate_up):
+    if plan[0] == "skinny":
         return ops.gemm_skinny(x, weight_gate_up, gated=True)
-    if _transposed_product_is_faster(x, weight_gate_up):
-        # the library with the weights as its first operand leaves the product transposed, [2I, M]
+    if plan[0] == "transposed":
         return ops.silu_mul_transposed(torch.mm(weight_gate_up, x.t()))
     return ops.silu_mul(linear(x, weight_gate_up))
 
 
-def _transposed_product_is_faster(x, weight):
+def gated_candidates(key):
+    _, rows, out_features, _, skinny_ok, transposable = key
+    plans = [gated_plan(rows, out_features, skinny_ok, transposable)]
+    for plan, ok in ((("skinny",), skinny_ok), (("library",), True), (("transposed",), transposable)):
+        if ok and plan not in plans:
+            plans.append(plan)
+    return plans
+
+
+def _gated_timing(key, operands, device):
+    _, rows, _, in_features, _, _ = key
+    x = (torch.randn((rows, in_features), device=device) * 0.5).to(torch.bfloat16)
+    return lambda plan, i: run_gated_plan(plan, x, operands[i][0])
+
+
+autotune.register_kind("gated", gated_candidates, _gated_timing)
+
+
+def _transposable(x, weight):
+    """Whether the library can take the weights as its first operand for these operands (any row count)."""
+    return (x.dtype == torch.bfloat16 and x.is_contiguous() and weight.shape[0] % 16 == 0 and x.shape[1] % 8 == 0
+            and x.shape[0] % 8 == 0)
+
+
+def _transposed_product_is_faster(rows):
     """Measured on MI355X at the 1.5B, 7B and 72B shapes' gate-up product: with a number of rows that is a multiple of
     256 (the portions that a token budget of 2,048 cuts) the library's tiles fit the rows when the weights are its
     first operand: level to 15 % faster (2,048 rows of the 1.5B shape: 115 -> 98 us; 256 rows, a decode step of 256
     requests: 3 to 8 %); with other row counts it is up to 20 % slower, so they keep the usual product."""
     every = TUNING.transposed_gate_up_row_multiple
-    return (x.dtype == torch.bfloat16 and x.shape[0] >= every and x.shape[0] % every == 0 and x.is_contiguous()
-            and weight.shape[0] % 16 == 0 and x.shape[1] % 8 == 0)
+    return rows >= every and rows % every == 0

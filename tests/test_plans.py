@@ -33,3 +33,65 @@ def test_nearest_divisor():
     assert L._nearest_divisor(296, 4.6, 16) == 4
     assert L._nearest_divisor(7, 3.0, 16) == 1          # 1 and 7 are the divisors; 1 is nearer
     assert L._nearest_divisor(24, 100.0, 3) == 3        # never above the cap
+
+
+def test_rules_as_plans():
+    """The rules' decisions as plans, at the sizes they were measured at."""
+    # decode rows of the 1.5B shape: the streaming kernel, K in parts where the norm that follows adds them
+    assert L.linear_plan(64, 1536, 8960, False, False, True, True) == ("skinny", 4, 10)
+    assert L.linear_plan(8, 1536, 8960, False, False, True, True) == ("skinny", 1, 5)
+    assert L.linear_plan(8, 1536, 8960, False, False, False, True) == ("skinny", 1, 1)     # nobody to add parts
+    assert L.linear_plan(8, 1536, 8960, False, True, True, True) == ("skinny", 1, 1)       # float32 out: no parts
+    # wide outputs go to the library from 17 rows on; prompt portions always
+    assert L.linear_plan(64, 17920, 1536, False, False, False, True) == ("library", 1)
+    assert L.linear_plan(16, 17920, 1536, False, False, False, True) == ("skinny", 1, 1)
+    assert L.linear_plan(2048, 1536, 8960, False, False, True, False) == ("library", 4)
+    assert L.linear_plan(2048, 1536, 8960, True, False, True, False) == ("library", 1)     # a bias: one product
+    assert L.linear_plan(4096, 1536, 8960, False, False, True, False) == ("library", 1)
+    assert L.gated_plan(8, 17920, True, True) == ("skinny",)
+    assert L.gated_plan(64, 17920, True, True) == ("library",)
+    assert L.gated_plan(2048, 17920, False, True) == ("transposed",)
+    assert L.gated_plan(2040, 17920, False, True) == ("library",)
+
+
+def test_candidates_hold_the_rules_plan_first_and_only_plans_that_fit():
+    for rows in (1, 8, 16, 17, 64, 128, 256):
+        for n, k in ((1536, 8960), (3584, 18944), (8192, 29568), (88, 520), (1536, 1536), (151936, 1536)):
+            for has_bias in (False, True):
+                for f32 in (False, True):
+                    for parts_ok in (False, True):
+                        skinny_ok = rows <= 64
+                        key = ("linear", rows, n, k, has_bias, f32, parts_ok, skinny_ok)
+                        plans = L.linear_candidates(key)
+                        assert plans[0] == L.linear_plan(rows, n, k, has_bias, f32, parts_ok, skinny_ok)
+                        assert len(set(plans)) == len(plans) and ("library", 1) in plans
+                        for plan in plans[1:]:
+                            if plan[0] == "skinny":
+                                assert skinny_ok and plan[1] in (1, 4) and (plan[1] == 1 or rows > 16)
+                                if plan[2] > 1:
+                                    assert parts_ok and not f32 and -(-k // 64) % plan[2] == 0 and plan[2] * 8 <= -(-k // 64)
+                            else:
+                                if plan[1] > 1:
+                                    assert parts_ok and not f32 and not has_bias
+                                    assert k % plan[1] == 0 and (k // plan[1]) % 8 == 0 and k // plan[1] >= 512
+    assert L.gated_candidates(("gated", 64, 17920, 1536, True, True)) == [("library",), ("skinny",), ("transposed",)]
+    assert L.gated_candidates(("gated", 2048, 17920, 1536, False, True)) == [("transposed",), ("library",)]
+    assert L.gated_candidates(("gated", 100, 17920, 1536, False, False)) == [("library",)]
+
+
+def test_kept_plans_answer_for_their_class_of_rows():
+    from ginfer_amd.kernels import autotune
+    assert [autotune.rows_class(r) for r in (1, 7, 16, 17, 32, 33, 64, 65, 200)] == [1, 7, 16, 32, 32, 48, 64, 80, 208]
+    autotune.clear()
+    assert not autotune.active() and autotune.choose(("linear", 32), ("w",)) is None
+    with autotune.collecting() as seen:
+        assert autotune.active()
+        assert autotune.choose(("linear", 32), ("w0",)) is None and autotune.choose(("linear", 32), ("w1",)) is None
+        assert autotune.choose(("gated", 32), ("w2",)) is None
+    assert seen == {("linear", 32): [("w0",), ("w1",)], ("gated", 32): [("w2",)]} and not autotune.active()
+    autotune.TABLE[("linear", 32)] = ("library", 2)
+    try:
+        assert autotune.active() and autotune.choose(("linear", 32), ("w",)) == ("library", 2)
+        assert autotune.choose(("linear", 48), ("w",)) is None
+    finally:
+        autotune.clear()
