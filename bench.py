@@ -162,7 +162,7 @@ def main():
         for _ in range(warmup):
             engine.step()
         sync()
-        del engine.step_log[:]
+        engine.step_log.clear()
         t0 = time.perf_counter()
         for _ in range(steps):
             engine.step()

@@ -376,6 +376,11 @@ class CacheManager:
         req.pending = n_new
         return req.length
 
+    def cancel(self, rid):
+        """The reserved tokens will not run after all.  Pages that the reservation took stay in the request's table, where
+        its next reservation finds them."""
+        self.requests[rid].pending = 0
+
     def tables_array(self, group, slots, width):
         """int32 [len(slots), width]: the block tables of the requests in these state slots."""
         mirror = self._table_np[group]

@@ -129,7 +129,7 @@ def cmd_benchmark(args):
     engine.generate([[rng.randrange(vocab) for _ in range(hi)] for _ in range(2)], _params(args, 2))
     for k in engine.stats:
         engine.stats[k] = 0 if isinstance(engine.stats[k], int) else 0.0
-    del engine.step_log[:]
+    engine.step_log.clear()
     t0 = time.perf_counter()
     if args.request_rate > 0:
         outs = _generate_as_they_arrive(engine, prompts, _params(args, len(prompts)), args.request_rate, rng)

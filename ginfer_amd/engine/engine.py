@@ -1,6 +1,7 @@
 """The engine: requests in, token ids out.  Field names of the configuration are the reference's
 (ginfer/engine/config.h:8-21); `generate` and `step` follow ginfer/engine/engine.cc:93-151, without the
 tokenizer: prompts are lists of token ids and so are the results."""
+import collections
 import time
 from dataclasses import dataclass
 
@@ -86,7 +87,7 @@ class Engine:
         # one record a step: wall time of Engine.step, the device's own time for the step's kernels (model and sampling,
         # between two events on the stream) and the step's tokens; the reference accounts wall time only
         # (ginfer/engine/engine.cc:93-121)
-        self.step_log = []
+        self.step_log = collections.deque(maxlen=1 << 16)      # the last 65,536 steps
         self.last_logits = None          # the logits of the step launched last (a buffer that the next step overwrites)
         if config.warmup:
             self._warm_up()

@@ -190,7 +190,7 @@ class ModelRunner:
             logits = self._run(host, borrow, device_tokens)
         except Exception:
             for rid in reserved_here:       # nothing is committed: the requests stay as long as they were
-                cache.requests[rid].pending = 0
+                cache.cancel(rid)
             raise
         # What this step reserved it also commits.  A caller that reserved the tokens itself (the scheduler) commits them
         # too, with the request's tokens: the cache manager then remembers the pages that are full now, for requests

@@ -257,6 +257,6 @@ class Scheduler:
                 reserved.append(sc.seq.request_id)
             except OutOfPages:
                 for rid in reserved:
-                    self.cache.requests[rid].pending = 0
+                    self.cache.cancel(rid)
                 return None
         return [Scheduled(sc.seq, 1, True) for _, sc in alive], [i for i, _ in alive]
