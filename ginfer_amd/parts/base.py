@@ -26,7 +26,8 @@ Norm          forward(residual float32 [T, H], delta [T, H] | None, rows=None) -
               adds delta into the 32-bit residual stream and returns the normalised rows; with `rows`
               (int32 indices) only those rows are returned and the residual is left as it is.
 Position      what the mixer's kernel needs to encode positions (for rotary kinds: `tables()`).
-Embedding     forward(token_ids int32 [T]) -> float32 [T, H] (the start of the residual stream)
+Embedding     forward(token_ids int32 [T], step) -> float32 [T, H] (the start of the residual stream; `step` is the
+              batch's `StepContext`, for an embedding that adds something by position)
 Head          forward(x [R, H]) -> float32 logits [R, V]
 Arrangement   how a layer's parts are ordered around the residual stream (see block.py).
 """

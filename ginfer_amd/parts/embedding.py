@@ -28,7 +28,7 @@ class Embedding(Part):
     def kernel_modules(self):
         return ["embedding"]
 
-    def forward(self, token_ids):
+    def forward(self, token_ids, step=None):
         return ops.embedding_gather(self.weight, token_ids)
 
 

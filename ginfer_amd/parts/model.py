@@ -152,7 +152,7 @@ class DecoderModel:
     # ---- forward
     def forward(self, step):
         """Logits float32 [R, V] at `step.logit_rows`."""
-        residual = self.embedding.forward(step.token_ids)
+        residual = self.embedding.forward(step.token_ids, step)
         delta = None
         for i, e in enumerate(self.schedule):
             cache = step.caches[i]

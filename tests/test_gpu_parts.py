@@ -715,3 +715,142 @@ def test_schedule_names_a_layer_twice_and_shares_a_cache(tmp_path):
         got = H.run_steps(runner, steps)
         for (rid, p), row in got.items():
             assert np.abs(row - ref[p]).max() / np.abs(ref).max() < 1e-4
+
+
+def _register_toy_ends():
+    """A third toy architecture defined here: a norm of another kind (mean taken off, gain and bias), an embedding that
+    scales the table's rows and adds a learned vector per position, and a head with a bias whose logits are capped
+    softly.  The layers between them are the package's own.  None of it touches the package's files."""
+    from ginfer_amd.config import register_architecture, PartSpec, prenorm_layer, ScheduleEntry, ModelSpec
+    from ginfer_amd.parts import register_norm, register_embedding, register_head, Part
+    from ginfer_amd.weights import WeightSpec
+
+    @register_norm("toy_centered_norm")
+    class CenteredNorm(Part):
+        """y = (h - mean(h)) / sqrt(var(h) + eps) * g + b, h = residual + delta, in 32-bit.  It says nothing of partial
+        sums or folding: the block hands it whole rows."""
+
+        def __init__(self, size, eps, dtype, device):
+            self.size, self.eps, self.dtype, self.device = int(size), float(eps), dtype, device
+
+        def weight_specs(self):
+            return {"weight": WeightSpec((self.size,), init="one_plus_normal", keep_32bit=True),
+                    "bias": WeightSpec((self.size,), std=0.1, keep_32bit=True)}
+
+        def bind_weights(self, t):
+            self.weight, self.bias = t["weight"], t["bias"]
+
+        def forward(self, residual, delta=None, rows=None):
+            if rows is not None:
+                h = residual[rows.long()] + (delta[rows.long()].float() if delta is not None else 0.0)
+            else:
+                if delta is not None:
+                    residual += delta.float()
+                h = residual
+            c = h - h.mean(dim=-1, keepdim=True)
+            y = c * torch.rsqrt(c.pow(2).mean(dim=-1, keepdim=True) + self.eps) * self.weight.float() + self.bias.float()
+            return y.to(self.dtype)
+
+    @register_embedding("toy_scaled_with_positions")
+    class ScaledWithPositions(Part):
+        """x[t] = sqrt(H) * E[id[t]] + P[position[t]]: it reads the positions from the step."""
+
+        def __init__(self, vocab_size, hidden_size, max_positions, dtype, device):
+            self.V, self.H, self.P, self.dtype, self.device = int(vocab_size), int(hidden_size), int(max_positions), dtype, device
+
+        def weight_specs(self):
+            return {"weight": WeightSpec((self.V, self.H)), "positions.weight": WeightSpec((self.P, self.H), std=0.05)}
+
+        def bind_weights(self, t):
+            self.weight, self.positions = t["weight"], t["positions.weight"]
+
+        def forward(self, token_ids, step):
+            return self.weight[token_ids.long()].float() * math.sqrt(self.H) + self.positions[step.positions.long()].float()
+
+    @register_head("toy_capped_head")
+    class CappedHead(Part):
+        """logits = cap * tanh((x . W^T + b) / cap), 32-bit."""
+
+        def __init__(self, vocab_size, hidden_size, cap, dtype, device):
+            self.V, self.H, self.cap, self.dtype, self.device = int(vocab_size), int(hidden_size), float(cap), dtype, device
+
+        def weight_specs(self):
+            return {"weight": WeightSpec((self.V, self.H), std=0.3), "bias": WeightSpec((self.V,), std=0.5, keep_32bit=True)}
+
+        def bind_weights(self, t):
+            self.weight, self.bias = t["weight"], t["bias"]
+
+        def forward(self, x):
+            z = x.float() @ self.weight.float().t() + self.bias.float()
+            return self.cap * torch.tanh(z / self.cap)
+
+    @register_architecture("ToyEndsLM")
+    @dataclass
+    class ToyEndsConfig:
+        hidden_size: int = 48
+        vocab_size: int = 211
+        architecture = "ToyEndsLM"
+
+        @classmethod
+        def from_dict(cls, d):
+            return cls(d["hidden_size"], d["vocab_size"])
+
+        def to_dict(self):
+            return dict(architectures=["ToyEndsLM"], hidden_size=self.hidden_size, vocab_size=self.vocab_size)
+
+        def model_spec(self):
+            Hd = self.hidden_size
+            norm = PartSpec("toy_centered_norm", dict(size=Hd, eps=1e-5))
+            rope = PartSpec("rope_neox", dict(theta=300.0, rotary_dim=16, max_positions=96))
+            attn = PartSpec("attention", dict(hidden_size=Hd, num_heads=3, num_kv_heads=1, head_dim=16, qkv_bias=True,
+                                              out_bias=False, window=None, position=rope, scale=None))
+            dense = PartSpec("swiglu", dict(hidden_size=Hd, intermediate_size=72))
+            layers = [prenorm_layer("model.layers.%d" % i, attn, dense, norm, norm) for i in range(2)]
+            return ModelSpec(hidden_size=Hd, vocab_size=self.vocab_size, layers=layers,
+                             schedule=[ScheduleEntry(0), ScheduleEntry(1)],
+                             embedding=PartSpec("toy_scaled_with_positions",
+                                                dict(vocab_size=self.vocab_size, hidden_size=Hd, max_positions=96)),
+                             final_norm=norm,
+                             head=PartSpec("toy_capped_head", dict(vocab_size=self.vocab_size, hidden_size=Hd, cap=3.0)),
+                             max_positions=96, eos_token_ids=[0])
+    return ToyEndsConfig
+
+
+def _toy_ends_plain(folder, ids):
+    w = pm.read_weights(folder)
+    T, Hd = len(ids), 48
+    cfg = dict(num_attention_heads=3, num_key_value_heads=1, head_dim=16)
+
+    def norm(h, prefix):
+        c = h - h.mean(dim=-1, keepdim=True)
+        return c / torch.sqrt(c.pow(2).mean(dim=-1, keepdim=True) + 1e-5) * w[prefix + ".weight"] + w[prefix + ".bias"]
+    sin, cos = pm.rope_tables(300.0, 16, T)
+    x = pm.embedding(w["model.embed_tokens.weight"], ids) * math.sqrt(Hd) + w["model.embed_tokens.positions.weight"][:T]
+    for layer in (0, 1):
+        p = "model.layers.%d" % layer
+        a, _ = pm.attention_block(norm(x, p + ".input_layernorm"), w, p + ".self_attn", cfg, list(range(T)), sin, cos, None)
+        h = x + a
+        x = h + pm.feed_forward(norm(h, p + ".post_attention_layernorm"), w, p + ".mlp")
+    z = pm.linear(norm(x, "model.norm"), w["lm_head.weight"]) + w["lm_head.bias"]
+    return (3.0 * torch.tanh(z / 3.0)).float().numpy()
+
+
+def test_toy_norm_embedding_and_head(tmp_path):
+    """The ends of a model and its norms as toys registered here: a norm with a mean and a bias (it takes neither
+    partial sums nor folding, so the block adds up what the products leave in parts), an embedding that reads the step's
+    positions, a head with a bias and a cap; stepped whole, in portions and mixed against their plain statement."""
+    from ginfer_amd import ModelRunner, write_random_model, config_from_folder
+    Toy = _register_toy_ends()
+    folder = write_random_model(str(tmp_path / "ends"), Toy(), seed=21, dtype="float32")
+    assert type(config_from_folder(folder)).__name__ == "ToyEndsConfig"
+    reqs = {"a": H.random_tokens(50, 211, 31), "b": H.random_tokens(9, 211, 32), "c": H.random_tokens(27, 211, 33)}
+    runner = ModelRunner(folder, dtype="float32", page_size=8, num_pages=30, max_requests=3)
+    assert not runner.use_graphs
+    refs = {rid: _toy_ends_plain(folder, ids) for rid, ids in reqs.items()}
+    assert max(np.abs(r).max() for r in refs.values()) > 1.5          # the cap is felt
+    for steps in (H.steps_whole(reqs), H.steps_portions(reqs, sizes=(5, 2, 17)), H.steps_mixed(reqs, max_live=3, seed=4)):
+        got = H.run_steps(runner, steps)
+        runner.cache.check()
+        for (rid, p), row in got.items():
+            err = np.abs(row - refs[rid][p]).max() / np.abs(refs[rid]).max()
+            assert err < 1e-4, "request %s position %d: %.3g" % (rid, p, err)
