@@ -82,6 +82,7 @@ class ModelRunner:
             prefix_caching = CacheManager.supports_prefix_caching(specs)
         self.graph_mixed_steps = bool(graph_mixed_steps)
         self.autotune = bool(autotune)
+        self._reserved_by_tuning = 0
         self._graphs, self._graph_seen, self._padded_buffers = {}, {}, {}
         self._graph_budget, self._graph_bytes, self._graph_bytes_seen = None, 0, {}
         # Padding pays while the host's launches (~5 ms a step) outlast the device's work on the padded rows, which may
@@ -327,6 +328,7 @@ class ModelRunner:
         if need > self._graph_budget:
             return None
         before = torch.cuda.memory_reserved(self.device)     # a recorded step keeps a pool of its own reserved
+        self._reserved_by_tuning = 0
         t0 = time.perf_counter()
         try:
             g = capture(key, host)
@@ -339,7 +341,7 @@ class ModelRunner:
             torch.cuda.synchronize()
             return None
         self.counts["recording_seconds"] = round(self.counts["recording_seconds"] + time.perf_counter() - t0, 4)
-        g["bytes"] = max(0, torch.cuda.memory_reserved(self.device) - before)
+        g["bytes"] = max(0, torch.cuda.memory_reserved(self.device) - before - self._reserved_by_tuning)
         self._graph_bytes += g["bytes"]
         kind = key[0] == "padded"
         self._graph_bytes_seen[kind] = max(self._graph_bytes_seen.get(kind, 0), g["bytes"])
@@ -451,9 +453,12 @@ class ModelRunner:
             with autotune.collecting() as seen:
                 self._run_once_unrecorded(ctx, count=False)
             t0 = time.perf_counter()
+            reserved = torch.cuda.memory_reserved(self.device)
             self.counts["autotuned_keys"] = self.counts.get("autotuned_keys", 0) + autotune.tune(
                 seen, self.device, verbose=bool(os.environ.get("GINFER_AMD_AUTOTUNE_VERBOSE")))
             self.counts["autotune_seconds"] = round(self.counts.get("autotune_seconds", 0.0) + time.perf_counter() - t0, 3)
+            # what the timing left in the allocator's hands is not the recorded step's
+            self._reserved_by_tuning += max(0, torch.cuda.memory_reserved(self.device) - reserved)
         ctx.extra = dict(extra)
         self._run_once_unrecorded(ctx)
         ctx.extra = dict(extra)
