@@ -107,10 +107,17 @@ def test_a_runner_that_times_its_plans(tmp_path):
     again = ModelRunner(folder, dtype="bfloat16", page_size=16, num_pages=2 * live, max_requests=live, autotune=True)
     got2 = H.run_steps(again, steps)
     assert again.counts.get("autotuned_keys", 0) == 0
+    # the kept plans in recorded steps and launched kernel by kernel: the same bits (prompts run kernel by kernel in both)
+    pair = [ModelRunner(folder, dtype="bfloat16", page_size=16, num_pages=2 * live, max_requests=live, autotune=True,
+                        use_graphs=g, graph_mixed_steps=False) for g in (True, False)]
+    a, b = (H.run_steps(r, steps) for r in pair)
+    assert pair[0].counts["replayed_decode"] >= 3 and pair[1].counts["replayed_decode"] == 0
+    for k in a:
+        assert np.array_equal(a[k], b[k]), "replayed and launched steps differ at %s" % (k,)
     pcfg, w = pm.read_config(folder), pm.read_weights(folder, torch.float32)
     for rid in list(reqs)[:3] + list(reqs)[-2:]:
         ref = pm.forward(pcfg, w, reqs[rid]).numpy()
         for p in range(prompt - 1, prompt + decoded):
-            for g in (got, got2):
+            for g in (got, got2, a):
                 err = np.abs(g[(rid, p)] - ref[p]).max() / np.abs(ref).max()
                 assert err <= H.TOL["bfloat16"], "request %s position %d: %.3g" % (rid, p, err)
