@@ -60,7 +60,7 @@ __global__ __launch_bounds__(64 * GA_MAX_WAVES) void paged_attention_generic_ker
     int hd, int page_size, int window, float scale, int tq, int hpw) {
   extern __shared__ float lds[];
   const int group = nh / nkv, head_blocks = (group + hpw - 1) / hpw;     // hpw heads of a kv group to a workgroup
-  const int waves = tq * hpw, threads = waves * WAVE;
+  const int waves = tq * hpw, threads = blockDim.x;        // wavefronts that compute; all threads load (see the launcher)
   const int ks = hd + KPAD;                      // a key's row in LDS, in floats
   float* k_s = lds;                              // [64][hd + KPAD]
   float* v_s = k_s + WAVE * ks;                  // [hd][64 + VPAD]
@@ -72,7 +72,7 @@ __global__ __launch_bounds__(64 * GA_MAX_WAVES) void paged_attention_generic_ker
   const int tl = wave / hpw, h = g * group + hl;                  // the wavefront's token of the workgroup, and head
   const int64_t t0 = (int64_t)blockIdx.x * tq;
   const int64_t t = t0 + tl;
-  const bool live = t < tokens && hl < group;
+  const bool live = wave < waves && t < tokens && hl < group;
   const int pos = live ? positions[t] : -1;
   const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
   if (live) {
@@ -245,7 +245,12 @@ extern "C" int ga_paged_attention_generic(void* out, int64_t out_stride, const v
   const size_t lds = sizeof(float) * ((size_t)WAVE * (hd + KPAD) + (size_t)hd * VS + (size_t)waves * hd + (size_t)waves * WAVE)
                      + sizeof(int32_t) * WAVE;
   if ((int64_t)nkv * head_blocks > 65535) return -3;
-  dim3 grid((tokens + tq - 1) / tq, nkv * head_blocks), block(WAVE * waves);
+  // A workgroup with few wavefronts that compute (a decoded token: the heads of one kv group) gets further ones that
+  // only help to load: a tile's loads are then all under way at once, and a tile's time is one trip to memory.
+  int total_waves = waves;
+  const int vectors = WAVE * hd / (is_bf16 ? 8 : 4);                  // 16-byte loads of a tile's keys (and of its values)
+  while (total_waves < GA_MAX_WAVES && total_waves * WAVE * GA_BATCH < vectors) ++total_waves;
+  dim3 grid((tokens + tq - 1) / tq, nkv * head_blocks), block(WAVE * total_waves);
   // 16-byte loads where a key's dimensions and a page's keys come in whole vectors at 16-byte addresses
   const int vec = is_bf16 ? 8 : 4;
   const bool wide = hd % vec == 0 && page_size % vec == 0 && WAVE % page_size == 0 &&

@@ -18,6 +18,9 @@
 #include "ginfer_amd.h"   // the entry points below are checked against their declarations
 
 #define GEMM_THREADS 256
+#ifndef GEMM_MATRIX_FROM_ROWS
+#define GEMM_MATRIX_FROM_ROWS 64    // more rows than this: the kernel on the matrix cores (the same bits)
+#endif
 
 // four consecutive elements as floats; `wide`: one load (the address is a multiple of four elements)
 template <typename T>
@@ -131,6 +134,106 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_nt_kernel(TC* __restrict__ 
   }
 }
 
+// The same product on the matrix cores, for many rows.  v_mfma_f32_32x32x2_f32 takes 32-bit operands and adds the two
+// products of its step of K into the accumulator one after the other, each as a fused multiply-add: measured on the
+// device, its results over a K of 512 equal the chain of fmaf over ascending k bit for bit, for every element of the
+// tile.  So this kernel gives the bits of the kernel above at some three times its rate.  A workgroup of four
+// wavefronts, 2 x 2 over a tile of TM x TN; a wavefront owns (TM / 2) x (TN / 2) as blocks of 32 x 32.  Lane l supplies
+// row l % 32 of a block's A and W for k = step + l / 32 and receives, in register r, row 4 (l / 32) + 8 (r / 4) + r % 4
+// and column l % 32 of the block.  Staging as above (k-major in LDS, the next step of K on its way meanwhile); rows
+// are padded by two words so that the transposing stores of a wavefront fall into different banks.
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+
+template <typename TA, typename TW, typename TC, int TM, int TN, int TK>
+__global__ __launch_bounds__(GEMM_THREADS) void gemm_nt_matrix_kernel(TC* __restrict__ C, int64_t ldc,
+                                                                      const TA* __restrict__ A, int64_t lda,
+                                                                      const TW* __restrict__ W,
+                                                                      const TW* __restrict__ bias, int M, int N,
+                                                                      int K, int wide_a, int wide_w) {
+  constexpr int BM = TM / 64, BN = TN / 64;         // blocks of 32 x 32 per wavefront, down and across
+  constexpr int GA = TM * TK / 4 / GEMM_THREADS, GW = TN * TK / 4 / GEMM_THREADS;
+  static_assert(GA >= 1 && GW >= 1 && TM % 64 == 0 && TN % 64 == 0 && TK % 2 == 0, "tile sizes");
+  __shared__ float a_s[TK][TM + 2];
+  __shared__ float w_s[TK][TN + 2];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int m0 = blockIdx.y * TM, n0 = blockIdx.x * TN;
+  const int wm = (wave >> 1) * (TM / 2), wn = (wave & 1) * (TN / 2);     // the wavefront's corner in the tile
+  const int l32 = lane & 31, half = lane >> 5;
+  f32x16 acc[BM][BN];
+#pragma unroll
+  for (int i = 0; i < BM; ++i)
+#pragma unroll
+    for (int j = 0; j < BN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  float ra[GA][4], rw[GW][4];
+  auto fetch = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < GA; ++i) {
+      const int gi = tid + i * GEMM_THREADS, row = gi / (TK / 4), k = k0 + (gi % (TK / 4)) * 4;
+      const int m = m0 + row;
+      const int valid = (m < M && k < K) ? (K - k < 4 ? K - k : 4) : 0;
+      if (valid) load4<TA>(ra[i], A + (int64_t)m * lda + k, valid, wide_a != 0);
+      else ra[i][0] = ra[i][1] = ra[i][2] = ra[i][3] = 0.f;
+    }
+#pragma unroll
+    for (int i = 0; i < GW; ++i) {
+      const int gi = tid + i * GEMM_THREADS, row = gi / (TK / 4), k = k0 + (gi % (TK / 4)) * 4;
+      const int n = n0 + row;
+      const int valid = (n < N && k < K) ? (K - k < 4 ? K - k : 4) : 0;
+      if (valid) load4<TW>(rw[i], W + (int64_t)n * K + k, valid, wide_w != 0);
+      else rw[i][0] = rw[i][1] = rw[i][2] = rw[i][3] = 0.f;
+    }
+  };
+  fetch(0);
+  for (int k0 = 0; k0 < K; k0 += TK) {
+#pragma unroll
+    for (int i = 0; i < GA; ++i) {
+      const int gi = tid + i * GEMM_THREADS, row = gi / (TK / 4), kk = (gi % (TK / 4)) * 4;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) a_s[kk + j][row] = ra[i][j];
+    }
+#pragma unroll
+    for (int i = 0; i < GW; ++i) {
+      const int gi = tid + i * GEMM_THREADS, row = gi / (TK / 4), kk = (gi % (TK / 4)) * 4;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) w_s[kk + j][row] = rw[i][j];
+    }
+    __syncthreads();
+    if (k0 + TK < K) fetch(k0 + TK);        // on its way while this step is multiplied
+#pragma unroll
+    for (int k = 0; k < TK; k += 2) {
+      float a[BM], w[BN];
+#pragma unroll
+      for (int i = 0; i < BM; ++i) a[i] = a_s[k + half][wm + i * 32 + l32];
+#pragma unroll
+      for (int j = 0; j < BN; ++j) w[j] = w_s[k + half][wn + j * 32 + l32];
+#pragma unroll
+      for (int i = 0; i < BM; ++i)
+#pragma unroll
+        for (int j = 0; j < BN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], w[j], acc[i][j], 0, 0, 0);
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < BM; ++i)
+#pragma unroll
+    for (int j = 0; j < BN; ++j) {
+      const int n = n0 + wn + j * 32 + l32;
+      if (n >= N) continue;
+      const float b = bias ? Num<TW>::ld(bias + n) : 0.f;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int m = m0 + wm + i * 32 + half * 4 + 8 * (r / 4) + (r % 4);
+        if (m >= M) continue;
+        float v = acc[i][j][r];
+        if (bias) v += b;
+        Num<TC>::st(C + (int64_t)m * ldc + n, v);
+      }
+    }
+}
+
 // in_bf16: A, W and bias are bfloat16 (else float); out_bf16: C is bfloat16 (else float).
 extern "C" int ga_gemm_nt(void* C, int64_t ldc, const void* A, int64_t lda, const void* W,
                           const void* bias, int M, int N, int K, int in_bf16, int out_bf16,
@@ -138,7 +241,13 @@ extern "C" int ga_gemm_nt(void* C, int64_t ldc, const void* A, int64_t lda, cons
   if (M <= 0 || N <= 0) return 0;
   if (K <= 0) return -1;
   const bool few = M <= 16;                 // a decode step's rows: 16 x 32 tiles, long steps of K
-  const int tm = few ? 16 : 64, tn = few ? 32 : 64;
+  // many rows: the matrix cores, in the largest of the tiles 128 x 128, 128 x 64, 64 x 64 that still makes 256 workgroups
+  const bool matrix = M > GEMM_MATRIX_FROM_ROWS;
+  const bool wide = matrix && (int64_t)((M + 127) / 128) * ((N + 127) / 128) >= 256;
+  const bool tall = matrix && !wide && (int64_t)((M + 127) / 128) * ((N + 63) / 64) >= 256;
+  // few rows and few columns: tiles of 16 columns make twice the workgroups
+  const bool narrow = few && (N + 31) / 32 < 256;
+  const int tm = few ? 16 : (wide || tall) ? 128 : 64, tn = few ? (narrow ? 16 : 32) : wide ? 128 : 64;
   dim3 grid((N + tn - 1) / tn, (M + tm - 1) / tm), block(GEMM_THREADS);
   if (grid.y > 65535) return -2;
   // 16-byte loads (8 bytes for bfloat16) need rows that start at multiples of four elements
@@ -147,9 +256,24 @@ extern "C" int ga_gemm_nt(void* C, int64_t ldc, const void* A, int64_t lda, cons
   const int wide_w = (K % 4 == 0 && (uintptr_t)W % unit == 0) ? 1 : 0;
 #define LAUNCH(TA, TW, TC)                                                                                   \
   do {                                                                                                       \
-    if (few)                                                                                                 \
+    if (narrow)                                                                                              \
+      hipLaunchKernelGGL((gemm_nt_kernel<TA, TW, TC, 16, 16, 128>), grid, block, 0, stream, (TC*)C, ldc,     \
+                         (const TA*)A, lda, (const TW*)W, (const TW*)bias, M, N, K, wide_a, wide_w);         \
+    else if (few)                                                                                            \
       hipLaunchKernelGGL((gemm_nt_kernel<TA, TW, TC, 16, 32, 128>), grid, block, 0, stream, (TC*)C, ldc,     \
                          (const TA*)A, lda, (const TW*)W, (const TW*)bias, M, N, K, wide_a, wide_w);         \
+    else if (matrix && wide)                                                                                 \
+      hipLaunchKernelGGL((gemm_nt_matrix_kernel<TA, TW, TC, 128, 128, 32>), grid, block, 0, stream,          \
+                         (TC*)C, ldc, (const TA*)A, lda, (const TW*)W, (const TW*)bias, M, N, K, wide_a,     \
+                         wide_w);                                                                            \
+    else if (matrix && tall)                                                                                 \
+      hipLaunchKernelGGL((gemm_nt_matrix_kernel<TA, TW, TC, 128, 64, 32>), grid, block, 0, stream,           \
+                         (TC*)C, ldc, (const TA*)A, lda, (const TW*)W, (const TW*)bias, M, N, K, wide_a,     \
+                         wide_w);                                                                            \
+    else if (matrix)                                                                                         \
+      hipLaunchKernelGGL((gemm_nt_matrix_kernel<TA, TW, TC, 64, 64, 32>), grid, block, 0, stream,            \
+                         (TC*)C, ldc, (const TA*)A, lda, (const TW*)W, (const TW*)bias, M, N, K, wide_a,     \
+                         wide_w);                                                                            \
     else                                                                                                     \
       hipLaunchKernelGGL((gemm_nt_kernel<TA, TW, TC, 64, 64, 32>), grid, block, 0, stream, (TC*)C, ldc,      \
                          (const TA*)A, lda, (const TW*)W, (const TW*)bias, M, N, K, wide_a, wide_w);         \

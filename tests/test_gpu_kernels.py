@@ -126,6 +126,24 @@ def test_gemm_nt_rows_do_not_depend_on_the_batch():
         assert torch.equal(ops.gemm_nt(a[r:r + 1].contiguous(), w, b)[0], full[r])
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("M,N,K,bias", [(65, 130, 77, True), (200, 1536, 521, False), (128, 128, 32, True),
+                                        (300, 4600, 1000, True), (2048, 1536, 1536, False), (257, 66, 3, True)])
+def test_gemm_nt_on_the_matrix_cores_gives_the_bits_of_the_fma_kernel(dtype, M, N, K, bias):
+    """More than 64 rows go through the 32-bit matrix-core instruction, up to 64 through plain fused multiply-adds; both
+    add an element's terms over ascending k into one accumulator, so the large product must equal, bit for bit, the
+    same rows multiplied 64 and 16 at a time, and one row alone."""
+    from ginfer_amd.kernels import ops
+    a, w = rnd((M, K), dtype, 16), rnd((N, K), dtype, 17)
+    b = rnd((N,), dtype, 18) if bias else None
+    full = ops.gemm_nt(a, w, b, out_dtype=torch.float32)
+    close(full, a.double() @ w.double().t() + (b.double() if bias else 0), 5e-5)
+    for rows in (64, 16):
+        pieces = torch.cat([ops.gemm_nt(a[r:r + rows].contiguous(), w, b, out_dtype=torch.float32) for r in range(0, M, rows)])
+        assert torch.equal(pieces, full), "rows %d at a time: %d elements differ" % (rows, int((pieces != full).sum()))
+    assert torch.equal(ops.gemm_nt(a[M - 1:].contiguous(), w, b, out_dtype=torch.float32)[0], full[M - 1])
+
+
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-4), (torch.bfloat16, 1e-2)])
 @pytest.mark.parametrize("T,nh,nkv,hd,rd,theta", [(128, 32, 8, 128, 128, 1e4), (64, 12, 12, 64, 64, 1e4),
                                                   (9, 6, 3, 48, 48, 5e5), (5, 4, 2, 32, 16, 1e6), (7, 3, 1, 24, 20, 1e4),
