@@ -51,7 +51,10 @@ struct VecLoad {
 
 #define GA_BATCH 4         // loads of keys, and as many of values, that a thread has under way at a time
 
-template <typename T, int VEC>
+// PIPE: the wavefronts beyond those that compute are loaders: they bring tile i + 1 into a second buffer while the
+// others multiply tile i, one barrier a tile (the launcher says when: few workgroups, both buffers fit, and at least
+// as many wavefronts load as compute).
+template <typename T, int VEC, bool PIPE>
 __global__ __launch_bounds__(64 * GA_MAX_WAVES) void paged_attention_generic_kernel(
     T* __restrict__ out, int64_t out_stride, const T* __restrict__ q, int64_t q_stride,
     const T* __restrict__ k_pages, const T* __restrict__ v_pages,
@@ -62,11 +65,11 @@ __global__ __launch_bounds__(64 * GA_MAX_WAVES) void paged_attention_generic_ker
   const int group = nh / nkv, head_blocks = (group + hpw - 1) / hpw;     // hpw heads of a kv group to a workgroup
   const int waves = tq * hpw, threads = blockDim.x;        // wavefronts that compute; all threads load (see the launcher)
   const int ks = hd + KPAD;                      // a key's row in LDS, in floats
-  float* k_s = lds;                              // [64][hd + KPAD]
-  float* v_s = k_s + WAVE * ks;                  // [hd][64 + VPAD]
-  float* q_s = v_s + hd * VS;                    // [waves][hd]
+  const int tile_floats = WAVE * ks + hd * VS;    // a tile in LDS: keys [64][hd + KPAD], then values [hd][64 + 4]
+  constexpr int nbuf = PIPE ? 2 : 1;
+  float* q_s = lds + nbuf * tile_floats;         // [waves][hd]
   float* p_s = q_s + waves * hd;                 // [waves][64]
-  int32_t* page_s = reinterpret_cast<int32_t*>(p_s + waves * WAVE);     // [64]: the page of every key of the tile, or -1
+  int32_t* page_s = reinterpret_cast<int32_t*>(p_s + waves * WAVE);     // [nbuf][64]: the page of every key of a tile, or -1
   const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
   const int g = blockIdx.y / head_blocks, hl = (blockIdx.y % head_blocks) * hpw + wave % hpw;
   const int tl = wave / hpw, h = g * group + hl;                  // the wavefront's token of the workgroup, and head
@@ -107,56 +110,57 @@ __global__ __launch_bounds__(64 * GA_MAX_WAVES) void paged_attention_generic_ker
       const int pi = (tile + (int)threadIdx.x) / page_size;
       return (pi >= first_page && pi <= last_page) ? bt[pi] : -1;
     };
-    int32_t my_page = tile_page((lo_min / WAVE) * WAVE);
     const int per_key = hd / VEC, per_dim = WAVE / VEC, nvec = WAVE * per_key;       // as many vectors of values as of keys
-    for (int tile = (lo_min / WAVE) * WAVE; tile <= pos_max; tile += WAVE) {
-      __syncthreads();                            // the tile before has been read (and q_s is written)
-      if (threadIdx.x < WAVE) page_s[threadIdx.x] = my_page;
-      __syncthreads();
-      my_page = tile_page(tile + WAVE);           // on its way while this tile is loaded and multiplied
-      // keys: VEC dimensions of one key to a load, consecutive threads on consecutive dimensions; values: VEC keys of
-      // one dimension to a load (a page keeps the keys of a dimension side by side).  A batch of both is under way
-      // before the first of it is put into LDS.
-      for (int base = threadIdx.x; base < nvec; base += threads * GA_BATCH) {
-        VecLoad<T, VEC> rk[GA_BATCH], rv[GA_BATCH];
-        bool okk[GA_BATCH], okv[GA_BATCH];
+    // keys: VEC dimensions of one key to a load, consecutive threads on consecutive dimensions; values: VEC keys of
+    // one dimension to a load (a page keeps the keys of a dimension side by side).  A batch of both is under way
+    // before the first of it is put into LDS.
+    constexpr int NB = GA_BATCH;
+    // the threads that load, and this thread's number among them
+    const int loaders = PIPE ? threads - waves * WAVE : threads;
+    const int ltid = PIPE ? (int)threadIdx.x - waves * WAVE : (int)threadIdx.x;
+    VecLoad<T, VEC> rk[NB], rv[NB];
+    bool okk[NB], okv[NB];
+    auto ask = [&](int tile, int base, const int32_t* pages) {
 #pragma unroll
-        for (int u = 0; u < GA_BATCH; ++u) {
-          const int v = base + u * threads;
-          const int j = v / per_key, d = (v - j * per_key) * VEC;
-          const int64_t page = v < nvec ? page_s[j] : -1;
-          okk[u] = page >= 0;
-          if (okk[u]) rk[u].load(k_pages + ((page * nkv + g) * page_size + ((tile + j) % page_size)) * hd + d);
-        }
+      for (int u = 0; u < NB; ++u) {
+        const int v = base + u * loaders;
+        const int j = v / per_key, d = (v - j * per_key) * VEC;
+        const int64_t page = v < nvec ? pages[j] : -1;
+        okk[u] = page >= 0;
+        if (okk[u]) rk[u].load(k_pages + ((page * nkv + g) * page_size + ((tile + j) % page_size)) * hd + d);
+      }
 #pragma unroll
-        for (int u = 0; u < GA_BATCH; ++u) {
-          const int v = base + u * threads;
-          const int d = v / per_dim, j = (v - d * per_dim) * VEC;
-          const int64_t page = v < nvec ? page_s[j] : -1;
-          okv[u] = page >= 0;
-          if (okv[u]) rv[u].load(v_pages + ((page * nkv + g) * hd + d) * page_size + ((tile + j) % page_size));
-        }
+      for (int u = 0; u < NB; ++u) {
+        const int v = base + u * loaders;
+        const int d = v / per_dim, j = (v - d * per_dim) * VEC;
+        const int64_t page = v < nvec ? pages[j] : -1;
+        okv[u] = page >= 0;
+        if (okv[u]) rv[u].load(v_pages + ((page * nkv + g) * hd + d) * page_size + ((tile + j) % page_size));
+      }
+    };
+    auto put = [&](int base, float* k_s, float* v_s) {
 #pragma unroll
-        for (int u = 0; u < GA_BATCH; ++u) {
-          const int v = base + u * threads;
-          const int j = v / per_key, d = (v - j * per_key) * VEC;
-          if (okk[u]) {
+      for (int u = 0; u < NB; ++u) {
+        const int v = base + u * loaders;
+        const int j = v / per_key, d = (v - j * per_key) * VEC;
+        if (okk[u]) {
 #pragma unroll
-            for (int i = 0; i < VEC; ++i) k_s[j * ks + d + i] = rk[u].v[i];
-          }
-        }
-#pragma unroll
-        for (int u = 0; u < GA_BATCH; ++u) {
-          const int v = base + u * threads;
-          const int d = v / per_dim, j = (v - d * per_dim) * VEC;
-          if (okv[u]) {
-#pragma unroll
-            for (int i = 0; i < VEC; ++i) v_s[d * VS + j + i] = rv[u].v[i];
-          }
+          for (int i = 0; i < VEC; ++i) k_s[j * ks + d + i] = rk[u].v[i];
         }
       }
-      __syncthreads();
-      if (!mine || tile > pos || tile + WAVE - 1 < lo) continue;      // not a tile of this wavefront's token
+#pragma unroll
+      for (int u = 0; u < NB; ++u) {
+        const int v = base + u * loaders;
+        const int d = v / per_dim, j = (v - d * per_dim) * VEC;
+        if (okv[u]) {
+#pragma unroll
+          for (int i = 0; i < VEC; ++i) v_s[d * VS + j + i] = rv[u].v[i];
+        }
+      }
+    };
+    // one tile of this wavefront's token, its keys and values in LDS
+    auto attend = [&](int tile, const float* k_s, const float* v_s) {
+      if (!mine || tile > pos || tile + WAVE - 1 < lo) return;        // not a tile of this wavefront's token
       const int c = tile + lane;
       const bool valid = c >= lo && c <= pos;
       float s = -INFINITY;
@@ -209,6 +213,55 @@ __global__ __launch_bounds__(64 * GA_MAX_WAVES) void paged_attention_generic_ker
         }
       }
       __builtin_amdgcn_wave_barrier();
+    };
+    const int first_tile = (lo_min / WAVE) * WAVE;
+    if (!PIPE) {
+      int32_t my_page = tile_page(first_tile);
+      float* k_s = lds;
+      float* v_s = lds + WAVE * ks;
+      for (int tile = first_tile; tile <= pos_max; tile += WAVE) {
+        __syncthreads();                            // the tile before has been read (and q_s is written)
+        if (threadIdx.x < WAVE) page_s[threadIdx.x] = my_page;
+        __syncthreads();
+        my_page = tile_page(tile + WAVE);           // on its way while this tile is loaded and multiplied
+        for (int base = threadIdx.x; base < nvec; base += threads * GA_BATCH) {
+          ask(tile, base, page_s);
+          put(base, k_s, v_s);
+        }
+        __syncthreads();
+        attend(tile, k_s, v_s);
+      }
+    } else {
+      // The pages of a tile are looked up two tiles ahead (by the first wavefront, which computes); the loaders put
+      // tile i + 1 into the buffer that tile i - 1 was read from.
+      const bool loader = wave >= waves;
+      __syncthreads();                              // the run before has been read (and q_s is written)
+      if (threadIdx.x < WAVE) page_s[threadIdx.x] = tile_page(first_tile);
+      __syncthreads();
+      if (loader) {
+        for (int base = ltid; base < nvec; base += loaders * GA_BATCH) {
+          ask(first_tile, base, page_s);
+          put(base, lds, lds + WAVE * ks);
+        }
+      }
+      if (threadIdx.x < WAVE) page_s[WAVE + threadIdx.x] = tile_page(first_tile + WAVE);
+      __syncthreads();
+      int b = 0;
+      for (int tile = first_tile; tile <= pos_max; tile += WAVE, b ^= 1) {
+        if (loader) {
+          if (tile + WAVE <= pos_max) {
+            for (int base = ltid; base < nvec; base += loaders * GA_BATCH) {
+              ask(tile + WAVE, base, page_s + (b ^ 1) * WAVE);
+              put(base, lds + (b ^ 1) * tile_floats, lds + (b ^ 1) * tile_floats + WAVE * ks);
+            }
+          }
+        } else {
+          const int32_t my_page = tile_page(tile + 2 * WAVE);
+          attend(tile, lds + b * tile_floats, lds + b * tile_floats + WAVE * ks);
+          if (threadIdx.x < WAVE) page_s[b * WAVE + threadIdx.x] = my_page;   // read again two tiles on
+        }
+        __syncthreads();
+      }
     }
     run_begin = run_end;
   }
@@ -242,33 +295,45 @@ extern "C" int ga_paged_attention_generic(void* out, int64_t out_stride, const v
   if (tq * hpw > GA_MAX_WAVES) tq = GA_MAX_WAVES / hpw;
   if (tq > tokens) tq = tokens;
   const int waves = tq * hpw;
-  const size_t lds = sizeof(float) * ((size_t)WAVE * (hd + KPAD) + (size_t)hd * VS + (size_t)waves * hd + (size_t)waves * WAVE)
-                     + sizeof(int32_t) * WAVE;
+  const size_t tile_bytes = sizeof(float) * ((size_t)WAVE * (hd + KPAD) + (size_t)hd * VS);
+  const size_t rest_bytes = sizeof(float) * ((size_t)waves * hd + (size_t)waves * WAVE) + sizeof(int32_t) * 2 * WAVE;
   if ((int64_t)nkv * head_blocks > 65535) return -3;
   // A workgroup with few wavefronts that compute (a decoded token: the heads of one kv group) gets further ones that
   // only help to load: a tile's loads are then all under way at once, and a tile's time is one trip to memory.
-  int total_waves = waves;
-  const int vectors = WAVE * hd / (is_bf16 ? 8 : 4);                  // 16-byte loads of a tile's keys (and of its values)
-  while (total_waves < GA_MAX_WAVES && total_waves * WAVE * GA_BATCH < vectors) ++total_waves;
-  dim3 grid((tokens + tq - 1) / tq, nkv * head_blocks), block(WAVE * total_waves);
   // 16-byte loads where a key's dimensions and a page's keys come in whole vectors at 16-byte addresses
   const int vec = is_bf16 ? 8 : 4;
   const bool wide = hd % vec == 0 && page_size % vec == 0 && WAVE % page_size == 0 &&
                     ((uintptr_t)k_pages % 16 == 0) && ((uintptr_t)v_pages % 16 == 0);
-#define LAUNCH(TT, VV)                                                                                               \
+  int total_waves = waves;
+  const int vectors = WAVE * hd / (wide ? vec : 1);                   // loads of a tile's keys (and as many of its values)
+  while (total_waves < GA_MAX_WAVES && total_waves * WAVE * GA_BATCH < vectors) ++total_waves;
+  dim3 grid((tokens + tq - 1) / tq, nkv * head_blocks), block(WAVE * total_waves);
+  // Few workgroups (a decode step: they cannot fill the chip, and each walks its keys alone): two tile buffers, the
+  // next tile loaded while this one is multiplied, where both fit and a thread's one batch of loads is a whole tile.
+  const bool pipelined = (int64_t)grid.x * grid.y <= 256 && 2 * tile_bytes + rest_bytes <= 150 * 1024 &&
+                         GA_MAX_WAVES - waves >= waves;
+  if (pipelined) block.x = WAVE * GA_MAX_WAVES;
+  const size_t lds = (pipelined ? 2 : 1) * tile_bytes + rest_bytes;
+#define LAUNCH(TT, VV, PP)                                                                                           \
   do {                                                                                                               \
-    const void* fn = (const void*)paged_attention_generic_kernel<TT, VV>;                                            \
+    const void* fn = (const void*)paged_attention_generic_kernel<TT, VV, PP>;                                        \
     if (lds > 48 * 1024 && hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) \
       return -4;                                                                                                     \
-    hipLaunchKernelGGL((paged_attention_generic_kernel<TT, VV>), grid, block, lds, stream, (TT*)out, out_stride,     \
+    hipLaunchKernelGGL((paged_attention_generic_kernel<TT, VV, PP>), grid, block, lds, stream, (TT*)out, out_stride, \
                        (const TT*)q, q_stride, (const TT*)k_pages, (const TT*)v_pages, (const int32_t*)block_table,  \
                        table_width, (const int32_t*)token_entry, (const int32_t*)positions, tokens, nh, nkv, hd,      \
                        page_size, window, scale, tq, hpw);                                                           \
   } while (0)
   if (is_bf16) {
-    if (wide) LAUNCH(bf16_t, 8); else LAUNCH(bf16_t, 1);
+    if (wide && pipelined) LAUNCH(bf16_t, 8, true);
+    else if (wide) LAUNCH(bf16_t, 8, false);
+    else if (pipelined) LAUNCH(bf16_t, 1, true);
+    else LAUNCH(bf16_t, 1, false);
   } else {
-    if (wide) LAUNCH(float, 4); else LAUNCH(float, 1);
+    if (wide && pipelined) LAUNCH(float, 4, true);
+    else if (wide) LAUNCH(float, 4, false);
+    else if (pipelined) LAUNCH(float, 1, true);
+    else LAUNCH(float, 1, false);
   }
 #undef LAUNCH
   return GA_CHECK_LAUNCH();

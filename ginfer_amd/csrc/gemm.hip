@@ -3,17 +3,18 @@
 // added in 32-bit before the one rounding (ginfer/core/op/kernels/cuda/gemm_kernel/
 // gemm_kernel.cu:100-121, ginfer/core/op/kernels/cuda/gemv_kernel.cu:52-55).
 //
-// gemm_nt_kernel is the true 32-bit product (plain FMA, no matrix unit, no reduced-precision
-// mode): a tile of C per workgroup, staged through LDS in steps of K.  Every element of C is ONE accumulator
-// summed over k in ascending order, so its bits do not depend on M, on the tile it falls in, on the tile's
-// shape or on the rest of the batch: the two shapes below (64 x 64 for many rows, 16 x 32 for the few rows
-// of a decode step, where only the columns can be shared out) give the same bits for the same row.  It is
-// templated on storage so that it also serves bfloat16 operands (the kernel tests' oracle and the fallback
-// for shapes the matrix-core kernels refuse).
+// Three kernels make the true 32-bit product (no reduced-precision mode anywhere).  In all of them every element of
+// C is ONE accumulator that takes its terms over ascending k as fused multiply-adds, so its bits do not depend on M,
+// on the tile it falls in, on the rest of the batch, or on which of the three ran:
+//   gemm_nt_kernel           17 to 64 rows: plain FMA, a tile of 64 x 64 per workgroup staged through LDS in steps of K;
+//   gemm_nt_matrix_kernel    more rows: the matrix cores' 32-bit instruction over tiles of up to 128 x 128;
+//   gemm_nt_few_rows_kernel  up to 16 rows (a decode step): the matrix cores again, a wavefront per 16 columns,
+//                            operands straight from memory.
+// They are templated on storage, so that they also serve bfloat16 operands (the kernel tests' oracle and the
+// fallback for shapes the bfloat16 kernels refuse).
 //
 // A step of K is asked for (in 16-byte loads where rows allow it, consecutive lanes on consecutive elements)
-// while the step before is being multiplied: the loads' way from memory, which a workgroup of a decode step
-// would otherwise wait out some hundred times in a row, runs beside the arithmetic.
+// while the step before is being multiplied.
 #include "common.cuh"
 #include "ginfer_amd.h"   // the entry points below are checked against their declarations
 
@@ -234,6 +235,127 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_nt_matrix_kernel(TC* __rest
     }
 }
 
+// Up to 16 rows (a decode step): one wavefront per 16 columns, no LDS.  v_mfma_f32_16x16x4_f32 takes, from lane l, row
+// l % 16 of A and of W at k = step + l / 16, and adds its four products into the accumulator in ascending k as fused
+// multiply-adds (the same measurement as above): the bits of the other two kernels again.  A lane loads four
+// consecutive elements of its row (16 bytes; the four lanes of a row 64 consecutive bytes), which is the operand of
+// four steps once the four lanes of the row have exchanged elements (a 4 x 4 transpose in two rounds of swaps between
+// lanes 16 and 32 apart).  Of FEW_SETS sets of FEW_DEPTH such loads of A and of W one is multiplied while the others
+// are under way.
+// Register r of lane l receives row 4 (l / 16) + r, column l % 16.
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+#define FEW_DEPTH 8
+#define FEW_SETS 2
+
+// x[c] of the lane 16 s + i (s = 0..3) becomes what was x[s] of the lane 16 c + i
+__device__ __forceinline__ void transpose_over_lane_rows(float (&x)[4], int s) {
+  const bool odd = s & 1, high = s & 2;
+#pragma unroll
+  for (int c = 0; c < 4; c += 2) {
+    const float give = odd ? x[c] : x[c + 1];
+    const float got = __shfl_xor(give, 16, 64);
+    if (odd) x[c] = got; else x[c + 1] = got;
+  }
+#pragma unroll
+  for (int c = 0; c < 2; ++c) {
+    const float give = high ? x[c] : x[c + 2];
+    const float got = __shfl_xor(give, 32, 64);
+    if (high) x[c] = got; else x[c + 2] = got;
+  }
+}
+
+// four consecutive elements at an address that is a multiple of four elements, no questions asked
+template <typename T>
+__device__ __forceinline__ void load4_aligned(float (&v)[4], const T* p) {
+  load4<T>(v, p, 4, true);
+}
+
+template <typename TA, typename TW, typename TC>
+__global__ __launch_bounds__(64) void gemm_nt_few_rows_kernel(TC* __restrict__ C, int64_t ldc,
+                                                              const TA* __restrict__ A, int64_t lda,
+                                                              const TW* __restrict__ W,
+                                                              const TW* __restrict__ bias, int M, int N, int K,
+                                                              int wide_a, int wide_w) {
+  const int lane = threadIdx.x, i = lane & 15, kq = lane >> 4;
+  const int n = blockIdx.x * 16 + i;
+  const bool a_ok = i < M, w_ok = n < N;
+  // a lane whose row does not exist reads row 0 and drops what it read: no branch in the loop
+  const TA* pa = A + (int64_t)(a_ok ? i : 0) * lda + 4 * kq;
+  const TW* pw = W + (int64_t)(w_ok ? n : 0) * K + 4 * kq;
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  // FEW_SETS sets of FEW_DEPTH loads of A and of W: one is multiplied while the others are on their way (a wavefront
+  // has the registers of its SIMD to itself: so few wavefronts run here that the bytes each keeps under way are what
+  // decides)
+  float a[FEW_SETS][FEW_DEPTH][4], w[FEW_SETS][FEW_DEPTH][4];
+  // whole chunks of 16 elements, with aligned rows, take the loop without branches; what is left of K (and everything,
+  // with rows that are not aligned) takes the careful loads afterwards: ascending k all the same
+  const int chunks = (wide_a && wide_w) ? K / 16 : 0;
+  auto multiply = [&](float (&x)[4], float (&y)[4]) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      x[e] = a_ok ? x[e] : 0.f;
+      y[e] = w_ok ? y[e] : 0.f;
+    }
+    transpose_over_lane_rows(x, kq);
+    transpose_over_lane_rows(y, kq);
+#pragma unroll
+    for (int st = 0; st < 4; ++st) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(x[st], y[st], acc, 0, 0, 0);
+  };
+  // the loads of the chunks first .. first + FEW_DEPTH - 1 (those of them that exist; `all`: they all do)
+  auto fetch = [&](float (&x)[FEW_DEPTH][4], float (&y)[FEW_DEPTH][4], int first, bool all) {
+#pragma unroll
+    for (int d = 0; d < FEW_DEPTH; ++d)
+      if (all || first + d < chunks) {
+        load4_aligned<TA>(x[d], pa + (first + d) * 16);
+        load4_aligned<TW>(y[d], pw + (first + d) * 16);
+      }
+  };
+  auto multiply_set = [&](float (&x)[FEW_DEPTH][4], float (&y)[FEW_DEPTH][4], int first, bool all) {
+#pragma unroll
+    for (int d = 0; d < FEW_DEPTH; ++d)
+      if (all || first + d < chunks) multiply(x[d], y[d]);
+  };
+#pragma unroll
+  for (int st = 0; st < FEW_SETS - 1; ++st) fetch(a[st], w[st], st * FEW_DEPTH, false);
+  int c0 = 0;
+  // while every set of a round and the sets asked for in it lie inside K nothing in the loop is conditional: the
+  // compiler then counts the loads and waits for just those of the set it multiplies
+  for (; c0 + (2 * FEW_SETS - 1) * FEW_DEPTH <= chunks; c0 += FEW_SETS * FEW_DEPTH) {
+#pragma unroll
+    for (int st = 0; st < FEW_SETS; ++st) {
+      fetch(a[(st + FEW_SETS - 1) % FEW_SETS], w[(st + FEW_SETS - 1) % FEW_SETS], c0 + (st + FEW_SETS - 1) * FEW_DEPTH, true);
+      multiply_set(a[st], w[st], c0 + st * FEW_DEPTH, true);
+    }
+  }
+  for (; c0 < chunks; c0 += FEW_SETS * FEW_DEPTH) {
+#pragma unroll
+    for (int st = 0; st < FEW_SETS; ++st) {
+      fetch(a[(st + FEW_SETS - 1) % FEW_SETS], w[(st + FEW_SETS - 1) % FEW_SETS], c0 + (st + FEW_SETS - 1) * FEW_DEPTH, false);
+      multiply_set(a[st], w[st], c0 + st * FEW_DEPTH, false);
+    }
+  }
+  for (int k0 = chunks * 16; k0 < K; k0 += 16) {
+    const int k = k0 + 4 * kq;
+    const int valid = k < K ? (K - k < 4 ? K - k : 4) : 0;
+    float x[4] = {0.f, 0.f, 0.f, 0.f}, y[4] = {0.f, 0.f, 0.f, 0.f};
+    if (valid) {
+      load4<TA>(x, pa + k0, valid, false);
+      load4<TW>(y, pw + k0, valid, false);
+    }
+    multiply(x, y);
+  }
+  if (!w_ok) return;
+  const float b = bias ? Num<TW>::ld(bias + n) : 0.f;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int m = 4 * kq + r;
+    if (m >= M) continue;
+    float v = acc[r];
+    if (bias) v += b;
+    Num<TC>::st(C + (int64_t)m * ldc + n, v);
+  }
+}
+
 // in_bf16: A, W and bias are bfloat16 (else float); out_bf16: C is bfloat16 (else float).
 extern "C" int ga_gemm_nt(void* C, int64_t ldc, const void* A, int64_t lda, const void* W,
                           const void* bias, int M, int N, int K, int in_bf16, int out_bf16,
@@ -245,9 +367,7 @@ extern "C" int ga_gemm_nt(void* C, int64_t ldc, const void* A, int64_t lda, cons
   const bool matrix = M > GEMM_MATRIX_FROM_ROWS;
   const bool wide = matrix && (int64_t)((M + 127) / 128) * ((N + 127) / 128) >= 256;
   const bool tall = matrix && !wide && (int64_t)((M + 127) / 128) * ((N + 63) / 64) >= 256;
-  // few rows and few columns: tiles of 16 columns make twice the workgroups
-  const bool narrow = few && (N + 31) / 32 < 256;
-  const int tm = few ? 16 : (wide || tall) ? 128 : 64, tn = few ? (narrow ? 16 : 32) : wide ? 128 : 64;
+  const int tm = few ? 16 : (wide || tall) ? 128 : 64, tn = few ? 16 : wide ? 128 : 64;
   dim3 grid((N + tn - 1) / tn, (M + tm - 1) / tm), block(GEMM_THREADS);
   if (grid.y > 65535) return -2;
   // 16-byte loads (8 bytes for bfloat16) need rows that start at multiples of four elements
@@ -256,11 +376,8 @@ extern "C" int ga_gemm_nt(void* C, int64_t ldc, const void* A, int64_t lda, cons
   const int wide_w = (K % 4 == 0 && (uintptr_t)W % unit == 0) ? 1 : 0;
 #define LAUNCH(TA, TW, TC)                                                                                   \
   do {                                                                                                       \
-    if (narrow)                                                                                              \
-      hipLaunchKernelGGL((gemm_nt_kernel<TA, TW, TC, 16, 16, 128>), grid, block, 0, stream, (TC*)C, ldc,     \
-                         (const TA*)A, lda, (const TW*)W, (const TW*)bias, M, N, K, wide_a, wide_w);         \
-    else if (few)                                                                                            \
-      hipLaunchKernelGGL((gemm_nt_kernel<TA, TW, TC, 16, 32, 128>), grid, block, 0, stream, (TC*)C, ldc,     \
+    if (few)                                                                                                 \
+      hipLaunchKernelGGL((gemm_nt_few_rows_kernel<TA, TW, TC>), grid, dim3(64), 0, stream, (TC*)C, ldc,      \
                          (const TA*)A, lda, (const TW*)W, (const TW*)bias, M, N, K, wide_a, wide_w);         \
     else if (matrix && wide)                                                                                 \
       hipLaunchKernelGGL((gemm_nt_matrix_kernel<TA, TW, TC, 128, 128, 32>), grid, block, 0, stream,          \
