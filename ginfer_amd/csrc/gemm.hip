@@ -362,7 +362,7 @@ extern "C" int ga_gemm_nt(void* C, int64_t ldc, const void* A, int64_t lda, cons
                           hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (K <= 0) return -1;
-  const bool few = M <= 16;                 // a decode step's rows: 16 x 32 tiles, long steps of K
+  const bool few = M <= 16;                 // a decode step's rows: a wavefront per 16 columns
   // many rows: the matrix cores, in the largest of the tiles 128 x 128, 128 x 64, 64 x 64 that still makes 256 workgroups
   const bool matrix = M > GEMM_MATRIX_FROM_ROWS;
   const bool wide = matrix && (int64_t)((M + 127) / 128) * ((N + 127) / 128) >= 256;
