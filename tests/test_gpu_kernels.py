@@ -126,6 +126,48 @@ def test_gemm_nt_rows_do_not_depend_on_the_batch():
         assert torch.equal(ops.gemm_nt(a[r:r + 1].contiguous(), w, b)[0], full[r])
 
 
+def _fma32(a, b, c):
+    """round_to_float32(a * b + c) with ONE rounding, for float32 values a, b, c: the sum is taken exactly (as a ratio
+    of integers) and rounded to 24 bits, ties to even."""
+    from fractions import Fraction
+    exact = Fraction(float(a)) * Fraction(float(b)) + Fraction(float(c))
+    if exact == 0:
+        return np.float32(0.0)
+    sign = -1 if exact < 0 else 1
+    mag = abs(exact)
+    e = mag.numerator.bit_length() - mag.denominator.bit_length()          # 2^e <= mag < 2^(e+2), roughly
+    while Fraction(2) ** e > mag:
+        e -= 1
+    while Fraction(2) ** (e + 1) <= mag:
+        e += 1
+    e = max(e, -126)                                                       # subnormals keep the exponent of 2^-126
+    scaled = mag / Fraction(2) ** (e - 23)                                 # 24 bits before the point
+    q, r = divmod(scaled.numerator, scaled.denominator)
+    twice = 2 * r
+    if twice > scaled.denominator or (twice == scaled.denominator and q % 2 == 1):
+        q += 1
+    return np.float32(sign * float(Fraction(q) * Fraction(2) ** (e - 23)))
+
+
+@pytest.mark.parametrize("M", [3, 40, 70])
+def test_gemm_nt_32_bit_is_the_chain_of_fused_multiply_adds_over_ascending_k(M):
+    """What the 32-bit product IS, stated without any kernel: every element starts at zero and takes its K terms in
+    ascending order, each as one fused multiply-add (one rounding); the bias is added last.  3 rows run on the
+    16x16x4 matrix instruction, 40 on plain FMA, 70 on the 32x32x2 matrix instruction: all three must give these bits."""
+    from ginfer_amd.kernels import ops
+    N, K = 5, 37
+    a, w, b = rnd((M, K), torch.float32, 31), rnd((N, K), torch.float32, 32), rnd((N,), torch.float32, 33)
+    got = ops.gemm_nt(a, w, b).cpu().numpy()
+    an, wn, bn = a.cpu().numpy(), w.cpu().numpy(), b.cpu().numpy()
+    for m in sorted({0, 1, M // 2, M - 1}):
+        for n in range(N):
+            acc = np.float32(0.0)
+            for k in range(K):
+                acc = _fma32(an[m, k], wn[n, k], acc)
+            want = np.float32(acc + bn[n])
+            assert got[m, n].tobytes() == want.tobytes(), "element (%d, %d): %r, the chain gives %r" % (m, n, got[m, n], want)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("M,N,K,bias", [(65, 130, 77, True), (200, 1536, 521, False), (128, 128, 32, True),
                                         (300, 4600, 1000, True), (2048, 1536, 1536, False), (257, 66, 3, True)])
