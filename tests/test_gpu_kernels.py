@@ -149,6 +149,32 @@ def _fma32(a, b, c):
     return np.float32(sign * float(Fraction(q) * Fraction(2) ** (e - 23)))
 
 
+@pytest.mark.parametrize("seed", range(30))
+def test_gemm_nt_at_drawn_sizes(seed):
+    """Rows, columns and K drawn at random (odd sizes, rows of a wider buffer that start at odd elements): the plain
+    product, and the same bits for the same rows multiplied one, 16 and 64 at a time."""
+    import random
+    from ginfer_amd.kernels import ops
+    rng = random.Random(700 + seed)
+    M = rng.choice([1, 2, 3, 7, 8, 15, 16, 17, 33, 64, 65, 100, 129, 300])
+    N = rng.choice([1, 5, 16, 17, 31, 64, 100, 130, 257, 1000])
+    K = rng.choice([1, 3, 4, 8, 15, 16, 17, 31, 32, 33, 64, 100, 127, 128, 129, 500, 1536])
+    dtype = rng.choice([torch.float32, torch.float32, torch.bfloat16])
+    a, w = rnd((M, K), dtype, 40 + seed), rnd((N, K), dtype, 80 + seed)
+    b = rnd((N,), dtype, 120 + seed) if rng.random() < 0.5 else None
+    if rng.random() < 0.4:
+        off = rng.choice([0, 1, 4])
+        wide = torch.zeros((M, K + 8), dtype=dtype, device=a.device)
+        wide[:, off:off + K] = a
+        a = wide[:, off:off + K]
+    full = ops.gemm_nt(a, w, b, out_dtype=torch.float32)
+    close(full, a.double() @ w.double().t() + (b.double() if b is not None else 0), 5e-5)
+    for rows in (1, 16, 64):
+        if rows < M:
+            pieces = torch.cat([ops.gemm_nt(a[r:r + rows], w, b, out_dtype=torch.float32) for r in range(0, M, rows)])
+            assert torch.equal(pieces, full), "%d x %d x %d %s, %d rows at a time" % (M, N, K, dtype, rows)
+
+
 @pytest.mark.parametrize("M", [3, 40, 70])
 def test_gemm_nt_32_bit_is_the_chain_of_fused_multiply_adds_over_ascending_k(M):
     """What the 32-bit product IS, stated without any kernel: every element starts at zero and takes its K terms in
@@ -339,6 +365,34 @@ def test_paged_attention_generic(dtype, tol, nh, nkv, hd, seqs):
         out = ops.paged_attention_generic(a["q"], a["k_pages"], a["v_pages"], a["block_table"], a["token_entry"],
                                           a["positions"], nh, nkv, hd, 1.0 / math.sqrt(hd))
         close(out, ref, tol)
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_paged_attention_generic_at_drawn_sizes_whatever_shares_a_workgroup(seed):
+    """Head layouts, head sizes, page sizes, windows and mixes of requests drawn at random, in 32-bit: the plain result,
+    and the same bits whether a workgroup holds one token, two, or what the library chooses (which also decides whether
+    the loading wavefronts and the second tile buffer of a step with few workgroups are used)."""
+    import random
+    from ginfer_amd.kernels import ops
+    rng = random.Random(300 + seed)
+    nkv, group = rng.choice([1, 2, 3, 4]), rng.choice([1, 2, 3, 6, 7, 8])
+    nh, hd, ps = nkv * group, rng.choice([16, 24, 32, 48, 64, 80, 128]), rng.choice([4, 8, 16, 32])
+    window = rng.choice([None, None, None, 5, 40, 100])
+    kind = rng.choice(["single tokens", "portions and single tokens", "a prompt"])
+    if kind == "single tokens":
+        seqs = [(1, rng.randint(1, 300)) for _ in range(rng.randint(1, 6))]
+    elif kind == "a prompt":
+        n = rng.randint(2, 120)
+        seqs = [(n, n + rng.choice([0, 0, 17, 64]))]
+    else:
+        seqs = [(ql, ql + rng.randint(0, 150)) for ql in (rng.choice([1, 1, 2, 5, 33]) for _ in range(rng.randint(2, 5)))]
+    a, ref, _ = _paged_case(seqs, nh, nkv, hd, ps, torch.float32, seed=seed, window=window)
+    outs = [ops.paged_attention_generic(a["q"], a["k_pages"], a["v_pages"], a["block_table"], a["token_entry"],
+                                        a["positions"], nh, nkv, hd, 1.0 / math.sqrt(hd), window=window,
+                                        tokens_per_workgroup=tq) for tq in (0, 1, 2)]
+    close(outs[0], ref, 1e-5)
+    what = "%s %s, %d heads in %d groups of size %d, pages of %d, window %s" % (kind, seqs, nh, nkv, hd, ps, window)
+    assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2]), what
 
 
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-5), (torch.bfloat16, 2e-2)])
