@@ -1,7 +1,9 @@
-// Paged attention, the general kernel: any mix of prompt portions and single decoded tokens, any
+// Paged attention, the general kernels: any mix of prompt portions and single decoded tokens, any
 // head size up to 256, full or windowed, 32-bit or bfloat16 storage with
-// 32-bit scores, softmax and accumulators.  It is the whole of the 32-bit path and the fallback of
-// the bfloat16 path.
+// 32-bit scores, softmax and accumulators.  They are the whole of the 32-bit path and the fallback of
+// the bfloat16 path.  Two kernels that give the same bits: a wavefront per (token, query head), described first, for
+// steps of single tokens and for every size; and the matrix cores' 32-bit instruction (further down) for steps that
+// hold prompt portions, at head sizes in steps of 16 up to 128.
 //
 // One wavefront per (token, query head).  A token is self-describing: `token_entry[t]` names its
 // row of the block table and `positions[t]` its absolute position p, so it attends to the keys
@@ -21,6 +23,8 @@
 // lane per dimension meets a bank twice), and every wavefront takes its operands from there.  What a wavefront computes, and in which order it adds,
 // does not depend on what shares the workgroup with it: its dot products run over the dimensions in ascending order,
 // its sums over the keys of a tile likewise, and tiles follow each other in ascending order.
+#include <type_traits>
+
 #include "common.cuh"
 #include "ginfer_amd.h"   // the entry points below are checked against their declarations
 
@@ -185,7 +189,7 @@ __global__ __launch_bounds__(64 * GA_MAX_WAVES) void paged_attention_generic_ker
       const float m_new = fmaxf(m, wave_max(s));   // finite: every tile holds at least one valid key
       const float p = valid ? expf(s - m_new) : 0.f;
       const float alpha = expf(m - m_new);         // exp(-inf) = 0 on the first tile
-      l = l * alpha + wave_sum(p);
+      l = __builtin_fmaf(l, alpha, wave_sum(p));
       m = m_new;
       p_s[wave * WAVE + lane] = p;                 // read by this wavefront alone: LDS keeps a wavefront's order
       __builtin_amdgcn_wave_barrier();
@@ -275,6 +279,324 @@ __global__ __launch_bounds__(64 * GA_MAX_WAVES) void paged_attention_generic_ker
   }
 }
 
+// The same attention on the matrix cores, for steps that hold prompt portions.  v_mfma_f32_16x16x4_f32 takes 32-bit
+// operands and adds its four products into the accumulator in ascending k as fused multiply-adds, so a score is the
+// chain over ascending dimensions, and an output element the chain over ascending keys, that the kernel above computes:
+// the same bits (a key that a token does not see enters its chain as a product with zero, which leaves the sum as it
+// is; only a sum that is exactly -0 would become +0).  A wavefront holds one head of MA_COLS neighbouring tokens: the
+// scores of a tile are [64 keys][16 tokens] in four accumulators, lane (token, kq) holding keys 16 b + 4 kq + r of its
+// token, so the maximum and the sum over a tile's keys are taken in registers and two exchanges, the sum in the order
+// of the butterfly above: key bits 5, 4, 3, 2, 1, 0.  The probabilities go through LDS, half a tile at a time, to
+// become the second operand of the product with the values.  Queries stay in registers.  A workgroup holds `tq`
+// groups of MA_COLS tokens and `hpw` heads of one kv head; its tokens fall into runs of one request as above, and a
+// token outside the run, or one that sees no key of the tile, keeps its state through the tile: scale one,
+// probabilities zero.  Keys and values beyond the run's range are put into LDS as zeros: what lies in a page beyond a
+// request's last key may be anything, and zero times it must be zero.  The wavefronts beyond those that compute are
+// loaders: they bring tile i + 1 into a second buffer while the others multiply tile i, one barrier a tile.
+#define MA_COLS 16
+#define MA_MAX_COMPUTE 12
+#define MA_LOADERS 4
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+template <typename T, int VEC, int HD>
+__global__ __launch_bounds__(64 * (MA_MAX_COMPUTE + MA_LOADERS)) void paged_attention_matrix_kernel(
+    T* __restrict__ out, int64_t out_stride, const T* __restrict__ q, int64_t q_stride,
+    const T* __restrict__ k_pages, const T* __restrict__ v_pages,
+    const int32_t* __restrict__ block_table, int table_width,
+    const int32_t* __restrict__ token_entry, const int32_t* __restrict__ positions, int tokens, int nh, int nkv,
+    int page_size, int window, float scale, int tq, int hpw) {
+  extern __shared__ float lds[];
+  constexpr int hd = HD;
+  // A row of keys in LDS holds dimension d at (d % 4) * (HD / 4) + d / 4, a row of values key j at (j % 4) * 16 + j / 4:
+  // lane (row, kq) of an operand wants every fourth element from kq on, and so reads four of them at a time; the rows'
+  // padding puts the 16 rows of a read on different banks.
+  constexpr int KS = HD + KPAD;
+  constexpr int NBLK = HD / 16;                  // blocks of 16 dimensions of the output
+  constexpr int tile_floats = WAVE * KS + HD * VS;
+  const int group = nh / nkv, head_blocks = (group + hpw - 1) / hpw;
+  const int waves = tq * hpw, span = tq * MA_COLS;          // wavefronts that compute; tokens of the workgroup
+  float* p_all = lds + 2 * tile_floats;          // [waves][32][MA_COLS]
+  int64_t* base_s = reinterpret_cast<int64_t*>(p_all + waves * (WAVE / 2) * MA_COLS);      // [2][64]
+  int32_t* plain_s = reinterpret_cast<int32_t*>(base_s + 2 * WAVE);                        // [2]
+  const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
+  const int col = lane & 15, kq = lane >> 4;
+  const bool loader = wave >= waves;
+  const int ct = wave / hpw;                                      // the wavefront's group of tokens
+  // the workgroups of the step's last tokens come first: they have the most keys to walk, and the compute units that
+  // finish the short ones early take what is left
+  const int ny = nkv * head_blocks, by = blockIdx.x % ny, bx = gridDim.x / ny - 1 - blockIdx.x / ny;
+  const int g = by / head_blocks, hl = (by % head_blocks) * hpw + wave % hpw;
+  const int h = g * group + hl;
+  const int64_t t0 = (int64_t)bx * span;
+  const int tl = ct * MA_COLS + col;                              // this lane's token of the workgroup: a column of the scores
+  const int64_t t = t0 + tl;
+  const bool live = !loader && hl < group && t < tokens;
+  const int pos = live ? positions[t] : -1;
+  const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  const int loaders = (int)blockDim.x - waves * WAVE, ltid = (int)threadIdx.x - waves * WAVE;
+  // The workgroup's tokens from `begin` on that are of one request: the run's end, and the range of keys that its
+  // tokens see.  Loaders and the others walk the same runs and tiles, and meet at the same barriers.
+  struct Run { int entry, end, lo_min, pos_max; };
+  auto next_run = [&](int begin) -> Run {
+    Run r{token_entry[t0 + begin], begin, 0x7fffffff, -1};
+    while (r.end < span && t0 + r.end < tokens && token_entry[t0 + r.end] == r.entry) {
+      const int p = positions[t0 + r.end];
+      const int l0 = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+      r.lo_min = l0 < r.lo_min ? l0 : r.lo_min;
+      r.pos_max = p > r.pos_max ? p : r.pos_max;
+      ++r.end;
+    }
+    return r;
+  };
+
+  if (loader) {
+    for (int run_begin = 0; run_begin < span && t0 + run_begin < tokens;) {
+      const Run run = next_run(run_begin);
+      const int lo_min = run.lo_min, pos_max = run.pos_max;
+      const int32_t* bt = block_table + (int64_t)run.entry * table_width;
+      const int first_page = lo_min / page_size, last_page = pos_max / page_size;
+      // where the page of key `tile + ltid` begins for this kv head, in elements (both caches keep page_size * hd
+      // elements per page and kv head), or -1 for a key without a page; by the first loading wavefront
+      auto tile_base = [&](int tile) -> int64_t {
+        if (tile > pos_max) return -1;
+        const int pi = (tile + ltid) / page_size;
+        if (pi < first_page || pi > last_page) return -1;
+        const int64_t page = bt[pi];
+        return page >= 0 ? (page * nkv + g) * page_size * hd : -1;
+      };
+      constexpr int per_key = HD / VEC, per_dim = WAVE / VEC, nvec = WAVE * per_key;
+      constexpr int NB = VEC == 1 ? 8 : 4;         // loads of keys, and as many of values, under way in a thread
+      // a tile into a buffer: all its loads of a round are under way before the first is put into LDS; what lies
+      // outside the run's keys, or has no page, becomes zero.  `plain`: every key of the tile has a page and is one of
+      // the run's: nothing to ask.
+      auto load_tile = [&](int tile, const int64_t* bases, float* k_s, float* v_s, auto plain_tag) {
+        constexpr bool plain = decltype(plain_tag)::value;
+        for (int base = ltid; base < nvec; base += loaders * NB) {
+          VecLoad<T, VEC> rk[NB], rv[NB];
+#pragma unroll
+          for (int u = 0; u < NB; ++u) {
+            const int v = base + u * loaders;
+            const int j = v / per_key, d = (v - j * per_key) * VEC;
+            // with 16-byte loads a page's size divides 64, and a tile begins where a page does
+            const int in_page = VEC > 1 ? (j & (page_size - 1)) : (tile + j) % page_size;
+            if (plain) {
+              if (nvec % (MA_LOADERS * WAVE * NB) == 0 || v < nvec) rk[u].load(k_pages + bases[j] + in_page * hd + d);
+            } else {
+              const int64_t at = v < nvec ? bases[j] : -1;
+              rk[u].zero();
+              if (at >= 0 && tile + j >= lo_min && tile + j <= pos_max) rk[u].load(k_pages + at + in_page * hd + d);
+            }
+          }
+#pragma unroll
+          for (int u = 0; u < NB; ++u) {
+            const int v = base + u * loaders;
+            const int d = v / per_dim, j = (v - d * per_dim) * VEC;
+            const int in_page = VEC > 1 ? (j & (page_size - 1)) : (tile + j) % page_size;
+            if (plain) {
+              if (nvec % (MA_LOADERS * WAVE * NB) == 0 || v < nvec) rv[u].load(v_pages + bases[j] + d * page_size + in_page);
+            } else {
+              const int64_t at = v < nvec ? bases[j] : -1;
+              rv[u].zero();
+              if (at >= 0) rv[u].load(v_pages + at + d * page_size + in_page);
+            }
+          }
+#pragma unroll
+          for (int u = 0; u < NB; ++u) {
+            const int v = base + u * loaders;
+            if (nvec % (MA_LOADERS * WAVE * NB) != 0 && v >= nvec) continue;
+            const int j = v / per_key, d = (v - j * per_key) * VEC;
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) k_s[j * KS + ((d + i) & 3) * (HD / 4) + ((d + i) >> 2)] = rk[u].v[i];
+          }
+#pragma unroll
+          for (int u = 0; u < NB; ++u) {
+            const int v = base + u * loaders;
+            if (nvec % (MA_LOADERS * WAVE * NB) != 0 && v >= nvec) continue;
+            const int d = v / per_dim, j = (v - d * per_dim) * VEC;
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) {
+              const int c = tile + j + i;
+              const bool out_of_range = !plain && (c < lo_min || c > pos_max);
+              v_s[d * VS + ((j + i) & 3) * (WAVE / 4) + ((j + i) >> 2)] = out_of_range ? 0.f : rv[u].v[i];
+            }
+          }
+        }
+      };
+      // a tile's bases into LDS, and whether the tile is plain
+      auto note_tile = [&](int tile, int slot) {
+        if (ltid >= WAVE) return;
+        const int64_t at = tile_base(tile);
+        base_s[slot * WAVE + ltid] = at;
+        const bool plain = __ballot(at >= 0) == ~0ull && tile >= lo_min && tile + WAVE - 1 <= pos_max;
+        if (ltid == 0) plain_s[slot] = plain ? 1 : 0;
+      };
+      auto load = [&](int tile, int slot) {
+        float* buf = lds + slot * tile_floats;
+        if (plain_s[slot]) load_tile(tile, base_s + slot * WAVE, buf, buf + WAVE * KS, std::true_type{});
+        else load_tile(tile, base_s + slot * WAVE, buf, buf + WAVE * KS, std::false_type{});
+      };
+      const int first_tile = (lo_min / WAVE) * WAVE;
+      __syncthreads();                              // the run before has been read
+      note_tile(first_tile, 0);
+      __syncthreads();
+      load(first_tile, 0);
+      note_tile(first_tile + WAVE, 1);
+      __syncthreads();
+      int b = 0;
+      for (int tile = first_tile; tile <= pos_max; tile += WAVE, b ^= 1) {
+        if (tile + WAVE <= pos_max) load(tile + WAVE, b ^ 1);
+        note_tile(tile + 2 * WAVE, b);               // read two tiles on
+        __syncthreads();
+      }
+      run_begin = run.end;
+    }
+    return;
+  }
+
+  float qr[HD / 4];                                    // the token's query at dimensions 4 i + kq
+#pragma unroll
+  for (int i = 0; i < HD / 4; ++i) qr[i] = 0.f;
+  if (live) {
+    const T* qp = q + t * q_stride + (int64_t)h * hd + kq;
+#pragma unroll
+    for (int i = 0; i < HD / 4; ++i) qr[i] = Num<T>::ld(qp + 4 * i);
+  }
+  float m = -INFINITY, l = 0.f;
+  f32x4 acc[NBLK];
+#pragma unroll
+  for (int i = 0; i < NBLK; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float* p_s = p_all + wave * (WAVE / 2) * MA_COLS;
+  for (int run_begin = 0; run_begin < span && t0 + run_begin < tokens;) {
+    const Run run = next_run(run_begin);
+    const bool mine = live && tl >= run_begin && tl < run.end;
+    // one tile for this wavefront's tokens, its keys and values in LDS
+    auto attend = [&](int tile, const float* k_s, const float* v_s) {
+      const bool active = mine && !(tile > pos || tile + WAVE - 1 < lo);
+      if (__ballot(active) == 0) return;                 // no token of this wavefront sees the tile
+      // scores: block b holds keys 16 b .. 16 b + 15 of the tile; lane (col, kq) gives key col's dimension 4 i + kq
+      f32x4 s[4];
+#pragma unroll
+      for (int b = 0; b < 4; ++b) s[b] = f32x4{0.f, 0.f, 0.f, 0.f};
+      const float* ka = k_s + col * KS + kq * (HD / 4);
+#pragma unroll
+      for (int n = 0; n < HD / 16; ++n) {
+        float4 a[4];
+#pragma unroll
+        for (int b = 0; b < 4; ++b) a[b] = *reinterpret_cast<const float4*>(ka + b * 16 * KS + 4 * n);
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+#pragma unroll
+          for (int b = 0; b < 4; ++b)
+            s[b] = __builtin_amdgcn_mfma_f32_16x16x4f32(reinterpret_cast<const float*>(&a[b])[e], qr[4 * n + e], s[b], 0, 0, 0);
+      }
+      // element r of block b: key 16 b + 4 kq + r of the tile, for this lane's token.  Where every token of the
+      // wavefront sees all 64 keys (most tiles of a long prompt) nothing needs a mask: the same arithmetic without
+      // the selects.
+      const bool whole = __ballot(active && tile >= lo && tile + WAVE - 1 <= pos) == ~0ull;
+      float m_new, alpha;
+      if (whole) {
+        float mx = -INFINITY;
+#pragma unroll
+        for (int b = 0; b < 4; ++b)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            s[b][r] = s[b][r] * scale;
+            mx = fmaxf(mx, s[b][r]);
+          }
+        mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+        mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
+        m_new = fmaxf(m, mx);
+        alpha = expf(m - m_new);                   // exp(-inf) = 0 on a token's first tile
+#pragma unroll
+        for (int b = 0; b < 4; ++b)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) s[b][r] = expf(s[b][r] - m_new);
+      } else {
+        float mx = -INFINITY;
+#pragma unroll
+        for (int b = 0; b < 4; ++b)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int c = tile + 16 * b + 4 * kq + r;
+            s[b][r] = (active && c >= lo && c <= pos) ? s[b][r] * scale : -INFINITY;
+            mx = fmaxf(mx, s[b][r]);
+          }
+        mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+        mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
+        m_new = fmaxf(m, mx);                      // finite for a token that sees the tile: it holds one of its keys
+        alpha = active ? expf(m - m_new) : 1.f;
+#pragma unroll
+        for (int b = 0; b < 4; ++b)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int c = tile + 16 * b + 4 * kq + r;
+            s[b][r] = (active && c >= lo && c <= pos) ? expf(s[b][r] - m_new) : 0.f;
+          }
+        m_new = active ? m_new : m;
+      }
+      float u[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) u[r] = (s[0][r] + s[2][r]) + (s[1][r] + s[3][r]);     // key bits 5, then 4
+#pragma unroll
+      for (int r = 0; r < 4; ++r) u[r] = u[r] + __shfl_xor(u[r], 32, WAVE);             // key bit 3
+#pragma unroll
+      for (int r = 0; r < 4; ++r) u[r] = u[r] + __shfl_xor(u[r], 16, WAVE);             // key bit 2
+      const float sum = (u[0] + u[2]) + (u[1] + u[3]);                                  // key bits 1 and 0
+      l = __builtin_fmaf(l, alpha, sum);
+      m = m_new;
+      if (__ballot(alpha != 1.f) != 0) {             // times one changes nothing
+#pragma unroll
+        for (int i = 0; i < NBLK; ++i)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) acc[i][r] = acc[i][r] * alpha;
+      }
+      // values: lane (col, kq) gives dimension 16 blk + col at key 4 j + kq, and its token's probability of that key
+      const float* va = v_s + col * VS + kq * (WAVE / 4);
+      const float* pb = p_s + kq * MA_COLS + col;
+#pragma unroll
+      for (int hf = 0; hf < 2; ++hf) {
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) p_s[(16 * b + 4 * kq + r) * MA_COLS + col] = s[2 * hf + b][r];
+        __builtin_amdgcn_wave_barrier();             // read by this wavefront alone: LDS keeps a wavefront's order
+#pragma unroll
+        for (int n = 0; n < 2; ++n) {
+          float4 v[NBLK];
+#pragma unroll
+          for (int i = 0; i < NBLK; ++i) v[i] = *reinterpret_cast<const float4*>(va + i * 16 * VS + 8 * hf + 4 * n);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const float pj = pb[4 * (4 * n + e) * MA_COLS];
+#pragma unroll
+            for (int i = 0; i < NBLK; ++i)
+              acc[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(reinterpret_cast<const float*>(&v[i])[e], pj, acc[i], 0, 0, 0);
+          }
+        }
+        __builtin_amdgcn_wave_barrier();
+      }
+    };
+    const int first_tile = (run.lo_min / WAVE) * WAVE;
+    __syncthreads();
+    __syncthreads();
+    __syncthreads();
+    int b = 0;
+    for (int tile = first_tile; tile <= run.pos_max; tile += WAVE, b ^= 1) {
+      const float* buf = lds + b * tile_floats;
+      attend(tile, buf, buf + WAVE * KS);
+      __syncthreads();
+    }
+    run_begin = run.end;
+  }
+  if (!live) return;
+  T* op = out + t * out_stride + (int64_t)h * hd;
+  const float inv = 1.0f / l;
+#pragma unroll
+  for (int i = 0; i < NBLK; ++i)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) Num<T>::st(op + i * 16 + 4 * kq + r, acc[i][r] * inv);
+}
+
 // out: [T, nh*hd] (row stride out_stride elements); q: rows of stride q_stride (the fused q|k|v
 // buffer); k_pages: [pages, nkv, page_size, hd]; v_pages: [pages, nkv, hd, page_size]; block_table: [entries, table_width];
 // token_entry, positions: [T].  tokens_per_workgroup: how many neighbouring tokens of the step share a workgroup and,
@@ -290,6 +612,75 @@ extern "C" int ga_paged_attention_generic(void* out, int64_t out_stride, const v
   if (tokens <= 0) return 0;
   if (hd > MAX_HD || hd <= 0 || nkv <= 0 || nh % nkv != 0 || page_size <= 0) return -1;
   const int group = nh / nkv;
+  // 16-byte loads where a key's dimensions and a page's keys come in whole vectors at 16-byte addresses
+  const int vec = is_bf16 ? 8 : 4;
+  const bool wide = hd % vec == 0 && page_size % vec == 0 && WAVE % page_size == 0 &&
+                    ((uintptr_t)k_pages % 16 == 0) && ((uintptr_t)v_pages % 16 == 0);
+  // Steps that hold prompt portions, at the head sizes it is built for: the kernel on the matrix cores.  A workgroup
+  // holds tq groups of tokens times hpw heads of a kv group, which share its tiles: as many wavefronts (12, 8, 4, 2,
+  // 1) as still leave one and a half workgroups to every compute unit, so that the units that finish the first tokens
+  // of a prompt, which see few keys, find more work (measured: that weighs more than the sharing); whole kv groups
+  // or divisors of them, so that no wavefront is without a head.
+  if (tokens_per_workgroup == 0 && tokens >= 2 * MA_COLS && hd % 16 == 0 && hd <= 128) {
+    int tq = 1, hpw = 1;
+    auto workgroups = [&](int tq_, int hpw_) {
+      return ((int64_t)(tokens + tq_ * MA_COLS - 1) / (tq_ * MA_COLS)) * nkv * ((group + hpw_ - 1) / hpw_);
+    };
+    static const int wavefronts[] = {MA_MAX_COMPUTE, 8, 4, 2, 1};
+    for (int most : wavefronts) {
+      int best = -1;
+      for (int h = 1; h <= group && h <= most; ++h) {
+        if (group % h != 0) continue;
+        const int t = most / h, key = 2 * (t * h + (h == group ? 1 : 0));      // a whole kv group counts for one more
+        if (key >= best) best = key, tq = t, hpw = h;                           // among equals, more heads
+      }
+      if (workgroups(tq, hpw) >= 384) break;
+    }
+    const int head_blocks = (group + hpw - 1) / hpw, waves = tq * hpw;
+    const size_t lds = sizeof(float) * (2 * ((size_t)WAVE * (hd + KPAD) + (size_t)hd * VS) + (size_t)waves * (WAVE / 2) * MA_COLS) +
+                       sizeof(int64_t) * (2 * WAVE + 1);
+    const int64_t workgroup_count = ((int64_t)(tokens + tq * MA_COLS - 1) / (tq * MA_COLS)) * nkv * head_blocks;
+    dim3 grid((unsigned)workgroup_count), block(WAVE * (waves + MA_LOADERS));
+    bool launched = workgroup_count <= 0x7fffffff;
+#define LAUNCH_MATRIX(TT, VV, HH)                                                                                    \
+  do {                                                                                                               \
+    const void* fn = (const void*)paged_attention_matrix_kernel<TT, VV, HH>;                                         \
+    if (lds > 48 * 1024 && hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) { \
+      (void)hipGetLastError();                                                                                       \
+      launched = false;                                                                                              \
+      break;                                                                                                         \
+    }                                                                                                                \
+    hipLaunchKernelGGL((paged_attention_matrix_kernel<TT, VV, HH>), grid, block, lds, stream, (TT*)out, out_stride,  \
+                       (const TT*)q, q_stride, (const TT*)k_pages, (const TT*)v_pages, (const int32_t*)block_table,  \
+                       table_width, (const int32_t*)token_entry, (const int32_t*)positions, tokens, nh, nkv,          \
+                       page_size, window, scale, tq, hpw);                                                           \
+  } while (0)
+#define LAUNCH_MATRIX_HD(TT, VV)                                                                                     \
+  do {                                                                                                               \
+    switch (hd) {                                                                                                    \
+      case 16: LAUNCH_MATRIX(TT, VV, 16); break;                                                                     \
+      case 32: LAUNCH_MATRIX(TT, VV, 32); break;                                                                     \
+      case 48: LAUNCH_MATRIX(TT, VV, 48); break;                                                                     \
+      case 64: LAUNCH_MATRIX(TT, VV, 64); break;                                                                     \
+      case 80: LAUNCH_MATRIX(TT, VV, 80); break;                                                                     \
+      case 96: LAUNCH_MATRIX(TT, VV, 96); break;                                                                     \
+      case 112: LAUNCH_MATRIX(TT, VV, 112); break;                                                                   \
+      default: LAUNCH_MATRIX(TT, VV, 128); break;                                                                    \
+    }                                                                                                                \
+  } while (0)
+    if (launched) {
+      if (is_bf16) {
+        if (wide) LAUNCH_MATRIX_HD(bf16_t, 8);
+        else LAUNCH_MATRIX_HD(bf16_t, 1);
+      } else {
+        if (wide) LAUNCH_MATRIX_HD(float, 4);
+        else LAUNCH_MATRIX_HD(float, 1);
+      }
+    }
+#undef LAUNCH_MATRIX_HD
+#undef LAUNCH_MATRIX
+    if (launched) return GA_CHECK_LAUNCH();         // else: the kernel below
+  }
   const int hpw = group < GA_MAX_WAVES ? group : GA_MAX_WAVES, head_blocks = (group + hpw - 1) / hpw;
   int tq = tokens_per_workgroup > 0 ? tokens_per_workgroup : 4;
   if (tq * hpw > GA_MAX_WAVES) tq = GA_MAX_WAVES / hpw;
@@ -300,10 +691,6 @@ extern "C" int ga_paged_attention_generic(void* out, int64_t out_stride, const v
   if ((int64_t)nkv * head_blocks > 65535) return -3;
   // A workgroup with few wavefronts that compute (a decoded token: the heads of one kv group) gets further ones that
   // only help to load: a tile's loads are then all under way at once, and a tile's time is one trip to memory.
-  // 16-byte loads where a key's dimensions and a page's keys come in whole vectors at 16-byte addresses
-  const int vec = is_bf16 ? 8 : 4;
-  const bool wide = hd % vec == 0 && page_size % vec == 0 && WAVE % page_size == 0 &&
-                    ((uintptr_t)k_pages % 16 == 0) && ((uintptr_t)v_pages % 16 == 0);
   int total_waves = waves;
   const int vectors = WAVE * hd / (wide ? vec : 1);                   // loads of a tile's keys (and as many of its values)
   while (total_waves < GA_MAX_WAVES && total_waves * WAVE * GA_BATCH < vectors) ++total_waves;

@@ -26,7 +26,7 @@ FLAGS = ["--offload-arch=" + ARCH, "-O3", "-std=c++17", "-shared", "-fPIC",
 MODULES = ("embedding", "norm", "rope_kv", "attention_generic", "attention_mfma", "gemm", "gemm_skinny",
            "activation", "sampling", "random_fill")
 # flags of single modules: the random-weights generator must round every operation by itself, as the host's twin does
-MODULE_FLAGS = {"random_fill": ["-ffp-contract=off"]}
+MODULE_FLAGS = {"random_fill": ["-ffp-contract=off"], "attention_generic": ["-ffp-contract=off"]}
 # headers beside common.cuh that a module includes (they enter its digest)
 MODULE_HEADERS = {"random_fill": ["random_normal.h"]}
 # plain C++ libraries for the host (no GPU runtime), built with the host compiler from csrc/host/

@@ -396,6 +396,39 @@ def test_paged_attention_generic_at_drawn_sizes_whatever_shares_a_workgroup(seed
 
 
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-5), (torch.bfloat16, 2e-2)])
+@pytest.mark.parametrize("seed", range(24))
+def test_paged_attention_on_the_matrix_cores_gives_the_bits_of_the_wavefront_per_token(dtype, tol, seed):
+    """Steps of 32 tokens and more that hold prompt portions, at head sizes in steps of 16 up to 128, run on the matrix
+    cores when the library chooses (tokens_per_workgroup 0); with one token to a workgroup they run a wavefront per
+    (token, head).  Both add a score's products over ascending dimensions and an output's over ascending keys as fused
+    multiply-adds, so they give the same bits: portions of several requests in one group of 32 tokens, single tokens
+    between them, windows, kv groups that do not fill a workgroup, pages smaller than a load."""
+    import random
+    from ginfer_amd.kernels import ops
+    rng = random.Random(900 + seed)
+    nkv, group = rng.choice([1, 2, 3]), rng.choice([1, 2, 3, 6, 7, 8, 12])
+    nh, hd, ps = nkv * group, (16, 32, 48, 64, 80, 96, 112, 128)[seed % 8], rng.choice([2, 4, 8, 16, 32, 64])
+    window = rng.choice([None, None, 7, 40, 100, 130])
+    kind = rng.choice(["a prompt", "portions", "portions and single tokens"])
+    if kind == "a prompt":
+        n = rng.randint(32, 300)
+        seqs = [(n, n + rng.choice([0, 0, 17, 64, 200]))]
+    elif kind == "portions":
+        seqs = [(ql, ql + rng.randint(0, 200)) for ql in (rng.choice([2, 5, 20, 33, 64, 90]) for _ in range(rng.randint(2, 4)))]
+    else:
+        seqs = [(ql, ql + rng.randint(0, 200)) for ql in (rng.choice([1, 1, 1, 2, 30, 45]) for _ in range(rng.randint(3, 7)))]
+    while sum(ql for ql, _ in seqs) < 32:
+        seqs.append((16, 16 + rng.randint(0, 100)))
+    a, ref, _ = _paged_case(seqs, nh, nkv, hd, ps, dtype, seed=seed, window=window)
+    outs = [ops.paged_attention_generic(a["q"], a["k_pages"], a["v_pages"], a["block_table"], a["token_entry"],
+                                        a["positions"], nh, nkv, hd, 1.0 / math.sqrt(hd), window=window,
+                                        tokens_per_workgroup=tq) for tq in (0, 1)]
+    what = "%s %s, %d heads in %d groups of size %d, pages of %d, window %s" % (kind, seqs, nh, nkv, hd, ps, window)
+    close(outs[0], ref, tol)
+    assert torch.equal(outs[0], outs[1]), what
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-5), (torch.bfloat16, 2e-2)])
 @pytest.mark.parametrize("window", [1, 5, 16, 40, 64, 100])
 def test_paged_attention_window(dtype, tol, window):
     from ginfer_amd.kernels import ops
