@@ -55,6 +55,18 @@ struct VecLoad {
 
 #define GA_BATCH 4         // loads of keys, and as many of values, that a thread has under way at a time
 
+// Whether the tokens around token t that are of its request (neighbours in the step: a request's tokens lie side by
+// side) are fewer than n.  The two kernels below share a step by this: runs of at least MA_MIN_RUN tokens go to the
+// matrix cores, shorter ones (the single tokens of decoding requests beside a prompt portion, which each walk the keys
+// of another request) to a wavefront per token and head.
+__device__ __forceinline__ bool run_is_shorter(const int32_t* __restrict__ token_entry, int64_t t, int tokens, int n) {
+  const int e = token_entry[t];
+  int len = 1;
+  for (int i = 1; len < n && t - i >= 0 && token_entry[t - i] == e; ++i) ++len;
+  for (int i = 1; len < n && t + i < tokens && token_entry[t + i] == e; ++i) ++len;
+  return len < n;
+}
+
 // PIPE: the wavefronts beyond those that compute are loaders: they bring tile i + 1 into a second buffer while the
 // others multiply tile i, one barrier a tile (the launcher says when: few workgroups, both buffers fit, and at least
 // as many wavefronts load as compute).
@@ -64,7 +76,7 @@ __global__ __launch_bounds__(64 * GA_MAX_WAVES) void paged_attention_generic_ker
     const T* __restrict__ k_pages, const T* __restrict__ v_pages,
     const int32_t* __restrict__ block_table, int table_width,
     const int32_t* __restrict__ token_entry, const int32_t* __restrict__ positions, int tokens, int nh, int nkv,
-    int hd, int page_size, int window, float scale, int tq, int hpw) {
+    int hd, int page_size, int window, float scale, int tq, int hpw, int min_run) {
   extern __shared__ float lds[];
   const int group = nh / nkv, head_blocks = (group + hpw - 1) / hpw;     // hpw heads of a kv group to a workgroup
   const int waves = tq * hpw, threads = blockDim.x;        // wavefronts that compute; all threads load (see the launcher)
@@ -91,6 +103,7 @@ __global__ __launch_bounds__(64 * GA_MAX_WAVES) void paged_attention_generic_ker
   float acc[MAX_HD / WAVE];
 #pragma unroll
   for (int i = 0; i < MAX_HD / WAVE; ++i) acc[i] = 0.f;
+  bool done = false;           // this wavefront's token was of a run that this kernel handles
 
   // The workgroup's tokens fall into runs of one request each (a prompt portion: one run; single tokens of several
   // requests: a run each).  A run's tiles are loaded once and serve every wavefront of the run.
@@ -105,7 +118,13 @@ __global__ __launch_bounds__(64 * GA_MAX_WAVES) void paged_attention_generic_ker
       pos_max = p > pos_max ? p : pos_max;
       ++run_end;
     }
+    // min_run > 0: runs of that many tokens and more are the other kernel's
+    if (min_run > 0 && !run_is_shorter(token_entry, t0 + run_begin, tokens, min_run)) {
+      run_begin = run_end;
+      continue;
+    }
     const bool mine = live && tl >= run_begin && tl < run_end;
+    done = done || mine;
     const int32_t* bt = block_table + (int64_t)run_entry * table_width;
     const int first_page = lo_min / page_size, last_page = pos_max / page_size;    // the pages that the run reads
     // the page of every key of a tile, asked for one tile ahead
@@ -269,7 +288,7 @@ __global__ __launch_bounds__(64 * GA_MAX_WAVES) void paged_attention_generic_ker
     }
     run_begin = run_end;
   }
-  if (!live) return;
+  if (!done) return;
   T* op = out + t * out_stride + (int64_t)h * hd;
   const float inv = 1.0f / l;
 #pragma unroll
@@ -296,6 +315,7 @@ __global__ __launch_bounds__(64 * GA_MAX_WAVES) void paged_attention_generic_ker
 #define MA_COLS 16
 #define MA_MAX_COMPUTE 12
 #define MA_LOADERS 4
+#define MA_MIN_RUN 8        // shorter runs of tokens are left to the kernel above
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
 template <typename T, int VEC, int HD>
@@ -336,9 +356,9 @@ __global__ __launch_bounds__(64 * (MA_MAX_COMPUTE + MA_LOADERS)) void paged_atte
   const int loaders = (int)blockDim.x - waves * WAVE, ltid = (int)threadIdx.x - waves * WAVE;
   // The workgroup's tokens from `begin` on that are of one request: the run's end, and the range of keys that its
   // tokens see.  Loaders and the others walk the same runs and tiles, and meet at the same barriers.
-  struct Run { int entry, end, lo_min, pos_max; };
+  struct Run { int entry, end, lo_min, pos_max; bool skipped; };
   auto next_run = [&](int begin) -> Run {
-    Run r{token_entry[t0 + begin], begin, 0x7fffffff, -1};
+    Run r{token_entry[t0 + begin], begin, 0x7fffffff, -1, run_is_shorter(token_entry, t0 + begin, tokens, MA_MIN_RUN)};
     while (r.end < span && t0 + r.end < tokens && token_entry[t0 + r.end] == r.entry) {
       const int p = positions[t0 + r.end];
       const int l0 = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
@@ -352,6 +372,10 @@ __global__ __launch_bounds__(64 * (MA_MAX_COMPUTE + MA_LOADERS)) void paged_atte
   if (loader) {
     for (int run_begin = 0; run_begin < span && t0 + run_begin < tokens;) {
       const Run run = next_run(run_begin);
+      if (run.skipped) {
+        run_begin = run.end;
+        continue;
+      }
       const int lo_min = run.lo_min, pos_max = run.pos_max;
       const int32_t* bt = block_table + (int64_t)run.entry * table_width;
       const int first_page = lo_min / page_size, last_page = pos_max / page_size;
@@ -466,9 +490,15 @@ __global__ __launch_bounds__(64 * (MA_MAX_COMPUTE + MA_LOADERS)) void paged_atte
 #pragma unroll
   for (int i = 0; i < NBLK; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
   float* p_s = p_all + wave * (WAVE / 2) * MA_COLS;
+  bool done = false;           // this lane's token was of a run that this kernel handles
   for (int run_begin = 0; run_begin < span && t0 + run_begin < tokens;) {
     const Run run = next_run(run_begin);
+    if (run.skipped) {
+      run_begin = run.end;
+      continue;
+    }
     const bool mine = live && tl >= run_begin && tl < run.end;
+    done = done || mine;
     // one tile for this wavefront's tokens, its keys and values in LDS
     auto attend = [&](int tile, const float* k_s, const float* v_s) {
       const bool active = mine && !(tile > pos || tile + WAVE - 1 < lo);
@@ -588,7 +618,7 @@ __global__ __launch_bounds__(64 * (MA_MAX_COMPUTE + MA_LOADERS)) void paged_atte
     }
     run_begin = run.end;
   }
-  if (!live) return;
+  if (!done) return;
   T* op = out + t * out_stride + (int64_t)h * hd;
   const float inv = 1.0f / l;
 #pragma unroll
@@ -600,8 +630,10 @@ __global__ __launch_bounds__(64 * (MA_MAX_COMPUTE + MA_LOADERS)) void paged_atte
 // out: [T, nh*hd] (row stride out_stride elements); q: rows of stride q_stride (the fused q|k|v
 // buffer); k_pages: [pages, nkv, page_size, hd]; v_pages: [pages, nkv, hd, page_size]; block_table: [entries, table_width];
 // token_entry, positions: [T].  tokens_per_workgroup: how many neighbouring tokens of the step share a workgroup and,
-// where they are of one request, its tiles of keys and values (1 for steps of single tokens; 0: the library chooses);
-// a token's result does not depend on it.
+// where they are of one request, its tiles of keys and values (1 for steps of single tokens; 0: the library chooses,
+// which for steps of 32 tokens and more means two kernels: the matrix cores for a request's 8 tokens and more, a
+// wavefront per token and head for fewer; -1: as 0, and the caller knows that every request of the step has at least 8
+// tokens in it, which saves the second kernel); a token's result does not depend on it.
 extern "C" int ga_paged_attention_generic(void* out, int64_t out_stride, const void* q,
                                           int64_t q_stride, const void* k_pages,
                                           const void* v_pages, const void* block_table,
@@ -612,6 +644,7 @@ extern "C" int ga_paged_attention_generic(void* out, int64_t out_stride, const v
   if (tokens <= 0) return 0;
   if (hd > MAX_HD || hd <= 0 || nkv <= 0 || nh % nkv != 0 || page_size <= 0) return -1;
   const int group = nh / nkv;
+  int min_run = 0;            // > 0: the runs of that many tokens and more have gone to the matrix cores
   // 16-byte loads where a key's dimensions and a page's keys come in whole vectors at 16-byte addresses
   const int vec = is_bf16 ? 8 : 4;
   const bool wide = hd % vec == 0 && page_size % vec == 0 && WAVE % page_size == 0 &&
@@ -621,6 +654,8 @@ extern "C" int ga_paged_attention_generic(void* out, int64_t out_stride, const v
   // 1) as still leave one and a half workgroups to every compute unit, so that the units that finish the first tokens
   // of a prompt, which see few keys, find more work (measured: that weighs more than the sharing); whole kv groups
   // or divisors of them, so that no wavefront is without a head.
+  const bool long_runs_only = tokens_per_workgroup < 0;
+  if (long_runs_only) tokens_per_workgroup = 0;
   if (tokens_per_workgroup == 0 && tokens >= 2 * MA_COLS && hd % 16 == 0 && hd <= 128) {
     int tq = 1, hpw = 1;
     auto workgroups = [&](int tq_, int hpw_) {
@@ -679,7 +714,12 @@ extern "C" int ga_paged_attention_generic(void* out, int64_t out_stride, const v
     }
 #undef LAUNCH_MATRIX_HD
 #undef LAUNCH_MATRIX
-    if (launched) return GA_CHECK_LAUNCH();         // else: the kernel below
+    if (launched) {
+      const int rc = GA_CHECK_LAUNCH();
+      if (rc != 0 || long_runs_only) return rc;
+      min_run = MA_MIN_RUN;                          // the kernel below takes the shorter runs, a token to a workgroup
+      tokens_per_workgroup = 1;
+    }
   }
   const int hpw = group < GA_MAX_WAVES ? group : GA_MAX_WAVES, head_blocks = (group + hpw - 1) / hpw;
   int tq = tokens_per_workgroup > 0 ? tokens_per_workgroup : 4;
@@ -697,7 +737,8 @@ extern "C" int ga_paged_attention_generic(void* out, int64_t out_stride, const v
   dim3 grid((tokens + tq - 1) / tq, nkv * head_blocks), block(WAVE * total_waves);
   // Few workgroups (a decode step: they cannot fill the chip, and each walks its keys alone): two tile buffers, the
   // next tile loaded while this one is multiplied, where both fit and a thread's one batch of loads is a whole tile.
-  const bool pipelined = (int64_t)grid.x * grid.y <= 256 && 2 * tile_bytes + rest_bytes <= 150 * 1024 &&
+  // (Beside the matrix kernel the workgroups that find work are those of a few single tokens: the same.)
+  const bool pipelined = ((int64_t)grid.x * grid.y <= 256 || min_run > 0) && 2 * tile_bytes + rest_bytes <= 150 * 1024 &&
                          GA_MAX_WAVES - waves >= waves;
   if (pipelined) block.x = WAVE * GA_MAX_WAVES;
   const size_t lds = (pipelined ? 2 : 1) * tile_bytes + rest_bytes;
@@ -709,7 +750,7 @@ extern "C" int ga_paged_attention_generic(void* out, int64_t out_stride, const v
     hipLaunchKernelGGL((paged_attention_generic_kernel<TT, VV, PP>), grid, block, lds, stream, (TT*)out, out_stride, \
                        (const TT*)q, q_stride, (const TT*)k_pages, (const TT*)v_pages, (const int32_t*)block_table,  \
                        table_width, (const int32_t*)token_entry, (const int32_t*)positions, tokens, nh, nkv, hd,      \
-                       page_size, window, scale, tq, hpw);                                                           \
+                       page_size, window, scale, tq, hpw, min_run);                                                  \
   } while (0)
   if (is_bf16) {
     if (wide && pipelined) LAUNCH(bf16_t, 8, true);

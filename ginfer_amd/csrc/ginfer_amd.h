@@ -68,7 +68,8 @@ int ga_silu_mul(void* out, const void* gu, int tokens, int inter, int is_bf16, h
 int ga_silu_mul_transposed(void* out, const void* gu_t, int tokens, int inter, hipStream_t stream);
 
 // ---- attention_generic.hip: every token attends to its request's pages; any head size up to 256, window or 0;
-// tokens_per_workgroup neighbouring tokens share a workgroup's tiles of keys and values (0: the library chooses)
+// tokens_per_workgroup neighbouring tokens share a workgroup's tiles of keys and values (0: the library chooses; -1: the
+// same, and every request of the step has at least 8 tokens in it)
 int ga_paged_attention_generic(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* k_pages,
                                const void* v_pages, const void* block_table, int table_width, const void* token_entry,
                                const void* positions, int tokens, int nh, int nkv, int hd, int page_size, int window,

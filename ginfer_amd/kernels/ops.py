@@ -216,7 +216,9 @@ def paged_attention_generic(q, k_pages, v_pages, block_table, token_entry, posit
     Token t attends to the keys of request token_entry[t] at positions
     [max(0, p - window + 1), p], p = positions[t].  Returns [T, nh*hd].  tokens_per_workgroup: how many neighbouring
     tokens share a workgroup and (where they are of one request) its tiles of keys and values; 1 suits steps of
-    single tokens, 0 leaves it to the library; no token's result depends on it."""
+    single tokens, 0 leaves it to the library (from 32 tokens on: the matrix cores for a request's 8 tokens and more,
+    a second kernel for the requests with fewer), -1 says besides that every request has at least 8 tokens in the
+    step; no token's result depends on it."""
     T = _check_attention_operands(q, k_pages, v_pages, block_table, token_entry, positions, num_heads,
                                   num_kv_heads, head_dim)
     _need(0 < head_dim <= 256,
@@ -608,6 +610,11 @@ def paged_attention(q, k_pages, v_pages, block_table, step, num_heads, num_kv_he
     if attention_mfma_supported(q.dtype, head_dim, k_pages.shape[2]):
         return paged_attention_mfma(q, k_pages, v_pages, block_table, step, num_heads, num_kv_heads, head_dim, scale,
                                     window)
+    if step.max_q_len == 1:
+        grouping = 1
+    elif "static_plan" not in (step.extra or {}) and min(step.host_q_len) >= 8:
+        grouping = -1          # the step's own sizes are known here (a recorded step of padded sizes serves many)
+    else:
+        grouping = 0
     return paged_attention_generic(q, k_pages, v_pages, block_table, step.token_entry, step.positions, num_heads,
-                                   num_kv_heads, head_dim, scale, window,
-                                   tokens_per_workgroup=1 if step.max_q_len == 1 else 0)
+                                   num_kv_heads, head_dim, scale, window, tokens_per_workgroup=grouping)

@@ -402,7 +402,8 @@ def test_paged_attention_on_the_matrix_cores_gives_the_bits_of_the_wavefront_per
     cores when the library chooses (tokens_per_workgroup 0); with one token to a workgroup they run a wavefront per
     (token, head).  Both add a score's products over ascending dimensions and an output's over ascending keys as fused
     multiply-adds, so they give the same bits: portions of several requests in one group of 32 tokens, single tokens
-    between them, windows, kv groups that do not fill a workgroup, pages smaller than a load."""
+    between them (runs of fewer than 8 tokens are left to the wavefronts per token in the same call), windows, kv groups
+    that do not fill a workgroup, pages smaller than a load."""
     import random
     from ginfer_amd.kernels import ops
     rng = random.Random(900 + seed)
@@ -416,7 +417,7 @@ def test_paged_attention_on_the_matrix_cores_gives_the_bits_of_the_wavefront_per
     elif kind == "portions":
         seqs = [(ql, ql + rng.randint(0, 200)) for ql in (rng.choice([2, 5, 20, 33, 64, 90]) for _ in range(rng.randint(2, 4)))]
     else:
-        seqs = [(ql, ql + rng.randint(0, 200)) for ql in (rng.choice([1, 1, 1, 2, 30, 45]) for _ in range(rng.randint(3, 7)))]
+        seqs = [(ql, ql + rng.randint(0, 200)) for ql in (rng.choice([1, 1, 1, 2, 7, 8, 9, 30, 45]) for _ in range(rng.randint(3, 7)))]
     while sum(ql for ql, _ in seqs) < 32:
         seqs.append((16, 16 + rng.randint(0, 100)))
     a, ref, _ = _paged_case(seqs, nh, nkv, hd, ps, dtype, seed=seed, window=window)
@@ -426,6 +427,11 @@ def test_paged_attention_on_the_matrix_cores_gives_the_bits_of_the_wavefront_per
     what = "%s %s, %d heads in %d groups of size %d, pages of %d, window %s" % (kind, seqs, nh, nkv, hd, ps, window)
     close(outs[0], ref, tol)
     assert torch.equal(outs[0], outs[1]), what
+    if min(ql for ql, _ in seqs) >= 8:                # the caller may then say so, and the second kernel is left out
+        alone = ops.paged_attention_generic(a["q"], a["k_pages"], a["v_pages"], a["block_table"], a["token_entry"],
+                                            a["positions"], nh, nkv, hd, 1.0 / math.sqrt(hd), window=window,
+                                            tokens_per_workgroup=-1)
+        assert torch.equal(alone, outs[1]), what
 
 
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-5), (torch.bfloat16, 2e-2)])
