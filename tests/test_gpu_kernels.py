@@ -434,6 +434,22 @@ def test_paged_attention_on_the_matrix_cores_gives_the_bits_of_the_wavefront_per
         assert torch.equal(alone, outs[1]), what
 
 
+@pytest.mark.parametrize("seqs,window", [([(2048, 2048)], None), ([(1, 900), (1500, 2100), (1, 64), (3, 700), (540, 540)], None),
+                                         ([(1100, 1700)], 600)])
+def test_paged_attention_on_the_matrix_cores_at_the_sizes_of_the_benchmark(seqs, window):
+    """The 32-bit attention at the 1.5B shape's heads (12 in 2 groups of size 128, pages of 16): a 2,048-token prompt, a
+    step that mixes long portions with single tokens, and a window; against the plain result, and the same bits from
+    the matrix cores and from a wavefront per token."""
+    from ginfer_amd.kernels import ops
+    nh, nkv, hd, ps = 12, 2, 128, 16
+    a, ref, _ = _paged_case(seqs, nh, nkv, hd, ps, torch.float32, seed=11, window=window)
+    outs = [ops.paged_attention_generic(a["q"], a["k_pages"], a["v_pages"], a["block_table"], a["token_entry"],
+                                        a["positions"], nh, nkv, hd, 1.0 / math.sqrt(hd), window=window,
+                                        tokens_per_workgroup=tq) for tq in (0, 1)]
+    close(outs[0], ref, 1e-5)
+    assert torch.equal(outs[0], outs[1])
+
+
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-5), (torch.bfloat16, 2e-2)])
 @pytest.mark.parametrize("window", [1, 5, 16, 40, 64, 100])
 def test_paged_attention_window(dtype, tol, window):
