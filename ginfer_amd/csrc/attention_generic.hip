@@ -298,6 +298,125 @@ __global__ __launch_bounds__(64 * GA_MAX_WAVES) void paged_attention_generic_ker
   }
 }
 
+// What the loading wavefronts of the matrix-core kernels do for one run of tokens: tiles of 64 keys and their values
+// from the pages into one of two buffers in LDS.  A row of keys in LDS holds dimension d at (d % 4) * (HD / 4) + d / 4,
+// a row of values key j at (j % 4) * 16 + j / 4: lane (row, kq) of a matrix operand wants every fourth element from
+// kq on, and so reads four of them at a time; the rows' padding puts the 16 rows of a read on different banks.
+template <typename T, int VEC, int HD, int NLOAD>
+struct TileLoader {
+  static constexpr int KS = HD + KPAD;
+  static constexpr int tile_floats = WAVE * KS + HD * VS;
+  static constexpr int per_key = HD / VEC, per_dim = WAVE / VEC, nvec = WAVE * per_key;
+  static constexpr int NB = VEC == 1 ? 8 : 4;       // loads of keys, and as many of values, under way in a thread
+  static constexpr int loaders = NLOAD * WAVE;
+  static constexpr bool whole_rounds = nvec % (loaders * NB) == 0;
+  const T* k_pages;
+  const T* v_pages;
+  const int32_t* bt;           // the request's row of the block table
+  int nkv, g, page_size, lo_min, pos_max, ltid;
+  float* lds;                  // two tile buffers
+  int64_t* base_s;             // [2][64]
+  int32_t* plain_s;            // [2]
+
+  // where the page of key `tile + ltid` begins for this kv head, in elements (both caches keep page_size * HD
+  // elements per page and kv head), or -1 for a key without a page; by the first loading wavefront
+  __device__ __forceinline__ int64_t tile_base(int tile) const {
+    if (tile > pos_max) return -1;
+    const int pi = (tile + ltid) / page_size;
+    if (pi < lo_min / page_size || pi > pos_max / page_size) return -1;
+    const int64_t page = bt[pi];
+    return page >= 0 ? (page * nkv + g) * page_size * HD : -1;
+  }
+  // a tile into a buffer: all its loads of a round are under way before the first is put into LDS; what lies
+  // outside the run's keys, or has no page, becomes zero (what lies in a page beyond a request's last key may be
+  // anything, and zero times it must be zero).  PLAIN: every key of the tile has a page and is one of the run's:
+  // nothing to ask.
+  template <bool PLAIN>
+  __device__ __forceinline__ void load_tile(int tile, const int64_t* bases, float* k_s, float* v_s) const {
+    for (int base = ltid; base < nvec; base += loaders * NB) {
+      VecLoad<T, VEC> rk[NB], rv[NB];
+#pragma unroll
+      for (int u = 0; u < NB; ++u) {
+        const int v = base + u * loaders;
+        const int j = v / per_key, d = (v - j * per_key) * VEC;
+        // with 16-byte loads a page's size divides 64, and a tile begins where a page does
+        const int in_page = VEC > 1 ? (j & (page_size - 1)) : (tile + j) % page_size;
+        if (PLAIN) {
+          if (whole_rounds || v < nvec) rk[u].load(k_pages + bases[j] + in_page * HD + d);
+        } else {
+          const int64_t at = v < nvec ? bases[j] : -1;
+          rk[u].zero();
+          if (at >= 0 && tile + j >= lo_min && tile + j <= pos_max) rk[u].load(k_pages + at + in_page * HD + d);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < NB; ++u) {
+        const int v = base + u * loaders;
+        const int d = v / per_dim, j = (v - d * per_dim) * VEC;
+        const int in_page = VEC > 1 ? (j & (page_size - 1)) : (tile + j) % page_size;
+        if (PLAIN) {
+          if (whole_rounds || v < nvec) rv[u].load(v_pages + bases[j] + d * page_size + in_page);
+        } else {
+          const int64_t at = v < nvec ? bases[j] : -1;
+          rv[u].zero();
+          if (at >= 0) rv[u].load(v_pages + at + d * page_size + in_page);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < NB; ++u) {
+        const int v = base + u * loaders;
+        if (!whole_rounds && v >= nvec) continue;
+        const int j = v / per_key, d = (v - j * per_key) * VEC;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) k_s[j * KS + ((d + i) & 3) * (HD / 4) + ((d + i) >> 2)] = rk[u].v[i];
+      }
+#pragma unroll
+      for (int u = 0; u < NB; ++u) {
+        const int v = base + u * loaders;
+        if (!whole_rounds && v >= nvec) continue;
+        const int d = v / per_dim, j = (v - d * per_dim) * VEC;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+          const int c = tile + j + i;
+          const bool out_of_range = !PLAIN && (c < lo_min || c > pos_max);
+          v_s[d * VS + ((j + i) & 3) * (WAVE / 4) + ((j + i) >> 2)] = out_of_range ? 0.f : rv[u].v[i];
+        }
+      }
+    }
+  }
+  // a tile's bases into LDS, and whether the tile is plain
+  __device__ __forceinline__ void note_tile(int tile, int slot) const {
+    if (ltid >= WAVE) return;
+    const int64_t at = tile_base(tile);
+    base_s[slot * WAVE + ltid] = at;
+    const bool plain = __ballot(at >= 0) == ~0ull && tile >= lo_min && tile + WAVE - 1 <= pos_max;
+    if (ltid == 0) plain_s[slot] = plain ? 1 : 0;
+  }
+  __device__ __forceinline__ void load(int tile, int slot) const {
+    float* buf = lds + slot * tile_floats;
+    if (plain_s[slot]) load_tile<true>(tile, base_s + slot * WAVE, buf, buf + WAVE * KS);
+    else load_tile<false>(tile, base_s + slot * WAVE, buf, buf + WAVE * KS);
+  }
+  // The run's tiles one after the other, tile i + 1 into the buffer that tile i - 1 was read from while the others
+  // multiply tile i: `barriers` barriers a tile, which the wavefronts that multiply meet as well (three before the
+  // first tile).
+  __device__ __forceinline__ void run(int barriers) const {
+    const int first_tile = (lo_min / WAVE) * WAVE;
+    __syncthreads();                              // the run before has been read
+    note_tile(first_tile, 0);
+    __syncthreads();
+    load(first_tile, 0);
+    note_tile(first_tile + WAVE, 1);
+    __syncthreads();
+    int b = 0;
+    for (int tile = first_tile; tile <= pos_max; tile += WAVE, b ^= 1) {
+      if (tile + WAVE <= pos_max) load(tile + WAVE, b ^ 1);
+      note_tile(tile + 2 * WAVE, b);               // read two tiles on
+      for (int i = 0; i < barriers; ++i) __syncthreads();
+    }
+  }
+};
+
 // The same attention on the matrix cores, for steps that hold prompt portions.  v_mfma_f32_16x16x4_f32 takes 32-bit
 // operands and adds its four products into the accumulator in ascending k as fused multiply-adds, so a score is the
 // chain over ascending dimensions, and an output element the chain over ascending keys, that the kernel above computes:
@@ -327,10 +446,7 @@ __global__ __launch_bounds__(64 * (MA_MAX_COMPUTE + MA_LOADERS)) void paged_atte
     int page_size, int window, float scale, int tq, int hpw) {
   extern __shared__ float lds[];
   constexpr int hd = HD;
-  // A row of keys in LDS holds dimension d at (d % 4) * (HD / 4) + d / 4, a row of values key j at (j % 4) * 16 + j / 4:
-  // lane (row, kq) of an operand wants every fourth element from kq on, and so reads four of them at a time; the rows'
-  // padding puts the 16 rows of a read on different banks.
-  constexpr int KS = HD + KPAD;
+  constexpr int KS = HD + KPAD;                  // the layout of a tile in LDS: TileLoader
   constexpr int NBLK = HD / 16;                  // blocks of 16 dimensions of the output
   constexpr int tile_floats = WAVE * KS + HD * VS;
   const int group = nh / nkv, head_blocks = (group + hpw - 1) / hpw;
@@ -353,7 +469,7 @@ __global__ __launch_bounds__(64 * (MA_MAX_COMPUTE + MA_LOADERS)) void paged_atte
   const bool live = !loader && hl < group && t < tokens;
   const int pos = live ? positions[t] : -1;
   const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
-  const int loaders = (int)blockDim.x - waves * WAVE, ltid = (int)threadIdx.x - waves * WAVE;
+  const int ltid = (int)threadIdx.x - waves * WAVE;          // a loading thread's number
   // The workgroup's tokens from `begin` on that are of one request: the run's end, and the range of keys that its
   // tokens see.  Loaders and the others walk the same runs and tiles, and meet at the same barriers.
   struct Run { int entry, end, lo_min, pos_max; bool skipped; };
@@ -376,102 +492,9 @@ __global__ __launch_bounds__(64 * (MA_MAX_COMPUTE + MA_LOADERS)) void paged_atte
         run_begin = run.end;
         continue;
       }
-      const int lo_min = run.lo_min, pos_max = run.pos_max;
-      const int32_t* bt = block_table + (int64_t)run.entry * table_width;
-      const int first_page = lo_min / page_size, last_page = pos_max / page_size;
-      // where the page of key `tile + ltid` begins for this kv head, in elements (both caches keep page_size * hd
-      // elements per page and kv head), or -1 for a key without a page; by the first loading wavefront
-      auto tile_base = [&](int tile) -> int64_t {
-        if (tile > pos_max) return -1;
-        const int pi = (tile + ltid) / page_size;
-        if (pi < first_page || pi > last_page) return -1;
-        const int64_t page = bt[pi];
-        return page >= 0 ? (page * nkv + g) * page_size * hd : -1;
-      };
-      constexpr int per_key = HD / VEC, per_dim = WAVE / VEC, nvec = WAVE * per_key;
-      constexpr int NB = VEC == 1 ? 8 : 4;         // loads of keys, and as many of values, under way in a thread
-      // a tile into a buffer: all its loads of a round are under way before the first is put into LDS; what lies
-      // outside the run's keys, or has no page, becomes zero.  `plain`: every key of the tile has a page and is one of
-      // the run's: nothing to ask.
-      auto load_tile = [&](int tile, const int64_t* bases, float* k_s, float* v_s, auto plain_tag) {
-        constexpr bool plain = decltype(plain_tag)::value;
-        for (int base = ltid; base < nvec; base += loaders * NB) {
-          VecLoad<T, VEC> rk[NB], rv[NB];
-#pragma unroll
-          for (int u = 0; u < NB; ++u) {
-            const int v = base + u * loaders;
-            const int j = v / per_key, d = (v - j * per_key) * VEC;
-            // with 16-byte loads a page's size divides 64, and a tile begins where a page does
-            const int in_page = VEC > 1 ? (j & (page_size - 1)) : (tile + j) % page_size;
-            if (plain) {
-              if (nvec % (MA_LOADERS * WAVE * NB) == 0 || v < nvec) rk[u].load(k_pages + bases[j] + in_page * hd + d);
-            } else {
-              const int64_t at = v < nvec ? bases[j] : -1;
-              rk[u].zero();
-              if (at >= 0 && tile + j >= lo_min && tile + j <= pos_max) rk[u].load(k_pages + at + in_page * hd + d);
-            }
-          }
-#pragma unroll
-          for (int u = 0; u < NB; ++u) {
-            const int v = base + u * loaders;
-            const int d = v / per_dim, j = (v - d * per_dim) * VEC;
-            const int in_page = VEC > 1 ? (j & (page_size - 1)) : (tile + j) % page_size;
-            if (plain) {
-              if (nvec % (MA_LOADERS * WAVE * NB) == 0 || v < nvec) rv[u].load(v_pages + bases[j] + d * page_size + in_page);
-            } else {
-              const int64_t at = v < nvec ? bases[j] : -1;
-              rv[u].zero();
-              if (at >= 0) rv[u].load(v_pages + at + d * page_size + in_page);
-            }
-          }
-#pragma unroll
-          for (int u = 0; u < NB; ++u) {
-            const int v = base + u * loaders;
-            if (nvec % (MA_LOADERS * WAVE * NB) != 0 && v >= nvec) continue;
-            const int j = v / per_key, d = (v - j * per_key) * VEC;
-#pragma unroll
-            for (int i = 0; i < VEC; ++i) k_s[j * KS + ((d + i) & 3) * (HD / 4) + ((d + i) >> 2)] = rk[u].v[i];
-          }
-#pragma unroll
-          for (int u = 0; u < NB; ++u) {
-            const int v = base + u * loaders;
-            if (nvec % (MA_LOADERS * WAVE * NB) != 0 && v >= nvec) continue;
-            const int d = v / per_dim, j = (v - d * per_dim) * VEC;
-#pragma unroll
-            for (int i = 0; i < VEC; ++i) {
-              const int c = tile + j + i;
-              const bool out_of_range = !plain && (c < lo_min || c > pos_max);
-              v_s[d * VS + ((j + i) & 3) * (WAVE / 4) + ((j + i) >> 2)] = out_of_range ? 0.f : rv[u].v[i];
-            }
-          }
-        }
-      };
-      // a tile's bases into LDS, and whether the tile is plain
-      auto note_tile = [&](int tile, int slot) {
-        if (ltid >= WAVE) return;
-        const int64_t at = tile_base(tile);
-        base_s[slot * WAVE + ltid] = at;
-        const bool plain = __ballot(at >= 0) == ~0ull && tile >= lo_min && tile + WAVE - 1 <= pos_max;
-        if (ltid == 0) plain_s[slot] = plain ? 1 : 0;
-      };
-      auto load = [&](int tile, int slot) {
-        float* buf = lds + slot * tile_floats;
-        if (plain_s[slot]) load_tile(tile, base_s + slot * WAVE, buf, buf + WAVE * KS, std::true_type{});
-        else load_tile(tile, base_s + slot * WAVE, buf, buf + WAVE * KS, std::false_type{});
-      };
-      const int first_tile = (lo_min / WAVE) * WAVE;
-      __syncthreads();                              // the run before has been read
-      note_tile(first_tile, 0);
-      __syncthreads();
-      load(first_tile, 0);
-      note_tile(first_tile + WAVE, 1);
-      __syncthreads();
-      int b = 0;
-      for (int tile = first_tile; tile <= pos_max; tile += WAVE, b ^= 1) {
-        if (tile + WAVE <= pos_max) load(tile + WAVE, b ^ 1);
-        note_tile(tile + 2 * WAVE, b);               // read two tiles on
-        __syncthreads();
-      }
+      const TileLoader<T, VEC, HD, MA_LOADERS> loading{k_pages, v_pages, block_table + (int64_t)run.entry * table_width,
+                                                       nkv, g, page_size, run.lo_min, run.pos_max, ltid, lds, base_s, plain_s};
+      loading.run(1);
       run_begin = run.end;
     }
     return;
@@ -627,6 +650,145 @@ __global__ __launch_bounds__(64 * (MA_MAX_COMPUTE + MA_LOADERS)) void paged_atte
     for (int r = 0; r < 4; ++r) Num<T>::st(op + i * 16 + 4 * kq + r, acc[i][r] * inv);
 }
 
+// Single tokens on the matrix cores: the heads of a kv group are the columns.  A workgroup holds one token and (up to
+// 16 heads of) one kv head; the scores of a tile are [64 keys][heads], and the four wavefronts that multiply take 16
+// keys each, then, for the product with the values, their share of the output's blocks of 16 dimensions each.  Between
+// the two they meet twice: once for the tile's maximum (each gives its 16 keys' maximum per head through LDS), once
+// for the probabilities, which all of them read from LDS: as the second operand of their products, and to add up a
+// head's 64 of them in the order of the butterfly (key bits 5 to 0), every wavefront for itself.  The keys and values
+// of a tile are read from LDS once, not once per head as with a wavefront per head, which is what bounds that kernel.
+// Scores, maxima, exponentials, sums and outputs are those of the other two kernels to the bit.
+#define HA_COMPUTE 4
+#define HA_LOADERS 8
+
+template <typename T, int VEC, int HD>
+__global__ __launch_bounds__(64 * (HA_COMPUTE + HA_LOADERS)) void paged_attention_heads_kernel(
+    T* __restrict__ out, int64_t out_stride, const T* __restrict__ q, int64_t q_stride,
+    const T* __restrict__ k_pages, const T* __restrict__ v_pages,
+    const int32_t* __restrict__ block_table, int table_width,
+    const int32_t* __restrict__ token_entry, const int32_t* __restrict__ positions, int tokens, int nh, int nkv,
+    int page_size, int window, float scale, int min_run) {
+  extern __shared__ float lds[];
+  constexpr int KS = HD + KPAD;                  // the layout of a tile in LDS: TileLoader
+  constexpr int NBLK = HD / 16;                  // blocks of 16 dimensions of the output
+  constexpr int BPW = (NBLK + HA_COMPUTE - 1) / HA_COMPUTE;       // ... of a wavefront: blocks wave, wave + 4, ...
+  constexpr int tile_floats = WAVE * KS + HD * VS;
+  const int group = nh / nkv, head_blocks = (group + 15) / 16;
+  float* p_s = lds + 2 * tile_floats;            // [64 keys][16 heads]
+  float* mx_s = p_s + WAVE * 16;                 // [4][16]
+  int64_t* base_s = reinterpret_cast<int64_t*>(mx_s + HA_COMPUTE * 16);      // [2][64]
+  int32_t* plain_s = reinterpret_cast<int32_t*>(base_s + 2 * WAVE);          // [2]
+  const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
+  const int col = lane & 15, kq = lane >> 4;
+  const int64_t t = blockIdx.x;
+  // min_run > 0: the tokens of runs of that many and more are another kernel's
+  if (min_run > 0 && !run_is_shorter(token_entry, t, tokens, min_run)) return;
+  const int g = blockIdx.y / head_blocks, hl = (blockIdx.y % head_blocks) * 16 + col;
+  const int h = g * group + hl;
+  const int pos = positions[t];
+  const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  if (wave >= HA_COMPUTE) {
+    const TileLoader<T, VEC, HD, HA_LOADERS> loading{k_pages, v_pages, block_table + (int64_t)token_entry[t] * table_width,
+                                                     nkv, g, page_size, lo, pos, (int)threadIdx.x - HA_COMPUTE * WAVE,
+                                                     lds, base_s, plain_s};
+    loading.run(3);
+    return;
+  }
+  const bool live = hl < group;                  // this lane's column has a head
+  float qr[HD / 4];                              // the head's query at dimensions 4 i + kq
+#pragma unroll
+  for (int i = 0; i < HD / 4; ++i) qr[i] = 0.f;
+  if (live) {
+    const T* qp = q + t * q_stride + (int64_t)h * HD + kq;
+#pragma unroll
+    for (int i = 0; i < HD / 4; ++i) qr[i] = Num<T>::ld(qp + 4 * i);
+  }
+  float m = -INFINITY, l = 0.f;
+  f32x4 acc[BPW];
+#pragma unroll
+  for (int i = 0; i < BPW; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+  __syncthreads();
+  __syncthreads();
+  __syncthreads();
+  int b = 0;
+  for (int tile = (lo / WAVE) * WAVE; tile <= pos; tile += WAVE, b ^= 1) {
+    const float* k_s = lds + b * tile_floats;
+    const float* v_s = k_s + WAVE * KS;
+    // scores of keys 16 wave .. 16 wave + 15 of the tile; lane (col, kq) gives key col's dimension 4 i + kq
+    f32x4 s = f32x4{0.f, 0.f, 0.f, 0.f};
+    const float* ka = k_s + (16 * wave + col) * KS + kq * (HD / 4);
+#pragma unroll
+    for (int n = 0; n < HD / 16; ++n) {
+      const float4 a = *reinterpret_cast<const float4*>(ka + 4 * n);
+      s = __builtin_amdgcn_mfma_f32_16x16x4f32(a.x, qr[4 * n], s, 0, 0, 0);
+      s = __builtin_amdgcn_mfma_f32_16x16x4f32(a.y, qr[4 * n + 1], s, 0, 0, 0);
+      s = __builtin_amdgcn_mfma_f32_16x16x4f32(a.z, qr[4 * n + 2], s, 0, 0, 0);
+      s = __builtin_amdgcn_mfma_f32_16x16x4f32(a.w, qr[4 * n + 3], s, 0, 0, 0);
+    }
+    // element r: key 16 wave + 4 kq + r of the tile, for this lane's head
+    float mx = -INFINITY;
+    bool valid[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int c = tile + 16 * wave + 4 * kq + r;
+      valid[r] = live && c >= lo && c <= pos;
+      s[r] = valid[r] ? s[r] * scale : -INFINITY;
+      mx = fmaxf(mx, s[r]);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+    mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
+    if (kq == 0) mx_s[wave * 16 + col] = mx;
+    __syncthreads();
+    const float m_new = fmaxf(fmaxf(m, fmaxf(mx_s[col], mx_s[16 + col])), fmaxf(mx_s[32 + col], mx_s[48 + col]));
+    const float alpha = live ? expf(m - m_new) : 1.f;       // exp(-inf) = 0 on the first tile
+#pragma unroll
+    for (int r = 0; r < 4; ++r) p_s[(16 * wave + 4 * kq + r) * 16 + col] = valid[r] ? expf(s[r] - m_new) : 0.f;
+    __syncthreads();
+    float u[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const float* pr = p_s + (4 * kq + r) * 16 + col;
+      u[r] = (pr[0] + pr[32 * 16]) + (pr[16 * 16] + pr[48 * 16]);                     // key bits 5, then 4
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) u[r] = u[r] + __shfl_xor(u[r], 32, WAVE);             // key bit 3
+#pragma unroll
+    for (int r = 0; r < 4; ++r) u[r] = u[r] + __shfl_xor(u[r], 16, WAVE);             // key bit 2
+    const float sum = (u[0] + u[2]) + (u[1] + u[3]);                                  // key bits 1 and 0
+    l = __builtin_fmaf(l, alpha, sum);
+    m = live ? m_new : m;
+    // values: lane (col, kq) gives dimension 16 blk + col at key 4 j + kq, and its head's probability of that key
+    const float* va = v_s + col * VS + kq * (WAVE / 4);
+    const float* pb = p_s + kq * 16 + col;
+#pragma unroll
+    for (int i = 0; i < BPW; ++i) {
+      const int blk = wave + HA_COMPUTE * i;
+      if (NBLK % HA_COMPUTE != 0 && blk >= NBLK) break;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) acc[i][r] = acc[i][r] * alpha;
+#pragma unroll
+      for (int n = 0; n < 4; ++n) {
+        const float4 v = *reinterpret_cast<const float4*>(va + blk * 16 * VS + 4 * n);
+        acc[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(v.x, pb[4 * (4 * n) * 16], acc[i], 0, 0, 0);
+        acc[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(v.y, pb[4 * (4 * n + 1) * 16], acc[i], 0, 0, 0);
+        acc[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(v.z, pb[4 * (4 * n + 2) * 16], acc[i], 0, 0, 0);
+        acc[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(v.w, pb[4 * (4 * n + 3) * 16], acc[i], 0, 0, 0);
+      }
+    }
+    __syncthreads();
+  }
+  if (!live) return;
+  T* op = out + t * out_stride + (int64_t)h * HD;
+  const float inv = 1.0f / l;
+#pragma unroll
+  for (int i = 0; i < BPW; ++i) {
+    const int blk = wave + HA_COMPUTE * i;
+    if (NBLK % HA_COMPUTE != 0 && blk >= NBLK) break;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) Num<T>::st(op + blk * 16 + 4 * kq + r, acc[i][r] * inv);
+  }
+}
+
 // out: [T, nh*hd] (row stride out_stride elements); q: rows of stride q_stride (the fused q|k|v
 // buffer); k_pages: [pages, nkv, page_size, hd]; v_pages: [pages, nkv, hd, page_size]; block_table: [entries, table_width];
 // token_entry, positions: [T].  tokens_per_workgroup: how many neighbouring tokens of the step share a workgroup and,
@@ -720,6 +882,48 @@ extern "C" int ga_paged_attention_generic(void* out, int64_t out_stride, const v
       min_run = MA_MIN_RUN;                          // the kernel below takes the shorter runs, a token to a workgroup
       tokens_per_workgroup = 1;
     }
+  }
+  // Single tokens (a decode step, or the short runs beside the matrix kernel's), 16-byte loads, the same head sizes:
+  // the heads of a kv group as the columns of matrix-core products.
+  if (tokens_per_workgroup == 1 && wide && hd % 16 == 0 && hd <= 128) {
+    const int head_blocks = (group + 15) / 16;
+    const size_t lds = sizeof(float) * (2 * ((size_t)WAVE * (hd + KPAD) + (size_t)hd * VS) + (size_t)WAVE * 16 + HA_COMPUTE * 16) +
+                       sizeof(int64_t) * (2 * WAVE + 1);
+    dim3 grid((unsigned)tokens, nkv * head_blocks), block(WAVE * (HA_COMPUTE + HA_LOADERS));
+    bool launched = (int64_t)nkv * head_blocks <= 65535;
+#define LAUNCH_HEADS(TT, VV, HH)                                                                                     \
+  do {                                                                                                               \
+    const void* fn = (const void*)paged_attention_heads_kernel<TT, VV, HH>;                                          \
+    if (lds > 48 * 1024 && hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) { \
+      (void)hipGetLastError();                                                                                       \
+      launched = false;                                                                                              \
+      break;                                                                                                         \
+    }                                                                                                                \
+    hipLaunchKernelGGL((paged_attention_heads_kernel<TT, VV, HH>), grid, block, lds, stream, (TT*)out, out_stride,   \
+                       (const TT*)q, q_stride, (const TT*)k_pages, (const TT*)v_pages, (const int32_t*)block_table,  \
+                       table_width, (const int32_t*)token_entry, (const int32_t*)positions, tokens, nh, nkv,          \
+                       page_size, window, scale, min_run);                                                           \
+  } while (0)
+#define LAUNCH_HEADS_HD(TT, VV)                                                                                      \
+  do {                                                                                                               \
+    switch (hd) {                                                                                                    \
+      case 16: LAUNCH_HEADS(TT, VV, 16); break;                                                                      \
+      case 32: LAUNCH_HEADS(TT, VV, 32); break;                                                                      \
+      case 48: LAUNCH_HEADS(TT, VV, 48); break;                                                                      \
+      case 64: LAUNCH_HEADS(TT, VV, 64); break;                                                                      \
+      case 80: LAUNCH_HEADS(TT, VV, 80); break;                                                                      \
+      case 96: LAUNCH_HEADS(TT, VV, 96); break;                                                                      \
+      case 112: LAUNCH_HEADS(TT, VV, 112); break;                                                                    \
+      default: LAUNCH_HEADS(TT, VV, 128); break;                                                                     \
+    }                                                                                                                \
+  } while (0)
+    if (launched) {
+      if (is_bf16) LAUNCH_HEADS_HD(bf16_t, 8);
+      else LAUNCH_HEADS_HD(float, 4);
+    }
+#undef LAUNCH_HEADS_HD
+#undef LAUNCH_HEADS
+    if (launched) return GA_CHECK_LAUNCH();         // else: the kernel below
   }
   const int hpw = group < GA_MAX_WAVES ? group : GA_MAX_WAVES, head_blocks = (group + hpw - 1) / hpw;
   int tq = tokens_per_workgroup > 0 ? tokens_per_workgroup : 4;

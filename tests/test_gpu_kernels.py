@@ -399,9 +399,10 @@ def test_paged_attention_generic_at_drawn_sizes_whatever_shares_a_workgroup(seed
 @pytest.mark.parametrize("seed", range(24))
 def test_paged_attention_on_the_matrix_cores_gives_the_bits_of_the_wavefront_per_token(dtype, tol, seed):
     """Steps of 32 tokens and more that hold prompt portions, at head sizes in steps of 16 up to 128, run on the matrix
-    cores when the library chooses (tokens_per_workgroup 0); with one token to a workgroup they run a wavefront per
-    (token, head).  Both add a score's products over ascending dimensions and an output's over ascending keys as fused
-    multiply-adds, so they give the same bits: portions of several requests in one group of 32 tokens, single tokens
+    cores when the library chooses (tokens_per_workgroup 0): a wavefront per head and 16 tokens; with one token to a
+    workgroup the heads of a kv group are the columns of the matrix cores' products (where pages allow 16-byte loads);
+    with two, a wavefront per (token, head) without the matrix cores.  All add a score's products over ascending
+    dimensions and an output's over ascending keys as fused multiply-adds, so they give the same bits: portions of several requests in one group of 32 tokens, single tokens
     between them (runs of fewer than 8 tokens are left to the wavefronts per token in the same call), windows, kv groups
     that do not fill a workgroup, pages smaller than a load."""
     import random
@@ -423,10 +424,10 @@ def test_paged_attention_on_the_matrix_cores_gives_the_bits_of_the_wavefront_per
     a, ref, _ = _paged_case(seqs, nh, nkv, hd, ps, dtype, seed=seed, window=window)
     outs = [ops.paged_attention_generic(a["q"], a["k_pages"], a["v_pages"], a["block_table"], a["token_entry"],
                                         a["positions"], nh, nkv, hd, 1.0 / math.sqrt(hd), window=window,
-                                        tokens_per_workgroup=tq) for tq in (0, 1)]
+                                        tokens_per_workgroup=tq) for tq in (0, 1, 2)]
     what = "%s %s, %d heads in %d groups of size %d, pages of %d, window %s" % (kind, seqs, nh, nkv, hd, ps, window)
     close(outs[0], ref, tol)
-    assert torch.equal(outs[0], outs[1]), what
+    assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2]), what
     if min(ql for ql, _ in seqs) >= 8:                # the caller may then say so, and the second kernel is left out
         alone = ops.paged_attention_generic(a["q"], a["k_pages"], a["v_pages"], a["block_table"], a["token_entry"],
                                             a["positions"], nh, nkv, hd, 1.0 / math.sqrt(hd), window=window,
@@ -445,9 +446,9 @@ def test_paged_attention_on_the_matrix_cores_at_the_sizes_of_the_benchmark(seqs,
     a, ref, _ = _paged_case(seqs, nh, nkv, hd, ps, torch.float32, seed=11, window=window)
     outs = [ops.paged_attention_generic(a["q"], a["k_pages"], a["v_pages"], a["block_table"], a["token_entry"],
                                         a["positions"], nh, nkv, hd, 1.0 / math.sqrt(hd), window=window,
-                                        tokens_per_workgroup=tq) for tq in (0, 1)]
+                                        tokens_per_workgroup=tq) for tq in (0, 1, 2)]
     close(outs[0], ref, 1e-5)
-    assert torch.equal(outs[0], outs[1])
+    assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])
 
 
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-5), (torch.bfloat16, 2e-2)])
