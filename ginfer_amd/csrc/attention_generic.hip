@@ -1,9 +1,9 @@
 // Paged attention, the general kernels: any mix of prompt portions and single decoded tokens, any
 // head size up to 256, full or windowed, 32-bit or bfloat16 storage with
 // 32-bit scores, softmax and accumulators.  They are the whole of the 32-bit path and the fallback of
-// the bfloat16 path.  Two kernels that give the same bits: a wavefront per (token, query head), described first, for
-// steps of single tokens and for every size; and the matrix cores' 32-bit instruction (further down) for steps that
-// hold prompt portions, at head sizes in steps of 16 up to 128.
+// the bfloat16 path.  Three kernels that give the same bits: a wavefront per (token, query head), described first, for
+// every size; and two on the matrix cores' 32-bit instruction (further down), at head sizes in steps of 16 up to 128:
+// one for the prompt portions of a step, one for its single tokens.
 //
 // One wavefront per (token, query head).  A token is self-describing: `token_entry[t]` names its
 // row of the block table and `positions[t]` its absolute position p, so it attends to the keys
