@@ -818,6 +818,12 @@ extern "C" int ga_paged_attention_generic(void* out, int64_t out_stride, const v
   // or divisors of them, so that no wavefront is without a head.
   const bool long_runs_only = tokens_per_workgroup < 0;
   if (long_runs_only) tokens_per_workgroup = 0;
+  // A step of few tokens, whatever they are: a workgroup per token and kv head (the heads kernel below) while there
+  // are no more than two of them to a compute unit.  Its four wavefronts share a tile's keys, where the kernel for
+  // prompt portions has one wavefront walk them; that one wins by the tiles its tokens share once there are many
+  // (measured at contexts of 512 and 4,096: 12 heads in 2 groups up to 256 tokens, 28 in 4 up to 128, 16 in 16 up to 32).
+  if (tokens_per_workgroup == 0 && wide && hd % 16 == 0 && hd <= 128 && (int64_t)tokens * nkv * ((group + 15) / 16) <= 512)
+    tokens_per_workgroup = 1;
   if (tokens_per_workgroup == 0 && tokens >= 2 * MA_COLS && hd % 16 == 0 && hd <= 128) {
     int tq = 1, hpw = 1;
     auto workgroups = [&](int tq_, int hpw_) {

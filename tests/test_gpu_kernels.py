@@ -419,8 +419,11 @@ def test_paged_attention_on_the_matrix_cores_gives_the_bits_of_the_wavefront_per
         seqs = [(ql, ql + rng.randint(0, 200)) for ql in (rng.choice([2, 5, 20, 33, 64, 90]) for _ in range(rng.randint(2, 4)))]
     else:
         seqs = [(ql, ql + rng.randint(0, 200)) for ql in (rng.choice([1, 1, 1, 2, 7, 8, 9, 30, 45]) for _ in range(rng.randint(3, 7)))]
-    while sum(ql for ql, _ in seqs) < 32:
-        seqs.append((16, 16 + rng.randint(0, 100)))
+    # enough tokens that the library does not give the whole step to the kernel for single tokens (it does up to 512
+    # workgroups of a token and a kv head)
+    while sum(ql for ql, _ in seqs) * nkv <= 512:
+        seqs.append((rng.choice([16, 64, 150]), rng.choice([16, 64, 150]) + rng.randint(0, 100)))
+    seqs = [(ql, max(ql, kv)) for ql, kv in seqs]
     a, ref, _ = _paged_case(seqs, nh, nkv, hd, ps, dtype, seed=seed, window=window)
     outs = [ops.paged_attention_generic(a["q"], a["k_pages"], a["v_pages"], a["block_table"], a["token_entry"],
                                         a["positions"], nh, nkv, hd, 1.0 / math.sqrt(hd), window=window,
