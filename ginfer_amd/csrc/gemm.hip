@@ -247,21 +247,25 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 #define FEW_DEPTH 8
 #define FEW_SETS 2
 
-// x[c] of the lane 16 s + i (s = 0..3) becomes what was x[s] of the lane 16 c + i
-__device__ __forceinline__ void transpose_over_lane_rows(float (&x)[4], int s) {
-  const bool odd = s & 1, high = s & 2;
-#pragma unroll
-  for (int c = 0; c < 4; c += 2) {
-    const float give = odd ? x[c] : x[c + 1];
-    const float got = __shfl_xor(give, 16, 64);
-    if (odd) x[c] = got; else x[c + 1] = got;
-  }
-#pragma unroll
-  for (int c = 0; c < 2; ++c) {
-    const float give = high ? x[c] : x[c + 2];
-    const float got = __shfl_xor(give, 32, 64);
-    if (high) x[c] = got; else x[c + 2] = got;
-  }
+// x[c] of the lane 16 s + i (s = 0..3) becomes what was x[s] of the lane 16 c + i: a 4 x 4 transpose between the
+// registers and the wavefront's four rows of 16 lanes, by gfx950's row swaps (v_permlane16_swap exchanges the odd rows
+// of its first operand with the even rows of its second, v_permlane32_swap the upper half of the first with the lower
+// half of the second): the 2 x 2 blocks transposed in themselves, then the two off the diagonal exchanged
+__device__ __forceinline__ void swap_rows_16(float& a, float& b) {
+  const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(a), __float_as_uint(b), false, false);
+  a = __uint_as_float(r[0]);
+  b = __uint_as_float(r[1]);
+}
+__device__ __forceinline__ void swap_rows_32(float& a, float& b) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(a), __float_as_uint(b), false, false);
+  a = __uint_as_float(r[0]);
+  b = __uint_as_float(r[1]);
+}
+__device__ __forceinline__ void transpose_over_lane_rows(float (&x)[4]) {
+  swap_rows_16(x[0], x[1]);
+  swap_rows_16(x[2], x[3]);
+  swap_rows_32(x[0], x[2]);
+  swap_rows_32(x[1], x[3]);
 }
 
 // four consecutive elements at an address that is a multiple of four elements, no questions asked
@@ -290,14 +294,11 @@ __global__ __launch_bounds__(64) void gemm_nt_few_rows_kernel(TC* __restrict__ C
   // whole chunks of 16 elements, with aligned rows, take the loop without branches; what is left of K (and everything,
   // with rows that are not aligned) takes the careful loads afterwards: ascending k all the same
   const int chunks = (wide_a && wide_w) ? K / 16 : 0;
+  // (a lane without a row of its own multiplies row 0's numbers: they meet nobody else's, a row of A and a row of W
+  // make one element of C, and that element is not stored)
   auto multiply = [&](float (&x)[4], float (&y)[4]) {
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      x[e] = a_ok ? x[e] : 0.f;
-      y[e] = w_ok ? y[e] : 0.f;
-    }
-    transpose_over_lane_rows(x, kq);
-    transpose_over_lane_rows(y, kq);
+    transpose_over_lane_rows(x);
+    transpose_over_lane_rows(y);
 #pragma unroll
     for (int st = 0; st < 4; ++st) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(x[st], y[st], acc, 0, 0, 0);
   };
