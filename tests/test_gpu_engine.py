@@ -43,6 +43,37 @@ LENGTHS = {"A": [5, 17, 33, 70, 131], "B": [1, 9, 40, 64, 100, 150], "C": [3, 50
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "C"])
+def test_long_prompts_whole_in_portions_and_decoded(folders, tmp_path, name, dtype):
+    """Prompts of several hundred tokens: whole, they are a step of so many tokens that the 32-bit attention runs its
+    kernel for prompt portions (a wavefront per head and 16 tokens); in portions and decoded, the kernel for single
+    tokens and small steps.  The same logits as the plain model, and in 32-bit the same bits whatever the cutting; C has
+    windows of 40 keys on three of its layers."""
+    if name == "A":
+        cfg = dict(H.TINY_A, max_position_embeddings=1024)
+        folder, lengths, ps = H.make_model_folder(tmp_path / "long_a", cfg, 5, "float32"), [700, 90], 16
+    else:
+        folder, lengths, ps = folders["C"], [380, 300], H.TINY["C"][2]
+    vocab = H.TINY[name][0]["vocab_size"]
+    reqs = {"r%d" % i: H.random_tokens(n, vocab, 40 + i) for i, n in enumerate(lengths)}
+    from ginfer_amd import ModelRunner
+    runner = ModelRunner(folder, dtype=dtype, page_size=ps, num_pages=-(-1024 // ps), max_requests=4)
+    results = {}
+    for what, steps in (("whole", H.steps_whole(reqs)), ("last 32 decoded", H.steps_last_decoded(reqs)),
+                        ("portions", H.steps_portions(reqs, sizes=(130, 2, 33, 300, 16, 7, 64, 5))),
+                        ("mixed", H.steps_mixed(reqs, max_live=2, seed=4))):
+        got = H.run_steps(runner, steps)
+        runner.cache.check()
+        assert not runner.cache.requests
+        H.compare_with_plain(got, reqs, folder, H.TOL[dtype], "%s %s %s" % (name, dtype, what))
+        results[what] = got
+    if dtype == "float32":
+        for what in ("last 32 decoded", "portions", "mixed"):
+            for key, row in results[what].items():
+                assert np.array_equal(row, results["whole"][key]), "%s: %r differs in bits from whole" % (what, key)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", ["A", "B", "C"])
 @pytest.mark.parametrize("weights", ["usual", "wide"])
 def test_whole_last_decoded_and_portions(folders, sharp_folders, name, dtype, weights):
