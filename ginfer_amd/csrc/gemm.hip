@@ -169,7 +169,22 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_nt_matrix_kernel(TC* __rest
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
   float ra[GA][4], rw[GW][4];
+  // a tile that lies inside C, with rows that allow 16-byte loads, asks nothing per load while its step lies inside K
+  const bool inside = wide_a && wide_w && m0 + TM <= M && n0 + TN <= N;
   auto fetch = [&](int k0) {
+    if (inside && k0 + TK <= K) {
+#pragma unroll
+      for (int i = 0; i < GA; ++i) {
+        const int gi = tid + i * GEMM_THREADS, row = gi / (TK / 4), k = k0 + (gi % (TK / 4)) * 4;
+        load4<TA>(ra[i], A + (int64_t)(m0 + row) * lda + k, 4, true);
+      }
+#pragma unroll
+      for (int i = 0; i < GW; ++i) {
+        const int gi = tid + i * GEMM_THREADS, row = gi / (TK / 4), k = k0 + (gi % (TK / 4)) * 4;
+        load4<TW>(rw[i], W + (int64_t)(n0 + row) * K + k, 4, true);
+      }
+      return;
+    }
 #pragma unroll
     for (int i = 0; i < GA; ++i) {
       const int gi = tid + i * GEMM_THREADS, row = gi / (TK / 4), k = k0 + (gi % (TK / 4)) * 4;
