@@ -6,10 +6,11 @@
 // Three kernels make the true 32-bit product (no reduced-precision mode anywhere).  In all of them every element of
 // C is ONE accumulator that takes its terms over ascending k as fused multiply-adds, so its bits do not depend on M,
 // on the tile it falls in, on the rest of the batch, or on which of the three ran:
-//   gemm_nt_kernel           17 to 64 rows: plain FMA, a tile of 64 x 64 per workgroup staged through LDS in steps of K;
-//   gemm_nt_matrix_kernel    more rows: the matrix cores' 32-bit instruction over tiles of up to 128 x 128;
-//   gemm_nt_few_rows_kernel  up to 16 rows (a decode step): the matrix cores again, a wavefront per 16 columns,
-//                            operands straight from memory.
+//   gemm_nt_few_rows_kernel  up to 64 rows (a decode step, a small portion): the matrix cores' 32-bit instruction, a
+//                            wavefront per 16 columns and up to four blocks of 16 rows, operands straight from memory;
+//   gemm_nt_matrix_kernel    more rows: the matrix cores again, over tiles of up to 128 x 128 through LDS;
+//   gemm_nt_kernel           plain FMA, a tile of 64 x 64 per workgroup staged through LDS in steps of K: 33 to 64 rows
+//                            times 65,536 columns and more (a head), where it is the fastest of the three.
 // They are templated on storage, so that they also serve bfloat16 operands (the kernel tests' oracle and the
 // fallback for shapes the bfloat16 kernels refuse).
 //
@@ -261,6 +262,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_nt_matrix_kernel(TC* __rest
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 #define FEW_DEPTH 8
 #define FEW_SETS 2
+#define FEW_DEPTH_BLOCKS 4     // ... with several blocks of rows (measured: 2, 4, 8)
 
 // x[c] of the lane 16 s + i (s = 0..3) becomes what was x[s] of the lane 16 c + i: a 4 x 4 transpose between the
 // registers and the wavefront's four rows of 16 lanes, by gfx950's row swaps (v_permlane16_swap exchanges the odd rows
@@ -289,73 +291,87 @@ __device__ __forceinline__ void load4_aligned(float (&v)[4], const T* p) {
   load4<T>(v, p, 4, true);
 }
 
-template <typename TA, typename TW, typename TC>
+template <typename TA, typename TW, typename TC, int RB>
 __global__ __launch_bounds__(64) void gemm_nt_few_rows_kernel(TC* __restrict__ C, int64_t ldc,
                                                               const TA* __restrict__ A, int64_t lda,
                                                               const TW* __restrict__ W,
                                                               const TW* __restrict__ bias, int M, int N, int K,
                                                               int wide_a, int wide_w) {
+  // RB blocks of 16 rows: the wavefront's 16 columns of W are loaded once for all of them, and the blocks' chains of
+  // matrix instructions run side by side
   const int lane = threadIdx.x, i = lane & 15, kq = lane >> 4;
   const int n = blockIdx.x * 16 + i;
-  const bool a_ok = i < M, w_ok = n < N;
+  const bool w_ok = n < N;
   // a lane whose row does not exist reads row 0 and drops what it read: no branch in the loop
-  const TA* pa = A + (int64_t)(a_ok ? i : 0) * lda + 4 * kq;
+  const TA* pa[RB];
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) pa[rb] = A + (int64_t)(16 * rb + i < M ? 16 * rb + i : 0) * lda + 4 * kq;
   const TW* pw = W + (int64_t)(w_ok ? n : 0) * K + 4 * kq;
-  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-  // FEW_SETS sets of FEW_DEPTH loads of A and of W: one is multiplied while the others are on their way (a wavefront
-  // has the registers of its SIMD to itself: so few wavefronts run here that the bytes each keeps under way are what
-  // decides)
-  float a[FEW_SETS][FEW_DEPTH][4], w[FEW_SETS][FEW_DEPTH][4];
+  f32x4 acc[RB];
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) acc[rb] = f32x4{0.f, 0.f, 0.f, 0.f};
+  // FEW_SETS sets of DEPTH loads of A's blocks and of W: one is multiplied while the others are on their way (a
+  // wavefront has the registers of its SIMD to itself: so few wavefronts run here that the bytes each keeps under way
+  // are what decides)
+  constexpr int DEPTH = RB == 1 ? FEW_DEPTH : FEW_DEPTH_BLOCKS;
+  float a[FEW_SETS][DEPTH][RB][4], w[FEW_SETS][DEPTH][4];
   // whole chunks of 16 elements, with aligned rows, take the loop without branches; what is left of K (and everything,
   // with rows that are not aligned) takes the careful loads afterwards: ascending k all the same
   const int chunks = (wide_a && wide_w) ? K / 16 : 0;
   // (a lane without a row of its own multiplies row 0's numbers: they meet nobody else's, a row of A and a row of W
   // make one element of C, and that element is not stored)
-  auto multiply = [&](float (&x)[4], float (&y)[4]) {
-    transpose_over_lane_rows(x);
+  auto multiply = [&](float (&x)[RB][4], float (&y)[4]) {
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) transpose_over_lane_rows(x[rb]);
     transpose_over_lane_rows(y);
 #pragma unroll
-    for (int st = 0; st < 4; ++st) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(x[st], y[st], acc, 0, 0, 0);
-  };
-  // the loads of the chunks first .. first + FEW_DEPTH - 1 (those of them that exist; `all`: they all do)
-  auto fetch = [&](float (&x)[FEW_DEPTH][4], float (&y)[FEW_DEPTH][4], int first, bool all) {
+    for (int st = 0; st < 4; ++st)
 #pragma unroll
-    for (int d = 0; d < FEW_DEPTH; ++d)
+      for (int rb = 0; rb < RB; ++rb) acc[rb] = __builtin_amdgcn_mfma_f32_16x16x4f32(x[rb][st], y[st], acc[rb], 0, 0, 0);
+  };
+  // the loads of the chunks first .. first + DEPTH - 1 (those of them that exist; `all`: they all do)
+  auto fetch = [&](float (&x)[DEPTH][RB][4], float (&y)[DEPTH][4], int first, bool all) {
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d)
       if (all || first + d < chunks) {
-        load4_aligned<TA>(x[d], pa + (first + d) * 16);
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) load4_aligned<TA>(x[d][rb], pa[rb] + (first + d) * 16);
         load4_aligned<TW>(y[d], pw + (first + d) * 16);
       }
   };
-  auto multiply_set = [&](float (&x)[FEW_DEPTH][4], float (&y)[FEW_DEPTH][4], int first, bool all) {
+  auto multiply_set = [&](float (&x)[DEPTH][RB][4], float (&y)[DEPTH][4], int first, bool all) {
 #pragma unroll
-    for (int d = 0; d < FEW_DEPTH; ++d)
+    for (int d = 0; d < DEPTH; ++d)
       if (all || first + d < chunks) multiply(x[d], y[d]);
   };
 #pragma unroll
-  for (int st = 0; st < FEW_SETS - 1; ++st) fetch(a[st], w[st], st * FEW_DEPTH, false);
+  for (int st = 0; st < FEW_SETS - 1; ++st) fetch(a[st], w[st], st * DEPTH, false);
   int c0 = 0;
   // while every set of a round and the sets asked for in it lie inside K nothing in the loop is conditional: the
   // compiler then counts the loads and waits for just those of the set it multiplies
-  for (; c0 + (2 * FEW_SETS - 1) * FEW_DEPTH <= chunks; c0 += FEW_SETS * FEW_DEPTH) {
+  for (; c0 + (2 * FEW_SETS - 1) * DEPTH <= chunks; c0 += FEW_SETS * DEPTH) {
 #pragma unroll
     for (int st = 0; st < FEW_SETS; ++st) {
-      fetch(a[(st + FEW_SETS - 1) % FEW_SETS], w[(st + FEW_SETS - 1) % FEW_SETS], c0 + (st + FEW_SETS - 1) * FEW_DEPTH, true);
-      multiply_set(a[st], w[st], c0 + st * FEW_DEPTH, true);
+      fetch(a[(st + FEW_SETS - 1) % FEW_SETS], w[(st + FEW_SETS - 1) % FEW_SETS], c0 + (st + FEW_SETS - 1) * DEPTH, true);
+      multiply_set(a[st], w[st], c0 + st * DEPTH, true);
     }
   }
-  for (; c0 < chunks; c0 += FEW_SETS * FEW_DEPTH) {
+  for (; c0 < chunks; c0 += FEW_SETS * DEPTH) {
 #pragma unroll
     for (int st = 0; st < FEW_SETS; ++st) {
-      fetch(a[(st + FEW_SETS - 1) % FEW_SETS], w[(st + FEW_SETS - 1) % FEW_SETS], c0 + (st + FEW_SETS - 1) * FEW_DEPTH, false);
-      multiply_set(a[st], w[st], c0 + st * FEW_DEPTH, false);
+      fetch(a[(st + FEW_SETS - 1) % FEW_SETS], w[(st + FEW_SETS - 1) % FEW_SETS], c0 + (st + FEW_SETS - 1) * DEPTH, false);
+      multiply_set(a[st], w[st], c0 + st * DEPTH, false);
     }
   }
   for (int k0 = chunks * 16; k0 < K; k0 += 16) {
     const int k = k0 + 4 * kq;
     const int valid = k < K ? (K - k < 4 ? K - k : 4) : 0;
-    float x[4] = {0.f, 0.f, 0.f, 0.f}, y[4] = {0.f, 0.f, 0.f, 0.f};
+    float x[RB][4], y[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) x[rb][0] = x[rb][1] = x[rb][2] = x[rb][3] = 0.f;
     if (valid) {
-      load4<TA>(x, pa + k0, valid, false);
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) load4<TA>(x[rb], pa[rb] + k0, valid, false);
       load4<TW>(y, pw + k0, valid, false);
     }
     multiply(x, y);
@@ -363,13 +379,15 @@ __global__ __launch_bounds__(64) void gemm_nt_few_rows_kernel(TC* __restrict__ C
   if (!w_ok) return;
   const float b = bias ? Num<TW>::ld(bias + n) : 0.f;
 #pragma unroll
-  for (int r = 0; r < 4; ++r) {
-    const int m = 4 * kq + r;
-    if (m >= M) continue;
-    float v = acc[r];
-    if (bias) v += b;
-    Num<TC>::st(C + (int64_t)m * ldc + n, v);
-  }
+  for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int m = 16 * rb + 4 * kq + r;
+      if (m >= M) continue;
+      float v = acc[rb][r];
+      if (bias) v += b;
+      Num<TC>::st(C + (int64_t)m * ldc + n, v);
+    }
 }
 
 // in_bf16: A, W and bias are bfloat16 (else float); out_bf16: C is bfloat16 (else float).
@@ -378,12 +396,15 @@ extern "C" int ga_gemm_nt(void* C, int64_t ldc, const void* A, int64_t lda, cons
                           hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (K <= 0) return -1;
-  const bool few = M <= 16;                 // a decode step's rows: a wavefront per 16 columns
+  // up to 64 rows: a wavefront per 16 columns, which it streams once for up to four blocks of 16 rows (with more than 32
+  // rows and very many columns, a head over a large vocabulary, the plain kernel is faster: measured at 151,936 columns)
+  const bool few = M <= GEMM_MATRIX_FROM_ROWS && !(M > 32 && N >= 65536);
+  const int row_blocks = (M + 15) / 16;
   // many rows: the matrix cores, in the largest of the tiles 128 x 128, 128 x 64, 64 x 64 that still makes 256 workgroups
   const bool matrix = M > GEMM_MATRIX_FROM_ROWS;
   const bool wide = matrix && (int64_t)((M + 127) / 128) * ((N + 127) / 128) >= 256;
   const bool tall = matrix && !wide && (int64_t)((M + 127) / 128) * ((N + 63) / 64) >= 256;
-  const int tm = few ? 16 : (wide || tall) ? 128 : 64, tn = few ? 16 : wide ? 128 : 64;
+  const int tm = (wide || tall) ? 128 : 64, tn = few ? 16 : wide ? 128 : 64;
   dim3 grid((N + tn - 1) / tn, (M + tm - 1) / tm), block(GEMM_THREADS);
   if (grid.y > 65535) return -2;
   // 16-byte loads (8 bytes for bfloat16) need rows that start at multiples of four elements
@@ -392,8 +413,17 @@ extern "C" int ga_gemm_nt(void* C, int64_t ldc, const void* A, int64_t lda, cons
   const int wide_w = (K % 4 == 0 && (uintptr_t)W % unit == 0) ? 1 : 0;
 #define LAUNCH(TA, TW, TC)                                                                                   \
   do {                                                                                                       \
-    if (few)                                                                                                 \
-      hipLaunchKernelGGL((gemm_nt_few_rows_kernel<TA, TW, TC>), grid, dim3(64), 0, stream, (TC*)C, ldc,      \
+    if (few && row_blocks == 1)                                                                              \
+      hipLaunchKernelGGL((gemm_nt_few_rows_kernel<TA, TW, TC, 1>), grid, dim3(64), 0, stream, (TC*)C, ldc,   \
+                         (const TA*)A, lda, (const TW*)W, (const TW*)bias, M, N, K, wide_a, wide_w);         \
+    else if (few && row_blocks == 2)                                                                         \
+      hipLaunchKernelGGL((gemm_nt_few_rows_kernel<TA, TW, TC, 2>), grid, dim3(64), 0, stream, (TC*)C, ldc,   \
+                         (const TA*)A, lda, (const TW*)W, (const TW*)bias, M, N, K, wide_a, wide_w);         \
+    else if (few && row_blocks == 3)                                                                         \
+      hipLaunchKernelGGL((gemm_nt_few_rows_kernel<TA, TW, TC, 3>), grid, dim3(64), 0, stream, (TC*)C, ldc,   \
+                         (const TA*)A, lda, (const TW*)W, (const TW*)bias, M, N, K, wide_a, wide_w);         \
+    else if (few)                                                                                            \
+      hipLaunchKernelGGL((gemm_nt_few_rows_kernel<TA, TW, TC, 4>), grid, dim3(64), 0, stream, (TC*)C, ldc,   \
                          (const TA*)A, lda, (const TW*)W, (const TW*)bias, M, N, K, wide_a, wide_w);         \
     else if (matrix && wide)                                                                                 \
       hipLaunchKernelGGL((gemm_nt_matrix_kernel<TA, TW, TC, 128, 128, 32>), grid, block, 0, stream,          \

@@ -179,7 +179,8 @@ def test_gemm_nt_at_drawn_sizes(seed):
 def test_gemm_nt_32_bit_is_the_chain_of_fused_multiply_adds_over_ascending_k(M):
     """What the 32-bit product IS, stated without any kernel: every element starts at zero and takes its K terms in
     ascending order, each as one fused multiply-add (one rounding); the bias is added last.  3 rows run on the
-    16x16x4 matrix instruction, 40 on plain FMA, 70 on the 32x32x2 matrix instruction: all three must give these bits."""
+    16x16x4 matrix instruction, 40 on the same with three blocks of rows to a wavefront, 70 on the 32x32x2 matrix
+    instruction: all must give these bits (the plain-FMA kernel is held against them in the test below)."""
     from ginfer_amd.kernels import ops
     N, K = 5, 37
     a, w, b = rnd((M, K), torch.float32, 31), rnd((N, K), torch.float32, 32), rnd((N,), torch.float32, 33)
@@ -196,17 +197,19 @@ def test_gemm_nt_32_bit_is_the_chain_of_fused_multiply_adds_over_ascending_k(M):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("M,N,K,bias", [(65, 130, 77, True), (200, 1536, 521, False), (128, 128, 32, True),
-                                        (300, 4600, 1000, True), (2048, 1536, 1536, False), (257, 66, 3, True)])
+                                        (300, 4600, 1000, True), (2048, 1536, 1536, False), (257, 66, 3, True),
+                                        (130, 66000, 40, True)])
 def test_gemm_nt_on_the_matrix_cores_gives_the_bits_of_the_fma_kernel(dtype, M, N, K, bias):
-    """More than 64 rows go through the 32-bit matrix-core instruction, up to 64 through plain fused multiply-adds; both
-    add an element's terms over ascending k into one accumulator, so the large product must equal, bit for bit, the
-    same rows multiplied 64 and 16 at a time, and one row alone."""
+    """More than 64 rows go through tiles of the 32-bit matrix-core instruction, up to 64 through a wavefront per 16
+    columns with one to four blocks of 16 rows (and, from 33 rows on with 65,536 columns and more, through plain fused
+    multiply-adds); all add an element's terms over ascending k into one accumulator, so the large product must equal,
+    bit for bit, the same rows multiplied 64, 48, 32 and 16 at a time, and one row alone."""
     from ginfer_amd.kernels import ops
     a, w = rnd((M, K), dtype, 16), rnd((N, K), dtype, 17)
     b = rnd((N,), dtype, 18) if bias else None
     full = ops.gemm_nt(a, w, b, out_dtype=torch.float32)
     close(full, a.double() @ w.double().t() + (b.double() if bias else 0), 5e-5)
-    for rows in (64, 16):
+    for rows in (64, 48, 32, 16):
         pieces = torch.cat([ops.gemm_nt(a[r:r + rows].contiguous(), w, b, out_dtype=torch.float32) for r in range(0, M, rows)])
         assert torch.equal(pieces, full), "rows %d at a time: %d elements differ" % (rows, int((pieces != full).sum()))
     assert torch.equal(ops.gemm_nt(a[M - 1:].contiguous(), w, b, out_dtype=torch.float32)[0], full[M - 1])
