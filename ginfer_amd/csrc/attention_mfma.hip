@@ -482,13 +482,28 @@ __global__ __launch_bounds__(64 * DEC_WAVES) void attn_decode_split_kernel(
 }
 
 // grid (decode tokens, nh), 64 threads: merges the splits of one (token, head) in ascending order.
+// EARLY > 0 (at most that many splits, the usual case): every partial output this lane will need is asked for at
+// once, before the weights are worked out: one trip to memory instead of one after the other.  The sums are the same,
+// in the same order.
 #define MAX_SPLITS 256
+template <int EARLY>
 __global__ __launch_bounds__(64) void attn_decode_combine_kernel(
     bf16_t* __restrict__ out, int64_t out_stride, const float* __restrict__ part_o,
     const float* __restrict__ part_ml, const int4* __restrict__ decode_info, int nh, int num_splits) {
   __shared__ float w_s[MAX_SPLITS];
   const int ti = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
   const int64_t base = ((int64_t)ti * nh + head) * num_splits;
+  constexpr int DPL = (HD + 63) / 64;
+  float o[DPL][EARLY > 0 ? EARLY : 1];
+  const int row = decode_info[ti].x;
+  if (EARLY > 0) {
+#pragma unroll
+    for (int i = 0; i < DPL; ++i) {
+      const int d = lane + 64 * i < HD ? lane + 64 * i : 0;
+#pragma unroll
+      for (int s = 0; s < EARLY; ++s) o[i][s] = part_o[(base + (s < num_splits ? s : 0)) * HD + d];
+    }
+  }
   float mx = -INFINITY;
   for (int s = lane; s < num_splits; s += 64) mx = fmaxf(mx, part_ml[(base + s) * 2]);
   mx = wave_max(mx);
@@ -502,7 +517,19 @@ __global__ __launch_bounds__(64) void attn_decode_combine_kernel(
   total = wave_sum(total);
   __syncthreads();
   const float inv = 1.f / total;
-  bf16_t* op = out + (int64_t)decode_info[ti].x * out_stride + (int64_t)head * HD;
+  bf16_t* op = out + (int64_t)row * out_stride + (int64_t)head * HD;
+  if (EARLY > 0) {
+#pragma unroll
+    for (int i = 0; i < DPL; ++i) {
+      const int d = lane + 64 * i;
+      float acc = 0.f;
+#pragma unroll
+      for (int s = 0; s < EARLY; ++s)
+        if (s < num_splits) acc += o[i][s] * w_s[s];
+      if (d < HD) op[d] = f32_to_bf16(acc * inv);
+    }
+    return;
+  }
   for (int d = lane; d < HD; d += 64) {
     float acc = 0.f;
 #pragma unroll 8
@@ -896,9 +923,15 @@ extern "C" int ga_attn_decode(void* out, int64_t out_stride, const void* q, int6
                      num_splits);
   int rc = GA_CHECK_LAUNCH();
   if (rc || num_splits == 1) return rc;
-  hipLaunchKernelGGL(attn_decode_combine_kernel, dim3(n_tokens, nh), dim3(64), 0, stream, (bf16_t*)out,
-                     out_stride, (const float*)workspace_o, (const float*)workspace_ml,
-                     (const int4*)decode_info, nh, num_splits);
+#define COMBINE(EARLY)                                                                                       \
+  hipLaunchKernelGGL(attn_decode_combine_kernel<EARLY>, dim3(n_tokens, nh), dim3(64), 0, stream, (bf16_t*)out, \
+                     out_stride, (const float*)workspace_o, (const float*)workspace_ml,                        \
+                     (const int4*)decode_info, nh, num_splits)
+  if (num_splits <= 8) COMBINE(8);
+  else if (num_splits <= 16) COMBINE(16);
+  else if (num_splits <= 32) COMBINE(32);
+  else COMBINE(0);
+#undef COMBINE
   return GA_CHECK_LAUNCH();
 }
 
