@@ -42,6 +42,7 @@ class _Request:
     tables: List[List[int]] = field(default_factory=list)   # per group: logical block -> page or -1
     contents: List[List[int]] = field(default_factory=list) # per group: content number of each remembered block
     gone: List[int] = field(default_factory=list)           # per group: every block before this one was given back
+    hit: int = 0                         # tokens taken over from a remembered prefix, not yet counted as a hit
 
 
 def _block_tokens(token_ids, block, page_size):
@@ -255,7 +256,8 @@ class CacheManager:
             self._mirror_table(gi, req)
         req.length = blocks * ps
         self._length_np[req.slot] = req.length
-        self.prefix_hit_tokens += req.length
+        req.hit = req.length             # counted once the request's first tokens are reserved: an admission that is
+                                         # taken back for lack of pages, and tried again step after step, is no hit
 
     def _remember(self, req, token_ids):
         """Remembers the request's full pages whose tokens are known and whose keys and values are committed."""
@@ -346,6 +348,16 @@ class CacheManager:
             raise ValueError("request %r has %d reserved tokens that were not committed" % (rid, req.pending))
         if n_new < 1:
             raise ValueError("append needs at least one token")
+        hit, req.hit = req.hit, 0
+        try:
+            first = self._append(req, rid, n_new)
+        except OutOfPages:
+            req.hit = hit
+            raise
+        self.prefix_hit_tokens += hit
+        return first
+
+    def _append(self, req, rid, n_new):
         if n_new == 1 and not self._any_window and req.length % self.page_size:
             req.pending = 1              # the common decode step: room is left in the last page
             return req.length

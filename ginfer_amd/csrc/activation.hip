@@ -1,7 +1,7 @@
 // SwiGLU on the fused gate-up product: out[t, i] = (g * (1 / (1 + exp(-g)))) * u with
 // g = gu[t, i], u = gu[t, I + i].  32-bit arithmetic, one rounding.
 // Formula: ginfer/core/op/kernels/cuda/swiglu_kernel.cu:24-27 (which skips a tail of numel % 8).
-#include "common.cuh"
+#include "common.h"
 #include "ginfer_amd.h"   // the entry points below are checked against their declarations
 
 template <typename T>

@@ -25,7 +25,7 @@
 // its sums over the keys of a tile likewise, and tiles follow each other in ascending order.
 #include <type_traits>
 
-#include "common.cuh"
+#include "common.h"
 #include "ginfer_amd.h"   // the entry points below are checked against their declarations
 
 #define MAX_HD 256
@@ -795,14 +795,18 @@ __global__ __launch_bounds__(64 * (HA_COMPUTE + HA_LOADERS)) void paged_attentio
 // where they are of one request, its tiles of keys and values (1 for steps of single tokens; 0: the library chooses,
 // which for steps of 32 tokens and more means two kernels: the matrix cores for a request's 8 tokens and more, a
 // wavefront per token and head for fewer; -1: as 0, and the caller knows that every request of the step has at least 8
-// tokens in it, which saves the second kernel); a token's result does not depend on it.
+// tokens in it, which saves the second kernel); a token's result does not depend on it.  few_tokens_workgroups: a step
+// that makes no more workgroups of a token and a kv head than this goes whole to the kernel for single tokens;
+// fill_workgroups: the kernel for portions takes as many wavefronts to a workgroup as still leave this many workgroups
+// (both decide speed only; the caller's table of thresholds holds them).
 extern "C" int ga_paged_attention_generic(void* out, int64_t out_stride, const void* q,
                                           int64_t q_stride, const void* k_pages,
                                           const void* v_pages, const void* block_table,
                                           int table_width, const void* token_entry,
                                           const void* positions, int tokens, int nh, int nkv, int hd,
                                           int page_size, int window, float scale, int is_bf16,
-                                          int tokens_per_workgroup, hipStream_t stream) {
+                                          int tokens_per_workgroup, int few_tokens_workgroups,
+                                          int fill_workgroups, hipStream_t stream) {
   if (tokens <= 0) return 0;
   if (hd > MAX_HD || hd <= 0 || nkv <= 0 || nh % nkv != 0 || page_size <= 0) return -1;
   const int group = nh / nkv;
@@ -822,7 +826,7 @@ extern "C" int ga_paged_attention_generic(void* out, int64_t out_stride, const v
   // are no more than two of them to a compute unit.  Its four wavefronts share a tile's keys, where the kernel for
   // prompt portions has one wavefront walk them; that one wins by the tiles its tokens share once there are many
   // (measured at contexts of 512 and 4,096: 12 heads in 2 groups up to 256 tokens, 28 in 4 up to 128, 16 in 16 up to 32).
-  if (tokens_per_workgroup == 0 && wide && hd % 16 == 0 && hd <= 128 && (int64_t)tokens * nkv * ((group + 15) / 16) <= 512)
+  if (tokens_per_workgroup == 0 && wide && hd % 16 == 0 && hd <= 128 && (int64_t)tokens * nkv * ((group + 15) / 16) <= few_tokens_workgroups)
     tokens_per_workgroup = 1;
   if (tokens_per_workgroup == 0 && tokens >= 2 * MA_COLS && hd % 16 == 0 && hd <= 128) {
     int tq = 1, hpw = 1;
@@ -837,7 +841,7 @@ extern "C" int ga_paged_attention_generic(void* out, int64_t out_stride, const v
         const int t = most / h, key = 2 * (t * h + (h == group ? 1 : 0));      // a whole kv group counts for one more
         if (key >= best) best = key, tq = t, hpw = h;                           // among equals, more heads
       }
-      if (workgroups(tq, hpw) >= 384) break;
+      if (workgroups(tq, hpw) >= fill_workgroups) break;
     }
     const int head_blocks = (group + hpw - 1) / hpw, waves = tq * hpw;
     const size_t lds = sizeof(float) * (2 * ((size_t)WAVE * (hd + KPAD) + (size_t)hd * VS) + (size_t)waves * (WAVE / 2) * MA_COLS) +

@@ -28,7 +28,7 @@
 // The decode kernel and the first prefill kernel stage nothing through LDS: each operand element is loaded
 // once per wavefront, and the heads of a group that run side by side hit the same lines in the vector cache.
 // The second prefill kernel (head sizes 64, 128, 256) has one wavefront load each tile into LDS for all heads.
-#include "common.cuh"
+#include "common.h"
 #include "ginfer_amd.h"   // the entry points below are checked against their declarations
 
 #ifndef HEAD_DIM

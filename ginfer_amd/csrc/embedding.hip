@@ -2,7 +2,7 @@
 // The residual stream is kept in 32-bit in both dtypes, so the gather widens as it copies.
 // Formula: ginfer/core/op/kernels/cuda/embedding_kernel.cu:16-24 (which copies in the table's
 // dtype and drops a tail of H % 8 elements; here every element is copied).
-#include "common.cuh"
+#include "common.h"
 #include "ginfer_amd.h"   // the entry points below are checked against their declarations
 
 template <typename T>

@@ -16,7 +16,7 @@
 //
 // A step of K is asked for (in 16-byte loads where rows allow it, consecutive lanes on consecutive elements)
 // while the step before is being multiplied.
-#include "common.cuh"
+#include "common.h"
 #include "ginfer_amd.h"   // the entry points below are checked against their declarations
 
 #define GEMM_THREADS 256

@@ -12,7 +12,7 @@
 // in any order as long as both operands agree, lane group g = l/16 takes the 16 elements
 // [k + 16g, k + 16g + 16) of every 64-element step as two products, so that the four lanes of a row read
 // 128 consecutive bytes.
-#include "common.cuh"
+#include "common.h"
 #include "ginfer_amd.h"   // the entry points below are checked against their declarations
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
@@ -94,7 +94,7 @@ struct SkinnyTrip {
     for (int u = 0; u < UNROLL; ++u)
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
-        const int kk = k + u * 64 + g * 16 + j * 8;
+        const int kk = k + u * 64 + j * 32 + g * 8;
         const bool ok = kk < ke;
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) a[u][j][nt] = (ok && wok[nt]) ? load8(wp[nt] + kk) : zero8();

@@ -34,7 +34,9 @@ int ga_rope_kv_write(void* qkv, const void* positions, const void* cos_t, const 
                      void* k_pages, void* v_pages, int tokens, int nh, int nkv, int hd, int rotary_dim, int page_size,
                      int write_kv, int is_bf16, hipStream_t stream);
 
-// ---- gemm.hip: C [M, N] = A [M, K] . W [N, K]^T + bias, plain 32-bit FMA (the 32-bit path; also bfloat16 in)
+// ---- gemm.hip: C [M, N] = A [M, K] . W [N, K]^T + bias in true 32-bit: the matrix cores' 32-bit instructions (and plain FMA
+// for 33 to 64 rows of very wide products), every element one accumulator over ascending k: the same bits whichever
+// kernel runs (the 32-bit path; also bfloat16 in)
 int ga_gemm_nt(void* C, int64_t ldc, const void* A, int64_t lda, const void* W, const void* bias, int M, int N, int K,
                int in_bf16, int out_bf16, hipStream_t stream);
 
@@ -69,11 +71,13 @@ int ga_silu_mul_transposed(void* out, const void* gu_t, int tokens, int inter, h
 
 // ---- attention_generic.hip: every token attends to its request's pages; any head size up to 256, window or 0;
 // tokens_per_workgroup neighbouring tokens share a workgroup's tiles of keys and values (0: the library chooses; -1: the
-// same, and every request of the step has at least 8 tokens in it)
+// same, and every request of the step has at least 8 tokens in it); few_tokens_workgroups, fill_workgroups: the two
+// thresholds by which the launcher chooses among its kernels (speed only)
 int ga_paged_attention_generic(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* k_pages,
                                const void* v_pages, const void* block_table, int table_width, const void* token_entry,
                                const void* positions, int tokens, int nh, int nkv, int hd, int page_size, int window,
-                               float scale, int is_bf16, int tokens_per_workgroup, hipStream_t stream);
+                               float scale, int is_bf16, int tokens_per_workgroup, int few_tokens_workgroups,
+                               int fill_workgroups, hipStream_t stream);
 
 // ---- attention_mfma.hip (one library per head size): bfloat16 on the matrix cores
 int ga_attn_head_dim();

@@ -8,7 +8,7 @@
 // residual stream untouched, so a row may be listed twice.
 // The sum over a row is taken in a fixed order that depends on H alone, so a row's result does not
 // depend on which other rows are in the batch.
-#include "common.cuh"
+#include "common.h"
 #include "ginfer_amd.h"   // the entry points below are checked against their declarations
 
 #define NORM_THREADS 256

@@ -1,7 +1,7 @@
 // Filling a tensor with normal numbers on the device: element i = mean + std * normal(key, i), the generator of
 // random_normal.h, which the host library random_fill_host.cpp shares: the same seed gives the same bits on both.
 // For models too large to pass through a file (a 72B shape is 145 GB of weights).
-#include "common.cuh"
+#include "common.h"
 #include "ginfer_amd.h"   // the entry points below are checked against their declarations
 #include "random_normal.h"
 

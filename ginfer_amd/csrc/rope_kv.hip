@@ -11,7 +11,7 @@
 // that the matrix-core attention kernels read 8 consecutive keys of one dimension in one 16-byte
 // load).  The slot of token t is slot_mapping[t] = page * page_size + slot_in_page, or -1 to write
 // nothing for that token.
-#include "common.cuh"
+#include "common.h"
 #include "ginfer_amd.h"   // the entry points below are checked against their declarations
 
 template <typename T>

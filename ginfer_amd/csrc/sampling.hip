@@ -8,7 +8,7 @@
 //     number the caller supplies, so the choice is a pure function of (logits, temperature, uniform):
 //     the cut into segments depends on the vocabulary alone, never on the rows beside it.
 // The reference samples greedily only (ginfer/engine/sampling_params.h:5-8).
-#include "common.cuh"
+#include "common.h"
 #include "ginfer_amd.h"   // the entry points below are checked against their declarations
 #include <atomic>
 #include <mutex>

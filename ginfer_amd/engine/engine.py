@@ -8,6 +8,7 @@ from dataclasses import dataclass
 import torch
 from typing import List, Optional
 
+from ..kernels.tuning import TUNING
 from ..sampling import SamplingParams, Sampler
 from .runner import ModelRunner, StepEntry
 from .scheduler import Scheduler
@@ -103,14 +104,14 @@ class Engine:
         greedy = [SamplingParams()]
         try:
             done = set()
-            for n in (2048, 1024, 512, 400, 256, 160, 96, 48, 8):
+            for n in TUNING.warmup_portion_lengths:
                 n = min(n, room)
                 if n < 1 or n in done:
                     continue
                 done.add(n)
                 # short portions three times: the second run records the padded step that a lone prompt of about this
                 # length will be laid into, the third replays it
-                runs = 3 if n < 512 else 1
+                runs = 3 if n < TUNING.warmup_record_below else 1
                 for k in range(runs):
                     logits = runner.step([StepEntry(rid, [0] * n, [n - 1])], borrow=True)
                     self.sampler.sample_on_device(logits, greedy, [0])

@@ -281,7 +281,7 @@ class ModelRunner:
 
     def _run(self, host, borrow, device_tokens=None):
         E, T = host["E"], host["T"]
-        graphable = self.use_graphs and T == E and E <= GRAPH_MAX_ROWS and len(host["rows"]) == E and \
+        graphable = self.use_graphs and T == E and E <= TUNING.graph_max_rows and len(host["rows"]) == E and \
             bool((host["rows"] == np.arange(E)).all())
         if graphable:
             bucket = _context_bucket(host["max_kv"])
@@ -291,7 +291,7 @@ class ModelRunner:
                 self._graphs[key] = g        # most recently used last
             else:
                 self._graph_seen[key] = self._graph_seen.get(key, 0) + 1
-                if self._graph_seen[key] >= GRAPH_AFTER:
+                if self._graph_seen[key] >= TUNING.graph_after:
                     g = self._record(self._capture, key, host)
             if g is not None:
                 g["buf"].fill(host)
@@ -321,7 +321,7 @@ class ModelRunner:
             self._graph_budget = min((free + torch.cuda.memory_reserved(self.device)
                                       - torch.cuda.memory_allocated(self.device)) // 2, total // 8)
         need = self._graph_bytes_seen.get(key[0] == "padded", 0)
-        while self._graphs and (len(self._graphs) >= GRAPH_KEEP or self._graph_bytes + need > self._graph_budget):
+        while self._graphs and (len(self._graphs) >= TUNING.graph_keep or self._graph_bytes + need > self._graph_budget):
             old = self._graphs.pop(next(iter(self._graphs)))
             self._graph_bytes -= old["bytes"]
             del old
@@ -356,7 +356,7 @@ class ModelRunner:
         and single-token records that fill the plan point at the first padding row.  Rows do not mix in any kernel,
         so what the padding computes stays in the padding.  None: the step runs launch by launch."""
         T, E, R = host["T"], host["E"], len(host["rows"])
-        if T + 1 > self._padded_max_rows or E > GRAPH_MAX_ROWS:
+        if T + 1 > self._padded_max_rows or E > TUNING.graph_max_rows:
             return None
         t_pad = 64                       # coarse sizes, so that few recorded steps serve many: rows 64, 128, 256, 512
         while t_pad < T + 1:
@@ -375,7 +375,7 @@ class ModelRunner:
             self._graphs[key] = g
         else:
             self._graph_seen[key] = self._graph_seen.get(key, 0) + 1
-            if self._graph_seen[key] >= GRAPH_AFTER:
+            if self._graph_seen[key] >= TUNING.graph_after:
                 g = self._record(self._capture_padded, key, host)
         if g is None:
             # not recorded yet: launched kernel by kernel, but with the same padded sizes, so that a step's bits do not
@@ -553,11 +553,6 @@ def _context_bucket(max_kv):
     while bucket < max_kv:
         bucket *= 2
     return bucket
-
-
-GRAPH_MAX_ROWS = 256     # decode batches up to this many requests are recorded
-GRAPH_AFTER = 2          # a batch shape is recorded the second time it is seen
-GRAPH_KEEP = 128         # recorded shapes kept at a time (least recently used goes first)
 
 
 class _StepBuffers:

@@ -27,7 +27,7 @@ MODULES = ("embedding", "norm", "rope_kv", "attention_generic", "attention_mfma"
            "activation", "sampling", "random_fill")
 # flags of single modules: the random-weights generator must round every operation by itself, as the host's twin does
 MODULE_FLAGS = {"random_fill": ["-ffp-contract=off"], "attention_generic": ["-ffp-contract=off"]}
-# headers beside common.cuh that a module includes (they enter its digest)
+# headers beside common.h that a module includes (they enter its digest)
 MODULE_HEADERS = {"random_fill": ["random_normal.h"]}
 # plain C++ libraries for the host (no GPU runtime), built with the host compiler from csrc/host/
 HOST_MODULES = ("random_fill_host",)
@@ -69,7 +69,7 @@ def _split(module):
 def _digest(module):
     src, defines, _ = _split(module)
     h = hashlib.sha256()
-    for name in [src + ".hip", "common.cuh", "ginfer_amd.h"] + MODULE_HEADERS.get(src, []):
+    for name in [src + ".hip", "common.h", "ginfer_amd.h"] + MODULE_HEADERS.get(src, []):
         with open(os.path.join(CSRC, name), "rb") as f:
             h.update(f.read())
     h.update(" ".join(FLAGS + MODULE_FLAGS.get(src, [])).encode())

@@ -232,7 +232,8 @@ def paged_attention_generic(q, k_pages, v_pages, block_table, token_entry, posit
         _ptr(out), _i64(out.stride(0)), _ptr(q), _i64(q.stride(0)), _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
         _i(block_table.shape[1]), _ptr(token_entry), _ptr(positions), _i(T), _i(num_heads), _i(num_kv_heads),
         _i(head_dim), _i(k_pages.shape[2]), _i(int(window) if window else 0), _f(scale), _i(_is_bf16(q.dtype)),
-        _i(int(tokens_per_workgroup)), _stream()), "paged_attention_generic")
+        _i(int(tokens_per_workgroup)), _i(TUNING.generic_few_tokens_workgroups), _i(TUNING.generic_fill_workgroups),
+        _stream()), "paged_attention_generic")
     return out
 
 

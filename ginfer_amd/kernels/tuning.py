@@ -7,7 +7,9 @@ the layer sizes of a 1.5B and a 7B model; a model of other sizes may want others
     TUNING.library_from_rows = 32                       # for the process
     GINFER_AMD_TUNING='{"library_from_rows": 32}'       # or from the environment, as JSON
 
-Nothing else in the package holds such a number.
+No part or dispatcher holds such a number of its own.  What the kernels fix when they are compiled is not in this table:
+the wavefronts of an attention workgroup (`PREFILL_WAVES`, `DEC_WAVES`), how late the running maximum of the softmax
+is raised (`LAZY_MAX`) and the like are macros at the top of the source that uses them, each with its measurement.
 """
 import json
 import os
@@ -57,11 +59,28 @@ class Tuning:
     prefill_wide_tiles_from: int = 1024      # tokens in a step from which prompt rows go 32 to a wavefront
     # heads of a kv group go side by side into a prefill workgroup only while the step still makes this many workgroups
     prefill_fill_workgroups: int = 256
+    # ---- the general attention kernels (the 32-bit path, odd head or page sizes; csrc/attention_generic.hip).  A step that
+    # makes no more workgroups of a token and a kv head than this goes whole to the kernel for single tokens (measured at
+    # contexts of 512 and 4,096: 12 heads in 2 groups up to 256 tokens); the kernel for portions takes as many wavefronts
+    # to a workgroup as still leave `generic_fill_workgroups` workgroups (one and a half to a compute unit).
+    generic_few_tokens_workgroups: int = 512
+    generic_fill_workgroups: int = 384
     # ---- recorded steps (engine/runner.py): steps with prompt portions are laid into recorded steps of padded sizes up
     # to `mixed_graph_max_tokens` rows, fewer for large models: padding pays while rows x weights stays under what the
     # device does in the time the host needs to launch a step kernel by kernel.
     mixed_graph_max_tokens: int = 512
     padded_rows_times_weights: float = 1.5e12
+    # decode batches up to `graph_max_rows` requests are recorded, a shape the `graph_after`-th time it is seen, and the
+    # `graph_keep` most recently used recorded shapes are kept
+    graph_max_rows: int = 256
+    graph_after: int = 2
+    graph_keep: int = 128
+    # ---- the engine's warm-up (engine/engine.py): prompt portions of these lengths run once before the first request
+    # (the BLAS library picks other kernels for other numbers of rows and loads each at its first use); the ones under
+    # `warmup_record_below` run three times, so that the padded step a lone prompt of about that length is laid into is
+    # recorded and replayed before a request pays for it
+    warmup_portion_lengths: tuple = (2048, 1024, 512, 400, 256, 160, 96, 48, 8)
+    warmup_record_below: int = 512
 
     def update(self, values):
         known = {f.name: f.type for f in fields(self)}

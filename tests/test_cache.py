@@ -188,10 +188,12 @@ def test_prefix_is_shared_exactly():
     assert m.table("a", 0) == [0, 1, 2]
     b = a[:16] + [7, 7, 7]
     m.admit("b", b)
-    assert m.length("b") == 16 and m.table("b", 0) == [0, 1] and m.prefix_hit_tokens == 16
+    assert m.length("b") == 16 and m.table("b", 0) == [0, 1]
+    assert m.prefix_hit_tokens == 0                # a hit counts once the request's first tokens are reserved
     assert m.groups[0].pool.holders(0) == 2 and m.groups[0].pool.holders(2) == 1
     m.check()
     _run(m, "b", b)
+    assert m.prefix_hit_tokens == 16
     assert m.table("b", 0) == [0, 1, 3]            # its own page from the first token that differs
     m.release("a", a)
     assert m.groups[0].pool.holders(0) == 1 and m.groups[0].pool.num_free == 5
@@ -259,6 +261,7 @@ def test_random_orders_with_shared_prefixes(seed):
     stems = [[rng.randrange(3) for _ in range(40)] for _ in range(3)]
     shadow = [dict() for _ in m.groups]
     live, tokens, next_id, hits = [], {}, 0, 0
+    found = {}                # what a request found in the cache counts as a hit once its first tokens are reserved
     for _ in range(800):
         op = rng.random()
         if op < 0.25 and m.can_admit():
@@ -271,7 +274,7 @@ def test_random_orders_with_shared_prefixes(seed):
             for gi in range(len(m.groups)):
                 for i, page in enumerate(m.table(next_id, gi)):
                     assert shadow[gi][page] == toks[:(i + 1) * ps]
-            hits += got
+            found[next_id] = got
             live.append(next_id)
             tokens[next_id] = toks
             next_id += 1
@@ -288,6 +291,8 @@ def test_random_orders_with_shared_prefixes(seed):
             except OutOfPages:
                 m.check()
                 continue
+            hits += found.pop(rid, 0)
+            assert hits == m.prefix_hit_tokens
             for gi in range(len(m.groups)):
                 t = m.table(rid, gi)
                 for blk in range(start // ps, (start + n - 1) // ps + 1):

@@ -116,10 +116,10 @@ def test_mixed_with_pages_used_again(folders, sharp_folders, name, dtype, weight
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
 def test_trace_run_program(folders, tmp_path, dtype, name):
-    """bin/trace_run as a user runs it: whole, then mixed with few pages, in one process (C: layers with a
-    window beside layers without, so two groups of pages)."""
+    """bin/trace_run as a user runs it: whole, then mixed with few pages, in one process (A: the head shares the
+    embedding's table; C: layers with a window beside layers without, so two groups of pages)."""
     reqs = _requests(name, [70, 33, 120, 64, 90], seed=70)
     whole = H.steps_whole(reqs)
     mixed = H.steps_mixed({k + "m": v for k, v in reqs.items()}, max_live=4, seed=5)
@@ -180,6 +180,23 @@ def test_greedy_generation_through_the_entry_point(folders, dtype):
         assert o.prompt_token_ids == p and len(o.token_ids) == 12 and o.finish_reason == "max_tokens"
         assert streamed[o.request_id] == o.token_ids          # every token was handed out as it came, in order
     _greedy_as_plain(folder, prompts, outs, dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_greedy_generation_with_a_tied_head(folders, dtype):
+    """The smallest configuration as it is stated for this engine: tied head, prompts of 5, 17 and 33 tokens, 8 greedy
+    tokens each, pages of 16, through the entry point."""
+    from ginfer_amd import Engine, EngineConfig, SamplingParams
+    name = "A"
+    vocab = H.TINY[name][0]["vocab_size"]
+    prompts = [H.random_tokens(n, vocab, 300 + n) for n in (5, 17, 33)]
+    eng = Engine(EngineConfig(model_path=folders[name], dtype=dtype, max_num_batched_tokens=32, max_num_seqs=4,
+                              max_seq_len=128, kvcache_block_size=16, num_kvcache_blocks=16))
+    assert eng.runner.model.head.weight.data_ptr() == eng.runner.model.embedding.weight.data_ptr()     # one table
+    outs = eng.generate(prompts, SamplingParams(max_tokens=8, ignore_eos=True))
+    eng.runner.cache.check()
+    assert [len(o.token_ids) for o in outs] == [8, 8, 8]
+    _greedy_as_plain(folders[name], prompts, outs, dtype)
 
 
 def _greedy_as_plain(folder, prompts, outs, dtype):
@@ -533,8 +550,8 @@ def test_real_layer_sizes(tmp_path):
 def test_recorded_shapes_are_bounded(folders, monkeypatch):
     """Every batch size gets a graph of its own; only the most recently used are kept."""
     from ginfer_amd import ModelRunner, StepEntry
-    from ginfer_amd.engine import runner as R
-    monkeypatch.setattr(R, "GRAPH_KEEP", 3)
+    from ginfer_amd.kernels.tuning import TUNING
+    monkeypatch.setattr(TUNING, "graph_keep", 3)
     r = ModelRunner(folders["A"], dtype="bfloat16", page_size=16, num_pages=64, max_requests=8)
     ref = ModelRunner(folders["A"], dtype="bfloat16", page_size=16, num_pages=64, max_requests=8, use_graphs=False)
     toks = H.random_tokens(400, 512, 5)

@@ -314,6 +314,30 @@ def test_a_request_starts_behind_the_prefix_that_the_cache_holds():
     assert all(g.pool.num_free == g.pool.num_pages for g in cache.groups)
 
 
+def test_a_sharer_that_waits_for_pages_counts_its_hit_once():
+    """8 pages of 8: a request of 56 tokens decodes and holds 7 pages (8 once it crosses a page's edge); a second one
+    shares its first 32 tokens and has to wait, admitted and sent back step after step, until pages are free.  The
+    tokens found in the cache count once, when its first portion is reserved."""
+    sched, cache = make(num_pages=8, page_size=8, budget=64, max_num_seqs=2, prefix_caching=True)
+    a = seq(0, 56, max_tokens=6)
+    b = Sequence(1, a.token_ids[:32] + [3] * 12, 44, SamplingParams(max_tokens=2))
+    waited, first_portion = [], []
+
+    def on_admit(step, batch, hits):
+        if b.state is State.WAITING and step >= 2:
+            waited.append(step)
+            assert cache.prefix_hit_tokens == 0 and hits == 0
+        for sc in batch:
+            if sc.seq is b and not first_portion:
+                first_portion.append((step, sc.num_tokens, hits))
+    done = run_as_the_engine(sched, cache, [a], arrivals={2: b}, on_admit=on_admit)
+    assert len(waited) >= 3, "the second request did not have to wait: %s" % waited
+    assert first_portion and first_portion[0][2] == 32       # the hit is booked with the first portion, 32 tokens
+    assert cache.prefix_hit_tokens == 32
+    assert {s.request_id: s.token_ids for s in done} == {0: expected(a), 1: expected(b)}
+    assert all(g.pool.num_free == g.pool.num_pages for g in cache.groups)
+
+
 def run_as_the_engine(sched, cache, seqs, arrivals=None, on_admit=None, max_steps=10000):
     """The engine's own order of calls around a step, without the device: schedule (which reserves), the runner's
     bookkeeping for the step's entries (which finds everything reserved and so commits nothing), advance (which commits
