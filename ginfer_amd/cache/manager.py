@@ -1,10 +1,11 @@
 """The cache manager: keys and values in pages with a block table per request, and slots for
 per-request state of fixed size.
 
-Schedule entries of the model that keep keys and values fall into *groups* by what they need
-(num_kv_heads, head_dim, window).  A group has a page pool of its own and every request has one block
-table per group; all entries of a group share the table (page p means page p of every entry's
-tensor).  Block table entry i covers positions [i * page_size, (i + 1) * page_size) of the request.
+What a schedule entry of the model keeps per request is a list of caches: any number of paged ones (keys and values,
+`KVCacheSpec`, or any per-token tensors, `PagedSpec`) and of state slots (`StateSpec`); most entries keep one.  The
+paged caches fall into *groups* by what they need (their spec: widths, window).  A group has a page pool of its own and
+every request has one block table per group; all caches of a group share the table (page p means page p of every
+cache's tensors).  Block table entry i covers positions [i * page_size, (i + 1) * page_size) of the request.
 A group with a window gives a page back as soon as every position in it lies behind the window of the
 next token to be computed; its table keeps a -1 there.  Pages return to the pool when a request is
 released and are used again by later requests.  The reference has one pool, one table per sequence,
@@ -20,9 +21,9 @@ reference compares a 64-bit chain hash and the page's own tokens).  Only for mod
 keeps all keys and that have no per-request state: a window gives pages of a prefix back, and state has to
 see every token.
 
-Device layout of one group: one allocation [entries_in_group, 2 (k, v), pages, nkv * page_size * hd]; an
-entry's keys are viewed [pages, nkv, page_size, hd] and its values [pages, nkv, hd, page_size]
-(transposed inside a page, which is what the matrix-core attention kernels read fastest).
+Device layout of one group: for each tensor of its spec one allocation [caches_in_group, pages, page_size * elements
+per token]; keys are viewed [pages, nkv, page_size, hd] and values [pages, nkv, value_dim, page_size] (transposed
+inside a page, which is what the matrix-core attention kernels read fastest).
 """
 from array import array
 from dataclasses import dataclass, field
@@ -30,7 +31,7 @@ from typing import Dict, List, Optional
 
 import numpy as np
 
-from ..parts.base import KVCacheSpec, StateSpec
+from ..parts.base import KVCacheSpec, PagedSpec, StateSpec
 from .pages import PagePool, SlotPool, OutOfPages
 
 
@@ -50,11 +51,26 @@ def _block_tokens(token_ids, block, page_size):
     return array("i", token_ids[block * page_size:(block + 1) * page_size]).tobytes()
 
 
+def _is_paged(spec):
+    return isinstance(spec, (KVCacheSpec, PagedSpec))
+
+
+def caches_of(entry_spec):
+    """What a schedule entry keeps, as a list: a single spec stands for a list of one, None for none."""
+    if entry_spec is None:
+        return []
+    if isinstance(entry_spec, (list, tuple)):
+        return list(entry_spec)
+    return [entry_spec]
+
+
 class CacheGroup:
-    def __init__(self, spec, entries, num_pages, page_size):
-        self.spec, self.entries, self.page_size = spec, list(entries), page_size
+    def __init__(self, spec, units, num_pages, page_size):
+        """units: the caches of the group as (schedule entry, place in the entry's list)."""
+        self.spec, self.units, self.page_size = spec, list(units), page_size
+        self.entries = [e for e, _ in self.units]
         self.pool = PagePool(num_pages)
-        self.tensor = None               # device tensor, set by allocate_device
+        self.tensors = None              # device tensors by name [caches, pages, page_size * elements], set by allocate_device
         # full pages whose tokens are known, for requests that share a prefix
         self._page_of = {}               # (content number of the block before or 0, the block's tokens) -> page
         self._key_of = {}                # page -> its key in _page_of
@@ -99,8 +115,8 @@ class CacheGroup:
 
 class CacheManager:
     def __init__(self, cache_specs, page_size, num_pages, max_requests, prefix_caching=False):
-        """cache_specs: per schedule entry KVCacheSpec | StateSpec | None (None: keeps nothing, or reads
-        another entry's cache).  num_pages: pages of every group's pool, or a list with one count per group (in the
+        """cache_specs: per schedule entry KVCacheSpec | PagedSpec | StateSpec | None, or a list of them (None: keeps
+        nothing, or reads another entry's cache).  num_pages: pages of every group's pool, or a list with one count per group (in the
         order of `group_specs(cache_specs)`; a group with a window needs few, see `plan_pages`).  prefix_caching:
         requests admitted with their tokens share the pages of a known prefix."""
         if prefix_caching and not self.supports_prefix_caching(cache_specs):
@@ -119,16 +135,17 @@ class CacheManager:
         else:
             counts = [int(num_pages)] * len(by_key)
         self.groups = [CacheGroup(k, v, n, self.page_size) for (k, v), n in zip(by_key.items(), counts)]
-        self.group_of = {}               # schedule entry -> (group index, index inside the group)
+        self.group_of = {}               # (schedule entry, place in its list) -> (group index, index inside the group)
         for gi, g in enumerate(self.groups):
-            for j, e in enumerate(g.entries):
-                self.group_of[e] = (gi, j)
-        self.state_entries = [i for i, s in enumerate(self.cache_specs) if isinstance(s, StateSpec)]
+            for j, unit in enumerate(g.units):
+                self.group_of[unit] = (gi, j)
+        self.state_units = [(i, k) for i, s in enumerate(self.cache_specs) for k, c in enumerate(caches_of(s))
+                            if isinstance(c, StateSpec)]
         self.slots = SlotPool(self.max_requests)
         # one more slot than requests: the rows that pad a recorded step read and write the state of this slot, which
         # no request ever holds
         self.pad_slot = self.max_requests
-        self.state_tensors = {}          # schedule entry -> device tensor [max_requests + 1, *shape]
+        self.state_tensors = {}          # (schedule entry, place in its list) -> device tensor [max_requests + 1, *shape]
         self.requests: Dict[object, _Request] = {}
         # host mirrors for building a step without a Python loop per request: per group the block tables
         # by state slot (int32, -1 where there is no page), and the lengths by state slot
@@ -138,21 +155,41 @@ class CacheManager:
 
     @staticmethod
     def group_specs(cache_specs):
-        """{KVCacheSpec: [schedule entries]} in the order in which the groups are made."""
-        by_key: Dict[KVCacheSpec, List[int]] = {}
+        """{paged spec: [(schedule entry, place in its list)]} in the order in which the groups are made."""
+        by_key = {}
         for i, s in enumerate(cache_specs):
-            if isinstance(s, KVCacheSpec):
-                by_key.setdefault(s, []).append(i)
+            for k, c in enumerate(caches_of(s)):
+                if _is_paged(c):
+                    by_key.setdefault(c, []).append((i, k))
         return by_key
 
     @staticmethod
-    def window_pages(window, page_size, max_requests, max_step_tokens, max_model_len):
-        """Pages that a group with this window can hold at most.  Between steps a request holds the pages of positions
-        [length - window + 1, length), at most (window - 1) // page + 2 of them (`commit` gives the others back); while it
-        runs n tokens of a step it holds those of [length - window + 1, length + n), at most ceil(n / page) + 1 more; over
+    def state_bytes(cache_specs, max_requests):
+        """Device bytes of the per-request state: every state tensor has a slot for each request and one more."""
+        import torch
+        total = 0
+        for s in cache_specs:
+            for c in caches_of(s):
+                if isinstance(c, StateSpec):
+                    n = 1
+                    for d in c.shape:
+                        n *= int(d)
+                    total += (max_requests + 1) * n * torch.empty(0, dtype=c.dtype).element_size()
+        return total
+
+    @staticmethod
+    def window_span_pages(window, page_size):
+        """Pages that `window` consecutive positions can touch: what a request of a group with this window holds between
+        steps (`commit` gives back what lies behind the window of the next token) and while one more token runs."""
+        return (window - 1) // page_size + 2
+
+    @classmethod
+    def window_pages(cls, window, page_size, max_requests, max_step_tokens, max_model_len):
+        """Pages that a group with this window can hold at most.  While a request runs n tokens of a step it holds the
+        pages of the positions [length - window + 1, length + n): at most `window_span_pages` + 1 + (n - 1) // page; over
         the requests of a step the n add up to the step's token budget.  Never more than all keys of every request."""
         per_request_all = -(-max_model_len // page_size)
-        per_request = min((window - 1) // page_size + 3, per_request_all)
+        per_request = min(cls.window_span_pages(window, page_size) + 1, per_request_all)
         return min(max_requests * per_request + -(-max_step_tokens // page_size), max_requests * per_request_all)
 
     @classmethod
@@ -163,8 +200,8 @@ class CacheManager:
         groups = cls.group_specs(cache_specs)
         if not groups:
             return []
-        page_bytes = [len(entries) * 2 * spec.num_kv_heads * page_size * spec.head_dim * element_size
-                      for spec, entries in groups.items()]
+        page_bytes = [len(units) * sum(w for _, w in spec.page_tensors()) * page_size * element_size
+                      for spec, units in groups.items()]
         counts, left = [None] * len(groups), int(pool_bytes)
         for gi, spec in enumerate(groups):
             if spec.window is not None:
@@ -185,30 +222,36 @@ class CacheManager:
 
     @staticmethod
     def supports_prefix_caching(cache_specs):
-        return (any(isinstance(s, KVCacheSpec) for s in cache_specs)
-                and not any(isinstance(s, StateSpec) or (isinstance(s, KVCacheSpec) and s.window is not None)
-                            for s in cache_specs))
+        flat = [c for s in cache_specs for c in caches_of(s)]
+        return (any(_is_paged(c) for c in flat)
+                and not any(isinstance(c, StateSpec) or (_is_paged(c) and c.window is not None) for c in flat))
 
     # ---- device memory
     def pool_bytes(self, element_size):
-        return sum(g.pool.num_pages * len(g.entries) * 2 * g.spec.num_kv_heads * self.page_size * g.spec.head_dim
+        return sum(g.pool.num_pages * len(g.units) * sum(w for _, w in g.spec.page_tensors()) * self.page_size
                    * element_size for g in self.groups)
 
     def allocate_device(self, dtype, device):
         import torch
         for g in self.groups:
-            g.tensor = torch.zeros((len(g.entries), 2, g.pool.num_pages,
-                                    g.spec.num_kv_heads * self.page_size * g.spec.head_dim), dtype=dtype, device=device)
-        for e in self.state_entries:
-            s = self.cache_specs[e]
-            self.state_tensors[e] = torch.zeros((self.max_requests + 1,) + tuple(s.shape), dtype=s.dtype, device=device)
+            g.tensors = {name: torch.zeros((len(g.units), g.pool.num_pages, self.page_size * width), dtype=dtype,
+                                           device=device) for name, width in g.spec.page_tensors()}
+        for unit in self.state_units:
+            s = caches_of(self.cache_specs[unit[0]])[unit[1]]
+            self.state_tensors[unit] = torch.zeros((self.max_requests + 1,) + tuple(s.shape), dtype=s.dtype, device=device)
 
-    def kv_views(self, entry):
-        """(k_pages [pages, nkv, page_size, hd], v_pages [pages, nkv, hd, page_size]) of a schedule entry."""
-        gi, j = self.group_of[entry]
+    def page_views(self, entry, place=0):
+        """{name: [pages, page_size * elements per token]} of one paged cache of a schedule entry."""
+        gi, j = self.group_of[(entry, place)]
+        return {name: t[j] for name, t in self.groups[gi].tensors.items()}
+
+    def kv_views(self, entry, place=0):
+        """(k_pages [pages, nkv, page_size, hd], v_pages [pages, nkv, value_dim, page_size]) of a cache of keys and values."""
+        gi, j = self.group_of[(entry, place)]
         g = self.groups[gi]
-        n, nkv, hd = g.pool.num_pages, g.spec.num_kv_heads, g.spec.head_dim
-        return (g.tensor[j, 0].view(n, nkv, self.page_size, hd), g.tensor[j, 1].view(n, nkv, hd, self.page_size))
+        n, nkv = g.pool.num_pages, g.spec.num_kv_heads
+        return (g.tensors["k"][j].view(n, nkv, self.page_size, g.spec.head_dim),
+                g.tensors["v"][j].view(n, nkv, g.spec.v_dim, self.page_size))
 
     # ---- requests
     def has(self, rid):

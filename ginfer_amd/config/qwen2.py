@@ -14,6 +14,12 @@ from typing import List, Optional
 from .registry import register_architecture, ConfigError
 from .spec import PartSpec, prenorm_layer, ScheduleEntry, ModelSpec
 
+# How this architecture's checkpoints spell the prefixes of a layer's parts and of the parts outside the layers
+# (ginfer/model/qwen2.cc:34-46 and ginfer/model/loader/model_loader.cc:108-119 bind the same names)
+LAYER_TENSOR_NAMES = dict(mixer="self_attn", feed_forward="mlp", mixer_norm="input_layernorm",
+                          feed_forward_norm="post_attention_layernorm")
+MODEL_TENSOR_NAMES = dict(embedding="model.embed_tokens", final_norm="model.norm", head="lm_head")
+
 _REQUIRED = ("num_hidden_layers", "vocab_size", "max_position_embeddings", "num_attention_heads",
              "num_key_value_heads", "hidden_size", "intermediate_size")
 
@@ -138,7 +144,7 @@ class Qwen2Config:
             ffn = PartSpec("swiglu", dict(hidden_size=self.hidden_size,
                                           intermediate_size=self.intermediate_size))
             layers.append(prenorm_layer("model.layers.%d" % i, mixer=mixer, feed_forward=ffn,
-                                        mixer_norm=norm, feed_forward_norm=norm))
+                                        mixer_norm=norm, feed_forward_norm=norm, names=LAYER_TENSOR_NAMES))
         spec = ModelSpec(
             hidden_size=self.hidden_size, vocab_size=self.vocab_size, layers=layers,
             schedule=[ScheduleEntry(i) for i in range(self.num_hidden_layers)],
@@ -148,6 +154,6 @@ class Qwen2Config:
             head=PartSpec("lm_head", dict(vocab_size=self.vocab_size, hidden_size=self.hidden_size,
                                           tied=self.tie_word_embeddings)),
             max_positions=self.max_position_embeddings,
-            eos_token_ids=list(self.eos_token_ids))
+            eos_token_ids=list(self.eos_token_ids), names=dict(MODEL_TENSOR_NAMES))
         spec.validate()
         return spec

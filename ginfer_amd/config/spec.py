@@ -46,14 +46,12 @@ class LayerSpec:
 
 
 def prenorm_layer(prefix, mixer, feed_forward, mixer_norm, feed_forward_norm, names=None):
-    """The usual block of four parts (norm, mixer, norm, feed-forward) with the tensor names that checkpoints of this
-    family of models use."""
-    spelt = dict(mixer="self_attn", feed_forward="mlp", mixer_norm="input_layernorm",
-                 feed_forward_norm="post_attention_layernorm")
-    spelt.update(names or {})
+    """The usual block of four parts (norm, mixer, norm, feed-forward).  names: role -> the prefix of its tensors inside
+    the layer as the architecture's checkpoints spell it (the architecture's configuration knows; a role that is not
+    listed is spelt as the role itself)."""
     return LayerSpec(prefix=prefix, parts=dict(mixer=mixer, feed_forward=feed_forward, mixer_norm=mixer_norm,
                                                feed_forward_norm=feed_forward_norm),
-                     arrangement="prenorm", names=spelt)
+                     arrangement="prenorm", names=dict(names or {}))
 
 
 @dataclass
@@ -75,9 +73,12 @@ class ModelSpec:
     head: PartSpec
     max_positions: int
     eos_token_ids: List[int]
-    # tensor-name prefixes of the parts outside the layers
-    names: Dict[str, str] = field(default_factory=lambda: dict(
-        embedding="model.embed_tokens", final_norm="model.norm", head="lm_head"))
+    # tensor-name prefixes of the parts outside the layers, as the architecture's checkpoints spell them (a part that is
+    # not listed is spelt as its role: "embedding", "final_norm", "head")
+    names: Dict[str, str] = field(default_factory=dict)
+
+    def name_of(self, role):
+        return self.names.get(role, role)
 
     def validate(self):
         for i, e in enumerate(self.schedule):

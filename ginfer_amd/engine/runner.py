@@ -20,6 +20,7 @@ import numpy as np
 import torch
 
 from ..cache import CacheManager
+from ..cache.manager import caches_of
 from ..config import config_from_folder
 from ..kernels import autotune, build
 from ..kernels.tuning import TUNING
@@ -109,44 +110,60 @@ class ModelRunner:
 
     def _plan_pool(self, specs, utilization):
         """Page counts per cache group from the device's memory, in the reference's order (ginfer/model/model.cc:48-120
-        makes the scratch memory first, ginfer/engine/model_runner.cc:52-70 then sizes the pool from what is free):
-        the largest step runs once over a small pool of its own, which tells what activations, logits and the library's
-        workspace take at their peak; the pool is free memory x utilization, and a utilization that leaves less than
-        that peak beside the pool is refused.  Groups with a window get what they can ever hold, the groups that keep
-        all keys share the rest (`CacheManager.plan_pages`)."""
+        makes the scratch memory first, ginfer/engine/model_runner.cc:52-70 then sizes the pool from what is free).
+        The largest step runs once over a small pool of its own: a prompt portion beside a single token of every other
+        request, every request sampled, which tells what activations, logits and the library's workspace take at
+        their peak.  From the memory that is free with the weights loaded, the per-request state (fixed: a slot for
+        every request and one more) is taken first; the pool is what is left x utilization; beside the pool there has
+        to be room for that peak (and for the tuner's buffers, with autotune), else the utilization is refused; what
+        is left beyond that, up to a bound, is what recorded steps may hold (`_record` never takes from the step's
+        own room).  Groups with a window get what they can ever hold, the groups that keep all keys share the rest
+        (`CacheManager.plan_pages`)."""
         if not 0.0 < utilization <= 1.0:
             raise ValueError("gpu_memory_utilization must lie in (0, 1], got %r" % (utilization,))
         esize = torch.empty(0, dtype=self.dtype).element_size()
         if not CacheManager.group_specs(specs):
             return 0
         T, R, ps = self.max_step_tokens, self.max_requests, self.page_size
-        # the largest step over a pool that just holds it: one portion of T tokens, then one token of R requests
-        probe_pages = -(-T // ps) + R + 1
+        # the largest step over a pool that just holds it: a portion beside one token of each of the other requests
+        singles = max(0, min(R - 1, T - 1))
+        portion = T - singles
+        probe_pages = -(-portion // ps) + singles + 1
         self._install_cache(specs, probe_pages, False)
         torch.cuda.synchronize(self.device)
         resident = torch.cuda.memory_allocated(self.device)
         torch.cuda.reset_peak_memory_stats(self.device)
         try:
-            self.step([StepEntry(("probe", 0), [0] * T, [T - 1])])
-            self.release(("probe", 0))
-            self.step([StepEntry(("probe", r), [0], [0]) for r in range(R)])
-            for r in range(R):
-                self.release(("probe", r))
+            entries = [StepEntry(("probe", 0), [0] * portion, [portion - 1])]
+            entries += [StepEntry(("probe", r), [0], [0]) for r in range(1, singles + 1)]
+            self.step(entries)
+            for e in entries:
+                self.release(e.request_id)
             torch.cuda.synchronize(self.device)
         finally:
             peak = torch.cuda.max_memory_allocated(self.device) - resident
             del self.cache, self._buffers
             torch.cuda.empty_cache()
         free, total = torch.cuda.mem_get_info(self.device)
-        pool = int(free * utilization)
+        state = CacheManager.state_bytes(specs, R)
         need = int(peak * 1.1) + (64 << 20)          # the step's own peak, a tenth more, and the allocator's rounding
-        if free - pool < need:
+        if self.autotune:
+            # the tuner's buffer that is overwritten between timings, and the outputs of the candidates it runs (a step's
+            # own peak bounds them)
+            need += autotune.FLUSH_BYTES + int(peak)
+        avail = free - state
+        pool = int(avail * utilization) if avail > 0 else 0
+        if avail - pool < need or pool <= 0:
             raise ValueError("gpu_memory_utilization %.3f leaves %d MB beside the cache, but a step of %d tokens and %d "
-                             "requests takes up to %d MB: at most %.3f fits (%d MB are free with the weights loaded)"
-                             % (utilization, (free - pool) >> 20, T, R, need >> 20, max(0.0, (free - need) / free),
-                                free >> 20))
+                             "requests takes up to %d MB: at most %.3f fits (%d MB are free with the weights loaded, "
+                             "%d MB of them go to the per-request state)"
+                             % (utilization, max(avail - pool, 0) >> 20, T, R, need >> 20,
+                                max(0.0, (avail - need) / avail) if avail > 0 else 0.0, free >> 20, state >> 20))
         counts = CacheManager.plan_pages(specs, ps, esize, pool, R, T, self.max_model_len)
-        self.memory_plan = dict(free_bytes=int(free), pool_bytes=pool, step_peak_bytes=int(peak), pages=list(counts))
+        # what recorded steps may hold: what is left beside pool, state and the step's own room, at most an eighth of the card
+        self._graph_budget = max(0, min(avail - pool - need, total // 8))
+        self.memory_plan = dict(free_bytes=int(free), state_bytes=int(state), pool_bytes=pool, step_peak_bytes=int(peak),
+                                step_room_bytes=int(need), graph_budget_bytes=int(self._graph_budget), pages=list(counts))
         return counts
 
     @property
@@ -260,18 +277,22 @@ class ModelRunner:
         """Uploads the host arrays through one packed buffer and wraps the device views."""
         buf.fill(host)
         cache, ps = self.cache, self.page_size
+        def view(owner, place, spec, owns):
+            if isinstance(spec, StateSpec):
+                return StateView(cache.state_tensors[(owner, place)], buf.dev["state_slots"], owns)
+            gi, _ = cache.group_of[(owner, place)]
+            if isinstance(spec, KVCacheSpec):
+                kp, vp = cache.kv_views(owner, place)
+                return KVView(kp, vp, buf.dev["table%d" % gi], buf.dev["slots%d" % gi], ps, owns)
+            return KVView(None, None, buf.dev["table%d" % gi], buf.dev["slots%d" % gi], ps, owns,
+                          pages=cache.page_views(owner, place))
         caches = []
         for i, sched in enumerate(self.model.schedule):
             owner = self._owner_of[i]
             spec = cache.cache_specs[owner]
-            if isinstance(spec, KVCacheSpec):
-                gi, _ = cache.group_of[owner]
-                kp, vp = cache.kv_views(owner)
-                caches.append(KVView(kp, vp, buf.dev["table%d" % gi], buf.dev["slots%d" % gi], ps, owner == i))
-            elif isinstance(spec, StateSpec):
-                caches.append(StateView(cache.state_tensors[owner], buf.dev["state_slots"], owner == i))
-            else:
-                caches.append(None)
+            views = [view(owner, k, c, owner == i) for k, c in enumerate(caches_of(spec))]
+            # a block that names a list of caches gets a list of views, any other its one view (or None)
+            caches.append(views if isinstance(spec, (list, tuple)) else (views[0] if views else None))
         # decode rows come first in cu order only when every entry is a single token; the list is general
         return StepContext(
             token_ids=buf.dev["ids"], positions=buf.dev["pos"], token_entry=buf.dev["ent"], cu_tokens=buf.dev["cu"],
@@ -316,7 +337,7 @@ class ModelRunner:
         its activations): the least recently used ones are forgotten first, by count and by bytes.  None: not
         recorded, the step runs launch by launch."""
         if self._graph_budget is None:
-            # half of what the cache pool left free, at most 1/8 of the card
+            # the pool was given, not planned: half of what is free now, at most 1/8 of the card
             free, total = torch.cuda.mem_get_info(self.device)
             self._graph_budget = min((free + torch.cuda.memory_reserved(self.device)
                                       - torch.cuda.memory_allocated(self.device)) // 2, total // 8)
@@ -332,6 +353,12 @@ class ModelRunner:
         t0 = time.perf_counter()
         try:
             g = capture(key, host)
+        except torch.cuda.OutOfMemoryError as e:
+            # the plan left recorded steps a budget that the device does not have: better said than run on slowly
+            self._graphs.pop(key, None)
+            raise RuntimeError("the device ran out of memory while a step of %s was being recorded (%d MB held by "
+                               "recorded steps, budget %d MB): lower gpu_memory_utilization or max_num_seqs, or run "
+                               "without recorded steps" % (key, self._graph_bytes >> 20, self._graph_budget >> 20)) from e
         except Exception as e:           # recording is a matter of speed only: the steps go on launch by launch
             import sys
             sys.stderr.write("[ginfer_amd] recording a step failed (%s: %s); steps are launched kernel by kernel from "

@@ -59,8 +59,8 @@ class Scheduler:
         grown = min(total, self.max_model_len)
         for gi, g in enumerate(self.cache.groups):
             need = -(-grown // ps)
-            if g.window is not None:         # token by token a window holds the pages of `window` positions, one more at most
-                need = min(need, -(-g.window // ps) + 1)
+            if g.window is not None:         # token by token a window holds the pages that `window` positions can touch
+                need = min(need, self.cache.window_span_pages(g.window, ps))
             if need > g.pool.num_pages:
                 raise ValueError("request %r can grow to %d tokens (%d pages%s) but cache group %d has %d pages; "
                                  "it could never finish" % (seq.request_id, grown, need,

@@ -16,9 +16,10 @@ Every part
 
 Mixer         forward(x [T, H], step, cache) -> [T, H], or float32 [parts, T, H]: partial sums that the
               norm which follows adds up in order (what a K-split matrix product leaves)
-              cache_spec() -> KVCacheSpec | StateSpec | None: what one run of this mixer keeps per
-              request; `cache` in forward is the matching view (`KVView`, `StateView` or None) of the
-              schedule entry that is running.  `step` is the `StepContext` of the batch.
+              cache_spec() -> KVCacheSpec | PagedSpec | StateSpec | None, or a list of them: what one run of
+              this mixer keeps per request (pages and, or, a state slot); `cache` in forward is the matching
+              view (`KVView`, `StateView` or None; a list of views for a list of specs) of the schedule entry
+              that is running.  `step` is the `StepContext` of the batch.
 FeedForward   forward(x [T, H]) -> [T, H] (or partial sums, as a mixer)
 Norm          forward(residual float32 [T, H], delta [T, H] | None, rows=None) -> [R or T, H]; a norm that
               sets `accepts_partial_sums` also takes delta as float32 [parts, T, H] (else the block adds
@@ -38,12 +39,34 @@ import torch
 
 
 @dataclass(frozen=True)
+class PagedSpec:
+    """Anything kept per token, in pages: `tensors` lists (name, elements per token) of every tensor a page holds; a
+    page of the group's pool is, for each of them, page_size * elements in a row, which the mixer views as it likes.
+    window: None keeps every token; an integer w keeps only what a token at position p can still see (positions > p - w).
+    Mixers with the same spec share a pool and a block table."""
+    tensors: Tuple[Tuple[str, int], ...]
+    window: Optional[int] = None
+
+    def page_tensors(self):
+        return tuple((str(n), int(w)) for n, w in self.tensors)
+
+
+@dataclass(frozen=True)
 class KVCacheSpec:
-    """Keys and values in pages: per token, num_kv_heads * head_dim of each.  window: None keeps all
-    keys; an integer w keeps only what queries can still see (positions > p - w)."""
+    """Keys and values in pages: per token and kv head a key of head_dim and a value of value_dim elements (the keys'
+    width unless given).  window: None keeps all keys; an integer w keeps only what queries can still see
+    (positions > p - w)."""
     num_kv_heads: int
     head_dim: int
     window: Optional[int] = None
+    value_dim: Optional[int] = None
+
+    @property
+    def v_dim(self):
+        return self.head_dim if self.value_dim is None else self.value_dim
+
+    def page_tensors(self):
+        return (("k", self.num_kv_heads * self.head_dim), ("v", self.num_kv_heads * self.v_dim))
 
 
 @dataclass(frozen=True)

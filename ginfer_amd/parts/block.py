@@ -9,7 +9,8 @@ class Arrangement:
     for exactly these roles and hands them over as a dictionary.  Every part becomes an attribute under its role's
     name.  forward(residual float32 [T, H], delta, step, cache) takes the output of the block before as a pending
     `delta` (it is added to the residual by the first norm that runs) and returns its own last output as the next one.
-    cache_spec(): what one run of the block keeps per request; the mixer's, unless the kind says otherwise."""
+    cache_spec(): what one run of the block keeps per request; the mixer's, unless the kind says otherwise (a block with
+    several parts that keep something returns the list of their specs and gets the list of views as `cache`)."""
 
     roles = {}
 

@@ -11,13 +11,16 @@ from .block import whole
 
 @dataclass
 class KVView:
-    """What an attention-like mixer sees of the cache for the schedule entry that is running."""
-    k_pages: torch.Tensor          # [pages, nkv, page_size, hd]
-    v_pages: torch.Tensor          # [pages, nkv, hd, page_size]: values are kept transposed
+    """What a mixer sees of one paged cache of the schedule entry that is running.  A cache of keys and values
+    (`KVCacheSpec`) comes as k_pages and v_pages; any other paged cache (`PagedSpec`) as `pages`, its tensors by name,
+    each [pages, page_size * elements per token], for the mixer to view as it likes."""
+    k_pages: Optional[torch.Tensor]    # [pages, nkv, page_size, hd]
+    v_pages: Optional[torch.Tensor]    # [pages, nkv, value_dim, page_size]: values are kept transposed
     block_table: torch.Tensor      # int32 [entries, width]; -1 where a page was given back
     slot_mapping: torch.Tensor     # int64 [T]: page * page_size + offset for every token of the step
     page_size: int
     owner: bool                    # False when this run reads another entry's cache and must not write
+    pages: Optional[dict] = None
 
 
 @dataclass
@@ -43,7 +46,7 @@ class StepContext:
     num_entries: int
     host_q_start: List[int]
     host_q_len: List[int]
-    caches: List[object]           # per schedule entry: KVView | StateView | None
+    caches: List[object]           # per schedule entry: KVView | StateView | None, or a list of views
     extra: Optional[dict] = None   # whatever a kernel dispatcher wants to remember within the step
 
     @property
@@ -98,9 +101,9 @@ class DecoderModel:
 
     # ---- weights
     def _named_parts(self):
-        names = self.spec.names
-        out = [(names["embedding"], self.embedding), (names["final_norm"], self.final_norm),
-               (names["head"], self.head)]
+        name_of = self.spec.name_of
+        out = [(name_of("embedding"), self.embedding), (name_of("final_norm"), self.final_norm),
+               (name_of("head"), self.head)]
         for ls, block in zip(self.spec.layers, self.blocks):
             for role, part in block.parts():
                 out.append((ls.prefix + "." + ls.name_of(role), part))
@@ -142,8 +145,8 @@ class DecoderModel:
 
     # ---- cache
     def cache_specs(self):
-        """Per schedule entry: what its run keeps per request, or None when it keeps nothing or reads
-        another entry's cache."""
+        """Per schedule entry: what its run keeps per request (a spec or a list of specs), or None when it keeps nothing
+        or reads another entry's cache."""
         out = []
         for e in self.schedule:
             out.append(None if e.cache_of is not None else self.blocks[e.layer].cache_spec())

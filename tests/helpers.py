@@ -28,6 +28,11 @@ TINY_C = dict(  # explicit head_dim 48 with nh*hd != hidden, widths no power of 
     num_attention_heads=6, num_key_value_heads=3, head_dim=48, intermediate_size=136, vocab_size=777,
     rope_theta=5e5, rms_norm_eps=3e-6, tie_word_embeddings=False, max_position_embeddings=384,
     use_sliding_window=True, sliding_window=40, max_window_layers=1, eos_token_id=5)
+# how the checkpoints of this family of models spell the parts' tensor prefixes (the plain implementation reads these names;
+# the toy architectures of the tests spell theirs alike)
+LAYER_NAMES = dict(mixer="self_attn", feed_forward="mlp", mixer_norm="input_layernorm",
+                   feed_forward_norm="post_attention_layernorm")
+MODEL_NAMES = dict(embedding="model.embed_tokens", final_norm="model.norm", head="lm_head")
 TINY = {"A": (TINY_A, 0, 16), "B": (TINY_B, 1, 8), "C": (TINY_C, 2, 16)}   # config, seed, page size
 
 

@@ -6,7 +6,7 @@ import pytest
 import torch
 
 from ginfer_amd.cache import CacheManager, PagePool, SlotPool, OutOfPages
-from ginfer_amd.parts import KVCacheSpec, StateSpec
+from ginfer_amd.parts import KVCacheSpec, PagedSpec, StateSpec
 
 FULL = KVCacheSpec(2, 16, None)
 WIN = KVCacheSpec(2, 16, 20)
@@ -57,8 +57,37 @@ def test_slot_pool():
 def test_groups_by_need():
     m = CacheManager([FULL, WIN, None, FULL, StateSpec((8,), torch.float32), WIN], page_size=8, num_pages=10, max_requests=3)
     assert [(g.spec, g.entries) for g in m.groups] == [(FULL, [0, 3]), (WIN, [1, 5])]
-    assert m.group_of == {0: (0, 0), 3: (0, 1), 1: (1, 0), 5: (1, 1)} and m.state_entries == [4]
+    assert m.group_of == {(0, 0): (0, 0), (3, 0): (0, 1), (1, 0): (1, 0), (5, 0): (1, 1)} and m.state_units == [(4, 0)]
     assert m.pool_bytes(2) == 10 * 4 * 2 * 2 * 8 * 16 * 2
+
+
+def test_an_entry_may_keep_several_caches_and_pages_of_any_width():
+    """A schedule entry's cache may be a list (pages and a state slot side by side); values may be narrower than keys;
+    a paged cache may hold any named per-token tensors.  Each distinct paged spec is a group with a pool of its own."""
+    narrow = KVCacheSpec(2, 16, None, value_dim=8)
+    latent = PagedSpec((("c", 24), ("r", 4)), window=16)
+    state = StateSpec((5,), torch.float32)
+    m = CacheManager([[narrow, state], FULL, None, [latent, narrow], state], page_size=8, num_pages=[6, 7, 5], max_requests=2)
+    assert [(g.spec, g.units) for g in m.groups] == [(narrow, [(0, 0), (3, 1)]), (FULL, [(1, 0)]), (latent, [(3, 0)])]
+    assert m.state_units == [(0, 1), (4, 0)]
+    # bytes: narrow 2 caches x (2*16 + 2*8) a token, full 1 x 2*2*16, latent 1 x 28; pages of 8 tokens, 2-byte elements
+    assert m.pool_bytes(2) == (6 * 2 * 48 + 7 * 64 + 5 * 28) * 8 * 2
+    assert CacheManager.state_bytes(m.cache_specs, 2) == 2 * 3 * 5 * 4
+    assert not CacheManager.supports_prefix_caching(m.cache_specs)
+    counts = CacheManager.plan_pages(m.cache_specs, 8, 2, 10 ** 6, 2, 32, 64)
+    assert counts[2] == CacheManager.window_pages(16, 8, 2, 32, 64) and counts[0] == counts[1] > 0
+    # a request takes pages in every group alike and gives them all back
+    m.admit("a")
+    m.append("a", 20)
+    m.commit("a")
+    assert [len([p for p in m.table("a", gi) if p >= 0]) for gi in range(3)] == [3, 3, 3]
+    m.append("a", 20)
+    m.commit("a")
+    assert [len([p for p in m.table("a", gi) if p >= 0]) for gi in range(3)] == [5, 5, 2]     # the window keeps positions 25 to 39
+    m.check()
+    m.release("a")
+    m.check()
+    assert all(g.pool.num_free == g.pool.num_pages for g in m.groups)
 
 
 def test_append_commit_release_and_reuse():

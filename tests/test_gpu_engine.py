@@ -989,7 +989,8 @@ def test_the_pool_is_planned_from_free_memory_after_the_largest_step(folders, mo
     all_keys = [g for g in groups if g.window is None]
     windowed = [g for g in groups if g.window is not None]
     assert len(all_keys) == 1 and len(windowed) == 1           # layer 0 keeps all keys, layers 1 to 3 a window of 40
-    assert windowed[0].pool.num_pages == CacheManager.window_pages(40, 16, 4, 128, 384) == 4 * (39 // 16 + 3) + 8
+    assert windowed[0].pool.num_pages == CacheManager.window_pages(40, 16, 4, 128, 384) \
+        == 4 * (CacheManager.window_span_pages(40, 16) + 1) + 128 // 16
     per_page = lambda g: len(g.entries) * 2 * g.spec.num_kv_heads * 16 * g.spec.head_dim * 2
     assert all_keys[0].pool.num_pages * per_page(all_keys[0]) > 0.9 * plan["pool_bytes"]
     assert r.cache.pool_bytes(2) <= plan["pool_bytes"]

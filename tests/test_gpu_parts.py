@@ -205,11 +205,11 @@ def _register_toy():
     class RunningMean(Part):
         """out[t] = W . mean(x[0..t]) of the request; the state is (sum, count)."""
 
-        def __init__(self, hidden_size, dtype, device):
-            self.H, self.dtype, self.device = hidden_size, dtype, device
+        def __init__(self, hidden_size, dtype, device, state_pad=0):
+            self.H, self.dtype, self.device, self.pad = hidden_size, dtype, device, int(state_pad)
 
         def cache_spec(self):
-            return StateSpec((self.H + 1,), torch.float32)
+            return StateSpec((self.H + 1 + self.pad,), torch.float32)        # the padding only makes the slot large
 
         def weight_specs(self):
             return {"mix.weight": WeightSpec((self.H, self.H))}
@@ -239,14 +239,16 @@ def _register_toy():
     class ToyConfig:
         hidden_size: int = 48
         vocab_size: int = 211
+        state_pad: int = 0
         architecture = "ToyStateLM"
 
         @classmethod
         def from_dict(cls, d):
-            return cls(d["hidden_size"], d["vocab_size"])
+            return cls(d["hidden_size"], d["vocab_size"], d.get("state_pad", 0))
 
         def to_dict(self):
-            return dict(architectures=["ToyStateLM"], hidden_size=self.hidden_size, vocab_size=self.vocab_size)
+            return dict(architectures=["ToyStateLM"], hidden_size=self.hidden_size, vocab_size=self.vocab_size,
+                        state_pad=self.state_pad)
 
         def model_spec(self):
             Hd = self.hidden_size
@@ -254,16 +256,16 @@ def _register_toy():
             pos = PartSpec("rope_neox", dict(theta=1e4, rotary_dim=16, max_positions=256))
             attn = PartSpec("attention", dict(hidden_size=Hd, num_heads=3, num_kv_heads=1, head_dim=16, qkv_bias=True,
                                               out_bias=False, window=None, position=pos, scale=None))
-            toy = PartSpec("toy_running_mean", dict(hidden_size=Hd))
+            toy = PartSpec("toy_running_mean", dict(hidden_size=Hd, state_pad=self.state_pad))
             ffn = PartSpec("swiglu", dict(hidden_size=Hd, intermediate_size=80))
-            layers = [prenorm_layer("model.layers.%d" % i, m, ffn, norm, norm) for i, m in enumerate([attn, toy, attn])]
+            layers = [prenorm_layer("model.layers.%d" % i, m, ffn, norm, norm, names=H.LAYER_NAMES) for i, m in enumerate([attn, toy, attn])]
             # layer 0, the toy layer, layer 2 reading run 0's cache, the toy layer again (a second state)
             schedule = [ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(2, cache_of=0), ScheduleEntry(1)]
             return ModelSpec(hidden_size=Hd, vocab_size=self.vocab_size, layers=layers, schedule=schedule,
                              embedding=PartSpec("embedding", dict(vocab_size=self.vocab_size, hidden_size=Hd)),
                              final_norm=norm, head=PartSpec("lm_head", dict(vocab_size=self.vocab_size, hidden_size=Hd,
                                                                             tied=True)),
-                             max_positions=256, eos_token_ids=[0])
+                             max_positions=256, eos_token_ids=[0], names=H.MODEL_NAMES)
     return ToyConfig
 
 
@@ -372,13 +374,13 @@ def _register_recordable_toy():
                                               out_bias=False, window=None, position=pos, scale=None))
             toy = PartSpec("toy_running_mean_recordable", dict(hidden_size=Hd))
             ffn = PartSpec("swiglu", dict(hidden_size=Hd, intermediate_size=80))
-            layers = [prenorm_layer("model.layers.%d" % i, m, ffn, norm, norm) for i, m in enumerate([attn, toy, attn])]
+            layers = [prenorm_layer("model.layers.%d" % i, m, ffn, norm, norm, names=H.LAYER_NAMES) for i, m in enumerate([attn, toy, attn])]
             schedule = [ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(2, cache_of=0), ScheduleEntry(1)]
             return ModelSpec(hidden_size=Hd, vocab_size=self.vocab_size, layers=layers, schedule=schedule,
                              embedding=PartSpec("embedding", dict(vocab_size=self.vocab_size, hidden_size=Hd)),
                              final_norm=norm, head=PartSpec("lm_head", dict(vocab_size=self.vocab_size, hidden_size=Hd,
                                                                             tied=True)),
-                             max_positions=256, eos_token_ids=[0])
+                             max_positions=256, eos_token_ids=[0], names=H.MODEL_NAMES)
     return ToyRecordableConfig
 
 
@@ -478,7 +480,7 @@ def _register_toy_arrangements():
                 LayerSpec("model.layers.0", dict(mixer=attn, feed_forward=ffn, mixer_norm=norm, post_mixer_norm=norm,
                                                  feed_forward_norm=norm, post_feed_forward_norm=norm),
                           arrangement="toy_sandwich", names=dict(mixer="self_attn", feed_forward="mlp")),
-                prenorm_layer("model.layers.1", attn, ffn, norm, norm),
+                prenorm_layer("model.layers.1", attn, ffn, norm, norm, names=H.LAYER_NAMES),
                 LayerSpec("model.layers.2", dict(mixer=attn, feed_forward=ffn, norm=norm), arrangement="toy_parallel",
                           names=dict(mixer="self_attn", feed_forward="mlp", norm="shared_layernorm")),
             ]
@@ -487,7 +489,7 @@ def _register_toy_arrangements():
                              embedding=PartSpec("embedding", dict(vocab_size=self.vocab_size, hidden_size=Hd)),
                              final_norm=norm, head=PartSpec("lm_head", dict(vocab_size=self.vocab_size, hidden_size=Hd,
                                                                             tied=False)),
-                             max_positions=128, eos_token_ids=[0])
+                             max_positions=128, eos_token_ids=[0], names=H.MODEL_NAMES)
     return ToyArrangedConfig
 
 
@@ -629,14 +631,14 @@ def _register_routed_toy():
                                                   out_bias=False, window=None, position=pos, scale=None))
             dense = PartSpec("swiglu", dict(hidden_size=Hd, intermediate_size=56))
             routed = PartSpec("toy_one_of_n", dict(hidden_size=Hd, intermediate_size=24, num_experts=3))
-            layers = [prenorm_layer("model.layers.0", attn(slow), routed, norm, norm),
-                      prenorm_layer("model.layers.1", attn(rope), dense, norm, norm)]
+            layers = [prenorm_layer("model.layers.0", attn(slow), routed, norm, norm, names=H.LAYER_NAMES),
+                      prenorm_layer("model.layers.1", attn(rope), dense, norm, norm, names=H.LAYER_NAMES)]
             return ModelSpec(hidden_size=Hd, vocab_size=self.vocab_size, layers=layers,
                              schedule=[ScheduleEntry(0), ScheduleEntry(1)],
                              embedding=PartSpec("embedding", dict(vocab_size=self.vocab_size, hidden_size=Hd)),
                              final_norm=norm, head=PartSpec("lm_head", dict(vocab_size=self.vocab_size, hidden_size=Hd,
                                                                             tied=False)),
-                             max_positions=128, eos_token_ids=[0])
+                             max_positions=128, eos_token_ids=[0], names=H.MODEL_NAMES)
     return ToyRoutedConfig
 
 
@@ -805,14 +807,14 @@ def _register_toy_ends():
             attn = PartSpec("attention", dict(hidden_size=Hd, num_heads=3, num_kv_heads=1, head_dim=16, qkv_bias=True,
                                               out_bias=False, window=None, position=rope, scale=None))
             dense = PartSpec("swiglu", dict(hidden_size=Hd, intermediate_size=72))
-            layers = [prenorm_layer("model.layers.%d" % i, attn, dense, norm, norm) for i in range(2)]
+            layers = [prenorm_layer("model.layers.%d" % i, attn, dense, norm, norm, names=H.LAYER_NAMES) for i in range(2)]
             return ModelSpec(hidden_size=Hd, vocab_size=self.vocab_size, layers=layers,
                              schedule=[ScheduleEntry(0), ScheduleEntry(1)],
                              embedding=PartSpec("toy_scaled_with_positions",
                                                 dict(vocab_size=self.vocab_size, hidden_size=Hd, max_positions=96)),
                              final_norm=norm,
                              head=PartSpec("toy_capped_head", dict(vocab_size=self.vocab_size, hidden_size=Hd, cap=3.0)),
-                             max_positions=96, eos_token_ids=[0])
+                             max_positions=96, eos_token_ids=[0], names=H.MODEL_NAMES)
     return ToyEndsConfig
 
 
@@ -854,3 +856,208 @@ def test_toy_norm_embedding_and_head(tmp_path):
         for (rid, p), row in got.items():
             err = np.abs(row - refs[rid][p]).max() / np.abs(refs[rid]).max()
             assert err < 1e-4, "request %s position %d: %.3g" % (rid, p, err)
+
+
+# ----------------------------------------------------------------------------- caches of other shapes
+
+def _register_toy_caches():
+    """Two toys whose caches are not the usual pair of equally wide keys and values under one mixer: attention whose
+    values are half as wide as its keys (written in plain torch over the pages it is handed), and a block that has this
+    attention and a running mean side by side, pages and a state slot for one run of one layer."""
+    from ginfer_amd.config import register_architecture, PartSpec, LayerSpec, prenorm_layer, ScheduleEntry, ModelSpec
+    from ginfer_amd.parts import register_mixer, register_arrangement, Part, KVCacheSpec, StateSpec
+    from ginfer_amd.parts.block import Arrangement, whole
+    from ginfer_amd.weights import WeightSpec
+
+    @register_mixer("toy_narrow_value_attention")
+    class NarrowValueAttention(Part):
+        """Causal attention without positions: keys of `key_dim`, values of `value_dim` per head, one kv head per head."""
+
+        def __init__(self, hidden_size, num_heads, key_dim, value_dim, dtype, device):
+            self.H, self.nh, self.kd, self.vd, self.dtype, self.device = hidden_size, num_heads, key_dim, value_dim, dtype, device
+
+        def cache_spec(self):
+            return KVCacheSpec(self.nh, self.kd, None, value_dim=self.vd)
+
+        def weight_specs(self):
+            return {"q.weight": WeightSpec((self.nh * self.kd, self.H)), "k.weight": WeightSpec((self.nh * self.kd, self.H)),
+                    "v.weight": WeightSpec((self.nh * self.vd, self.H)), "o.weight": WeightSpec((self.H, self.nh * self.vd))}
+
+        def bind_weights(self, t):
+            self.w = {n.split(".")[0]: v for n, v in t.items()}
+
+        def forward(self, x, step, cache):
+            nh, kd, vd, ps = self.nh, self.kd, self.vd, cache.page_size
+            assert tuple(cache.k_pages.shape[1:]) == (nh, ps, kd) and tuple(cache.v_pages.shape[1:]) == (nh, vd, ps)
+            xf = x.float()
+            q = (xf @ self.w["q"].float().t()).view(-1, nh, kd)
+            k = (xf @ self.w["k"].float().t()).view(-1, nh, kd)
+            v = (xf @ self.w["v"].float().t()).view(-1, nh, vd)
+            page, off = cache.slot_mapping // ps, cache.slot_mapping % ps
+            cache.k_pages[page, :, off, :] = k.to(cache.k_pages.dtype)
+            cache.v_pages[page, :, :, off] = v.to(cache.v_pages.dtype)
+            out = torch.empty((x.shape[0], nh * vd), dtype=torch.float32, device=x.device)
+            o = 0
+            for e in range(step.num_entries):
+                n, start = step.host_q_len[e], step.host_q_start[e]
+                total = start + n
+                pages = cache.block_table[e, :-(-total // ps)].long()
+                keys = cache.k_pages[pages].float().permute(1, 0, 2, 3).reshape(nh, -1, kd)[:, :total]          # [nh, total, kd]
+                vals = cache.v_pages[pages].float().permute(1, 0, 3, 2).reshape(nh, -1, vd)[:, :total]          # [nh, total, vd]
+                s = torch.einsum("thd,hkd->htk", q[o:o + n], keys) / kd ** 0.5
+                seen = torch.arange(total, device=x.device)[None, :] <= (start + torch.arange(n, device=x.device))[:, None]
+                p = torch.softmax(s.masked_fill(~seen[None], float("-inf")), dim=-1)
+                out[o:o + n] = torch.einsum("htk,hkd->thd", p, vals).reshape(n, nh * vd)
+                o += n
+            return (out @ self.w["o"].float().t()).to(self.dtype)
+
+    @register_arrangement("toy_attention_beside_a_mean")
+    class AttentionBesideMean(Arrangement):
+        """h = x + attention(norm(x)) + running_mean(norm(x)); x' = h + feed_forward(norm2(h)).  One run keeps pages for
+        the attention and a state slot for the mean: the list of both is its cache."""
+        roles = {"mixer": "mixer", "mean": "mixer", "feed_forward": "feed_forward", "norm": "norm", "feed_forward_norm": "norm"}
+
+        def cache_spec(self):
+            return [self.mixer.cache_spec(), self.mean.cache_spec()]
+
+        def forward(self, residual, delta, step, cache):
+            pages, slot = cache
+            n = self.norm.forward(residual, whole(delta, self.norm))
+            a = self.mixer.forward(n, step, pages) + self.mean.forward(n, step, slot)
+            return self.feed_forward.forward(self.feed_forward_norm.forward(residual, a))
+
+    @register_architecture("ToyCachesLM")
+    @dataclass
+    class ToyCachesConfig:
+        hidden_size: int = 40
+        vocab_size: int = 173
+        architecture = "ToyCachesLM"
+
+        @classmethod
+        def from_dict(cls, d):
+            return cls(d["hidden_size"], d["vocab_size"])
+
+        def to_dict(self):
+            return dict(architectures=["ToyCachesLM"], hidden_size=self.hidden_size, vocab_size=self.vocab_size)
+
+        def model_spec(self):
+            Hd = self.hidden_size
+            norm = PartSpec("rmsnorm", dict(size=Hd, eps=1e-5))
+            narrow = PartSpec("toy_narrow_value_attention", dict(hidden_size=Hd, num_heads=2, key_dim=16, value_dim=8))
+            mean = PartSpec("toy_running_mean", dict(hidden_size=Hd))
+            ffn = PartSpec("swiglu", dict(hidden_size=Hd, intermediate_size=56))
+            layers = [
+                prenorm_layer("model.layers.0", narrow, ffn, norm, norm, names=H.LAYER_NAMES),
+                LayerSpec("model.layers.1", dict(mixer=narrow, mean=mean, feed_forward=ffn, norm=norm, feed_forward_norm=norm),
+                          arrangement="toy_attention_beside_a_mean",
+                          names=dict(mixer="self_attn", mean="mean", feed_forward="mlp", norm="input_layernorm",
+                                     feed_forward_norm="post_attention_layernorm")),
+            ]
+            return ModelSpec(hidden_size=Hd, vocab_size=self.vocab_size, layers=layers,
+                             schedule=[ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(0)],
+                             embedding=PartSpec("embedding", dict(vocab_size=self.vocab_size, hidden_size=Hd)),
+                             final_norm=norm, head=PartSpec("lm_head", dict(vocab_size=self.vocab_size, hidden_size=Hd,
+                                                                            tied=False)),
+                             max_positions=160, eos_token_ids=[0], names=H.MODEL_NAMES)
+    return ToyCachesConfig
+
+
+def _toy_caches_plain(folder, ids):
+    """The model of `_register_toy_caches` on a whole sequence, written out plainly in 64-bit."""
+    w = pm.read_weights(folder)
+    T = len(ids)
+    x = pm.embedding(w["model.embed_tokens.weight"], ids)
+
+    def narrow_attention(n, p):
+        q = pm.linear(n, w[p + ".q.weight"]).view(T, 2, 16)
+        k = pm.linear(n, w[p + ".k.weight"]).view(T, 2, 16)
+        v = pm.linear(n, w[p + ".v.weight"]).view(T, 2, 8)
+        s = torch.einsum("thd,khd->htk", q, k) / 4.0
+        s = s.masked_fill(torch.triu(torch.ones(T, T, dtype=torch.bool), diagonal=1)[None], float("-inf"))
+        return pm.linear(torch.einsum("htk,khd->thd", torch.softmax(s, dim=-1), v).reshape(T, 16), w[p + ".o.weight"])
+
+    for layer in (0, 1, 0):
+        p = "model.layers.%d" % layer
+        n = pm.rms_norm(x, w[p + ".input_layernorm.weight"], 1e-5)
+        a = narrow_attention(n, p + ".self_attn")
+        if layer == 1:
+            mean = torch.cumsum(n, dim=0) / torch.arange(1, T + 1, dtype=n.dtype)[:, None]
+            a = a + mean @ w[p + ".mean.mix.weight"].t()
+        h = x + a
+        x = h + pm.feed_forward(pm.rms_norm(h, w[p + ".post_attention_layernorm.weight"], 1e-5), w, p + ".mlp")
+    return pm.linear(pm.rms_norm(x, w["model.norm.weight"], 1e-5), w["lm_head.weight"]).float().numpy()
+
+
+def test_toy_caches_of_other_shapes_are_built_and_stepped(tmp_path):
+    """Values half as wide as keys, and a block that keeps pages and a state slot side by side: registered here, built
+    and stepped whole, in portions and mixed, against their plain statement.  Layer 0 runs twice (two caches of its
+    own); the runs of the narrow attention share one group of pages, whose pages hold 2 x 16 + 2 x 8 elements a token."""
+    from ginfer_amd import ModelRunner, write_random_model
+    _register_toy()                       # the running mean
+    Toy = _register_toy_caches()
+    folder = write_random_model(str(tmp_path / "toy"), Toy(), seed=9, dtype="float32")
+    reqs = {"a": H.random_tokens(45, 173, 1), "b": H.random_tokens(19, 173, 2), "c": H.random_tokens(33, 173, 3),
+            "d": H.random_tokens(27, 173, 4)}
+    runner = ModelRunner(folder, dtype="float32", page_size=8, num_pages=14, max_requests=3)
+    cache = runner.cache
+    assert [type(s).__name__ if not isinstance(s, list) else [type(c).__name__ for c in s] for s in cache.cache_specs] \
+        == ["KVCacheSpec", ["KVCacheSpec", "StateSpec"], "KVCacheSpec"]
+    assert len(cache.groups) == 1 and cache.groups[0].units == [(0, 0), (1, 0), (2, 0)] and cache.state_units == [(1, 1)]
+    assert cache.groups[0].tensors["k"].shape == (3, 14, 8 * 32) and cache.groups[0].tensors["v"].shape == (3, 14, 8 * 16)
+    assert cache.pool_bytes(4) == 14 * 3 * 48 * 8 * 4
+    assert not runner.use_graphs          # the toys say nothing of recording
+    refs = {rid: _toy_caches_plain(folder, ids) for rid, ids in reqs.items()}
+    for steps in (H.steps_whole(reqs), H.steps_portions(reqs, sizes=(5, 2, 11, 3)), H.steps_mixed(reqs, max_live=3, seed=2)):
+        got = H.run_steps(runner, steps)
+        cache.check()
+        assert got
+        for (rid, p), row in got.items():
+            err = np.abs(row - refs[rid][p]).max() / np.abs(refs[rid]).max()
+            assert err < 1e-4, "request %s position %d: %.3g" % (rid, p, err)
+
+
+def test_the_pool_is_planned_around_the_state_of_a_stateful_model(tmp_path, monkeypatch):
+    """Per-request state enters the memory plan before the pool of pages is sized: a toy whose state slots are large
+    (a quarter of a gigabyte each, two runs of the layer, a slot per request and one more) is planned as if 3 GB were
+    free, and generates to the end through the engine."""
+    from ginfer_amd import ModelRunner, Engine, EngineConfig, SamplingParams, write_random_model
+    from ginfer_amd.cache import CacheManager
+    Toy = _register_toy()
+    pad = (1 << 26) - 49
+    folder = write_random_model(str(tmp_path / "toy"), Toy(state_pad=pad), seed=4, dtype="float32")
+    real = torch.cuda.mem_get_info
+    torch.cuda.empty_cache()
+    if real()[0] < (6 << 30):
+        pytest.skip("needs 6 GB of free device memory")
+    monkeypatch.setattr(torch.cuda, "mem_get_info", lambda *a, **k: (3 << 30, real(*a, **k)[1]))     # as if 3 GB were free
+    r = ModelRunner(folder, dtype="float32", page_size=8, max_requests=3, max_num_batched_tokens=32, gpu_memory_utilization=0.5)
+    plan = r.memory_plan
+    state = 2 * 4 * (1 << 26) * 4                            # two runs, four slots, 2^26 floats
+    assert plan["state_bytes"] == state == CacheManager.state_bytes(r.cache.cache_specs, 3)
+    assert plan["pool_bytes"] == ((3 << 30) - state) // 2    # half of what the state leaves, not of all that is free
+    assert r.cache.pool_bytes(4) <= plan["pool_bytes"]
+    assert plan["step_room_bytes"] >= plan["step_peak_bytes"] > 0
+    assert 0 <= plan["graph_budget_bytes"] <= (3 << 30) - state - plan["pool_bytes"] - plan["step_room_bytes"]
+    assert sum(t.numel() * t.element_size() for t in r.cache.state_tensors.values()) == state
+    del r
+    torch.cuda.empty_cache()
+    # a utilisation that would have fitted without the state is refused, and the message names the state
+    with pytest.raises(ValueError, match="per-request state"):
+        monkeypatch.setattr(torch.cuda, "mem_get_info", lambda *a, **k: (state + (32 << 20), real(*a, **k)[1]))
+        ModelRunner(folder, dtype="float32", page_size=8, max_requests=3, max_num_batched_tokens=32, gpu_memory_utilization=0.5)
+    torch.cuda.empty_cache()
+    monkeypatch.setattr(torch.cuda, "mem_get_info", lambda *a, **k: (3 << 30, real(*a, **k)[1]))
+    eng = Engine(EngineConfig(model_path=folder, dtype="float32", max_num_batched_tokens=32, max_num_seqs=3, max_seq_len=120,
+                              kvcache_block_size=8, gpu_memory_utilization=0.5))
+    prompts = [H.random_tokens(n, 211, 60 + n) for n in (40, 7, 61, 23)]
+    outs = eng.generate(prompts, SamplingParams(max_tokens=10, ignore_eos=True))
+    eng.runner.cache.check()
+    assert all(g.pool.num_free == g.pool.num_pages for g in eng.runner.cache.groups)
+    for p, o in zip(prompts, outs):
+        assert len(o.token_ids) == 10
+        ids = p + o.token_ids
+        logits = _toy_plain(folder, ids[:-1])
+        for k, tok in enumerate(o.token_ids):
+            row = logits[len(p) - 1 + k]
+            best = int(np.argmax(row))
+            assert tok == best or float(row[best] - row[tok]) <= 1e-4 * float(np.abs(row).max()), (len(p), k, tok, best)
