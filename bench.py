@@ -4,6 +4,11 @@ on one MI355X, with the achieved fraction of the HBM and matrix-core rooflines.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B] [--context C]
 
+Beside the headline (batch 8, context 4,096) `points` holds decode at batch 1 and 64 and, in the default run, two
+further sizes, each with its fraction of the HBM peak computed as `roofline` is (weights once + the live requests'
+cache, over the step's time): batch 8 at context 32,768, and batch 64 at context 4,096 of the 7B shape (a second
+engine, weights drawn on the device).
+
 A step is one decode step of the engine: `Engine.step()` on requests that the engine itself has prefilled to the
 context, every request of the batch getting one token from the paged cache, its next token coming back to the
 host; the engine launches the next step before this step's tokens have been waited for.  Prints ONE JSON line;
@@ -61,6 +66,12 @@ def main():
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--points", default="1,64", help="other decode batch sizes to report")
+    ap.add_argument("--long-context", type=int, default=None,
+                    help="context of the further decode point at the headline's batch (default: 32768 in the default run "
+                         "of the 1.5b shape, else none; 0: none)")
+    ap.add_argument("--second-shape", default=None, choices=sorted(SHAPES) + ["none"],
+                    help="shape of the further decode point at batch 64, context 4096 (default: 7b in the default run of "
+                         "the 1.5b shape, else none)")
     ap.add_argument("--model-dir", default=None, help="a model folder: reused if it holds a model, else written (implies --file-weights)")
     ap.add_argument("--shape", default="1.5b", choices=sorted(SHAPES), help="layer sizes (the headline is 1.5b)")
     ap.add_argument("--no-measured-peaks", action="store_true",
@@ -105,15 +116,19 @@ def main():
     points = sorted({int(p) for p in args.points.split(",") if p} | {args.batch})
     max_b = max(points)
     page = 16
+    default_run = args.shape == "1.5b" and args.dtype == "bfloat16" and args.layers == full_layers and args.context == 4096
+    long_context = args.long_context if args.long_context is not None else (32768 if default_run else 0)
+    second_shape = args.second_shape or ("7b" if default_run and not args.autotune else "none")
     ctx_pages = -(-(args.context + 24) // page)
-    pages = max_b * ctx_pages + -(-args.prefill_tokens // page) + 8
+    pages = max(max_b * ctx_pages, args.batch * -(-(long_context + 24) // page)) + -(-args.prefill_tokens // page) + 8
+    longest = max(args.context, args.prefill_tokens, long_context)
     # The engine itself is what is timed: requests are added, the scheduler cuts their prompts into steps and reserves
     # their pages, the runner replays recorded decode steps, the sampler picks, tokens come back to the host every step.
     engine = Engine(EngineConfig(
         model_path=folder, model_config=config_from_dict(cfg) if device_weights else None,
         random_seed=0 if device_weights else None, dtype=args.dtype,
-        max_num_batched_tokens=max(2048, args.prefill_tokens, args.context + max_b), max_num_seqs=max_b,
-        max_seq_len=max(args.context, args.prefill_tokens) + max_b + 24, kvcache_block_size=page, num_kvcache_blocks=pages,
+        max_num_batched_tokens=max(2048, longest + max_b), max_num_seqs=max_b,
+        max_seq_len=longest + max_b + 24, kvcache_block_size=page, num_kvcache_blocks=pages,
         enable_prefix_caching=False, warmup=not args.no_engine_warmup, autotune=args.autotune))
     g = torch.Generator().manual_seed(0)
     vocab = cfg["vocab_size"]
@@ -121,7 +136,9 @@ def main():
     def sync():
         torch.cuda.synchronize()
 
-    def finite():
+    first_engine = engine
+
+    def finite(engine):
         if not bool(torch.isfinite(engine.last_logits).all()):
             sys.exit("bench.py: the step that was just timed made logits that are not finite")
 
@@ -137,15 +154,17 @@ def main():
         sync()
         times.append(time.perf_counter() - t0)
         assert len(done) == 1 and len(done[0].token_ids) == 1 and not engine.has_unfinished()
-        finite()
+        finite(engine)
     prefill_s = min(times[1:])
     peak = PEAK_FLOPS["bf16" if args.dtype == "bfloat16" else "fp32"]
     prefill = {"value": round(T / prefill_s, 1), "tokens": T, "ms": round(prefill_s * 1e3, 3),
                "frac": round(prefill_flops(T) / prefill_s / peak, 4)}
 
     # ---- decode: B requests whose prompts the engine prefills, so that the timed steps end at --context
-    def decode(B, steps, warmup):
+    def decode(B, steps, warmup, context=args.context, engine=None):
+        engine = engine or first_engine
         sched = engine.scheduler
+        vocab = engine.runner.vocab_size
         # Requests are added one by one, each prompt running whole in one step beside a token for every request added
         # before it (steps are not launched ahead meanwhile, so it is exactly one step); a request added earlier gets a
         # shorter prompt by as many tokens as it decodes until the last one is in: all reach the same length.
@@ -153,7 +172,7 @@ def main():
         params = SamplingParams(max_tokens=steps + warmup + B + 16, ignore_eos=True)
         ids = []
         for i in range(B):
-            n = args.context - steps - warmup - (B - 1 - i)
+            n = context - steps - warmup - (B - 1 - i)
             ids.append(engine.add_request(torch.randint(0, vocab, (n,), generator=g).tolist(), params))
             engine.step()
         assert not sched.waiting and len(sched.running) == B and all(s.decoding and s.remaining == 1 for s in sched.running)
@@ -168,14 +187,14 @@ def main():
             engine.step()
         sync()
         dt = (time.perf_counter() - t0) / steps
-        finite()
+        finite(engine)
         log = list(engine.step_log)
         assert len(log) == steps and all(p == 0 and d == B for _, _, p, d in log), "a timed step was no decode step of %d" % B
         assert engine.stats["steps_launched_ahead"] - ahead >= steps, "the timed steps were not launched ahead"
         device_ms = 1e3 * sum(d for _, d, _, _ in log) / steps
         # tokens of a request in the cache after the last timed step (the step launched ahead of it included)
         cached = [engine.runner.cache.length(rid) for rid in ids]
-        assert max(cached) - min(cached) <= 1 and abs(max(cached) - args.context) <= 2, cached
+        assert max(cached) - min(cached) <= 1 and abs(max(cached) - context) <= 2, cached
         mean_ctx = sum(cached) / float(B) - steps / 2.0
         for rid in ids:
             engine.abort(rid)
@@ -204,12 +223,43 @@ def main():
             out[name] = round(work / ((time.perf_counter() - t0) / 10), 1)
         return out
 
+    def hbm_frac(weights, kv_token, B, mean_ctx, dt):
+        return (weights + B * mean_ctx * kv_token) / dt / HBM_PEAK
+
     results = {}
     for B in points:
         results[B] = decode(B, args.steps, args.warmup)
     dt, mean_ctx, device_ms = results[args.batch]
     step_bytes = weight_bytes + args.batch * mean_ctx * kv_per_token
     achieved = step_bytes / dt / 1e9
+    more = {}
+    for B in points:
+        if B != args.batch:
+            more["decode_b%d" % B] = round(B / results[B][0], 1)
+            more["decode_b%d_hbm_frac" % B] = round(hbm_frac(weight_bytes, kv_per_token, B, results[B][1], results[B][0]), 4)
+    few = min(args.steps, 20), min(args.warmup, 5)
+    if long_context:
+        d, ctx, _ = decode(args.batch, few[0], few[1], context=long_context)
+        more["decode_b%d_ctx%d" % (args.batch, long_context)] = round(args.batch / d, 1)
+        more["decode_b%d_ctx%d_hbm_frac" % (args.batch, long_context)] = round(
+            hbm_frac(weight_bytes, kv_per_token, args.batch, ctx, d), 4)
+    measured = None if args.no_measured_peaks else measured_peaks()
+    if second_shape != "none":
+        # a second engine at another shape of the same architecture, its weights drawn on the device
+        del engine, first_engine
+        import gc
+        gc.collect()
+        torch.cuda.empty_cache()
+        name2, shape2 = SHAPES[second_shape]
+        w2, kv2, _ = model_numbers(shape2, shape2["num_hidden_layers"])
+        B2, C2 = 64, 4096
+        engine2 = Engine(EngineConfig(
+            model_path=None, model_config=config_from_dict(shape2), random_seed=0, dtype=args.dtype,
+            max_num_batched_tokens=C2 + B2, max_num_seqs=B2, max_seq_len=C2 + B2 + 24, kvcache_block_size=page,
+            num_kvcache_blocks=B2 * -(-(C2 + 24) // page) + 8, enable_prefix_caching=False, warmup=False))
+        d, ctx, _ = decode(B2, few[0], few[1], context=C2, engine=engine2)
+        more["decode_b%d_%s" % (B2, second_shape)] = round(B2 / d, 1)
+        more["decode_b%d_%s_hbm_frac" % (B2, second_shape)] = round(hbm_frac(w2, kv2, B2, ctx, d), 4)
     out = {
         "metric": "decode tok/s at batch %d (Qwen2 %s shape, context %d)" % (args.batch, args.shape.upper(), args.context),
         "value": round(args.batch / dt, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -224,10 +274,10 @@ def main():
         "prefill": prefill,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                      "frac": round(achieved * 1e9 / HBM_PEAK, 4)},
-        "points": {"decode_b%d" % B: round(B / results[B][0], 1) for B in points if B != args.batch},
+        "points": more,
     }
-    if not args.no_measured_peaks:
-        out["measured"] = measured_peaks()
+    if measured is not None:
+        out["measured"] = measured
     print(json.dumps(out))
     if tmp is not None:
         tmp.cleanup()
