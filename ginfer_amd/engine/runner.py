@@ -22,7 +22,7 @@ import torch
 from ..cache import CacheManager
 from ..cache.manager import caches_of
 from ..config import config_from_folder
-from ..kernels import autotune, build
+from ..kernels import autotune as tuner, build
 from ..kernels.tuning import TUNING
 from ..parts.base import KVCacheSpec, StateSpec
 from ..parts.model import build_model, StepContext, KVView, StateView
@@ -56,7 +56,8 @@ class ModelRunner:
         tokens, max_requests requests) has run, times gpu_memory_utilization.  strict_weights: a tensor in the folder
         that the model does not read is an error, not a warning.  autotune: before a step of some number of rows is
         recorded, the products that can be done in several ways are timed in each and the fastest kept
-        (kernels/autotune.py); takes a second or so per number of rows, once."""
+        (kernels/autotune.py); takes a second or so per number of rows, once.  True: the runner keeps its own table of
+        plans (`plans`); a table of another runner (its `plans`) may be given instead, to share what it measured."""
         self.device = device or require_gpu()
         if dtype not in DTYPES:
             raise ValueError("dtype must be one of %s, got %r" % (sorted(DTYPES), dtype))
@@ -82,7 +83,9 @@ class ModelRunner:
         if prefix_caching is None:       # where the model allows it
             prefix_caching = CacheManager.supports_prefix_caching(specs)
         self.graph_mixed_steps = bool(graph_mixed_steps)
-        self.autotune = bool(autotune)
+        # the plans this runner's products run by: its own table, one handed over, or none (by the rules)
+        self.plans = autotune if isinstance(autotune, tuner.Table) else (tuner.Table() if autotune else None)
+        self.autotune = self.plans is not None
         self._reserved_by_tuning = 0
         self._graphs, self._graph_seen, self._padded_buffers = {}, {}, {}
         self._graph_budget, self._graph_bytes, self._graph_bytes_seen = None, 0, {}
@@ -150,7 +153,7 @@ class ModelRunner:
         if self.autotune:
             # the tuner's buffer that is overwritten between timings, and the outputs of the candidates it runs (a step's
             # own peak bounds them)
-            need += autotune.FLUSH_BYTES + int(peak)
+            need += tuner.FLUSH_BYTES + int(peak)
         avail = free - state
         pool = int(avail * utilization) if avail > 0 else 0
         if avail - pool < need or pool <= 0:
@@ -330,7 +333,12 @@ class ModelRunner:
         if device_tokens is not None:
             buf.dev["ids"].copy_(device_tokens)
         self.counts["launched"] += 1
-        return self.model.forward(ctx)
+        return self._forward(ctx)
+
+    def _forward(self, ctx):
+        """The model's forward, its products running by this runner's plans (none: by the rules)."""
+        with tuner.using(self.plans):
+            return self.model.forward(ctx)
 
     def _record(self, capture, key, host):
         """Records a step unless the device memory that recorded steps may hold is used up (each holds its buffers and
@@ -417,7 +425,7 @@ class ModelRunner:
             self._padded_buffers[key] = buf
             ctx = self._padded_context(host, buf, t_pad, e_pad, width, bucket)
             self.counts["launched"] += 1
-            return self.model.forward(ctx)[:R]
+            return self._forward(ctx)[:R]
         g["buf"].fill(self._pad(host, t_pad, e_pad, g["width"]))
         g["graph"].replay()
         self.counts["replayed_padded"] += 1
@@ -449,7 +457,7 @@ class ModelRunner:
         self._settle(ctx, dict(ctx.extra))
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
-            logits = self.model.forward(ctx)
+            logits = self._forward(ctx)
         g = dict(graph=graph, buf=buf, logits=logits, ctx=ctx, width=width)
         self._graphs[key] = g
         return g
@@ -466,7 +474,7 @@ class ModelRunner:
         self._settle(ctx, {"decode_info": buf.dev["decode_info"], "decode_span": bucket})
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
-            logits = self.model.forward(ctx)
+            logits = self._forward(ctx)
         g = dict(graph=graph, buf=_GraphBuffers(buf, width, self._widen), logits=logits, ctx=ctx)
         self._graphs[key] = g
         return g
@@ -477,12 +485,12 @@ class ModelRunner:
         same `extra` (a run leaves its plans of rows and tiles there)."""
         if self.autotune:
             ctx.extra = dict(extra)
-            with autotune.collecting() as seen:
+            with tuner.collecting() as seen:
                 self._run_once_unrecorded(ctx, count=False)
             t0 = time.perf_counter()
             reserved = torch.cuda.memory_reserved(self.device)
-            self.counts["autotuned_keys"] = self.counts.get("autotuned_keys", 0) + autotune.tune(
-                seen, self.device, verbose=bool(os.environ.get("GINFER_AMD_AUTOTUNE_VERBOSE")))
+            self.counts["autotuned_keys"] = self.counts.get("autotuned_keys", 0) + tuner.tune(
+                seen, self.device, self.plans, verbose=bool(os.environ.get("GINFER_AMD_AUTOTUNE_VERBOSE")))
             self.counts["autotune_seconds"] = round(self.counts.get("autotune_seconds", 0.0) + time.perf_counter() - t0, 3)
             # what the timing left in the allocator's hands is not the recorded step's
             self._reserved_by_tuning += max(0, torch.cuda.memory_reserved(self.device) - reserved)
@@ -499,7 +507,7 @@ class ModelRunner:
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
-            self.model.forward(ctx)
+            self._forward(ctx)
         torch.cuda.current_stream().wait_stream(side)
         for e, t in saved.items():
             self.cache.state_tensors[e].copy_(t)

@@ -11,8 +11,12 @@ or simply to be sure, the runner can measure instead, before it records a step o
   3. from then on `choose` answers with the kept plan for that key.
 
 A plan decides speed only: every candidate computes the same product with 32-bit accumulation, so results differ in
-rounding at most.  The table lives for the process; it is empty, and `choose` a dictionary miss, unless a runner was
-built with autotune=True.
+rounding at most.  The kept plans live in a `Table` that belongs to the runner that measured them (a second runner
+may be handed the same table); `choose` answers from the table that is in use (`using(table)`, which the runner puts
+around every forward), so a runner built without autotune runs by the rules whatever other runners of the process have
+measured.  A key is measured when a step with it is about to be recorded, the second time the step's sizes are seen:
+the first step of those sizes has run by the rules, so in bfloat16 a runner with autotune gives up the promise that a
+step's bits do not depend on whether its sizes have been seen before (the plans differ in rounding).
 """
 import contextlib
 import sys
@@ -20,10 +24,17 @@ import time
 
 import torch
 
-TABLE = {}            # key -> plan
-REPORT = []           # (key, chosen plan, {plan: microseconds}) of every tuned key, for the curious
+class Table(dict):
+    """key -> kept plan; `report` lists (key, chosen plan, {plan: microseconds}) of every key measured into it."""
+
+    def __init__(self):
+        super().__init__()
+        self.report = []
+
+
 KINDS = {}            # kind of product -> ProductKind
 _collected = None     # while collecting: key -> list of operand tuples
+_current = None       # the table in use (a runner's, around its forward), or None: by the rules
 MAX_ROTATION = 32     # weights that a timing graph walks through
 FLUSH_BYTES = 1 << 29 # written before every timed replay: more than the caches hold, so that every weight comes from memory
 MARGIN = 0.10         # a plan must beat the rules' plan by this fraction to replace it: the timing stands for the step only so far
@@ -53,14 +64,26 @@ def collecting():
         _collected = prev
 
 
+@contextlib.contextmanager
+def using(table):
+    """The products inside run by the plans of `table` (None: by the rules)."""
+    global _current
+    prev, _current = _current, table
+    try:
+        yield table
+    finally:
+        _current = prev
+
+
 def choose(key, operands):
-    """The kept plan for `key`, or None (run by the rules).  `operands` is remembered while collecting."""
+    """The kept plan for `key` in the table in use, or None (run by the rules).  `operands` is remembered while
+    collecting."""
     if _collected is not None:
         seen = _collected.setdefault(key, [])
         if len(seen) < 4 * MAX_ROTATION:
             seen.append(operands)
         return None
-    return TABLE.get(key)
+    return _current.get(key) if _current is not None else None
 
 
 def rows_class(rows):
@@ -71,7 +94,7 @@ def rows_class(rows):
 
 
 def active():
-    return bool(TABLE) or _collected is not None
+    return bool(_current) or _collected is not None
 
 
 def _graph_time(run, n, flush, replays=5):
@@ -104,17 +127,18 @@ def _graph_time(run, n, flush, replays=5):
     return best
 
 
-def tune(collected, device, verbose=False):
-    """Measures the candidate plans of every collected key that has none yet.  Returns the number of keys tuned."""
+def tune(collected, device, table, verbose=False):
+    """Measures the candidate plans of every collected key that `table` has no plan for yet, and keeps the fastest
+    there.  Returns the number of keys measured."""
     done = 0
     flush = None
     for key, operands_list in collected.items():
-        if key in TABLE or key[0] not in KINDS:
+        if key in table or key[0] not in KINDS:
             continue
         kind = KINDS[key[0]]
         plans = kind.candidates(key)
         if len(plans) < 2:
-            TABLE[key] = plans[0] if plans else None
+            table[key] = plans[0] if plans else None
             continue
         # the operands of different layers, one of each (by the address of the first tensor)
         unique, seen = [], set()
@@ -142,16 +166,11 @@ def tune(collected, device, verbose=False):
         best = min(times, key=times.get)
         if by_rules in times and times[best] > times[by_rules] * (1.0 - MARGIN):
             best = by_rules
-        TABLE[key] = best
-        REPORT.append((key, best, times))
+        table[key] = best
+        table.report.append((key, best, times))
         done += 1
         if verbose:
             sys.stderr.write("[ginfer_amd] autotune %s: %s %.1f us (rules: %s %.1f us; %d plans in %.2f s)\n"
                              % (key, best, times[best], by_rules, times.get(by_rules, float("nan")), len(times),
                                 time.perf_counter() - t0))
     return done
-
-
-def clear():
-    TABLE.clear()
-    del REPORT[:]

@@ -10,14 +10,6 @@ import plain_model as pm
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(autouse=True)
-def _empty_table():
-    from ginfer_amd.kernels import autotune
-    autotune.clear()
-    yield
-    autotune.clear()
-
-
 def _operands(rows, n, k, seed, bias):
     g = torch.Generator().manual_seed(seed)
     d = torch.device("cuda:0")
@@ -97,18 +89,23 @@ def test_a_runner_that_times_its_plans(tmp_path):
     got = H.run_steps(runner, steps)
     runner.cache.check()
     assert runner.counts["autotuned_keys"] >= 3 and runner.counts["replayed_decode"] >= 3, runner.counts
-    keys = [key for key, _, _ in autotune.REPORT]
+    assert isinstance(runner.plans, autotune.Table)
+    keys = [key for key, _, _ in runner.plans.report]
     assert ("linear", 48, 3584, 18944, False, False, True, True) in keys, keys
-    for key, plan, times in autotune.REPORT:
+    for key, plan, times in runner.plans.report:
         print("%s -> %s (%d plans, %.1f to %.1f us)" % (key, plan, len(times), min(times.values()), max(times.values())))
-        assert autotune.TABLE[key] == plan and plan in times
-    # a second runner in the same process finds the plans and times nothing (its first steps already run by them,
-    # where the first runner's ran by the rules: the two agree up to rounding only)
-    again = ModelRunner(folder, dtype="bfloat16", page_size=16, num_pages=2 * live, max_requests=live, autotune=True)
+        assert runner.plans[key] == plan and plan in times
+    # the plans are the runner's own: a runner built without autotune runs by the rules, whatever this one has measured
+    plain = ModelRunner(folder, dtype="bfloat16", page_size=16, num_pages=2 * live, max_requests=live)
+    assert plain.plans is None and not autotune.active()
+    del plain
+    # a second runner that is handed the first one's table finds the plans and times nothing (its first steps already run
+    # by them, where the first runner's ran by the rules: the two agree up to rounding only)
+    again = ModelRunner(folder, dtype="bfloat16", page_size=16, num_pages=2 * live, max_requests=live, autotune=runner.plans)
     got2 = H.run_steps(again, steps)
-    assert again.counts.get("autotuned_keys", 0) == 0
+    assert again.counts.get("autotuned_keys", 0) == 0 and again.plans is runner.plans
     # the kept plans in recorded steps and launched kernel by kernel: the same bits (prompts run kernel by kernel in both)
-    pair = [ModelRunner(folder, dtype="bfloat16", page_size=16, num_pages=2 * live, max_requests=live, autotune=True,
+    pair = [ModelRunner(folder, dtype="bfloat16", page_size=16, num_pages=2 * live, max_requests=live, autotune=runner.plans,
                         use_graphs=g, graph_mixed_steps=False) for g in (True, False)]
     a, b = (H.run_steps(r, steps) for r in pair)
     assert pair[0].counts["replayed_decode"] >= 3 and pair[1].counts["replayed_decode"] == 0

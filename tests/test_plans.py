@@ -82,16 +82,18 @@ def test_candidates_hold_the_rules_plan_first_and_only_plans_that_fit():
 def test_kept_plans_answer_for_their_class_of_rows():
     from ginfer_amd.kernels import autotune
     assert [autotune.rows_class(r) for r in (1, 7, 16, 17, 32, 33, 64, 65, 200)] == [1, 7, 16, 32, 32, 48, 64, 80, 208]
-    autotune.clear()
     assert not autotune.active() and autotune.choose(("linear", 32), ("w",)) is None
     with autotune.collecting() as seen:
         assert autotune.active()
         assert autotune.choose(("linear", 32), ("w0",)) is None and autotune.choose(("linear", 32), ("w1",)) is None
         assert autotune.choose(("gated", 32), ("w2",)) is None
     assert seen == {("linear", 32): [("w0",), ("w1",)], ("gated", 32): [("w2",)]} and not autotune.active()
-    autotune.TABLE[("linear", 32)] = ("library", 2)
-    try:
+    table = autotune.Table()
+    table[("linear", 32)] = ("library", 2)
+    assert not autotune.active() and autotune.choose(("linear", 32), ("w",)) is None      # no table is in use
+    with autotune.using(table):
         assert autotune.active() and autotune.choose(("linear", 32), ("w",)) == ("library", 2)
         assert autotune.choose(("linear", 48), ("w",)) is None
-    finally:
-        autotune.clear()
+        with autotune.using(None):                                                          # a runner without plans
+            assert not autotune.active() and autotune.choose(("linear", 32), ("w",)) is None
+    assert not autotune.active()

@@ -33,12 +33,15 @@ def _both(lib, logits, temperature, uniform):
     torch.cuda.synchronize()
     assert lib.ga_sample_rows(ptr(want), ptr(logits), _i64(logits.stride(0)), _i(R), _i(V), ptr(temperature), ptr(uniform),
                               ptr(scratch), _stream()) == 0
-    before = torch.cuda.memory_allocated(), torch.cuda.memory_reserved()
+    # what the driver itself has free, with the device idle on both sides of the call: torch's own counters would not see
+    # an allocation that the library made behind its back
+    torch.cuda.synchronize()
+    before = torch.cuda.mem_get_info()[0], torch.cuda.memory_allocated(), torch.cuda.memory_reserved()
     rc = lib.ga_sample_rows_static(ptr(got), ptr(logits), _i64(logits.stride(0)), _i(R), _i(V), ptr(temperature),
                                    ptr(uniform), _stream())
     assert rc == 0, lib.ga_sample_rows_static_error(_i(rc))
-    assert (torch.cuda.memory_allocated(), torch.cuda.memory_reserved()) == before
     torch.cuda.synchronize()
+    assert (torch.cuda.mem_get_info()[0], torch.cuda.memory_allocated(), torch.cuda.memory_reserved()) == before
     return want.cpu().tolist(), got.cpu().tolist()
 
 
