@@ -178,7 +178,7 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(TC* __restrict_
                                                                  const bf16_t* __restrict__ W,
                                                                  const bf16_t* __restrict__ bias, int M, int N,
                                                                  int K, int ksteps, NormIn norm_in,
-                                                                 NormOut norm_out) {
+                                                                 NormOut norm_out, int fold_cols) {
   static_assert(PACK == 1 || MB == 1, "a packed tile holds at most 8 rows of A");
   __shared__ float red[SK_WAVES][NT * 16][MB * 16 + 1];
   __shared__ float rstd[16];
@@ -188,7 +188,12 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(TC* __restrict_
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r = lane & 15, g = lane >> 4;
   const int grp = wave / KS, ks = wave % KS;
   constexpr int NCOL = GATED ? CP : NT * CP;       // output columns of a group
-  const int n0 = (blockIdx.x * GROUPS + grp) * NCOL;
+  // A product that folds the norm after it owns `fold_cols` (<= CP) columns per workgroup: as many as spread the
+  // columns over all compute units (every workgroup reads all rows of A, so fewer, larger workgroups cost more
+  // than the empty tile rows of more, smaller ones).
+  const bool fuse_out = !GATED && NT == 1 && KS == SK_WAVES && MB == 1 && norm_out.residual != nullptr;
+  const int my_cols = fuse_out ? fold_cols : NCOL;
+  const int n0 = fuse_out ? blockIdx.x * fold_cols : (blockIdx.x * GROUPS + grp) * NCOL;
   const KRange<PACK> kr((blockIdx.y * KS + ks) * PACK, P::seg(r), ksteps, gridDim.y * KS * PACK, K);
   const int shift = kr.shift;
 
@@ -197,7 +202,7 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(TC* __restrict_
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) {
     const int n = GATED ? n0 + P::col(r) : n0 + nt * CP + P::col(r);
-    wok[nt] = n < N;
+    wok[nt] = n < N && (!fuse_out || P::col(r) < my_cols);
     wp[nt] = W + ((int64_t)(wok[nt] ? n : 0) + (GATED ? (int64_t)nt * N : 0)) * K + shift;
   }
   const bf16_t* ap[MB];
@@ -217,10 +222,9 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(TC* __restrict_
   NormInLoads in_loads;
   if (MB == 1) in_loads.load(norm_in, M, wave, lane);
   float out_res = 0.f, out_gain = 0.f;       // NormOut: thread t holds row t / CP, column t % CP of the workgroup
-  const bool fuse_out = !GATED && NT == 1 && KS == SK_WAVES && MB == 1 && norm_out.residual != nullptr;
   if (fuse_out) {
-    const int m = threadIdx.x / CP, n = blockIdx.x * CP + threadIdx.x % CP;
-    if (threadIdx.x < CP * CP && m < M && n < N) {
+    const int m = threadIdx.x / CP, n = n0 + threadIdx.x % CP;
+    if (threadIdx.x < CP * CP && m < M && n < N && threadIdx.x % CP < my_cols) {
       out_res = norm_out.residual[(int64_t)m * norm_out.ldr + n];
       out_gain = norm_out.gain_f32 ? reinterpret_cast<const float*>(norm_out.gain)[n]
                                    : bf16_to_f32(reinterpret_cast<const bf16_t*>(norm_out.gain)[n]);
@@ -250,8 +254,8 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(TC* __restrict_
   if (fuse_out) {
     // CP columns of up to CP rows: the threads of a row are CP neighbouring lanes, which add up their squares
     if (threadIdx.x >= CP * CP) return;
-    const int nl = threadIdx.x % CP, m = threadIdx.x / CP, n = blockIdx.x * CP + nl;
-    const bool ok = m < M && n < N;
+    const int nl = threadIdx.x % CP, m = threadIdx.x / CP, n = n0 + nl;
+    const bool ok = m < M && n < N && nl < my_cols;
     float h = 0.f;
     if (ok) {
       float v = total(0, 0, nl, m);
@@ -298,10 +302,24 @@ static int auto_pack(int M, int workgroups_of_full_tiles) {
   return (M <= 8 && workgroups_of_full_tiles < 192) ? 2 : 1;
 }
 
+// Columns that a workgroup of a product that folds the norm after it owns: the columns of a tile (16, or 8 when
+// packed), or fewer where that spreads the product over more compute units.  Every such workgroup reads all rows of A,
+// which with a long K is as much as its weights, and a compute unit takes in some 35 GB/s of such operands whatever it
+// does with them: measured on MI355X (the 1.5B shape's down and output projections at 8 rows; 192 workgroups of 8 columns
+// against 256 of 6): a decode step of 28 layers 1.745 -> 1.724 ms.  Never more workgroups than GA_FOLD_TARGET.
+#define GA_FOLD_TARGET 256
+static int fold_cols(int M, int N) {
+  const int cp = 16 / auto_pack(M, (N + 15) / 16);
+  const int full = (N + cp - 1) / cp;
+  if (full >= GA_FOLD_TARGET) return cp;
+  int cols = (N + GA_FOLD_TARGET - 1) / GA_FOLD_TARGET;          // as few columns as make GA_FOLD_TARGET workgroups
+  return cols < 1 ? 1 : (cols > cp ? cp : cols);
+}
+
 // Partial sums a row gets from a product of M rows and N columns that feeds a norm.
 extern "C" int ga_skinny_norm_parts(int M, int N) {
-  const int cp = 16 / auto_pack(M, (N + 15) / 16);
-  return (N + cp - 1) / cp;
+  const int cols = fold_cols(M, N);
+  return (N + cols - 1) / cols;
 }
 
 // A [M, K] (row stride lda), W [N, K] contiguous, bias [N] or null.  grid_splits == 1: C [M, N] (row
@@ -343,10 +361,15 @@ extern "C" int ga_gemm_skinny(void* C, int64_t ldc, const void* A, int64_t lda, 
   const int ncol = gated ? cp : nt * cp;
   const int ksteps = (K + 63) / 64;
   dim3 grid((N + groups * ncol - 1) / (groups * ncol), grid_splits), block(SK_THREADS);
+  int fcols = 0;
+  if (norm_out.residual) {
+    fcols = fold_cols(M, N);
+    grid.x = (N + fcols - 1) / fcols;
+  }
 #define LAUNCH(NT, MB, KS, TC, G, PK)                                                                     \
   hipLaunchKernelGGL((gemm_skinny_kernel<NT, MB, KS, TC, G, PK>), grid, block, 0, stream, (TC*)C, ldc,   \
                      (const bf16_t*)A, lda, (const bf16_t*)W, (const bf16_t*)bias, M, N, K, ksteps,      \
-                     norm_in, norm_out)
+                     norm_in, norm_out, fcols)
 #define PICK_KS(NT, MB, TC, G, PK)                                                                        \
   switch (ks) {                                                                                           \
     case 1: LAUNCH(NT, MB, 1, TC, G, PK); break;                                                          \
