@@ -539,6 +539,64 @@ __global__ __launch_bounds__(64) void attn_decode_combine_kernel(
 }
 
 // ----------------------------------------------------------------------------- prefill
+// Where a tile's keys are dealt to several workgroups (a short prompt makes too few tiles to go round, and its last
+// tiles see many times the keys of its first): parts[tile] = (first key, end of keys: multiples of 32, index of the
+// tile's first row among the rows whose results come in parts, part + (number of parts << 16)).  Such a workgroup
+// leaves its rows unnormalised, with their maxima and sums, where the kernel that merges the splits of single tokens
+// finds them: part_o [rows in parts][nh][parts][HD], part_ml [..][2].
+struct KeyPart {
+  int begin, end, first_row, part, parts;
+};
+__device__ __forceinline__ KeyPart key_part(const int32_t* __restrict__ parts, int bx, int begin, int end) {
+  KeyPart kp = {begin, end, -1, 0, 1};
+  if (parts) {
+    const int32_t* p = parts + (int64_t)bx * 4;
+    const int n = __builtin_amdgcn_readfirstlane(p[3]) >> 16;
+    if (n > 1) {
+      kp.begin = __builtin_amdgcn_readfirstlane(p[0]);
+      kp.end = __builtin_amdgcn_readfirstlane(p[1]);
+      kp.first_row = __builtin_amdgcn_readfirstlane(p[2]);
+      kp.part = __builtin_amdgcn_readfirstlane(p[3]) & 0xffff;
+      kp.parts = n;
+    }
+  }
+  return kp;
+}
+
+// The rows of a prefill wavefront, merged over its workgroup's streams: normalised into `out`, or (a tile whose keys
+// are in parts) as they are, with maxima and sums, into the workspace.
+template <int NB>
+__device__ __forceinline__ void write_rows(const f32x4 (&o)[NB][DB], const float (&m)[NB], const float (&l)[NB],
+                                           bf16_t* __restrict__ out, int64_t out_stride, float* __restrict__ part_o,
+                                           float* __restrict__ part_ml, const KeyPart& kp, int row0, int rows, int head,
+                                           int nh, int c, int g) {
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) {
+    const int j = nb * 16 + c;
+    if (j >= rows) continue;
+    if (kp.first_row >= 0) {
+      const int64_t slot = ((int64_t)(kp.first_row + j) * nh + head) * kp.parts + kp.part;
+      float* op = part_o + slot * HD + g * 4;
+#pragma unroll
+      for (int db = 0; db < DB; ++db) *reinterpret_cast<f32x4*>(op + db * 16) = o[nb][db];
+      if (g == 0) {
+        part_ml[slot * 2] = m[nb];
+        part_ml[slot * 2 + 1] = l[nb];
+      }
+      continue;
+    }
+    const float inv = 1.f / l[nb];
+    bf16_t* op = out + (int64_t)(row0 + j) * out_stride + (int64_t)head * HD + g * 4;
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+      union { uint2 u; bf16_t e[4]; } pk;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) pk.e[i] = f32_to_bf16(o[nb][db][i] * inv);
+      *reinterpret_cast<uint2*>(op + db * 16) = pk.u;
+    }
+  }
+}
+
 // grid (tiles, nkv * head_blocks); a workgroup holds hpw * splits wavefronts: hpw query heads of one kv
 // head, and for each head `splits` wavefronts that take the key tiles s, s + splits, ... of the same
 // 16*NB rows, so that the longest rows of a causal prompt are not one wavefront's serial work.  The
@@ -549,20 +607,21 @@ __global__ __launch_bounds__(64 * PREFILL_WAVES) void attn_prefill_kernel(
     bf16_t* __restrict__ out, int64_t out_stride, const bf16_t* __restrict__ q, int64_t q_stride,
     const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
     const int32_t* __restrict__ block_table, int table_width, const int32_t* __restrict__ tiles, int nh,
-    int nkv, int head_blocks, int hpw, int splits, int ps_shift, int window, float scale) {
+    int nkv, int head_blocks, int hpw, int splits, int ps_shift, int window, float scale,
+    const int32_t* __restrict__ parts, float* __restrict__ part_o, float* __restrict__ part_ml) {
   extern __shared__ float lds[];          // [hpw][splits-1][NB] x { o[HD][17], m[16], l[16] }
   constexpr int STATE = HD * 17 + 32;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c = lane & 15, g = lane >> 4;
-  // Workgroups go to the 8 XCDs in turn, each with an L2 of its own.  Where the grid's y (kv head x head block)
-  // divides 8 and its x is a multiple of 8 / y, the workgroups are renumbered so that an XCD sees one y only: its
-  // L2 then holds the keys and values of one kv head instead of all of them.  The tiles of a y keep their order
-  // (heaviest first).  With linear = 8a + b the new place is (y = b / per, x = a * per + b % per): one to one
-  // exactly when x's extent is a multiple of per (else the last x would fall outside, and the grid stays as it is).
+  // Workgroups are handed out in the order of their linear number and go to the 8 XCDs in turn, each with an L2 of its
+  // own.  They are renumbered with the grid's y (kv head x head block) running fastest, linear = x * extent of y + y
+  // (one to one for any extents): the heaviest tiles of every y go out first, so that in a step of more workgroups than
+  // the chip holds the long walks do not start last; and where y's extent divides 8 an XCD sees one y only, its L2
+  // holding the keys and values of one kv head instead of all of them.
   int by = blockIdx.y, bx = blockIdx.x;
-  if (gridDim.y > 1 && 8 % gridDim.y == 0 && gridDim.x % (8 / gridDim.y) == 0) {
-    const int linear = blockIdx.x + blockIdx.y * gridDim.x, per = 8 / gridDim.y;
-    by = (linear % 8) / per;
-    bx = (linear / 8) * per + (linear % 8) % per;
+  if (gridDim.y > 1) {
+    const int linear = blockIdx.x + blockIdx.y * gridDim.x;
+    by = linear % gridDim.y;
+    bx = linear / gridDim.y;
   }
   const int kvh = by / head_blocks, hb = by % head_blocks;
   const int group = nh / nkv;
@@ -571,6 +630,8 @@ __global__ __launch_bounds__(64 * PREFILL_WAVES) void attn_prefill_kernel(
   const int head = kvh * group + hb * hpw + hl;
   const int32_t* tile = tiles + (int64_t)bx * 4;
   const int entry = tile[0], row0 = tile[1], rows = tile[2], pos0 = tile[3];
+  const int kv_min_t = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;
+  const KeyPart kp = key_part(parts, bx, (kv_min_t / 32) * 32, ((pos0 + rows - 1) / 32 + 1) * 32);
 
   f32x4 o[NB][DB];
   float m[NB], l[NB];
@@ -593,7 +654,7 @@ __global__ __launch_bounds__(64 * PREFILL_WAVES) void attn_prefill_kernel(
     attend_tiles<NB, PREFILL_DEPTH>(o, m, l, qr, cpos, clo, k_pages, v_pages,
                                     block_table + (int64_t)__builtin_amdgcn_readfirstlane(entry) * table_width,
                                     table_width, kvh, nkv, ps_shift, kv_min, kv_max, full_lo, pos0,
-                                    (kv_min / 32) * 32 + 32 * split, (kv_max / 32 + 1) * 32, 32 * splits, scale);
+                                    kp.begin + 32 * split, kp.end, 32 * splits, scale);
     finish_sums<NB>(l);
   }
   if (splits > 1) {
@@ -633,24 +694,12 @@ __global__ __launch_bounds__(64 * PREFILL_WAVES) void attn_prefill_kernel(
 #pragma unroll
           for (int i = 0; i < 4; ++i) o[nb][db][i] += sn[(db * 16 + g * 4 + i) * 17 + c] * f;
       }
+      m[nb] = mx;                              // what sums and outputs are relative to now (a tile in parts hands it on)
     }
   } else if (!head_ok) {
     return;
   }
-#pragma unroll
-  for (int nb = 0; nb < NB; ++nb) {
-    const int j = nb * 16 + c;
-    if (j >= rows) continue;
-    const float inv = 1.f / l[nb];
-    bf16_t* op = out + (int64_t)(row0 + j) * out_stride + (int64_t)head * HD + g * 4;
-#pragma unroll
-    for (int db = 0; db < DB; ++db) {
-      union { uint2 u; bf16_t e[4]; } pk;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) pk.e[i] = f32_to_bf16(o[nb][db][i] * inv);
-      *reinterpret_cast<uint2*>(op + db * 16) = pk.u;
-    }
-  }
+  write_rows<NB>(o, m, l, out, out_stride, part_o, part_ml, kp, row0, rows, head, nh, c, g);
 }
 
 // ----------------------------------------------------------------------------- prefill, operands through LDS
@@ -725,7 +774,8 @@ __global__ __launch_bounds__(64 * PREFILL_WAVES) void attn_prefill_shared_kernel
     bf16_t* __restrict__ out, int64_t out_stride, const bf16_t* __restrict__ q, int64_t q_stride,
     const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
     const int32_t* __restrict__ block_table, int table_width, const int32_t* __restrict__ tiles, int nh,
-    int nkv, int head_blocks, int hpw, int splits, int ps_shift, int window, float scale) {
+    int nkv, int head_blocks, int hpw, int splits, int ps_shift, int window, float scale,
+    const int32_t* __restrict__ parts, float* __restrict__ part_o, float* __restrict__ part_ml) {
   static_assert(STAGES == 2 || STAGES == 3, "two or three stages");
   extern __shared__ __attribute__((aligned(16))) unsigned char ring[];
   float* lds = reinterpret_cast<float*>(ring);      // after the loop: [hpw][splits-1][NB] x { o[HD][17], m[16], l[16] }
@@ -733,10 +783,10 @@ __global__ __launch_bounds__(64 * PREFILL_WAVES) void attn_prefill_shared_kernel
   const int lane = threadIdx.x & 63, c = lane & 15, g = lane >> 4;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   int by = blockIdx.y, bx = blockIdx.x;             // renumbered as in the kernel above
-  if (gridDim.y > 1 && 8 % gridDim.y == 0 && gridDim.x % (8 / gridDim.y) == 0) {
-    const int linear = blockIdx.x + blockIdx.y * gridDim.x, per = 8 / gridDim.y;
-    by = (linear % 8) / per;
-    bx = (linear / 8) * per + (linear % 8) % per;
+  if (gridDim.y > 1) {
+    const int linear = blockIdx.x + blockIdx.y * gridDim.x;
+    by = linear % gridDim.y;
+    bx = linear / gridDim.y;
   }
   const int kvh = by / head_blocks, hb = by % head_blocks;
   const int group = nh / nkv;
@@ -753,7 +803,8 @@ __global__ __launch_bounds__(64 * PREFILL_WAVES) void attn_prefill_shared_kernel
   const int kv_max = pos0 + rows - 1;
   // every row of the tile sees the keys from the last row's window start up to the first row's position
   const int full_lo = (window > 0 && kv_max - window + 1 > 0) ? kv_max - window + 1 : 0;
-  const int first = (kv_min / 32) * 32, tile_end = (kv_max / 32 + 1) * 32, stride = 32 * splits;
+  const KeyPart kp = key_part(parts, bx, (kv_min / 32) * 32, (kv_max / 32 + 1) * 32);
+  const int first = kp.begin, tile_end = kp.end, stride = 32 * splits;
   const int iterations = (tile_end - first + stride - 1) / stride;       // of stream 0, the longest
   const int begin = first + 32 * stream;
   unsigned char* my_ring = ring + (size_t)stream * STAGES * STAGE_BYTES;
@@ -873,24 +924,12 @@ __global__ __launch_bounds__(64 * PREFILL_WAVES) void attn_prefill_shared_kernel
 #pragma unroll
           for (int i = 0; i < 4; ++i) o[nb][db][i] += sn[(db * 16 + g * 4 + i) * 17 + c] * f;
       }
+      m[nb] = mx;                              // what sums and outputs are relative to now (a tile in parts hands it on)
     }
   } else if (!head_ok) {
     return;
   }
-#pragma unroll
-  for (int nb = 0; nb < NB; ++nb) {
-    const int j = nb * 16 + c;
-    if (j >= rows) continue;
-    const float inv = 1.f / l[nb];
-    bf16_t* op = out + (int64_t)(row0 + j) * out_stride + (int64_t)head * HD + g * 4;
-#pragma unroll
-    for (int db = 0; db < DB; ++db) {
-      union { uint2 u; bf16_t e[4]; } pk;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) pk.e[i] = f32_to_bf16(o[nb][db][i] * inv);
-      *reinterpret_cast<uint2*>(op + db * 16) = pk.u;
-    }
-  }
+  write_rows<NB>(o, m, l, out, out_stride, part_o, part_ml, kp, row0, rows, head, nh, c, g);
 }
 #endif
 
@@ -935,12 +974,40 @@ extern "C" int ga_attn_decode(void* out, int64_t out_stride, const void* q, int6
   return GA_CHECK_LAUNCH();
 }
 
+static int attn_prefill_tiles(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* k_pages,
+                              const void* v_pages, const void* block_table, int table_width, const void* tiles,
+                              int n_tiles, int tile_rows, int nh, int nkv, int page_size, int window, float scale,
+                              int fill_workgroups, int prefer_workgroups, const void* parts, void* part_o,
+                              void* part_ml, hipStream_t stream);
+
+// parts: null, or for every tile int32 x 4 = (first key, end of keys, index of the tile's first row among the rows that
+// come in parts, part + (number of parts << 16)); a tile whose keys are dealt to several workgroups stands in `tiles` once
+// per part.  part_rows: int32 x 4 per row that comes in parts (its row of the step first), n_part_rows of them, each in
+// num_parts parts; part_o: n_part_rows * nh * num_parts * head_dim floats, part_ml: n_part_rows * nh * num_parts * 2.
 extern "C" int ga_attn_prefill(void* out, int64_t out_stride, const void* q, int64_t q_stride,
                                const void* k_pages, const void* v_pages, const void* block_table,
                                int table_width, const void* tiles, int n_tiles, int tile_rows, int nh, int nkv,
-                               int page_size, int window, float scale, int fill_workgroups, hipStream_t stream) {
+                               int page_size, int window, float scale, int fill_workgroups, int prefer_workgroups,
+                               const void* parts, const void* part_rows, int n_part_rows, int num_parts, void* part_o,
+                               void* part_ml, hipStream_t stream) {
   if (n_tiles <= 0) return 0;
   if (nkv <= 0 || nh % nkv) return -1;
+  if (parts && (n_part_rows <= 0 || num_parts < 2 || num_parts > 8 || !part_rows || !part_o || !part_ml)) return -8;
+  if (!parts) n_part_rows = 0;
+  int rc = attn_prefill_tiles(out, out_stride, q, q_stride, k_pages, v_pages, block_table, table_width, tiles, n_tiles,
+                              tile_rows, nh, nkv, page_size, window, scale, fill_workgroups, prefer_workgroups, parts, part_o,
+                              part_ml, stream);
+  if (rc || n_part_rows == 0) return rc;
+  hipLaunchKernelGGL(attn_decode_combine_kernel<8>, dim3(n_part_rows, nh), dim3(64), 0, stream, (bf16_t*)out, out_stride,
+                     (const float*)part_o, (const float*)part_ml, (const int4*)part_rows, nh, num_parts);
+  return GA_CHECK_LAUNCH();
+}
+
+static int attn_prefill_tiles(void* out, int64_t out_stride, const void* q, int64_t q_stride,
+                              const void* k_pages, const void* v_pages, const void* block_table,
+                              int table_width, const void* tiles, int n_tiles, int tile_rows, int nh, int nkv,
+                              int page_size, int window, float scale, int fill_workgroups, int prefer_workgroups,
+                              const void* parts, void* part_o, void* part_ml, hipStream_t stream) {
   if (tile_rows != 16 && tile_rows != 16 * PREFILL_NB) return -6;
   int ps_shift = 0;
   while ((1 << ps_shift) < page_size) ++ps_shift;
@@ -952,9 +1019,17 @@ extern "C" int ga_attn_prefill(void* out, int64_t out_stride, const void* q, int
     // at least two heads of a group side by side, and tiles enough to fill the chip with such workgroups: the
     // kernel that shares the operands through LDS.  A workgroup's wavefronts: heads x streams of tiles, and a
     // producer for every stream.
+    // Among the divisors of the group that still make fill_workgroups workgroups: the largest that makes prefer_workgroups
+    // (one and a half rounds of the chip: the workgroups of the second half-round fill in behind the short walks of the
+    // first), else the smallest (the most workgroups).  Measured on MI355X, 12 heads in 2 groups of head size 128, one
+    // prompt: 2,048 tokens 3 heads side by side (256 workgroups) 40.5 us, 2 (384) 38.1; 4,096 tokens 6 heads (256) 125 us,
+    // 3 (512) 82; 8,192 tokens 6 heads (512) 261 us, 3 (1,024) 272.
     int heads = 1;
-    for (int d = 2; d < PREFILL_WAVES; ++d)
-      if (group % d == 0 && (int64_t)n_tiles * nkv * (group / d) >= fill_workgroups) heads = d;
+    for (int d = PREFILL_WAVES - 1; d >= 2; --d)
+      if (group % d == 0 && (int64_t)n_tiles * nkv * (group / d) >= fill_workgroups) {
+        heads = d;                                                         // ends at the smallest such divisor
+        if ((int64_t)n_tiles * nkv * (group / d) >= prefer_workgroups) break;
+      }
     if (heads >= 2) {
       int streams = PREFILL_WAVES / (heads + 1), stages = 3;
       const size_t room = 150 * 1024;
@@ -975,7 +1050,8 @@ extern "C" int ga_attn_prefill(void* out, int64_t out_stride, const void* q, int
     hipLaunchKernelGGL((attn_prefill_shared_kernel<NB, ST>), grid, block, lds, stream, (bf16_t*)out,           \
                        out_stride, (const bf16_t*)q, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages, \
                        (const int32_t*)block_table, table_width, (const int32_t*)tiles, nh, nkv, head_blocks,  \
-                       heads, streams, ps_shift, window, scale * LOG2E);                                       \
+                       heads, streams, ps_shift, window, scale * LOG2E, (const int32_t*)parts, (float*)part_o, \
+                       (float*)part_ml);                                                                       \
   } while (0)
       if (nb == 1) {
         if (stages == 3) LAUNCH_SHARED(1, 3); else LAUNCH_SHARED(1, 2);
@@ -1005,7 +1081,8 @@ extern "C" int ga_attn_prefill(void* out, int64_t out_stride, const void* q, int
   hipLaunchKernelGGL(attn_prefill_kernel<NB>, grid, block, lds, stream, (bf16_t*)out, out_stride,         \
                      (const bf16_t*)q, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages,           \
                      (const int32_t*)block_table, table_width, (const int32_t*)tiles, nh, nkv, head_blocks, \
-                     hpw, splits, ps_shift, window, scale * LOG2E)
+                     hpw, splits, ps_shift, window, scale * LOG2E, (const int32_t*)parts, (float*)part_o,   \
+                     (float*)part_ml)
   if (lds > 48 * 1024) {                     // more dynamic LDS than the default limit: ask for it
     const void* fn = nb == 1 ? (const void*)attn_prefill_kernel<1> : (const void*)attn_prefill_kernel<PREFILL_NB>;
     if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) return -7;

@@ -88,11 +88,16 @@ int ga_attn_decode(void* out, int64_t out_stride, const void* q, int64_t q_strid
                    const void* v_pages, const void* block_table, int table_width, const void* decode_info, int n_tokens,
                    int nh, int nkv, int page_size, int window, float scale, int split_keys, int num_splits,
                    void* workspace_o, void* workspace_ml, hipStream_t stream);
-// rows of prompt portions, in tiles of int32 x 4 = (entry, first row of the step, rows, first position)
+// rows of prompt portions, in tiles of int32 x 4 = (entry, first row of the step, rows, first position).  parts (or
+// null): per tile int32 x 4 = (first key, end of keys, index of the tile's first row among the rows that come in parts,
+// part + (number of parts << 16)): the keys of such a tile are dealt to several workgroups, whose partial results
+// (part_o: n_part_rows * nh * num_parts * head_dim floats, part_ml: ... * 2) a second kernel merges; part_rows: int32 x 4
+// per row in parts, its row of the step first
 int ga_attn_prefill(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* k_pages,
                     const void* v_pages, const void* block_table, int table_width, const void* tiles, int n_tiles,
                     int tile_rows, int nh, int nkv, int page_size, int window, float scale, int fill_workgroups,
-                    hipStream_t stream);
+                    int prefer_workgroups, const void* parts, const void* part_rows, int n_part_rows, int num_parts, void* part_o,
+                    void* part_ml, hipStream_t stream);
 
 // ---- random_fill.hip: out[i] = mean + std * normal(key, i) for n elements, float or bfloat16: the counter-based
 // generator of random_normal.h, which gives the host library (host/random_fill_host.cpp) the same bits

@@ -512,11 +512,12 @@ def plan_rows(q_len, q_start, tile_rows):
 PLAN_TILE_ROWS = 16       # rows of a prompt portion per wavefront in steps of fewer than TUNING.prefill_wide_tiles_from tokens
 
 
-def _attention_plan(step, tile_rows, device):
+def _attention_plan(step, tile_rows, device, split_for=None):
     """Which rows of the step are single new tokens and how the rows of prompt portions fall into tiles;
     made once per step and shared by all layers.  A recorded step brings its plan along (`static_plan` in the
-    step's extra: device arrays of fixed size that the runner refills, counts that include padding)."""
-    key = ("attention_plan", tile_rows)
+    step's extra: device arrays of fixed size that the runner refills, counts that include padding).  split_for:
+    (window, workgroups per tile, streams of a workgroup) where the kernel takes tiles whose keys are in parts."""
+    key = ("attention_plan", tile_rows, split_for)
     plan = step.extra.get(key)
     if plan is not None:
         return plan
@@ -526,7 +527,7 @@ def _attention_plan(step, tile_rows, device):
               static["tile_rows"], tile_rows)
         plan = dict(n_decode=static["n_decode"], decode_pos=None, n_tiles=static["n_tiles"],
                     decode_span=step.extra.get("decode_span"), decode_info=step.extra.get("decode_info"),
-                    tiles=static["tiles"])
+                    tiles=static["tiles"], parts=None, part_rows=None, n_part_rows=0, num_parts=1)
         step.extra[key] = plan
         return plan
     import numpy as np
@@ -536,12 +537,64 @@ def _attention_plan(step, tile_rows, device):
     if decode_info is None and decode_rows:
         decode_info = torch.tensor([[r, p, e, 0] for r, p, e in zip(decode_rows, decode_pos, entries)], dtype=torch.int32,
                                    device=device)
-    plan = dict(
-        n_decode=len(decode_rows), decode_pos=decode_pos, n_tiles=len(tiles), decode_span=step.extra.get("decode_span"),
-        decode_info=decode_info,
-        tiles=(torch.tensor(np.asarray(tiles, dtype=np.int32).reshape(-1, 4), device=device) if tiles else None))
+    plan = dict(n_decode=len(decode_rows), decode_pos=decode_pos, n_tiles=len(tiles), decode_span=step.extra.get("decode_span"),
+                decode_info=decode_info, tiles=None, parts=None, part_rows=None, n_part_rows=0, num_parts=1)
+    if tiles:
+        split = key_parts(tiles, tile_rows, *split_for) if split_for is not None else None
+        if split is None:
+            plan["tiles"] = torch.tensor(np.asarray(tiles, dtype=np.int32).reshape(-1, 4), device=device)
+        else:
+            # the tiles, their parts and the rows that come in parts, in one transfer
+            pieces, parts, rows, num_parts = split
+            both = np.concatenate([np.asarray(pieces, dtype=np.int32).reshape(-1), np.asarray(parts, dtype=np.int32).reshape(-1),
+                                   np.asarray(rows, dtype=np.int32).reshape(-1)])
+            dev_all = torch.tensor(both, device=device)
+            n, r = len(pieces), len(rows)
+            plan.update(n_tiles=n, tiles=dev_all[:4 * n].view(n, 4), parts=dev_all[4 * n:8 * n].view(n, 4),
+                        part_rows=dev_all[8 * n:].view(r, 4), n_part_rows=r, num_parts=num_parts)
     step.extra[key] = plan
     return plan
+
+
+def key_parts(tiles, tile_rows, window, workgroups_per_tile, streams, compute_units=256):
+    """Whether the keys of a step's heaviest tiles should be dealt to several workgroups, and how.  A short prompt alone
+    in a step makes about as many workgroups as there are compute units, one round, so the kernel lasts as long as its
+    heaviest tile's walk over the keys, twice the mean of a causal prompt's tiles.  tiles: (entry, first row, rows, first
+    position), heaviest first.  None: leave the tiles whole.  Else (tiles with one entry per part, parts as the kernel takes
+    them, the rows that come in parts as int32 x 4, number of parts): the tiles with more than the mean share of keys per
+    compute unit fall into equal parts of at most that share.  Switched off in the table of thresholds
+    (`prefill_split_imbalance` 0): measured on MI355X it does not pay (a 2,048-token prompt of 12 heads in 2 groups, head
+    size 128: 40.8 us whole, 45.6 in parts: the workgroups beyond one round of the chip pay a workgroup's fixed part, some
+    8 us, a second time, and the merge and 10 MB of partial results cost what the shorter walks save)."""
+    def key_tiles(t):
+        lo = max(0, t[3] - window + 1) if window else 0
+        return (t[3] + t[2] - 1) // 32 + 1 - lo // 32, (lo // 32) * 32
+    counts = [key_tiles(t)[0] for t in tiles]
+    heaviest = max(counts)
+    share = sum(counts) * workgroups_per_tile / float(compute_units)          # tiles of 32 keys per compute unit, on average
+    if (TUNING.prefill_split_imbalance <= 0 or len(tiles) * workgroups_per_tile > TUNING.prefill_split_max_workgroups
+            or heaviest < TUNING.prefill_split_min_key_tiles * streams or heaviest <= TUNING.prefill_split_imbalance * share):
+        return None
+    share = max(share, 1.0)
+    num_parts = min(8, -(-heaviest // int(share)))
+    if num_parts < 2:
+        return None
+    out, rows_in_parts = [], []
+    for t, k in zip(tiles, counts):
+        first = key_tiles(t)[1]
+        if k <= 1.15 * share:
+            out.append((k, t, (first, first + 32 * k, -1, 1 << 16)))
+            continue
+        at = len(rows_in_parts)
+        rows_in_parts += [(t[1] + j, 0, 0, 0) for j in range(t[2])]
+        per = -(-k // num_parts)
+        per = -(-per // streams) * streams                    # whole rounds of the workgroup's streams
+        for part in range(num_parts):
+            b, e = min(part * per, k), min((part + 1) * per, k)
+            # a part without keys still writes its rows' (empty) results, which the merge expects
+            out.append((e - b, t, (first + 32 * b, first + 32 * e, at, part | (num_parts << 16))))
+    out.sort(key=lambda x: -x[0])                             # the longest walks first
+    return [x[1] for x in out], [x[2] for x in out], rows_in_parts, num_parts
 
 
 def _decode_splits(plan, window, nkv, head_blocks):
@@ -580,7 +633,9 @@ def paged_attention_mfma(q, k_pages, v_pages, block_table, step, num_heads, num_
     # rows of a prompt portion per wavefront: 32 where the kernel has it and the step is long, else 16
     wide = T >= TUNING.prefill_wide_tiles_from
     tile_rows = lib.ga_attn_prefill_max_tile_rows() if wide else 16
-    plan = _attention_plan(step, tile_rows, q.device)
+    plan = _attention_plan(step, tile_rows, q.device,
+                           split_for=_prefill_workgroups(step, tile_rows, num_heads // num_kv_heads, num_kv_heads, head_dim,
+                                                         int(window) if window else 0))
     _need(sum(step.host_q_len) == T, "the step's entries do not add up to its tokens")
     if out is None:
         out = torch.empty((T, num_heads * head_dim), dtype=q.dtype, device=q.device)
@@ -597,11 +652,47 @@ def paged_attention_mfma(q, k_pages, v_pages, block_table, step, num_heads, num_
             _i(block_table.shape[1]), _ptr(plan["decode_info"]), _i(plan["n_decode"]), _i(num_heads), _i(num_kv_heads), _i(page_size), _i(w), _f(scale), _i(split_keys),
             _i(num_splits), _ptr(ws_o), _ptr(ws_ml), _stream()), "attn_decode")
     if plan["n_tiles"]:
+        part_o = part_ml = None
+        if plan["n_part_rows"]:
+            n = plan["n_part_rows"] * num_heads * plan["num_parts"]
+            part_o = torch.empty((n * head_dim,), dtype=torch.float32, device=q.device)
+            part_ml = torch.empty((n * 2,), dtype=torch.float32, device=q.device)
         _check(lib.ga_attn_prefill(
             _ptr(out), _i64(out.stride(0)), _ptr(q), _i64(q.stride(0)), _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
             _i(block_table.shape[1]), _ptr(plan["tiles"]), _i(plan["n_tiles"]), _i(tile_rows), _i(num_heads), _i(num_kv_heads),
-            _i(page_size), _i(w), _f(scale), _i(TUNING.prefill_fill_workgroups), _stream()), "attn_prefill")
+            _i(page_size), _i(w), _f(scale), _i(TUNING.prefill_fill_workgroups), _i(TUNING.prefill_prefer_workgroups),
+            _ptr(plan["parts"]), _ptr(plan["part_rows"]),
+            _i(plan["n_part_rows"]), _i(plan["num_parts"]), _ptr(part_o), _ptr(part_ml), _stream()), "attn_prefill")
     return out
+
+
+def _prefill_workgroups(step, tile_rows, group, nkv, head_dim, window):
+    """(window, workgroups per tile, streams of tiles in a workgroup) as the prefill launcher will choose them for this
+    step, or None where the step brings its plan along (a recorded step) or has no prompt portion: what `key_parts`
+    needs to know.  Follows ga_attn_prefill's choice of heads per workgroup (csrc/attention_mfma.hip)."""
+    if "static_plan" in (step.extra or {}):
+        return None
+    n_tiles = sum(-(-n // tile_rows) for n in step.host_q_len if n > 1)
+    if n_tiles == 0:
+        return None
+    fill, waves = TUNING.prefill_fill_workgroups, 8
+    if head_dim in (64, 128, 256):
+        heads = 1
+        for d in range(waves - 1, 1, -1):
+            if group % d == 0 and n_tiles * nkv * (group // d) >= fill:
+                heads = d
+                if n_tiles * nkv * (group // d) >= TUNING.prefill_prefer_workgroups:
+                    break
+        if heads >= 2:
+            return window, nkv * (group // heads), max(1, waves // (heads + 1))
+    hpw = 1
+    for d in range(2, waves + 1):
+        if group % d == 0 and n_tiles * nkv * (group // d) >= fill:
+            hpw = d
+    splits = waves // hpw
+    if hpw > 1 and splits > 4:
+        splits = 4
+    return window, nkv * (group // hpw), splits
 
 
 def paged_attention(q, k_pages, v_pages, block_table, step, num_heads, num_kv_heads, head_dim, scale, window=None):

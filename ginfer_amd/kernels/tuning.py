@@ -56,9 +56,22 @@ class Tuning:
     decode_target_workgroups: int = 256      # key splits are chosen so that a decode step makes about this many workgroups
     decode_min_split_keys: int = 128         # one tile of 32 keys for each wavefront of a workgroup
     decode_max_splits: int = 256
-    prefill_wide_tiles_from: int = 1024      # tokens in a step from which prompt rows go 32 to a wavefront
-    # heads of a kv group go side by side into a prefill workgroup only while the step still makes this many workgroups
+    # tokens in a step from which prompt rows go 32 to a wavefront (12 heads in 2 groups of 128, one prompt alone: 1,024
+    # tokens 20.9 us with 16 rows, 24.8 with 32; 1,536: 27.2 and 29.8; 2,048: 39.4 and 38.1; 4,096: 110 and 82)
+    prefill_wide_tiles_from: int = 2048
+    # heads of a kv group go side by side into a prefill workgroup only while the step still makes `prefill_fill_workgroups`
+    # workgroups; among the groupings that do, the one with the most heads that still makes `prefill_prefer_workgroups`
+    # (one and a half rounds of the chip), else the one with the fewest heads
     prefill_fill_workgroups: int = 256
+    prefill_prefer_workgroups: int = 384
+    # The keys of a step's heaviest prompt tiles can be dealt to several workgroups (merged by a second kernel): when the
+    # step makes at most `prefill_split_max_workgroups` workgroups, the heaviest tile's walk is at least
+    # `prefill_split_min_key_tiles` tiles of 32 keys long per stream of its workgroup, and longer than
+    # `prefill_split_imbalance` times a compute unit's mean share.  0 (the default): never.  Measured with 1.5 at one prompt
+    # alone in a step, 12 heads in 2 groups of 128: 2,048 tokens 40.8 us whole, 45.6 in parts; 7B's heads 69.4 and 70.6.
+    prefill_split_max_workgroups: int = 512
+    prefill_split_min_key_tiles: int = 12
+    prefill_split_imbalance: float = 0.0
     # ---- the general attention kernels (the 32-bit path, odd head or page sizes; csrc/attention_generic.hip).  A step that
     # makes no more workgroups of a token and a kv head than this goes whole to the kernel for single tokens (measured at
     # contexts of 512 and 4,096: 12 heads in 2 groups up to 256 tokens); the kernel for portions takes as many wavefronts

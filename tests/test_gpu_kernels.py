@@ -654,6 +654,61 @@ def test_paged_attention_mfma_heads_side_by_side_finds_one_far_key(where, wide, 
         assert (last_rows - 7.0).abs().max() < 0.1
 
 
+def _force_key_parts(monkeypatch, ops, share):
+    """Makes the dispatcher deal the keys of every tile that has more than `share` tiles of 32 keys to several workgroups,
+    whatever the step's size (the rule itself looks for a short prompt alone in a step)."""
+    real = ops.key_parts
+    monkeypatch.setattr(ops.TUNING, "prefill_split_max_workgroups", 1 << 30)
+    monkeypatch.setattr(ops.TUNING, "prefill_split_min_key_tiles", 0)
+    monkeypatch.setattr(ops.TUNING, "prefill_split_imbalance", 1e-9)
+    units = {}
+    monkeypatch.setattr(ops, "key_parts", lambda tiles, tile_rows, window, wgs, streams, compute_units=256:
+                        real(tiles, tile_rows, window, wgs, streams,
+                             compute_units=max(1, int(units.setdefault("n", sum((t[3] + t[2] - 1) // 32 + 1 for t in tiles) * wgs / share)))))
+
+
+@pytest.mark.parametrize("wide", [False, True])
+@pytest.mark.parametrize("shared", [False, True])
+@pytest.mark.parametrize("nh,nkv,hd", [(12, 2, 128), (6, 3, 64), (6, 1, 48), (4, 2, 256), (5, 1, 80)])
+@pytest.mark.parametrize("seqs,window,share", [([(300, 700)], None, 5), ([(257, 1300), (40, 40), (1, 90)], None, 9),
+                                               ([(200, 330), (64, 64)], 100, 2), ([(150, 150)], None, 1.5),
+                                               ([(96, 2100)], None, 30)])
+def test_paged_attention_mfma_keys_in_parts(nh, nkv, hd, seqs, window, share, shared, wide, monkeypatch):
+    """The keys of the heaviest prompt tiles dealt to several workgroups, merged by the kernel that merges the splits of
+    single tokens: forced here at small sizes, for the kernel that keeps its operands in registers and the one that
+    shares them through LDS, beside tiles that stay whole and single tokens; up to eight parts."""
+    from ginfer_amd.kernels import ops
+    monkeypatch.setattr(ops.TUNING, "prefill_wide_tiles_from", 0 if wide else 1 << 30)
+    monkeypatch.setattr(ops.TUNING, "prefill_fill_workgroups", 1 if shared else 1 << 30)
+    _force_key_parts(monkeypatch, ops, share)
+    a, ref, _ = _paged_case(seqs, nh, nkv, hd, 16, torch.bfloat16, seed=hd + len(seqs), window=window)
+    step = _Step(seqs, a)
+    out = ops.paged_attention_mfma(a["q"], a["k_pages"], a["v_pages"], a["block_table"], step, nh, nkv, hd,
+                                   1.0 / math.sqrt(hd), window=window)
+    plans = [v for k, v in step.extra.items() if k[0] == "attention_plan"]
+    assert plans and plans[0]["n_part_rows"] > 0 and plans[0]["num_parts"] >= 2, "the keys were not dealt out"
+    close(out, ref, 2e-2)
+
+
+@pytest.mark.parametrize("where", ["first", "part_edge", "before_part_edge", "last"])
+def test_paged_attention_mfma_keys_in_parts_finds_one_far_key(where, monkeypatch):
+    from ginfer_amd.kernels import ops
+    monkeypatch.setattr(ops.TUNING, "prefill_wide_tiles_from", 0)
+    monkeypatch.setattr(ops.TUNING, "prefill_fill_workgroups", 1)
+    _force_key_parts(monkeypatch, ops, 6)
+    nh, nkv, hd, ps, kv = 6, 2, 64, 16, 640
+    seqs = [(40, kv)]
+    # with a share of 6 tiles the 20 tiles of 32 keys fall into 4 parts of 6 (rounded to the workgroup's streams): edges at 192, 384, 576
+    place = {"first": 0, "part_edge": 384, "before_part_edge": 383, "last": kv - 1}[where]
+    a, ref, _ = _paged_case(seqs, nh, nkv, hd, ps, torch.bfloat16, seed=5, spike=lambda e, ql, n: place)
+    step = _Step(seqs, a)
+    out = ops.paged_attention_mfma(a["q"], a["k_pages"], a["v_pages"], a["block_table"], step, nh, nkv, hd, 1.0 / math.sqrt(hd))
+    plan = [v for k, v in step.extra.items() if k[0] == "attention_plan"][0]
+    assert plan["num_parts"] >= 3
+    close(out, ref, 2e-2)
+    assert (out.float().cpu()[39] - 7.0).abs().max() < 0.1
+
+
 @pytest.mark.parametrize("wide", [False, True])
 @pytest.mark.parametrize("hd", list(range(16, 257, 16)))
 def test_paged_attention_mfma_every_head_size(hd, wide, monkeypatch):
@@ -830,7 +885,7 @@ def test_gemm_skinny_folds_the_norm_after_it(M, N, K, bias, gain_dtype):
     if M > 1:
         res1 = res0[M - 1:M].clone()
         alone = ops.gemm_skinny(a[M - 1:M], w, b, into_norm=(res1, gain, eps))
-        if M <= 8 or alone.sumsq.shape[1] == rows.sumsq.shape[1]:       # the same tiling: bit for bit
+        if M <= 8:                                                       # the same tiling (packed tiles): bit for bit
             assert torch.equal(alone.scaled[0], rows.scaled[M - 1]) and torch.equal(alone.sumsq[0], rows.sumsq[M - 1])
             assert torch.equal(res1[0], res[M - 1])
         else:            # from 9 rows on the tiles are not packed: the same sums in another order

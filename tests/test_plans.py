@@ -97,3 +97,36 @@ def test_kept_plans_answer_for_their_class_of_rows():
         with autotune.using(None):                                                          # a runner without plans
             assert not autotune.active() and autotune.choose(("linear", 32), ("w",)) is None
     assert not autotune.active()
+
+
+def test_keys_of_a_short_prompt_are_dealt_out_and_those_of_other_steps_are_not(monkeypatch):
+    """The rule that deals a tile's keys to several workgroups: one prompt of 2,048 tokens alone in a step (one round of
+    workgroups, the last tile walking twice the mean) is split, every part within the mean share, the parts of a tile
+    covering its keys once; shorter and longer prompts, and steps of many requests, stay whole."""
+    from ginfer_amd.kernels import ops
+    tiles = ops.plan_rows([2048], [0], 32)[3]
+    assert ops.key_parts(tiles, 32, 0, 4, 2) is None          # switched off in the table of thresholds: it was measured slower
+    monkeypatch.setattr(ops.TUNING, "prefill_split_imbalance", 1.5)
+    pieces, parts, rows, n = ops.key_parts(tiles, 32, 0, 4, 2)
+    assert n == 2 and len(pieces) == len(parts) > len(tiles) and len(rows) % 32 == 0
+    share = sum(range(1, 65)) * 4 / 256.0
+    assert max((e - b) // 32 for b, e, _, _ in parts) <= 1.15 * share + 2
+    by_tile = {}
+    for t, (b, e, at, packed) in zip(pieces, parts):
+        by_tile.setdefault(t, []).append((b, e, at, packed & 0xffff, packed >> 16))
+    assert set(by_tile) == set(tiles)
+    for t, ps in by_tile.items():
+        ps.sort()
+        assert ps[0][0] == 0 and ps[-1][1] == ((t[3] + t[2] - 1) // 32 + 1) * 32
+        assert all(x[1] == y[0] for x, y in zip(ps, ps[1:])) and [x[3] for x in ps] == list(range(len(ps)))
+        if len(ps) > 1:
+            assert all(x[4] == n and x[2] == ps[0][2] for x in ps)
+            assert [r[0] for r in rows[ps[0][2]:ps[0][2] + t[2]]] == list(range(t[1], t[1] + t[2]))
+        else:
+            assert ps[0][2] == -1
+    assert [e - b for b, e, _, _ in parts] == sorted((e - b for b, e, _, _ in parts), reverse=True)      # longest walks first
+    assert ops.key_parts(ops.plan_rows([1024], [0], 32)[3], 32, 0, 12, 8) is None
+    assert ops.key_parts(ops.plan_rows([4096], [0], 32)[3], 32, 0, 4, 2) is None
+    assert ops.key_parts(ops.plan_rows([512] * 4, [0] * 4, 32)[3], 32, 0, 4, 2) is None
+    # a window bounds every tile's keys: nothing to deal out
+    assert ops.key_parts(tiles, 32, 256, 4, 2) is None
