@@ -13,7 +13,7 @@ is raised (`LAZY_MAX`) and the like are macros at the top of the source that use
 """
 import json
 import os
-from dataclasses import dataclass, fields
+from dataclasses import dataclass, field, fields
 
 
 @dataclass
@@ -42,9 +42,36 @@ class Tuning:
     library_split_min_rows: int = 65
     library_split_max_rows: int = 256
     library_split_max_out_features: int = 4096
+    # From more than `library_from_rows` rows on, the library's one product is slow where K is long and the rows are few (it
+    # does not split K by itself: 5,120 columns of a K of 27,648 at 64 rows 173 us, in eight pieces 75).  A long K (at
+    # least `library_long_k_from`, and twice the columns or more) with at least `library_long_k_min_out_features` columns
+    # goes to the library in `library_long_k_pieces` pieces (or one fewer where only that cuts K into whole steps of 64),
+    # also where the streaming kernel would take it (2,048 columns of a K of 11,008 at 64 rows: 39 -> 30 us); up to
+    # `library_long_k_few_rows` rows only a K of `library_long_k_few_rows_from` or more with `library_min_out_features`
+    # columns, and in two pieces (5,120 columns of a K of 27,648 at 32 rows: 163 -> 94 us; more pieces lose there).  Measured at the down projections
+    # of the 3B, 7B, 14B, 32B and 72B shapes at 32 to 256 rows: 5 to 64 % less time than the plan before, the 7B shape's
+    # 64 rows aside (59 against 60 us; its own best is below).  A product about as long as it is wide with
+    # `library_square_min_features` columns and elements of K or more takes eight pieces beyond `library_long_k_few_rows`
+    # rows while it has under `library_square_max_out_features` columns, and four pieces from 128 rows on beyond that
+    # (5,120 squared: 5 to 34 % less; 8,192 squared at 256 rows 91 -> 62 us).
+    library_long_k_from: int = 8192
+    library_long_k_min_out_features: int = 2048
+    library_long_k_pieces: int = 8
+    library_long_k_few_rows: int = 32
+    library_long_k_few_rows_from: int = 16384
+    library_square_min_features: int = 4096
+    library_square_max_out_features: int = 8192
+    library_square_many_rows: int = 128
+    # Sizes at which the library's own choice of kernel makes an exception of one plan: "class of the row count,output
+    # columns,elements of K" of a product whose consumer adds partial sums -> the plan measured fastest there, which
+    # stands before the rules (found with --autotune at the 7B shape: decode at batch 64 7.57 -> 7.20 ms a step).
+    measured_plans: dict = field(default_factory=lambda: {
+        "64,3584,18944": ("library", 2), "64,3584,3584": ("library", 2), "128,3584,3584": ("library", 2)})
     # The same for the rows of prompt portions up to this many, in four pieces (the float32 parts cost the norm that
     # adds them more to read, so the gain is smaller and ends at 4,096 rows).
     library_split_portion_max_rows: int = 2048
+    # with more output columns than `library_split_max_out_features`, a long K (as above) goes in halves up to this many rows
+    library_split_wide_max_rows: int = 1024
     # The gate-up product lies transposed (weights as the library's first operand) for row counts from this on that
     # are a multiple of it: the library's tiles then fit the rows.
     transposed_gate_up_row_multiple: int = 256
@@ -100,6 +127,8 @@ class Tuning:
         for k, v in values.items():
             if k not in known:
                 raise KeyError("no tuning value %r (known: %s)" % (k, ", ".join(sorted(known))))
+            if isinstance(getattr(self, k), dict):
+                v = {str(size): tuple(plan) for size, plan in dict(v).items()}
             setattr(self, k, type(getattr(self, k))(v))
 
 

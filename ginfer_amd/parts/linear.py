@@ -37,6 +37,13 @@ def linear_plan(rows, out_features, in_features, has_bias, float32_out, parts_ok
     package's weight-streaming kernel, ("library", pieces of K) for the BLAS library.  More than one part or piece
     means float32 partial sums [parts, M, N] for the consumer to add."""
     may_split = parts_ok and not float32_out
+    if may_split and not has_bias:
+        measured = TUNING.measured_plans.get("%d,%d,%d" % (autotune.rows_class(rows), out_features, in_features))
+        if measured is not None and (skinny_ok or measured[0] != "skinny"):
+            return tuple(measured)
+        pieces = _library_long_k_pieces(rows, out_features, in_features)
+        if pieces > 1:
+            return ("library", pieces)
     if skinny_ok and not _library_is_faster(rows, out_features):
         # tilings measured on MI355X (graph replays, weights not cache-resident): up to 16 rows one
         # 16-row tile of W per wavefront streams best; beyond, four tiles halve the re-reading of x; a
@@ -157,6 +164,40 @@ def _library_is_faster(rows, out_features):
     return rows > TUNING.library_from_rows and out_features >= TUNING.library_min_out_features
 
 
+def _library_long_k_pieces(rows, out_features, in_features):
+    """Into how many pieces of K the library's product of a few rows is cut where its one product is slow because K
+    is long, or 1 where this rule has nothing to say (measured on MI355X at the layer sizes of models from 3B to 72B;
+    the figures stand beside the thresholds in kernels/tuning.py)."""
+    T = TUNING
+    if rows <= T.library_from_rows or rows > T.library_split_max_rows:
+        return 1
+    if in_features >= T.library_long_k_from and in_features >= 2 * out_features:
+        if out_features < T.library_long_k_min_out_features:
+            return 1
+        if rows <= T.library_long_k_few_rows:                # the fewest rows: two pieces, and only where the library is taken anyway
+            halves = in_features >= T.library_long_k_few_rows_from and out_features >= T.library_min_out_features
+            return 2 if halves and in_features % 16 == 0 else 1
+        tries = (T.library_long_k_pieces, T.library_long_k_pieces - 1)
+        for pieces in tries:                                   # whole steps of 64 first
+            if pieces > 1 and in_features % (pieces * 64) == 0:
+                return pieces
+        for pieces in tries + (5, 4, 2):
+            if pieces > 1 and in_features % (pieces * 8) == 0:
+                return pieces
+        return 1
+    if min(out_features, in_features) >= T.library_square_min_features and rows > T.library_long_k_few_rows:
+        if out_features < T.library_square_max_out_features:
+            tries = (8, 4, 2)
+        elif rows >= T.library_square_many_rows:
+            tries = (4, 2)
+        else:
+            return 1
+        for pieces in tries:
+            if in_features % (pieces * 8) == 0:
+                return pieces
+    return 1
+
+
 def _library_split(rows, out_features, in_features):
     """Into how many pieces of K the library's product is cut.  Measured on MI355X: with up to 256 rows, few
     output columns and a long K (the down projection of a busy decode step) the library's single product leaves
@@ -164,6 +205,14 @@ def _library_split(rows, out_features, in_features):
     gain less, while the float32 parts cost the norm more to read: four pieces take the down projection of the 1.5B
     shape and the norm after it from 50.7 to 39.0 us at 1,024 rows and from 76.0 to 69.8 at 2,048 (the library's one
     product makes 264 tiles for 256 compute units there); at 4,096 rows nothing is gained."""
+    if in_features >= TUNING.split_k_from and out_features > TUNING.library_split_max_out_features:
+        # more columns than that: only a long K, and only the shorter portions, in halves (5,120 columns of a K of 13,824:
+        # 512 rows 127 -> 98 us, 1,024 rows 168 -> 143; 8,192 columns of a K of 29,568: 347 -> 256 and 381 -> 378;
+        # at 2,048 rows one product is the fastest of all)
+        long_k = in_features >= TUNING.library_long_k_from and in_features >= 2 * out_features
+        if long_k and TUNING.library_split_max_rows < rows <= TUNING.library_split_wide_max_rows and in_features % 16 == 0:
+            return 2
+        return 1
     if not (in_features >= TUNING.split_k_from and out_features <= TUNING.library_split_max_out_features):
         return 1
     if TUNING.library_split_min_rows <= rows <= TUNING.library_split_max_rows:

@@ -27,6 +27,50 @@ def test_measured_shapes_keep_their_plans():
     assert L._library_split(4096, 1536, 8960) == 1 and L._library_split(2048, 1536, 1536) == 1
 
 
+def test_a_long_k_of_few_rows_goes_to_the_library_in_pieces():
+    """The down projections of larger models at 17 to 256 rows: the library with K in eight pieces (seven where only
+    that cuts K into whole steps of 64), also where the streaming kernel could take the rows; the sizes that were
+    measured as exceptions keep their own plan; small models are left as they were."""
+    plan = lambda rows, n, k: L.linear_plan(rows, n, k, False, False, True, rows <= 64)
+    assert plan(64, 2048, 11008) == ("library", 8) and plan(256, 2048, 11008) == ("library", 8)
+    assert plan(48, 3584, 18944) == ("library", 8) and plan(256, 3584, 18944) == ("library", 8)
+    assert plan(64, 5120, 27648) == ("library", 8) and plan(128, 5120, 13824) == ("library", 8)
+    assert plan(64, 8192, 29568) == ("library", 7) and plan(256, 8192, 29568) == ("library", 7)
+    # the fewest rows: two pieces where the library is taken anyway and K is very long, else as before
+    assert plan(32, 5120, 27648) == ("library", 2) and plan(24, 8192, 29568) == ("library", 2)
+    assert plan(32, 5120, 13824) == ("library", 1) and plan(32, 3584, 18944) == ("skinny", 4, 4)
+    assert plan(32, 2048, 11008) == ("skinny", 4, 4)
+    # about as long as wide
+    assert plan(64, 5120, 5120) == ("library", 8) and plan(256, 5120, 5120) == ("library", 8)
+    assert plan(64, 8192, 8192) == ("library", 1) and plan(128, 8192, 8192) == ("library", 4)
+    assert plan(32, 5120, 5120) == ("library", 1)
+    # measured exceptions (the library's own choice of kernel at these very sizes)
+    assert plan(64, 3584, 18944) == ("library", 2) and plan(64, 3584, 3584) == ("library", 2)
+    assert plan(50, 3584, 18944) == ("library", 2)                  # rows share a plan in classes of 16
+    assert L.linear_plan(64, 3584, 18944, False, False, False, True)[0] == "skinny"     # nobody to add parts: no pieces
+    assert L.linear_plan(64, 3584, 18944, True, False, True, True)[0] == "skinny"       # a bias: one product
+    # the 0.5B and 1.5B shapes: as measured there
+    assert plan(64, 1536, 8960) == ("skinny", 4, 10) and plan(256, 1536, 8960) == ("library", 5)
+    assert plan(64, 896, 4864) == ("skinny", 1, 4) and plan(64, 1536, 1536) == ("skinny", 1, 2)
+    # prompt portions of many columns: a long K in halves up to 1,024 rows
+    assert plan(512, 5120, 13824) == ("library", 2) and plan(1024, 8192, 29568) == ("library", 2)
+    assert plan(2048, 5120, 13824) == ("library", 1) and plan(512, 8192, 8192) == ("library", 1)
+    assert plan(512, 3584, 18944) == ("library", 4) and plan(2048, 2048, 11008) == ("library", 4)
+    # decode rows up to 16 fold their norms and never come here in pieces
+    assert plan(16, 5120, 27648)[0] == "skinny"
+    # every such plan is one the tuner would also try
+    for rows, n, k in ((64, 2048, 11008), (64, 8192, 29568), (32, 5120, 27648), (128, 8192, 8192), (64, 3584, 18944)):
+        key = ("linear", rows, n, k, False, False, True, rows <= 64)
+        assert L.linear_candidates(key)[0] == plan(rows, n, k)
+
+
+def test_measured_plans_can_be_set_from_json():
+    from ginfer_amd.kernels.tuning import Tuning
+    t = Tuning()
+    t.update({"measured_plans": {"64,1024,8192": ["library", 4]}})
+    assert t.measured_plans == {"64,1024,8192": ("library", 4)}
+
+
 def test_nearest_divisor():
     assert L._nearest_divisor(140, 10.7, 16) == 10
     assert L._nearest_divisor(140, 5.3, 16) == 5
