@@ -115,11 +115,10 @@ struct SkinnyTrip {
   }
 };
 
-template <int NT, int MB>
+template <int NT, int MB, int UNROLL = ((NT * MB <= 4) ? 4 : 2)>
 __device__ __forceinline__ void skinny_accumulate(f32x4 (&acc)[NT][MB], const bf16_t* const (&wp)[NT],
                                                   const bool (&wok)[NT], const bf16_t* const (&ap)[MB],
                                                   const bool (&aok)[MB], int kb, int kend, int ke, int g) {
-  constexpr int UNROLL = (NT * MB <= 4) ? 4 : 2;
   for (int k = kb; k < kend; k += 64 * UNROLL) {
     SkinnyTrip<NT, MB, UNROLL> trip;
     trip.load(wp, wok, ap, aok, k, ke, g);
@@ -292,6 +291,67 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(TC* __restrict_
   }
 }
 
+// The gated product of up to 16 rows, dealt EVENLY to the compute units.  A workgroup of the kernel above owns 16
+// columns, whatever their number: the 8,960 columns of a 1.5B model make 560 workgroups for 256 compute units, and a
+// unit that gets three of them streams half as much again as one that gets two.  Here the grid is a multiple of the
+// number of compute units and workgroup b owns the columns [b N / G, (b + 1) N / G), up to NT tiles of 16 of the gate
+// and as many of the up matrix: every unit streams the same bytes.  K is dealt to the 8 wavefronts and their parts are
+// added exactly as above, so the results are the same bits.  How many columns a workgroup should own is a trade: every
+// workgroup reads all rows of A (as much as M / 2 of its columns' weights), while more, smaller workgroups keep more
+// loads on their way; the launcher's rule states what was measured.
+template <int NT, typename TC>
+__global__ __launch_bounds__(SK_THREADS) void gemm_gated_even_kernel(TC* __restrict__ C, int64_t ldc,
+                                                                     const bf16_t* __restrict__ A, int64_t lda,
+                                                                     const bf16_t* __restrict__ W, int M, int N, int K,
+                                                                     int ksteps, NormIn norm_in) {
+  __shared__ float red[SK_WAVES][2 * NT * 16][16 + 1];
+  __shared__ float rstd[16];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r = lane & 15, g = lane >> 4;
+  const int c0 = (int)(((int64_t)blockIdx.x * N) / gridDim.x), c1 = (int)(((int64_t)(blockIdx.x + 1) * N) / gridDim.x);
+  const int cols = c1 - c0;                                  // <= NT * 16 by the launcher's choice of the grid
+  const KRange<1> kr(wave, 0, ksteps, SK_WAVES, K);
+  const bf16_t* wp[2 * NT];
+  bool wok[2 * NT];
+#pragma unroll
+  for (int t = 0; t < 2 * NT; ++t) {
+    const int cl = (t % NT) * 16 + r;                        // the lane's column within the workgroup's range
+    wok[t] = cl < cols;
+    wp[t] = W + ((int64_t)(wok[t] ? c0 + cl : 0) + (t >= NT ? (int64_t)N : 0)) * K + kr.shift;
+  }
+  const bf16_t* ap[1];
+  bool aok[1];
+  aok[0] = r < M;
+  ap[0] = A + (int64_t)(aok[0] ? r : 0) * lda + kr.shift;
+  f32x4 acc[2 * NT][1];
+#pragma unroll
+  for (int t = 0; t < 2 * NT; ++t) acc[t][0] = f32x4{0.f, 0.f, 0.f, 0.f};
+  NormInLoads in_loads;
+  in_loads.load(norm_in, M, wave, lane);
+  // steps of K asked for at once: fewer with more tiles, whose loads fill the registers
+  skinny_accumulate<2 * NT, 1, (NT == 1 ? 4 : NT == 2 ? 2 : 1)>(acc, wp, wok, ap, aok, 0, kr.kend, kr.ke, g);
+  in_loads.finish(norm_in, rstd, M, wave, lane);
+#pragma unroll
+  for (int t = 0; t < 2 * NT; ++t)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) red[wave][t * 16 + g * 4 + i][r] = acc[t][0][i];
+  __syncthreads();
+  const bool scale_rows = norm_in.sumsq != nullptr;
+  for (int idx = threadIdx.x; idx < cols * M; idx += SK_THREADS) {
+    const int cl = idx % cols, m = idx / cols;
+    float v = 0.f, u = 0.f;
+#pragma unroll
+    for (int w = 0; w < SK_WAVES; ++w) v += red[w][cl][m];            // in wavefront order, as in the kernel above
+#pragma unroll
+    for (int w = 0; w < SK_WAVES; ++w) u += red[w][NT * 16 + cl][m];
+    if (scale_rows) {
+      v *= rstd[m];
+      u *= rstd[m];
+    }
+    v = (v * (1.0f / (1.0f + expf(-v)))) * u;
+    Num<TC>::st(C + (int64_t)m * ldc + c0 + cl, v);
+  }
+}
+
 // GaSkinnyNorm, what ga_gemm_skinny takes beside the product itself, is declared in ginfer_amd.h.
 
 // Tiles of a product of M rows when the caller leaves the choice to the library: packed where they can be and
@@ -308,6 +368,23 @@ static int auto_pack(int M, int workgroups_of_full_tiles) {
 // does with them: measured on MI355X (the 1.5B shape's down and output projections at 8 rows; 192 workgroups of 8 columns
 // against 256 of 6): a decode step of 28 layers 1.745 -> 1.724 ms.  Never more workgroups than GA_FOLD_TARGET.
 #define GA_FOLD_TARGET 256
+// The gated product of up to 16 rows goes to the kernel that deals its columns evenly from this many (activation)
+// columns on: a workgroup then has at least 8 of them.
+#define GA_GATED_EVEN_MIN_COLUMNS 2048
+// Its workgroups: the multiple of GA_FOLD_TARGET that comes nearest to 12 columns a workgroup with up to 4 rows (and up
+// to 8 rows of a K of up to 2,048), 28 with up to 8 rows, 32 beyond, and never more than 48 (three tiles).  Measured on
+// MI355X as replays of a graph that walks 28 layers' weights, in us, before -> after (columns a workgroup), at 1, 8 and
+// 16 rows: 8,960 x 1,536: 16.7 -> 13.2 (12), 18.2 -> 15.7 (12), 20.5 -> 17.1 (35); 4,864 x 896: 8.5 -> 6.5 (10),
+// 9.2 -> 7.2 (10), 10.0 -> 8.0 (19); 11,008 x 2,048: 22.7 -> 18.9 (11), 24.8 -> 23.3 (11), 27.2 -> 26.7 (43);
+// 18,944 x 3,584: 57.4 -> 51.0 (13), 63.1 -> 60.3 (25), 71.7 -> 63.5 (37); 13,824 x 5,120: 63.9 -> 54.8 (11),
+// 71.6 -> 63.6 (27), 82.3 -> 68.7 (27); 29,568 x 8,192: 183 -> 169 (12), 200 -> 191 (29), 234 -> 206 (29).
+static int gated_even_workgroups(int M, int N, int K) {
+  const int target = M <= 4 ? 12 : M <= 8 ? (K <= 2048 ? 12 : 28) : 32;
+  int rounds = (N + GA_FOLD_TARGET * target / 2) / (GA_FOLD_TARGET * target);
+  if (rounds < 1) rounds = 1;
+  while ((N + GA_FOLD_TARGET * rounds - 1) / (GA_FOLD_TARGET * rounds) > 48) ++rounds;
+  return GA_FOLD_TARGET * rounds;
+}
 static int fold_cols(int M, int N) {
   const int cp = 16 / auto_pack(M, (N + 15) / 16);
   const int full = (N + cp - 1) / cp;
@@ -357,6 +434,22 @@ extern "C" int ga_gemm_skinny(void* C, int64_t ldc, const void* A, int64_t lda, 
   const int groups = SK_WAVES / ks;
   if (pack == 0) pack = (grid_splits == 1 && !gated) ? auto_pack(M, (N + groups * nt * 16 - 1) / (groups * nt * 16)) : 1;
   if (pack != 1 && (pack != 2 || M > 8)) return -2;
+  if (gated && mb == 1 && pack == 1 && N >= GA_GATED_EVEN_MIN_COLUMNS) {
+    const int workgroups = gated_even_workgroups(M, N, K);
+    const int most = (N + workgroups - 1) / workgroups, tiles = (most + 15) / 16;
+    const int ksteps = (K + 63) / 64;
+    dim3 grid(workgroups), block(SK_THREADS);
+#define LAUNCH_EVEN(NT, TC)                                                                                  \
+  hipLaunchKernelGGL((gemm_gated_even_kernel<NT, TC>), grid, block, 0, stream, (TC*)C, ldc, (const bf16_t*)A, \
+                     lda, (const bf16_t*)W, M, N, K, ksteps, norm_in)
+    if (out_f32) {
+      if (tiles == 1) LAUNCH_EVEN(1, float); else if (tiles == 2) LAUNCH_EVEN(2, float); else LAUNCH_EVEN(3, float);
+    } else {
+      if (tiles == 1) LAUNCH_EVEN(1, bf16_t); else if (tiles == 2) LAUNCH_EVEN(2, bf16_t); else LAUNCH_EVEN(3, bf16_t);
+    }
+#undef LAUNCH_EVEN
+    return GA_CHECK_LAUNCH();
+  }
   const int cp = 16 / pack;
   const int ncol = gated ? cp : nt * cp;
   const int ksteps = (K + 63) / 64;

@@ -821,8 +821,11 @@ def test_gemm_skinny_tilings_and_split_parts(M, N, K, nt, ks, gs, pack):
     close(out, ref, 1e-5)
 
 
-@pytest.mark.parametrize("M", [1, 8, 17, 64])
-@pytest.mark.parametrize("I,K", [(8960, 1536), (160, 64), (136, 88), (448, 192)])
+@pytest.mark.parametrize("M", [1, 5, 8, 16, 17, 64])
+@pytest.mark.parametrize("I,K", [(8960, 1536), (160, 64), (136, 88), (448, 192),
+                                 # from 2,048 columns on, up to 16 rows: the kernel that deals the columns evenly to a
+                                 # multiple of 256 workgroups (one, two and three tiles a workgroup, uneven shares)
+                                 (2056, 64), (6200, 40), (9000, 200), (12400, 24)])
 def test_gemm_skinny_gated(M, I, K):
     from ginfer_amd.kernels import ops
     a, w = rnd((M, K), torch.bfloat16, 50), rnd((2 * I, K), torch.bfloat16, 51, scale=0.3)
