@@ -514,7 +514,7 @@ __global__ __launch_bounds__(SK_THREADS) void qkv_rope_skinny_kernel(
     const bf16_t* __restrict__ bias, const int32_t* __restrict__ positions, const float* __restrict__ cos_t,
     const float* __restrict__ sin_t, const int64_t* __restrict__ slot_mapping, bf16_t* __restrict__ k_pages,
     bf16_t* __restrict__ v_pages, int M, int K, int nh, int nkv, int hd, int page_size, int write_kv,
-    int ksteps, NormIn norm_in) {
+    int ksteps, NormIn norm_in, int ucols) {
   static_assert(PACK == 1 || MB == 1, "a packed tile holds at most 8 rows of A");
   static_assert(PACK == 1 || !HALF, "a tile is packed or half empty, not both");
   __shared__ float red[SK_WAVES][32][MB * 16 + 1];
@@ -524,8 +524,10 @@ __global__ __launch_bounds__(SK_THREADS) void qkv_rope_skinny_kernel(
   constexpr int GROUPS = SK_WAVES / KS;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r = lane & 15, g = lane >> 4;
   const int grp = wave / KS, ks = wave % KS;
-  const int half = hd >> 1, upq = half / CP;            // units per q or k head
-  const int upv = hd / (2 * CP);                        // units per v head
+  // a unit's two tiles hold `ucols` (<= CP) columns each: fewer than a tile's where that spreads the product over more
+  // compute units (the lanes of the other columns load nothing)
+  const int half = hd >> 1, upq = half / ucols;         // units per q or k head
+  const int upv = hd / (2 * ucols);                     // units per v head
   const int qk_units = (nh + nkv) * upq, units = qk_units + nkv * upv;
   const int unit = blockIdx.x * GROUPS + grp;
   const bool unit_ok = unit < units;
@@ -533,18 +535,18 @@ __global__ __launch_bounds__(SK_THREADS) void qkv_rope_skinny_kernel(
   int row0 = 0, row1 = 0;
   if (unit_ok) {
     if (unit < qk_units) {
-      row0 = (unit / upq) * hd + (unit % upq) * CP;
+      row0 = (unit / upq) * hd + (unit % upq) * ucols;
       row1 = row0 + half;
     } else {
       const int u = unit - qk_units;
-      row0 = (nh + nkv) * hd + u * 2 * CP;
-      row1 = row0 + CP;
+      row0 = (nh + nkv) * hd + u * 2 * ucols;
+      row1 = row0 + ucols;
     }
   }
   const KRange<PACK> kr(ks * PACK, P::seg(r), ksteps, KS * PACK, K);
   const int shift = kr.shift;
   const int wrow = HALF ? (r & 7) : P::col(r);
-  const bool lane_ok = unit_ok && (!HALF || r < 8);
+  const bool lane_ok = unit_ok && (!HALF || r < 8) && wrow < ucols;
   const bf16_t* wp[2] = {W + (int64_t)(row0 + wrow) * K + shift, W + (int64_t)(row1 + wrow) * K + shift};
   const bool wok[2] = {lane_ok, lane_ok};
   const bf16_t* ap[MB];
@@ -564,7 +566,7 @@ __global__ __launch_bounds__(SK_THREADS) void qkv_rope_skinny_kernel(
 #pragma unroll
   for (int it = 0; it < ITEMS; ++it) {
     const int idx = threadIdx.x + it * SK_THREADS;
-    const int nl = idx % CP, rest = idx / CP;
+    const int nl = idx % ucols, rest = idx / ucols;
     const int gi = rest % GROUPS, m = rest / GROUPS;
     const int u = blockIdx.x * GROUPS + gi;
     e_slot[it] = -1;
@@ -573,7 +575,7 @@ __global__ __launch_bounds__(SK_THREADS) void qkv_rope_skinny_kernel(
     if (m < M && u < units) {
       if (write_kv) e_slot[it] = slot_mapping[m];
       if (u < qk_units) {
-        const int head = u / upq, j = (u % upq) * CP + nl;
+        const int head = u / upq, j = (u % upq) * ucols + nl;
         const int p = positions[m];
         e_cos[it] = cos_t[(int64_t)p * half + j];
         e_sin[it] = sin_t[(int64_t)p * half + j];
@@ -583,9 +585,9 @@ __global__ __launch_bounds__(SK_THREADS) void qkv_rope_skinny_kernel(
         }
       } else if (bias) {
         const int v = u - qk_units;
-        const int at = (nh + nkv + v / upv) * hd + (v % upv) * 2 * CP + nl;
+        const int at = (nh + nkv + v / upv) * hd + (v % upv) * 2 * ucols + nl;
         e_blo[it] = bf16_to_f32(bias[at]);
-        e_bhi[it] = bf16_to_f32(bias[at + CP]);
+        e_bhi[it] = bf16_to_f32(bias[at + ucols]);
       }
     }
   }
@@ -609,7 +611,7 @@ __global__ __launch_bounds__(SK_THREADS) void qkv_rope_skinny_kernel(
 #pragma unroll
   for (int it = 0; it < ITEMS; ++it) {
     const int idx = threadIdx.x + it * SK_THREADS;
-    const int nl = idx % CP, rest = idx / CP;
+    const int nl = idx % ucols, rest = idx / ucols;
     const int gi = rest % GROUPS, m = rest / GROUPS;
     const int u = blockIdx.x * GROUPS + gi;
     if (m >= M || u >= units) continue;
@@ -632,7 +634,7 @@ __global__ __launch_bounds__(SK_THREADS) void qkv_rope_skinny_kernel(
     int64_t page = 0, off = 0;
     if (slot >= 0) slot_page(slot, page_size, page, off);
     if (u < qk_units) {
-      const int head = u / upq, j = (u % upq) * CP + nl;
+      const int head = u / upq, j = (u % upq) * ucols + nl;
       const float c = e_cos[it], sn = e_sin[it];
       const bf16_t olo = f32_to_bf16(lo * c - hi * sn), ohi = f32_to_bf16(lo * sn + hi * c);
       if (head < nh) {
@@ -646,10 +648,10 @@ __global__ __launch_bounds__(SK_THREADS) void qkv_rope_skinny_kernel(
       }
     } else if (slot >= 0) {
       const int v = u - qk_units;
-      const int gh = v / upv, d = (v % upv) * 2 * CP + nl;
+      const int gh = v / upv, d = (v % upv) * 2 * ucols + nl;
       bf16_t* o = v_pages + ((page * nkv + gh) * (int64_t)hd + d) * page_size + off;
       o[0] = f32_to_bf16(lo);
-      o[(int64_t)CP * page_size] = f32_to_bf16(hi);
+      o[(int64_t)ucols * page_size] = f32_to_bf16(hi);
     }
   }
 }
@@ -658,6 +660,7 @@ __global__ __launch_bounds__(SK_THREADS) void qkv_rope_skinny_kernel(
 // positions int32 [M]; cos_t, sin_t float [positions, hd/2]; slot_mapping int64 [M] (-1: no cache write);
 // k_pages [pages, nkv, page_size, hd], v_pages [pages, nkv, hd, page_size].  norm: null, or the sums of the
 // norm whose (h * g) the rows of A are (its in_ fields only).  pack: 0 (the library chooses), 1 or 2.
+#define GA_QKV_SPREAD_BELOW 192
 extern "C" int ga_qkv_rope_skinny(void* q_out, const void* A, int64_t lda, const void* W, const void* bias,
                                   const void* positions, const void* cos_t, const void* sin_t,
                                   const void* slot_mapping, void* k_pages, void* v_pages, int M, int K, int nh,
@@ -678,14 +681,19 @@ extern "C" int ga_qkv_rope_skinny(void* q_out, const void* A, int64_t lda, const
   // with more than 8 rows and so few columns that full tiles leave most of the chip idle: half tiles (measured on
   // MI355X: 64 rows 11.4 us against 15.9 with 64 workgroups of full tiles; with 144 of them, slower)
   const bool half_tiles = pack == 1 && M > 8 && (nh + 2 * nkv) * hd / 32 < 128;
-  const int units = (nh + 2 * nkv) * hd / (2 * (half_tiles ? 8 : 16 / pack));
+  // columns of a unit's tile: all of a tile's, or half of them where a packed tile's 8 would leave the product on fewer
+  // than GA_QKV_SPREAD_BELOW workgroups (2,048 columns of a K of 1,536 at 8 rows: 128 workgroups of 8 + 8 columns
+  // 7.15 us in a decode step, 256 of 4 + 4 see the measurement beside the macro)
+  int ucols = half_tiles ? 8 : 16 / pack;
+  if (pack == 2 && (nh + 2 * nkv) * hd / (2 * ucols) < GA_QKV_SPREAD_BELOW && (hd / 2) % (ucols / 2) == 0) ucols /= 2;
+  const int units = (nh + 2 * nkv) * hd / (2 * ucols);
   const int ksteps = (K + 63) / 64;
   dim3 grid((units + groups - 1) / groups), block(SK_THREADS);
 #define LAUNCH(MB, PK, HF)                                                                                \
   hipLaunchKernelGGL((qkv_rope_skinny_kernel<MB, 8, PK, HF>), grid, block, 0, stream, (bf16_t*)q_out,    \
                      (const bf16_t*)A, lda, (const bf16_t*)W, (const bf16_t*)bias, (const int32_t*)positions, \
                      (const float*)cos_t, (const float*)sin_t, (const int64_t*)slot_mapping, (bf16_t*)k_pages, \
-                     (bf16_t*)v_pages, M, K, nh, nkv, hd, page_size, write_kv, ksteps, norm_in)
+                     (bf16_t*)v_pages, M, K, nh, nkv, hd, page_size, write_kv, ksteps, norm_in, ucols)
   switch (mb) {
     case 1:
       if (pack == 2) LAUNCH(1, 2, false); else if (half_tiles) LAUNCH(1, 1, true); else LAUNCH(1, 1, false);
