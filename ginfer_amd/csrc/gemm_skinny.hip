@@ -299,55 +299,63 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(TC* __restrict_
 // added exactly as above, so the results are the same bits.  How many columns a workgroup should own is a trade: every
 // workgroup reads all rows of A (as much as M / 2 of its columns' weights), while more, smaller workgroups keep more
 // loads on their way; the launcher's rule states what was measured.
-template <int NT, typename TC>
-__global__ __launch_bounds__(SK_THREADS) void gemm_gated_even_kernel(TC* __restrict__ C, int64_t ldc,
-                                                                     const bf16_t* __restrict__ A, int64_t lda,
-                                                                     const bf16_t* __restrict__ W, int M, int N, int K,
-                                                                     int ksteps, NormIn norm_in) {
-  __shared__ float red[SK_WAVES][2 * NT * 16][16 + 1];
+// The same dealing serves a plain product of many columns (the head): TILES tiles of 16 columns of W a workgroup, the
+// bias added to the sums.  GATED: the first half of the tiles is the gate's, the second the up matrix's.
+template <int TILES, typename TC, bool GATED>
+__global__ __launch_bounds__(SK_THREADS) void gemm_even_kernel(TC* __restrict__ C, int64_t ldc,
+                                                               const bf16_t* __restrict__ A, int64_t lda,
+                                                               const bf16_t* __restrict__ W,
+                                                               const bf16_t* __restrict__ bias, int M, int N, int K,
+                                                               int ksteps, NormIn norm_in) {
+  static_assert(!GATED || TILES % 2 == 0, "as many tiles of the gate as of the up matrix");
+  constexpr int PER = GATED ? TILES / 2 : TILES;             // tiles of one matrix
+  __shared__ float red[SK_WAVES][TILES * 16][16 + 1];
   __shared__ float rstd[16];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r = lane & 15, g = lane >> 4;
   const int c0 = (int)(((int64_t)blockIdx.x * N) / gridDim.x), c1 = (int)(((int64_t)(blockIdx.x + 1) * N) / gridDim.x);
-  const int cols = c1 - c0;                                  // <= NT * 16 by the launcher's choice of the grid
+  const int cols = c1 - c0;                                  // <= PER * 16 by the launcher's choice of the grid
   const KRange<1> kr(wave, 0, ksteps, SK_WAVES, K);
-  const bf16_t* wp[2 * NT];
-  bool wok[2 * NT];
+  const bf16_t* wp[TILES];
+  bool wok[TILES];
 #pragma unroll
-  for (int t = 0; t < 2 * NT; ++t) {
-    const int cl = (t % NT) * 16 + r;                        // the lane's column within the workgroup's range
+  for (int t = 0; t < TILES; ++t) {
+    const int cl = (t % PER) * 16 + r;                       // the lane's column within the workgroup's range
     wok[t] = cl < cols;
-    wp[t] = W + ((int64_t)(wok[t] ? c0 + cl : 0) + (t >= NT ? (int64_t)N : 0)) * K + kr.shift;
+    wp[t] = W + ((int64_t)(wok[t] ? c0 + cl : 0) + (GATED && t >= PER ? (int64_t)N : 0)) * K + kr.shift;
   }
   const bf16_t* ap[1];
   bool aok[1];
   aok[0] = r < M;
   ap[0] = A + (int64_t)(aok[0] ? r : 0) * lda + kr.shift;
-  f32x4 acc[2 * NT][1];
+  f32x4 acc[TILES][1];
 #pragma unroll
-  for (int t = 0; t < 2 * NT; ++t) acc[t][0] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int t = 0; t < TILES; ++t) acc[t][0] = f32x4{0.f, 0.f, 0.f, 0.f};
   NormInLoads in_loads;
   in_loads.load(norm_in, M, wave, lane);
   // steps of K asked for at once: fewer with more tiles, whose loads fill the registers
-  skinny_accumulate<2 * NT, 1, (NT == 1 ? 4 : NT == 2 ? 2 : 1)>(acc, wp, wok, ap, aok, 0, kr.kend, kr.ke, g);
+  skinny_accumulate<TILES, 1, (TILES <= 2 ? 4 : TILES <= 4 ? 2 : 1)>(acc, wp, wok, ap, aok, 0, kr.kend, kr.ke, g);
   in_loads.finish(norm_in, rstd, M, wave, lane);
 #pragma unroll
-  for (int t = 0; t < 2 * NT; ++t)
+  for (int t = 0; t < TILES; ++t)
 #pragma unroll
     for (int i = 0; i < 4; ++i) red[wave][t * 16 + g * 4 + i][r] = acc[t][0][i];
   __syncthreads();
   const bool scale_rows = norm_in.sumsq != nullptr;
   for (int idx = threadIdx.x; idx < cols * M; idx += SK_THREADS) {
     const int cl = idx % cols, m = idx / cols;
-    float v = 0.f, u = 0.f;
+    float v = 0.f;
 #pragma unroll
     for (int w = 0; w < SK_WAVES; ++w) v += red[w][cl][m];            // in wavefront order, as in the kernel above
+    if (scale_rows) v *= rstd[m];
+    if (GATED) {
+      float u = 0.f;
 #pragma unroll
-    for (int w = 0; w < SK_WAVES; ++w) u += red[w][NT * 16 + cl][m];
-    if (scale_rows) {
-      v *= rstd[m];
-      u *= rstd[m];
+      for (int w = 0; w < SK_WAVES; ++w) u += red[w][PER * 16 + cl][m];
+      if (scale_rows) u *= rstd[m];
+      v = (v * (1.0f / (1.0f + expf(-v)))) * u;
+    } else if (bias) {
+      v += bf16_to_f32(bias[c0 + cl]);
     }
-    v = (v * (1.0f / (1.0f + expf(-v)))) * u;
     Num<TC>::st(C + (int64_t)m * ldc + c0 + cl, v);
   }
 }
@@ -378,6 +386,20 @@ static int auto_pack(int M, int workgroups_of_full_tiles) {
 // 9.2 -> 7.2 (10), 10.0 -> 8.0 (19); 11,008 x 2,048: 22.7 -> 18.9 (11), 24.8 -> 23.3 (11), 27.2 -> 26.7 (43);
 // 18,944 x 3,584: 57.4 -> 51.0 (13), 63.1 -> 60.3 (25), 71.7 -> 63.5 (37); 13,824 x 5,120: 63.9 -> 54.8 (11),
 // 71.6 -> 63.6 (27), 82.3 -> 68.7 (27); 29,568 x 8,192: 183 -> 169 (12), 200 -> 191 (29), 234 -> 206 (29).
+// The plain product of up to 16 rows and at least this many columns (the head) is dealt the same way, to workgroups of
+// up to 6 tiles; 0: the kernel above keeps it.  Its thousands of small workgroups are even enough by their number, so
+// less is gained: measured on MI355X at 151,936 x 1,536 with 32-bit sums out, in us, before -> after (columns a
+// workgroup) at 1, 8 and 16 rows: 92.5 -> 86.0 (25), 109.9 -> 106.9 (75), 129.4 -> 113.5 (75); 152,064 x 3,584:
+// 186 -> 183 (16), 237 -> 227 (85), 298 -> 240 (85); 152,064 x 8,192: 410 and 410 (16), 486 -> 481 (60), 625 -> 515 (85).
+#define GA_PLAIN_EVEN_MIN_COLUMNS 16384
+static int plain_even_workgroups(int M, int N, int K) {
+  if (M <= 4 && K > 2048) return 0;
+  const int target = M <= 4 ? 24 : 80;
+  int rounds = (N + GA_FOLD_TARGET * target / 2) / (GA_FOLD_TARGET * target);
+  if (rounds < 1) rounds = 1;
+  while ((N + GA_FOLD_TARGET * rounds - 1) / (GA_FOLD_TARGET * rounds) > 96) ++rounds;
+  return GA_FOLD_TARGET * rounds;
+}
 static int gated_even_workgroups(int M, int N, int K) {
   const int target = M <= 4 ? 12 : M <= 8 ? (K <= 2048 ? 12 : 28) : 32;
   int rounds = (N + GA_FOLD_TARGET * target / 2) / (GA_FOLD_TARGET * target);
@@ -434,19 +456,24 @@ extern "C" int ga_gemm_skinny(void* C, int64_t ldc, const void* A, int64_t lda, 
   const int groups = SK_WAVES / ks;
   if (pack == 0) pack = (grid_splits == 1 && !gated) ? auto_pack(M, (N + groups * nt * 16 - 1) / (groups * nt * 16)) : 1;
   if (pack != 1 && (pack != 2 || M > 8)) return -2;
-  if (gated && mb == 1 && pack == 1 && N >= GA_GATED_EVEN_MIN_COLUMNS) {
-    const int workgroups = gated_even_workgroups(M, N, K);
-    const int most = (N + workgroups - 1) / workgroups, tiles = (most + 15) / 16;
+  const bool plain_even = !gated && grid_splits == 1 && !norm_out.residual && ks == SK_WAVES &&
+                          N >= GA_PLAIN_EVEN_MIN_COLUMNS && plain_even_workgroups(M, N, K) > 0;
+  if (mb == 1 && pack == 1 && ((gated && N >= GA_GATED_EVEN_MIN_COLUMNS) || plain_even)) {
+    const int workgroups = gated ? gated_even_workgroups(M, N, K) : plain_even_workgroups(M, N, K);
+    const int most = (N + workgroups - 1) / workgroups, per = (most + 15) / 16;      // tiles of one matrix
     const int ksteps = (K + 63) / 64;
     dim3 grid(workgroups), block(SK_THREADS);
-#define LAUNCH_EVEN(NT, TC)                                                                                  \
-  hipLaunchKernelGGL((gemm_gated_even_kernel<NT, TC>), grid, block, 0, stream, (TC*)C, ldc, (const bf16_t*)A, \
-                     lda, (const bf16_t*)W, M, N, K, ksteps, norm_in)
-    if (out_f32) {
-      if (tiles == 1) LAUNCH_EVEN(1, float); else if (tiles == 2) LAUNCH_EVEN(2, float); else LAUNCH_EVEN(3, float);
-    } else {
-      if (tiles == 1) LAUNCH_EVEN(1, bf16_t); else if (tiles == 2) LAUNCH_EVEN(2, bf16_t); else LAUNCH_EVEN(3, bf16_t);
-    }
+#define LAUNCH_EVEN(TILES, TC, G)                                                                              \
+  hipLaunchKernelGGL((gemm_even_kernel<TILES, TC, G>), grid, block, 0, stream, (TC*)C, ldc, (const bf16_t*)A, \
+                     lda, (const bf16_t*)W, (const bf16_t*)bias, M, N, K, ksteps, norm_in)
+#define PICK_EVEN(TC)                                                                                          \
+  if (gated) {                                                                                                 \
+    if (per == 1) LAUNCH_EVEN(2, TC, true); else if (per == 2) LAUNCH_EVEN(4, TC, true); else LAUNCH_EVEN(6, TC, true); \
+  } else {                                                                                                     \
+    if (per <= 2) LAUNCH_EVEN(2, TC, false); else if (per <= 4) LAUNCH_EVEN(4, TC, false); else LAUNCH_EVEN(6, TC, false); \
+  }
+    if (out_f32) { PICK_EVEN(float) } else { PICK_EVEN(bf16_t) }
+#undef PICK_EVEN
 #undef LAUNCH_EVEN
     return GA_CHECK_LAUNCH();
   }

@@ -760,7 +760,9 @@ def test_paged_attention_mfma_finds_one_far_key(where, wide, monkeypatch):
 
 @pytest.mark.parametrize("M", [1, 2, 8, 16, 17, 33, 64])
 @pytest.mark.parametrize("N,K,bias", [(2048, 1536, True), (1536, 1536, False), (17920, 1536, False), (1536, 8960, False),
-                                      (1000, 192, True), (197, 4216, False), (33, 8, True), (777, 88, False), (5000, 72, True)])
+                                      (1000, 192, True), (197, 4216, False), (33, 8, True), (777, 88, False), (5000, 72, True),
+                                      # from 16,384 columns on, up to 16 rows: dealt evenly to a multiple of 256 workgroups
+                                      (20000, 72, True), (40010, 40, True), (16390, 200, False)])
 def test_gemm_skinny(M, N, K, bias):
     from ginfer_amd.kernels import ops
     a, w = rnd((M, K), torch.bfloat16, 30), rnd((N, K), torch.bfloat16, 31)
