@@ -7,9 +7,12 @@ the layer sizes of a 1.5B and a 7B model; a model of other sizes may want others
     TUNING.library_from_rows = 32                       # for the process
     GINFER_AMD_TUNING='{"library_from_rows": 32}'       # or from the environment, as JSON
 
-No part or dispatcher holds such a number of its own.  What the kernels fix when they are compiled is not in this table:
-the wavefronts of an attention workgroup (`PREFILL_WAVES`, `DEC_WAVES`), how late the running maximum of the softmax
-is raised (`LAZY_MAX`) and the like are macros at the top of the source that uses them, each with its measurement.
+No part or dispatcher in Python holds such a number of its own.  What the kernels fix when they are compiled is not in
+this table: the wavefronts of an attention workgroup (`PREFILL_WAVES`, `DEC_WAVES`), how late the running maximum of the
+softmax is raised (`LAZY_MAX`) and the like are macros at the top of the source that uses them, each with its
+measurement; and how a launcher lays ONE kernel over the chip for the sizes it is given (packed tiles, the columns a
+workgroup owns where a product is dealt evenly to the compute units: `auto_pack`, `fold_cols`, `gated_even_workgroups`
+in csrc/gemm_skinny.hip) is a rule in that source, beside the figures it was measured with.
 """
 import json
 import os
