@@ -33,6 +33,12 @@ int ga_add_rmsnorm(void* out, void* residual, const void* delta, int delta_parts
 int ga_rope_kv_write(void* qkv, const void* positions, const void* cos_t, const void* sin_t, const void* slot_mapping,
                      void* k_pages, void* v_pages, int tokens, int nh, int nkv, int hd, int rotary_dim, int page_size,
                      int write_kv, int is_bf16, hipStream_t stream);
+// the same on 32-bit partial sums of the projection, parts [n_parts][tokens][(nh + 2 nkv) hd] added in order, then the bias
+// (bfloat16 or null): q to q_out [tokens][nh hd] in bfloat16, k and v into the pages
+int ga_rope_kv_from_parts(void* q_out, const void* parts, int n_parts, const void* bias, const void* positions,
+                          const void* cos_t, const void* sin_t, const void* slot_mapping, void* k_pages, void* v_pages,
+                          int tokens, int nh, int nkv, int hd, int rotary_dim, int page_size, int write_kv,
+                          hipStream_t stream);
 
 // ---- gemm.hip: C [M, N] = A [M, K] . W [N, K]^T + bias in true 32-bit: the matrix cores' 32-bit instructions (and plain FMA
 // for 33 to 64 rows of very wide products), every element one accumulator over ascending k: the same bits whichever

@@ -245,3 +245,121 @@ extern "C" int ga_rope_kv_write(void* qkv, const void* positions, const void* co
                        rotary_dim, page_size, write_kv);
   return GA_CHECK_LAUNCH();
 }
+
+// The same epilogue on a projection that arrives as 32-bit partial sums of a product whose K was split over workgroups
+// (parts [n_parts][tokens][(nh + 2 nkv) hd]): the parts are added in ascending order, the bias in 32-bit, q and k are
+// rotated on the 32-bit sums (one rounding fewer than rotating the rounded projection), q goes to q_out
+// [tokens][nh hd] in bfloat16, k and v straight into the pages.  A workgroup takes one token and one of
+// FROM_PARTS_CHUNKS shares of its items (an item: 4 consecutive pairs (j, j + half) of a q or k head, 4 elements of an
+// unrotated tail, or 4 elements of a v head), so that few tokens still make workgroups enough.
+#define FROM_PARTS_CHUNKS 2
+#define FROM_PARTS_MOST 8            // parts at most: their loads are all asked for before the first is added
+__global__ __launch_bounds__(256) void rope_kv_from_parts_kernel(
+    bf16_t* __restrict__ q_out, const float* __restrict__ parts, int n_parts, const bf16_t* __restrict__ bias,
+    const int32_t* __restrict__ positions, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+    const int64_t* __restrict__ slot_mapping, bf16_t* __restrict__ k_pages, bf16_t* __restrict__ v_pages, int nh, int nkv,
+    int hd, int rotary_dim, int page_size, int write_kv, int tokens) {
+  constexpr int V = 4;
+  const int64_t t = blockIdx.x;
+  const int half = rotary_dim >> 1;
+  const int rot_chunks = half / V, tail_chunks = (hd - rotary_dim) / V, v_chunks = hd / V;
+  const int per_head = rot_chunks + tail_chunks;
+  const int qk_items = (nh + nkv) * per_head;
+  const int total = qk_items + nkv * v_chunks;
+  const int width = (nh + 2 * nkv) * hd;
+  const int p = positions[t];
+  const float* c = cos_t + (int64_t)p * half;
+  const float* s = sin_t + (int64_t)p * half;
+  const int64_t part_stride = (int64_t)tokens * width;
+  const float* row = parts + t * (int64_t)width;
+  int64_t page = -1, off = 0;
+  if (write_kv) {
+    const int64_t slot = slot_mapping[t];
+    if (slot >= 0) slot_page(slot, page_size, page, off);
+  }
+  // the parts' four values of column `at`, all asked for at once (n_parts is the same for every lane)
+  auto ask = [&](float4 (&v)[FROM_PARTS_MOST], int at) {
+#pragma unroll
+    for (int q = 0; q < FROM_PARTS_MOST; ++q)
+      if (q < n_parts) v[q] = *reinterpret_cast<const float4*>(row + q * part_stride + at);
+  };
+  // ... added in ascending order, then the bias
+  auto add_up = [&](float (&x)[V], const float4 (&v)[FROM_PARTS_MOST], int at) {
+    x[0] = x[1] = x[2] = x[3] = 0.f;
+#pragma unroll
+    for (int q = 0; q < FROM_PARTS_MOST; ++q)
+      if (q < n_parts) {
+        x[0] += v[q].x; x[1] += v[q].y; x[2] += v[q].z; x[3] += v[q].w;
+      }
+    if (bias) {
+      union { uint2 u; bf16_t e[V]; } bv;
+      bv.u = *reinterpret_cast<const uint2*>(bias + at);
+#pragma unroll
+      for (int i = 0; i < V; ++i) x[i] += bf16_to_f32(bv.e[i]);
+    }
+  };
+  for (int item = blockIdx.y * blockDim.x + threadIdx.x; item < total; item += gridDim.y * blockDim.x) {
+    if (item < qk_items) {
+      const int head = item / per_head, ch = item % per_head;
+      bf16_t* dst = head < nh ? q_out + t * (int64_t)nh * hd + (int64_t)head * hd
+                              : (page >= 0 ? k_pages + ((page * nkv + (head - nh)) * page_size + off) * hd : nullptr);
+      if (!dst) continue;
+      if (ch < rot_chunks) {
+        const int j = ch * V;
+        float4 plo[FROM_PARTS_MOST], phi[FROM_PARTS_MOST];
+        ask(plo, head * hd + j);
+        ask(phi, head * hd + j + half);
+        const float4 cv = *reinterpret_cast<const float4*>(c + j), sv = *reinterpret_cast<const float4*>(s + j);
+        float lo[V], hi[V];
+        add_up(lo, plo, head * hd + j);
+        add_up(hi, phi, head * hd + j + half);
+        const float ce[V] = {cv.x, cv.y, cv.z, cv.w}, se[V] = {sv.x, sv.y, sv.z, sv.w};
+        union { uint2 u; bf16_t e[V]; } olo, ohi;
+#pragma unroll
+        for (int i = 0; i < V; ++i) {
+          olo.e[i] = f32_to_bf16(lo[i] * ce[i] - hi[i] * se[i]);
+          ohi.e[i] = f32_to_bf16(lo[i] * se[i] + hi[i] * ce[i]);
+        }
+        *reinterpret_cast<uint2*>(dst + j) = olo.u;
+        *reinterpret_cast<uint2*>(dst + j + half) = ohi.u;
+      } else {
+        const int j = rotary_dim + (ch - rot_chunks) * V;
+        float4 px[FROM_PARTS_MOST];
+        ask(px, head * hd + j);
+        float x[V];
+        add_up(x, px, head * hd + j);
+        union { uint2 u; bf16_t e[V]; } o;
+#pragma unroll
+        for (int i = 0; i < V; ++i) o.e[i] = f32_to_bf16(x[i]);
+        *reinterpret_cast<uint2*>(dst + j) = o.u;
+      }
+    } else if (page >= 0) {
+      const int vi = item - qk_items;
+      const int g = vi / v_chunks, j = (vi % v_chunks) * V;
+      float4 px[FROM_PARTS_MOST];
+      ask(px, (nh + nkv + g) * hd + j);
+      float x[V];
+      add_up(x, px, (nh + nkv + g) * hd + j);
+      bf16_t* dst = v_pages + ((page * nkv + g) * (int64_t)hd + j) * page_size + off;
+#pragma unroll
+      for (int i = 0; i < V; ++i) dst[(int64_t)i * page_size] = f32_to_bf16(x[i]);
+    }
+  }
+}
+
+// parts float [n_parts][tokens][(nh + 2 nkv) hd]; bias bfloat16 [(nh + 2 nkv) hd] or null; q_out bfloat16 [tokens][nh hd];
+// the rest as ga_rope_kv_write.  rotary_dim / 2, head_dim - rotary_dim and head_dim multiples of 4; at most 8 parts.
+extern "C" int ga_rope_kv_from_parts(void* q_out, const void* parts, int n_parts, const void* bias,
+                                     const void* positions, const void* cos_t, const void* sin_t,
+                                     const void* slot_mapping, void* k_pages, void* v_pages, int tokens, int nh, int nkv,
+                                     int hd, int rotary_dim, int page_size, int write_kv, hipStream_t stream) {
+  if (tokens <= 0) return 0;
+  if (n_parts < 1 || n_parts > FROM_PARTS_MOST || nh <= 0 || nkv <= 0) return -1;
+  if ((rotary_dim / 2) % 4 || (hd - rotary_dim) % 4 || hd % 4 || rotary_dim <= 0 || rotary_dim > hd) return -2;
+  dim3 grid(tokens, FROM_PARTS_CHUNKS), block(256);
+  hipLaunchKernelGGL(rope_kv_from_parts_kernel, grid, block, 0, stream, (bf16_t*)q_out, (const float*)parts, n_parts,
+                     (const bf16_t*)bias, (const int32_t*)positions, (const float*)cos_t, (const float*)sin_t,
+                     (const int64_t*)slot_mapping, (bf16_t*)k_pages, (bf16_t*)v_pages, nh, nkv, hd, rotary_dim, page_size,
+                     write_kv, tokens);
+  return GA_CHECK_LAUNCH();
+}

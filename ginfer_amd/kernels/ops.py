@@ -179,6 +179,44 @@ def rope_kv_write(qkv, positions, cos, sin, slot_mapping, k_pages, v_pages, num_
                                 _i(_is_bf16(qkv.dtype)), _stream()), "rope_kv_write")
 
 
+def rope_kv_from_parts(parts, bias, positions, cos, sin, slot_mapping, k_pages, v_pages, num_heads, num_kv_heads, head_dim,
+                       write_kv=True):
+    """The epilogue of a q|k|v projection that arrives as float32 partial sums [parts, T, (nh + 2 nkv) hd] of a product
+    whose K was split over workgroups: the parts added in order, the bias (bfloat16 [width] or None), q and k rotated on
+    the 32-bit sums; returns q [T, nh*hd] in bfloat16 and writes k and v into the paged cache at slot_mapping."""
+    _dev(parts, bias, positions, cos, sin, slot_mapping, k_pages, v_pages)
+    width = (num_heads + 2 * num_kv_heads) * head_dim
+    _need(parts.dtype == torch.float32 and parts.dim() == 3 and parts.shape[2] == width and parts.is_contiguous(),
+          "parts must be contiguous float32 [parts, T, %d]",
+          width)
+    T = parts.shape[1]
+    _need(positions.dtype == torch.int32 and positions.shape == (T,) and positions.is_contiguous(),
+          "positions must be contiguous int32 [T]")
+    _need(cos.dtype == torch.float32 and sin.dtype == torch.float32 and cos.shape == sin.shape and cos.dim() == 2
+          and cos.is_contiguous() and sin.is_contiguous(), "cos and sin must be contiguous float32 [P, rotary_dim/2]")
+    rotary_dim = 2 * cos.shape[1]
+    _need(0 < rotary_dim <= head_dim and (rotary_dim // 2) % 4 == 0 and (head_dim - rotary_dim) % 4 == 0 and head_dim % 4 == 0,
+          "this kernel takes rotary_dim / 2, head_dim - rotary_dim and head_dim in multiples of 4; got %d of %d",
+          rotary_dim, head_dim)
+    _need(1 <= parts.shape[0] <= 8, "this kernel adds up to 8 parts, got %d", parts.shape[0])
+    if bias is not None:
+        _need(bias.dtype == torch.bfloat16 and bias.shape == (width,) and bias.is_contiguous(),
+              "qkv bias must be bfloat16 [%d]",
+              width)
+    page_size = 1
+    if write_kv:
+        _need(slot_mapping is not None and slot_mapping.dtype == torch.int64 and slot_mapping.shape == (T,)
+              and slot_mapping.is_contiguous(), "slot_mapping must be contiguous int64 [T]")
+        page_size = _check_pages(k_pages, v_pages, torch.bfloat16, num_kv_heads, head_dim)
+    q = torch.empty((T, num_heads * head_dim), dtype=torch.bfloat16, device=parts.device)
+    lib = build.load("rope_kv")
+    _check(lib.ga_rope_kv_from_parts(_ptr(q), _ptr(parts), _i(parts.shape[0]), _ptr(bias), _ptr(positions), _ptr(cos),
+                                     _ptr(sin), _ptr(slot_mapping), _ptr(k_pages), _ptr(v_pages), _i(T), _i(num_heads),
+                                     _i(num_kv_heads), _i(head_dim), _i(rotary_dim), _i(page_size),
+                                     _i(1 if write_kv else 0), _stream()), "rope_kv_from_parts")
+    return q
+
+
 def _check_pages(k_pages, v_pages, dtype, nkv, hd):
     """k_pages [pages, nkv, page_size, hd], v_pages [pages, nkv, hd, page_size] (values transposed)."""
     _need(k_pages is not None and v_pages is not None, "cache pages are missing")

@@ -82,6 +82,13 @@ class Tuning:
     # of at least that, the library's product followed by the rotation kernel is faster (the fused kernel cannot split K).
     fused_qkv_up_to_rows: int = 16
     fused_qkv_unless_in_features: int = 3072
+    # With a shorter K than that, from this many rows on the product goes to the weight-streaming kernel with K split over
+    # workgroups, into K // `qkv_in_parts_min_k` parts (at most `qkv_in_parts_most`), which the rotation kernel adds up
+    # (2,048 columns of a K of 1,536 in a decode step of 64 rows: the fused kernel 13.6 us, product 6.7 + rotation over the
+    # parts 5.9; decode at batch 64 18,340 -> 18,450 tok/s, at batch 48 15,760 -> 15,900).
+    qkv_in_parts_from_rows: int = 48
+    qkv_in_parts_min_k: int = 384
+    qkv_in_parts_most: int = 4
     # ---- attention on the matrix cores (kernels/ops.py)
     decode_target_workgroups: int = 256      # key splits are chosen so that a decode step makes about this many workgroups
     decode_min_split_keys: int = 128         # one tile of 32 keys for each wavefront of a workgroup

@@ -19,6 +19,23 @@ def _library_then_rotation_is_faster(rows, in_features):
     return rows > TUNING.fused_qkv_up_to_rows and in_features >= TUNING.fused_qkv_unless_in_features
 
 
+def _projection_in_parts(x, w_qkv, head_dim, rotary_dim):
+    """Into how many parts of K the q|k|v product of these rows is split, its parts to be added by the rotation kernel;
+    0: not this way.  The fused kernel cannot split K, and each of its workgroups reads all rows of x, which from some
+    48 rows on is most of what it reads.  Measured on MI355X in a decode step of 64 rows (2,048 columns of a K of 1,536):
+    the fused kernel 13.6 us, the product in four parts 6.7 + the rotation kernel over them 5.9; with fewer rows the fused
+    kernel's time falls faster than the pair's (32 rows: 9.2 us)."""
+    if isinstance(x, ops.ScaledRows) or x.dtype != torch.bfloat16:
+        return 0
+    rows, K = x.shape
+    if not (TUNING.qkv_in_parts_from_rows <= rows <= ops.SKINNY_MAX_ROWS) or K >= TUNING.fused_qkv_unless_in_features:
+        return 0
+    if not ops.gemm_skinny_supported(x, w_qkv) or (rotary_dim // 2) % 4 or (head_dim - rotary_dim) % 4 or head_dim % 4:
+        return 0
+    parts = min(TUNING.qkv_in_parts_most, 8, K // TUNING.qkv_in_parts_min_k)
+    return parts if parts >= 2 else 0
+
+
 @register_mixer("attention")
 class Attention(Part):
     """q/k/v projections (one fused product over the stacked weights; results equal the three separate
@@ -78,7 +95,14 @@ class Attention(Part):
         """into_norm = (residual, norm): where the output projection's kernel can, the result is added to the
         residual here and the rows of `norm` come back as ops.ScaledRows; else the result comes back as ever."""
         cos, sin = self.position.tables()
-        if (ops.qkv_rope_skinny_supported(x, self.w_qkv, self.hd, self.position.rotary_dim)
+        parts = _projection_in_parts(x, self.w_qkv, self.hd, self.position.rotary_dim)
+        if parts:
+            # a decode step of many rows: the product with K split over workgroups (every workgroup then reads a share
+            # of the rows only), its 32-bit parts added up by the kernel that rotates and writes the cache
+            sums = ops.gemm_skinny(x, self.w_qkv, None, out_dtype=torch.float32, nt=2, grid_splits=parts)
+            qkv = ops.rope_kv_from_parts(sums, self.b_qkv, step.positions, cos, sin, cache.slot_mapping, cache.k_pages,
+                                         cache.v_pages, self.nh, self.nkv, self.hd, write_kv=cache.owner)
+        elif (ops.qkv_rope_skinny_supported(x, self.w_qkv, self.hd, self.position.rotary_dim)
                 and not _library_then_rotation_is_faster(x.shape[0], x.shape[1])):
             # few rows (decode): projection, rotation and cache write in one kernel
             qkv = ops.qkv_rope_skinny(x, self.w_qkv, self.b_qkv, step.positions, cos, sin, cache.slot_mapping,

@@ -909,6 +909,50 @@ def test_folded_norm_refuses_what_it_cannot_take():
         ops.gemm_skinny(a, w, into_norm=(res, gain, 1e-6))
 
 
+@pytest.mark.parametrize("M,parts", [(1, 1), (7, 3), (48, 4), (64, 2)])
+@pytest.mark.parametrize("nh,nkv,hd,rd,theta,bias", [(12, 2, 128, 128, 1e4, True), (5, 1, 96, 96, 5e5, False), (4, 4, 64, 32, 1e4, True),
+                                                     (3, 3, 48, 16, 1e6, True)])
+@pytest.mark.parametrize("ps", [8, 12])
+def test_rope_kv_from_parts(M, parts, nh, nkv, hd, rd, theta, bias, ps):
+    """The rotation kernel on 32-bit partial sums of the projection: parts added in order, bias, rotation of q and k
+    (a rotation of part of the head too), q out, k and v into their pages; nothing else touched."""
+    from ginfer_amd.kernels import ops
+    pages = 40
+    width = (nh + 2 * nkv) * hd
+    p = rnd((parts, M, width), torch.float32, 70)
+    b = rnd((width,), torch.bfloat16, 71) if bias else None
+    positions = torch.randint(0, 300, (M,), dtype=torch.int32, device=dev())
+    sin, cos = pm.rope_tables(theta, rd, 300)
+    slots = torch.randperm(pages * ps)[:M].to(torch.int64)
+    if M > 1:
+        slots[1] = -1
+    kp, vp = rnd((pages, nkv, ps, hd), torch.bfloat16, 63), rnd((pages, nkv, hd, ps), torch.bfloat16, 64)
+    kp0, vp0 = kp.clone().cpu(), vp.clone().cpu()
+    q = ops.rope_kv_from_parts(p, b, positions, cos.to(dev()), sin.to(dev()), slots.to(dev()), kp, vp, nh, nkv, hd)
+    assert q.dtype == torch.bfloat16 and q.shape == (M, nh * hd)
+    y = p.double().cpu().sum(0) + (b.double().cpu() if bias else 0)
+    pos = positions.cpu().tolist()
+    qr = pm.apply_rope(y[:, :nh * hd].view(M, nh, hd), pos, sin.double(), cos.double()).reshape(M, -1)
+    kr = pm.apply_rope(y[:, nh * hd:(nh + nkv) * hd].view(M, nkv, hd), pos, sin.double(), cos.double())
+    v = y[:, (nh + nkv) * hd:].view(M, nkv, hd)
+    close(q, qr, 1e-2)
+    kpc, vpc = kp.float().cpu(), vp.float().cpu()
+    touched_k, touched_v = torch.zeros_like(kpc, dtype=torch.bool), torch.zeros_like(vpc, dtype=torch.bool)
+    for t in range(M):
+        s = int(slots[t])
+        if s < 0:
+            continue
+        close(kpc[s // ps, :, s % ps, :], kr[t], 1e-2)
+        close(vpc[s // ps, :, :, s % ps], v[t], 1e-2)
+        touched_k[s // ps, :, s % ps, :] = True
+        touched_v[s // ps, :, :, s % ps] = True
+    assert torch.equal(kp.cpu()[~touched_k], kp0[~touched_k]) and torch.equal(vp.cpu()[~touched_v], vp0[~touched_v])
+    kp1, vp1 = kp0.clone().to(dev()), vp0.clone().to(dev())
+    q2 = ops.rope_kv_from_parts(p, b, positions, cos.to(dev()), sin.to(dev()), slots.to(dev()), kp1, vp1, nh, nkv, hd,
+                                write_kv=False)
+    assert torch.equal(q2, q) and torch.equal(kp1.cpu(), kp0) and torch.equal(vp1.cpu(), vp0)
+
+
 @pytest.mark.parametrize("M,pack", [(1, 1), (1, 2), (5, 2), (8, 1), (8, 2), (12, 1), (33, 1), (64, 1)])
 @pytest.mark.parametrize("nh,nkv,hd,K,theta", [(12, 2, 128, 1536, 1e4), (6, 1, 32, 192, 1e6), (4, 4, 64, 88, 1e4), (5, 1, 96, 72, 5e5),
                                                (28, 4, 128, 72, 1e4)])     # the last: so many columns that tiles stay full
